@@ -1,0 +1,208 @@
+/* C ABI of libmtrt_hip.so — the MI355X (gfx950) replacement for the executor
+ * runtime's CUDA kernel-launch layer plus the hand-written kernel clusters that
+ * stand in for the reference's generated PTX.
+ *
+ * Part 1 keeps the reference's symbol names, argument order and argument widths,
+ * so host code emitted by the reference compiler for its C backend links against
+ * this library unchanged; handles are opaque pointers (the reference's CUmodule,
+ * CUfunction, CUstream and cudaEvent_t are pointers too).  Where the reference
+ * takes PTX text these entry points take a gfx950 code object (the output of
+ * `hipcc --genco --offload-arch=gfx950`, bundled or bare): there is no JIT step.
+ * As in the reference, every failure in part 1 is fatal: the message is printed
+ * to stderr as "<file>#<line>: <text>" and the process aborts
+ * (mlir-tensorrt/executor/lib/Runtime/Backend/C/CUDAModule.cpp:27-53).
+ *
+ * Part 2 is the cluster layer: one entry point per kernel cluster of the
+ * quantization hot path.  The reference has no such functions — its compiler
+ * picks a grid and block for each generated kernel and emits a
+ * get-function + launch pair (mlir-tensorrt/compiler/lib/Passes/1_Core/KernelToCUDA/
+ * KernelToCUDA.cpp:151-186); these entry points are that emitted code written by
+ * hand for the hand-written kernels: they validate shapes and alignment, pick the
+ * kernel variant and launch shape for gfx950, build the void** argument array in
+ * the reference's device ABI (bare pointers, 64-bit sizes, scalars by value:
+ * mlir-tensorrt/kernel/lib/Kernel/Transforms/ExpandMemRefArgs.cpp:65-120) and go
+ * through the same module / function / launch path as part 1.  They return a
+ * status (0 = ok, codes as mlir-tensorrt/executor/lib/Runtime/StandaloneCPP/
+ * MTRTRuntimeStatus.h:31-41) and leave a message for mtrt_hip_last_error().
+ * All pointers are device pointers unless stated; nothing is synchronised: work
+ * is enqueued on `stream` (NULL = the default stream).
+ */
+#ifndef MTRT_HIP_H
+#define MTRT_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#define MTRT_CAPI_EXPORTED __attribute__((visibility("default")))
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct mtrt_opaque_module *mtrt_module_t;     /* hipModule_t   (reference: CUmodule)    */
+typedef struct mtrt_opaque_function *mtrt_function_t; /* hipFunction_t (reference: CUfunction)  */
+typedef struct mtrt_opaque_stream *mtrt_stream_t;     /* hipStream_t   (reference: CUstream)    */
+typedef struct mtrt_opaque_event *mtrt_event_t;       /* hipEvent_t    (reference: cudaEvent_t) */
+
+/* ------------------------------------------------------------------------- */
+/* Part 1 — launch ABI, same names as the reference C backend                  */
+/* (mlir-tensorrt/executor/lib/Runtime/Backend/C/CUDAModule.h:55-123)          */
+/* ------------------------------------------------------------------------- */
+
+/* CUDAModule.h:55-59 */
+MTRT_CAPI_EXPORTED int32_t mtrt_cuda_get_active_device(void);
+MTRT_CAPI_EXPORTED int32_t mtrt_cuda_set_active_device(int32_t device);
+MTRT_CAPI_EXPORTED int32_t mtrt_cuda_get_device(int32_t device);
+
+/* CUDAModule.h:61-65.  The reference header declares stream_create without a
+ * parameter while its LLVM lowering passes an i32 device
+ * (mlir-tensorrt/compiler/lib/Passes/2_Host/HostToLLVM/CUDAToLLVM/CUDAToLLVM.cpp:67-68);
+ * under the SysV x86-64 ABI an ignored integer argument is harmless, so the
+ * header form is kept. */
+MTRT_CAPI_EXPORTED mtrt_stream_t mtrt_cuda_stream_create(void);
+MTRT_CAPI_EXPORTED void mtrt_cuda_stream_destroy(mtrt_stream_t stream);
+MTRT_CAPI_EXPORTED void mtrt_cuda_stream_sync(mtrt_stream_t stream);
+
+/* CUDAModule.h:71-85 */
+MTRT_CAPI_EXPORTED mtrt_event_t mtrt_cuda_event_create(int32_t device);
+MTRT_CAPI_EXPORTED void mtrt_cuda_event_release(mtrt_event_t event);
+MTRT_CAPI_EXPORTED void mtrt_cuda_stream_record_event(mtrt_stream_t stream, mtrt_event_t event);
+MTRT_CAPI_EXPORTED void mtrt_cuda_stream_wait_event(mtrt_stream_t stream, mtrt_event_t event);
+MTRT_CAPI_EXPORTED void mtrt_cuda_event_sync(mtrt_event_t event);
+MTRT_CAPI_EXPORTED float mtrt_cuda_event_elapsed_msec(mtrt_event_t start, mtrt_event_t end);
+
+/* CUDAModule.h:87-96.  Pinned or managed requests return host-coherent memory
+ * (the reference returns cudaMallocManaged memory for both); device requests
+ * are stream-ordered allocations. */
+MTRT_CAPI_EXPORTED void *mtrt_cuda_alloc_async(mtrt_stream_t stream, int64_t size, int32_t alignment,
+                                               int8_t isHostPinned, int8_t isManaged);
+MTRT_CAPI_EXPORTED void mtrt_cuda_memcpy_async(mtrt_stream_t stream, void *src, void *dest,
+                                               int64_t size);
+MTRT_CAPI_EXPORTED void mtrt_cuda_free(mtrt_stream_t stream, void *ptr, int8_t isHostPinned,
+                                       int8_t isManaged);
+
+/* CUDAModule.h:98-102.  `ptxData`/`ptxLen` hold a gfx950 code object, not PTX. */
+MTRT_CAPI_EXPORTED mtrt_module_t mtrt_cuda_module_load_from_ptx(const char *ptxData, size_t ptxLen);
+MTRT_CAPI_EXPORTED mtrt_module_t mtrt_cuda_module_load_from_ptx_file(const char *filename,
+                                                                     size_t filenameLength);
+/* CUDAModule.h:104 */
+MTRT_CAPI_EXPORTED void mtrt_cuda_module_unload(mtrt_module_t module);
+/* CUDAModule.h:106-108.  `name` is NOT NUL-terminated; `length` bytes are used. */
+MTRT_CAPI_EXPORTED mtrt_function_t mtrt_cuda_module_get_function(mtrt_module_t module,
+                                                                 const char *name, int64_t length);
+/* CUDAModule.h:110-115.  args[i] points at the storage of the i-th kernel
+ * operand (the driver's kernelParams convention); valid only during the call. */
+MTRT_CAPI_EXPORTED void mtrt_cuda_launch_kernel(mtrt_function_t func, int32_t gridX, int32_t gridY,
+                                                int32_t gridZ, int32_t blockX, int32_t blockY,
+                                                int32_t blockZ, int32_t dynamicSharedMemory,
+                                                mtrt_stream_t stream, void **args);
+/* CUDAModule.h:117-119 */
+MTRT_CAPI_EXPORTED int32_t mtrt_cuda_get_current_device(void);
+MTRT_CAPI_EXPORTED int32_t mtrt_cuda_get_program_device(int32_t logicalId);
+
+/* ------------------------------------------------------------------------- */
+/* Part 2 — kernel clusters of the quantization hot path                       */
+/* ------------------------------------------------------------------------- */
+
+/* element types */
+enum mtrt_hip_dtype {
+  MTRT_F32 = 0,
+  MTRT_F16 = 1,
+  MTRT_BF16 = 2,
+  MTRT_I8 = 3,
+  MTRT_F8E4M3FN = 4,
+  MTRT_I4 = 5,        /* one int4 per byte, low nibble: the executor's host/buffer storage
+                         (mlir-tensorrt/executor/lib/Runtime/Backend/Common/DataTypes.cpp:494-519) */
+  MTRT_I4_PACKED = 6  /* two per byte, element 2i in the low nibble: what the reference hands to
+                         TensorRT (mlir-tensorrt/tensorrt/lib/Target/TensorRTEncodingOpInterface/
+                         NetworkEncoder.cpp:552-595) */
+};
+
+/* how `scale` is addressed; the data tensor is viewed as row-major [d0, d1] */
+enum mtrt_hip_scale_kind {
+  MTRT_SCALE_UNIFORM = 0, /* per-tensor: scale[0]; `nb` ignored                             */
+  MTRT_SCALE_ROW = 1,     /* scale[row % nb]: per-channel on a non-last axis (d0 = outer*C,
+                             nb = C) or blocks along the last axis (d1 = block, nb = d0)    */
+  MTRT_SCALE_COL = 2      /* scale[(row / nb) * d1 + col]: per-channel on the last axis
+                             (nb = d0) or blocks of nb rows along axis 0                    */
+};
+
+enum mtrt_hip_flags {
+  MTRT_Q_ROUND_TO_INT = 1, /* f8 target: apply round_nearest_even before the clamp, the form
+                              StablehloRaiseQDQ.cpp:233-265 matches; integer targets always round */
+  MTRT_F8_REFHOST = 2      /* f8 target: reproduce the reference HOST class bit for bit
+                              (DataTypes.cpp:43-122) instead of IEEE RNE + saturate           */
+};
+
+/* status codes, MTRTRuntimeStatus.h:31-41 */
+enum mtrt_hip_status {
+  MTRT_OK = 0,
+  MTRT_INVALID_ARGUMENT = 1,
+  MTRT_NOT_FOUND = 2,
+  MTRT_IO_ERROR = 3,
+  MTRT_DRIVER_ERROR = 4,
+  MTRT_RUNTIME_ERROR = 5,
+  MTRT_INTERNAL_ERROR = 7,
+  MTRT_UNIMPLEMENTED = 8
+};
+
+/* Thread-local message of the most recent failed part-2 call on this thread
+ * (MTRTRuntimeStatus.h:48-53 convention); "" if none. */
+MTRT_CAPI_EXPORTED const char *mtrt_hip_last_error(void);
+
+/* Loads the built-in kernel module on the current device (idempotent; every
+ * part-2 entry point does it on first use).  Fails with MTRT_RUNTIME_ERROR when
+ * there is no usable gfx950 device: there is no CPU fallback. */
+MTRT_CAPI_EXPORTED int32_t mtrt_hip_init(void);
+/* The built-in module, for callers that launch its kernels themselves through
+ * mtrt_cuda_module_get_function + mtrt_cuda_launch_kernel.  NULL on failure. */
+MTRT_CAPI_EXPORTED mtrt_module_t mtrt_hip_builtin_module(void);
+/* The code object bytes of the built-in module (what a reference executable
+ * would carry in the data segment that holds PTX today:
+ * mlir-tensorrt/compiler/lib/Passes/2_Host/HostToExecutor/CUDAToExecutor/CUDAToExecutor.cpp:858-866). */
+MTRT_CAPI_EXPORTED const char *mtrt_hip_builtin_code_object(size_t *size);
+
+/* {abs, reduce-max} cluster + scale = amax / qmax (one f32 divide).
+ * Either output may be NULL.  Replaces the generated reduction kernel of
+ * mlir-tensorrt/kernel/lib/Kernel/TransformSchedules/FallbackSchedule.cpp:147-343. */
+MTRT_CAPI_EXPORTED int32_t mtrt_hip_amax(mtrt_stream_t stream, const void *x, int32_t dtype,
+                                         int64_t n, float qmax, float *amax_out, float *scale_out);
+
+/* tensorrt.quantize semantics (TensorRTOps.td:3133-3194) in the StableHLO form
+ * of StablehloRaiseQDQ.cpp:233-265: q = convert(clamp(lo, rne(f32(x) / scale), hi)).
+ * x_dtype in {F32,F16,BF16}; q_dtype in {I8,F8E4M3FN,I4,I4_PACKED}; scale is f32. */
+MTRT_CAPI_EXPORTED int32_t mtrt_hip_quantize(mtrt_stream_t stream, const void *x, int32_t x_dtype,
+                                             void *q, int32_t q_dtype, const float *scale,
+                                             int32_t scale_kind, int64_t d0, int64_t d1, int64_t nb,
+                                             int32_t flags);
+/* tensorrt.dequantize semantics (TensorRTOps.td:3408-3445; StablehloRaiseQDQ.cpp:407-418):
+ * y = narrow(f32(q) * scale). */
+MTRT_CAPI_EXPORTED int32_t mtrt_hip_dequantize(mtrt_stream_t stream, const void *q, int32_t q_dtype,
+                                               void *y, int32_t y_dtype, const float *scale,
+                                               int32_t scale_kind, int64_t d0, int64_t d1,
+                                               int64_t nb);
+/* quantize followed by dequantize in one pass over x (the fake-quant pair of
+ * tripy/nvtripy/frontend/module/linear.py:112-151); writes q and y (same type as x). */
+MTRT_CAPI_EXPORTED int32_t mtrt_hip_quantize_dequantize(mtrt_stream_t stream, const void *x,
+                                                        int32_t x_dtype, void *q, int32_t q_dtype,
+                                                        void *y, const float *scale,
+                                                        int32_t scale_kind, int64_t d0, int64_t d1,
+                                                        int64_t nb, int32_t flags);
+
+/* LayerNorm over the last dimension, one launch
+ * (RaiseNormalizations.pdll:277-308; TensorRTOps.td:1303-1373); x, gamma, beta, y share dtype. */
+MTRT_CAPI_EXPORTED int32_t mtrt_hip_layernorm(mtrt_stream_t stream, const void *x, const void *gamma,
+                                              const void *beta, void *y, int32_t dtype, int64_t rows,
+                                              int64_t d, float eps);
+/* softmax over the last dimension, one launch (StablehloMatchers.cpp:311-335; TensorRTOps.td:1769-1796) */
+MTRT_CAPI_EXPORTED int32_t mtrt_hip_softmax(mtrt_stream_t stream, const void *x, void *y,
+                                            int32_t dtype, int64_t rows, int64_t d);
+
+/* Name of the kernel that the most recent successful part-2 call on this thread
+ * launched last (for profiles and tests). */
+MTRT_CAPI_EXPORTED const char *mtrt_hip_last_kernel(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MTRT_HIP_H */

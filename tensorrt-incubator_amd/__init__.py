@@ -1,0 +1,202 @@
+"""Host-side Python access to libmtrt_hip.so (ctypes, no torch types cross the ABI).
+
+The directory name carries a hyphen, so the package is loaded by path under the
+module name `tensorrt_incubator_amd` (see `__graft_entry__.load_package`).
+
+torch is used only to own device memory and streams: every wrapper below passes
+raw device pointers, extents and the current stream handle to the C ABI declared
+in include/mtrt_hip.h.  There is no fallback: if the shared library is missing or
+no gfx950 device is usable, the calls raise.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_DIR = os.path.join(_HERE, "lib")
+LIB_PATH = os.path.join(LIB_DIR, "libmtrt_hip.so")
+KERNEL_MODULE_PATH = os.path.join(LIB_DIR, "mtrt_kernels.hsaco")
+FIXTURE_MODULE_PATH = os.path.join(LIB_DIR, "mtrt_test_fixtures.hsaco")
+
+# enum mtrt_hip_dtype
+F32, F16, BF16, I8, F8E4M3FN, I4, I4_PACKED = range(7)
+# enum mtrt_hip_scale_kind
+SCALE_UNIFORM, SCALE_ROW, SCALE_COL = range(3)
+# enum mtrt_hip_flags
+Q_ROUND_TO_INT = 1
+F8_REFHOST = 2
+
+_c = ctypes
+_vp, _i32, _i64, _f32, _sz, _i8 = _c.c_void_p, _c.c_int32, _c.c_int64, _c.c_float, _c.c_size_t, _c.c_int8
+
+# name -> (restype, argtypes); mirrors include/mtrt_hip.h one to one
+PROTOTYPES = {
+    "mtrt_cuda_get_active_device": (_i32, []),
+    "mtrt_cuda_set_active_device": (_i32, [_i32]),
+    "mtrt_cuda_get_device": (_i32, [_i32]),
+    "mtrt_cuda_stream_create": (_vp, []),
+    "mtrt_cuda_stream_destroy": (None, [_vp]),
+    "mtrt_cuda_stream_sync": (None, [_vp]),
+    "mtrt_cuda_event_create": (_vp, [_i32]),
+    "mtrt_cuda_event_release": (None, [_vp]),
+    "mtrt_cuda_stream_record_event": (None, [_vp, _vp]),
+    "mtrt_cuda_stream_wait_event": (None, [_vp, _vp]),
+    "mtrt_cuda_event_sync": (None, [_vp]),
+    "mtrt_cuda_event_elapsed_msec": (_f32, [_vp, _vp]),
+    "mtrt_cuda_alloc_async": (_vp, [_vp, _i64, _i32, _i8, _i8]),
+    "mtrt_cuda_memcpy_async": (None, [_vp, _vp, _vp, _i64]),
+    "mtrt_cuda_free": (None, [_vp, _vp, _i8, _i8]),
+    "mtrt_cuda_module_load_from_ptx": (_vp, [_c.c_char_p, _sz]),
+    "mtrt_cuda_module_load_from_ptx_file": (_vp, [_c.c_char_p, _sz]),
+    "mtrt_cuda_module_unload": (None, [_vp]),
+    "mtrt_cuda_module_get_function": (_vp, [_vp, _c.c_char_p, _i64]),
+    "mtrt_cuda_launch_kernel": (None, [_vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp, _c.POINTER(_vp)]),
+    "mtrt_cuda_get_current_device": (_i32, []),
+    "mtrt_cuda_get_program_device": (_i32, [_i32]),
+    "mtrt_hip_last_error": (_c.c_char_p, []),
+    "mtrt_hip_last_kernel": (_c.c_char_p, []),
+    "mtrt_hip_init": (_i32, []),
+    "mtrt_hip_builtin_module": (_vp, []),
+    "mtrt_hip_builtin_code_object": (_vp, [_c.POINTER(_sz)]),
+    "mtrt_hip_amax": (_i32, [_vp, _vp, _i32, _i64, _f32, _vp, _vp]),
+    "mtrt_hip_quantize": (_i32, [_vp, _vp, _i32, _vp, _i32, _vp, _i32, _i64, _i64, _i64, _i32]),
+    "mtrt_hip_dequantize": (_i32, [_vp, _vp, _i32, _vp, _i32, _vp, _i32, _i64, _i64, _i64]),
+    "mtrt_hip_quantize_dequantize": (_i32, [_vp, _vp, _i32, _vp, _i32, _vp, _vp, _i32, _i64, _i64, _i64, _i32]),
+    "mtrt_hip_layernorm": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i64, _i64, _f32]),
+    "mtrt_hip_softmax": (_i32, [_vp, _vp, _vp, _i32, _i64, _i64]),
+}
+
+_lib = None
+
+
+class MtrtHipError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__("mtrt_hip status %d: %s" % (code, message))
+        self.code = code
+        self.message = message
+
+
+def lib():
+    """The loaded C-ABI library with prototypes applied; raises if it is not built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "%s is missing: run `python tensorrt-incubator_amd/build.py` (there is no fallback path)" % LIB_PATH)
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in PROTOTYPES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def check(status):
+    if status != 0:
+        raise MtrtHipError(status, lib().mtrt_hip_last_error().decode())
+
+
+def last_kernel():
+    return lib().mtrt_hip_last_kernel().decode()
+
+
+# --------------------------------------------------------------------------
+# torch-tensor conveniences (device memory + stream plumbing only)
+# --------------------------------------------------------------------------
+
+def _torch():
+    import torch
+    return torch
+
+
+def float_dtype_of(t):
+    torch = _torch()
+    return {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}[t.dtype]
+
+
+def _stream():
+    return _torch().cuda.current_stream().cuda_stream
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def code_tensor(q_dtype, numel, device):
+    """Uninitialised storage for `numel` quantized codes (uint8/int8 bytes)."""
+    torch = _torch()
+    if q_dtype == I8:
+        return torch.empty(numel, dtype=torch.int8, device=device)
+    if q_dtype == I4_PACKED:
+        return torch.empty((numel + 1) // 2, dtype=torch.uint8, device=device)
+    return torch.empty(numel, dtype=torch.uint8, device=device)
+
+
+def amax(x, qmax):
+    """Returns (amax, scale) as two 0-d f32 device tensors; scale = amax / qmax."""
+    torch = _torch()
+    assert x.is_cuda and x.is_contiguous()
+    out = torch.empty(2, dtype=torch.float32, device=x.device)
+    check(lib().mtrt_hip_amax(_stream(), x.data_ptr(), float_dtype_of(x), x.numel(), float(qmax),
+                              out.data_ptr(), out.data_ptr() + 4))
+    return out[0], out[1]
+
+
+def quantize(x, scale, q_dtype, kind=SCALE_UNIFORM, d0=None, d1=None, nb=1, flags=0, out=None):
+    assert x.is_cuda and x.is_contiguous() and scale.is_cuda and scale.dtype == _torch().float32
+    d0, d1 = _view2d(x, d0, d1)
+    q = code_tensor(q_dtype, d0 * d1, x.device) if out is None else out
+    check(lib().mtrt_hip_quantize(_stream(), x.data_ptr(), float_dtype_of(x), q.data_ptr(), q_dtype,
+                                  scale.data_ptr(), kind, d0, d1, nb, flags))
+    return q
+
+
+def dequantize(q, scale, q_dtype, out_torch_dtype, shape, kind=SCALE_UNIFORM, d0=None, d1=None, nb=1, out=None):
+    torch = _torch()
+    assert q.is_cuda and q.is_contiguous() and scale.dtype == torch.float32
+    y = torch.empty(shape, dtype=out_torch_dtype, device=q.device) if out is None else out
+    d0, d1 = _view2d(y, d0, d1)
+    check(lib().mtrt_hip_dequantize(_stream(), q.data_ptr(), q_dtype, y.data_ptr(), float_dtype_of(y),
+                                    scale.data_ptr(), kind, d0, d1, nb))
+    return y
+
+
+def quantize_dequantize(x, scale, q_dtype, kind=SCALE_UNIFORM, d0=None, d1=None, nb=1, flags=0, q_out=None, y_out=None):
+    torch = _torch()
+    assert x.is_cuda and x.is_contiguous() and scale.dtype == torch.float32
+    d0, d1 = _view2d(x, d0, d1)
+    q = code_tensor(q_dtype, d0 * d1, x.device) if q_out is None else q_out
+    y = torch.empty_like(x) if y_out is None else y_out
+    check(lib().mtrt_hip_quantize_dequantize(_stream(), x.data_ptr(), float_dtype_of(x), q.data_ptr(), q_dtype,
+                                             y.data_ptr(), scale.data_ptr(), kind, d0, d1, nb, flags))
+    return q, y
+
+
+def layernorm(x, gamma, beta, eps, out=None):
+    torch = _torch()
+    assert x.is_cuda and x.is_contiguous() and gamma.dtype == x.dtype and beta.dtype == x.dtype
+    d = x.shape[-1]
+    rows = x.numel() // d if d else 0
+    y = torch.empty_like(x) if out is None else out
+    check(lib().mtrt_hip_layernorm(_stream(), x.data_ptr(), gamma.data_ptr(), beta.data_ptr(), y.data_ptr(),
+                                   float_dtype_of(x), rows, d, float(eps)))
+    return y
+
+
+def softmax(x, out=None):
+    torch = _torch()
+    assert x.is_cuda and x.is_contiguous()
+    d = x.shape[-1]
+    rows = x.numel() // d if d else 0
+    y = torch.empty_like(x) if out is None else out
+    check(lib().mtrt_hip_softmax(_stream(), x.data_ptr(), y.data_ptr(), float_dtype_of(x), rows, d))
+    return y
+
+
+def _view2d(t, d0, d1):
+    if d0 is None or d1 is None:
+        if t.dim() == 0:
+            return 1, 1
+        d1 = t.shape[-1]
+        d0 = t.numel() // d1 if d1 else 0
+    return int(d0), int(d1)

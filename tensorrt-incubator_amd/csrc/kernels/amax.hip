@@ -1,0 +1,152 @@
+// amax cluster: amax = reduce_max(abs(f32(x))) over the whole tensor, plus the
+// host-sized follow-up op scale = amax / qmax folded into the same launch.
+//
+// Reference program: the {abs, reduce-max} codegen cluster that the kernel backend
+// forms for a dynamic-scale quantization
+//   mlir-tensorrt/compiler/lib/Backends/Kernel/KernelBackend.cpp:52-83
+//   mlir-tensorrt/compiler/lib/Backends/Kernel/KernelSegmentation.cpp:53-113
+// and scale = amax / maxbound as in tripy/examples/nanogpt/weight_loader.py:67-68.
+// The reference's generated reduction has every thread walk a whole row serially
+// (mlir-tensorrt/kernel/lib/Utils/TilingUtils.cpp:669-677); here the tensor is
+// streamed once with 128-bit loads by a grid sized to the chip, reduced per wave
+// with cross-lane exchanges, per workgroup through LDS, and across workgroups with
+// one device-scope atomic max per workgroup.  max is exact under any order, so the
+// result is bit-identical to the sequential host reduction.
+//
+// abs/max run on the BIT PATTERN: for non-NaN floats, |x| orders like the unsigned
+// integer (bits & 0x7fffffff), so v_and + v_max_u32 replace fabs + fmax and the
+// bf16/f16 inputs need no conversion in the loop.  A NaN input yields a NaN amax
+// (its pattern is the largest), unlike the host's std::max which would drop it
+// (CoreModule.cpp:540-551); the programs this serves are NaN-free.
+//
+// scratch: two 32-bit words owned by the caller's stream (running max, arrival
+// ticket), both zero on entry; the last workgroup to arrive publishes the results
+// and restores the zeros, so back-to-back launches on one stream need no memset.
+#include "common.hpp"
+
+using namespace mtrt_dev;
+
+namespace amax_cluster {
+
+constexpr int kAmaxThreads = 256;
+constexpr int kAmaxUnroll = 4;     // 128-bit loads in flight per lane per step
+
+template <typename X> struct AbsBits;
+template <> struct AbsBits<F32> {  // returns max over the 4 floats, as f32 bit pattern
+  static __device__ __forceinline__ uint32_t of(u32x4 t) {
+    uint32_t a = t.x & 0x7FFFFFFFu, b = t.y & 0x7FFFFFFFu, c = t.z & 0x7FFFFFFFu, d = t.w & 0x7FFFFFFFu;
+    a = a > b ? a : b; c = c > d ? c : d;
+    return a > c ? a : c;
+  }
+  static __device__ __forceinline__ uint32_t one(const float* p) { return f32_to_bits(*p) & 0x7FFFFFFFu; }
+  static __device__ __forceinline__ float finish(uint32_t m) { return bits_to_f32(m); }
+  static constexpr int kPerVec = 4;
+};
+template <> struct AbsBits<BF16> { // 8 bf16 per vector; result kept as f32 bit pattern (bf16 << 16)
+  static __device__ __forceinline__ uint32_t of(u32x4 t) {
+    uint32_t m = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t lo = (t[j] << 16) & 0x7FFF0000u, hi = t[j] & 0x7FFF0000u;
+      m = m > lo ? m : lo; m = m > hi ? m : hi;
+    }
+    return m;
+  }
+  static __device__ __forceinline__ uint32_t one(const uint16_t* p) { return (uint32_t(*p) << 16) & 0x7FFF0000u; }
+  static __device__ __forceinline__ float finish(uint32_t m) { return bits_to_f32(m); }
+  static constexpr int kPerVec = 8;
+};
+template <> struct AbsBits<F16> {  // 8 f16 per vector; result kept as f16 bit pattern
+  static __device__ __forceinline__ uint32_t of(u32x4 t) {
+    uint32_t m = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t lo = t[j] & 0x7FFFu, hi = (t[j] >> 16) & 0x7FFFu;
+      m = m > lo ? m : lo; m = m > hi ? m : hi;
+    }
+    return m;
+  }
+  static __device__ __forceinline__ uint32_t one(const uint16_t* p) { return uint32_t(*p) & 0x7FFFu; }
+  static __device__ __forceinline__ float finish(uint32_t m) { return f16_bits_to_f32(m); }
+  static constexpr int kPerVec = 8;
+};
+
+template <typename X>
+__device__ __forceinline__ void amax_body(const typename X::storage* __restrict__ x, int64_t n, float qmax,
+                                          float* __restrict__ amax_out, float* __restrict__ scale_out,
+                                          uint32_t* __restrict__ scratch) {
+  using A = AbsBits<X>;
+  // Elements before the first 16-byte boundary ("head") and after the last full
+  // vector ("tail") are taken one per lane by workgroup 0; everything between is
+  // streamed as 128-bit vectors.
+  constexpr int kElemBytes = 16 / A::kPerVec;
+  int64_t head = int64_t((16u - uint32_t(reinterpret_cast<uintptr_t>(x) & 15u)) & 15u) / kElemBytes;
+  head = head < n ? head : n;
+  const int64_t nvec = (n - head) / A::kPerVec;
+  const u32x4* __restrict__ xv = reinterpret_cast<const u32x4*>(x + head);
+  const int64_t stride = int64_t(gridDim.x) * kAmaxThreads;
+  uint32_t m = 0;
+  int64_t i = int64_t(blockIdx.x) * kAmaxThreads + threadIdx.x;
+  // main loop: kAmaxUnroll independent 128-bit loads per lane per trip
+  for (; i + (kAmaxUnroll - 1) * stride < nvec; i += kAmaxUnroll * stride) {
+    u32x4 t[kAmaxUnroll];
+#pragma unroll
+    for (int u = 0; u < kAmaxUnroll; ++u) t[u] = __builtin_nontemporal_load(xv + i + u * stride);
+#pragma unroll
+    for (int u = 0; u < kAmaxUnroll; ++u) { const uint32_t a = A::of(t[u]); m = m > a ? m : a; }
+  }
+  for (; i < nvec; i += stride) { const uint32_t a = A::of(__builtin_nontemporal_load(xv + i)); m = m > a ? m : a; }
+  if (blockIdx.x == 0 && threadIdx.x < 2 * A::kPerVec) {
+    const int64_t tail0 = head + nvec * A::kPerVec;
+    const int64_t e = threadIdx.x < A::kPerVec ? int64_t(threadIdx.x) : tail0 + (threadIdx.x - A::kPerVec);
+    const bool live = threadIdx.x < A::kPerVec ? (e < head) : (e < n);
+    if (live) { const uint32_t a = A::one(x + e); m = m > a ? m : a; }
+  }
+
+  m = wave_reduce(m, MaxU32());
+  __shared__ uint32_t wave_max[kAmaxThreads / kWave];
+  const int wave = threadIdx.x / kWave;
+  if ((threadIdx.x & (kWave - 1)) == 0) wave_max[wave] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int w = 1; w < kAmaxThreads / kWave; ++w) m = m > wave_max[w] ? m : wave_max[w];
+    // Cross-workgroup step.  Device-scope atomics execute at the memory side, the
+    // one place all eight XCDs agree on, so no cache write-back or invalidate is
+    // needed (an acquire/release pair at device scope would flush and invalidate this
+    // XCD's L2 once per workgroup, which costs more than the reduction itself).
+    // Ordering is by completion: the max RETURNS its old value and the empty asm
+    // consumes it, so the wave waits for that value before it issues the ticket;
+    // every max is therefore performed before the ticket of the same workgroup, and
+    // all of them before the last ticket.
+    const uint32_t before = __hip_atomic_fetch_max(&scratch[0], m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __asm__ volatile("" ::"v"(before) : "memory");
+    const uint32_t ticket = __hip_atomic_fetch_add(&scratch[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (ticket == gridDim.x - 1) {
+      // read-modify-write, so the value comes from the memory side, not from a cache
+      const uint32_t total = __hip_atomic_fetch_max(&scratch[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const float amax = A::finish(total);
+      if (amax_out) *amax_out = amax;
+      if (scale_out) *scale_out = amax / qmax;         // one IEEE divide, as the host does it
+      __hip_atomic_exchange(&scratch[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_exchange(&scratch[1], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+}
+
+}  // namespace amax_cluster
+using namespace amax_cluster;
+
+// (x, n, qmax, amax_out, scale_out, scratch) ; x needs only its natural element alignment.
+extern "C" __global__ void __launch_bounds__(kAmaxThreads) mtrt_amax_f32(
+    const float* x, int64_t n, float qmax, float* amax_out, float* scale_out, uint32_t* scratch) {
+  amax_body<F32>(x, n, qmax, amax_out, scale_out, scratch);
+}
+extern "C" __global__ void __launch_bounds__(kAmaxThreads) mtrt_amax_bf16(
+    const uint16_t* x, int64_t n, float qmax, float* amax_out, float* scale_out, uint32_t* scratch) {
+  amax_body<BF16>(x, n, qmax, amax_out, scale_out, scratch);
+}
+extern "C" __global__ void __launch_bounds__(kAmaxThreads) mtrt_amax_f16(
+    const uint16_t* x, int64_t n, float qmax, float* amax_out, float* scale_out, uint32_t* scratch) {
+  amax_body<F16>(x, n, qmax, amax_out, scale_out, scratch);
+}

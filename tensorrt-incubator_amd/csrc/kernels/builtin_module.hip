@@ -1,0 +1,6 @@
+// The built-in kernel module: every cluster kernel in one gfx950 code object, so
+// the host side loads one module and resolves kernels by name.
+#include "amax.hip"
+#include "qdq.hip"
+#include "norm.hip"
+#include "util.hip"

@@ -1,0 +1,264 @@
+// Fused elementwise+reduce clusters over the last dimension: LayerNorm and softmax.
+//
+// LayerNorm (the decomposition the reference recognises,
+//   mlir-tensorrt/tensorrt/lib/TensorRT/Transforms/RaiseNormalizations.pdll:277-308;
+//   user API tripy/nvtripy/frontend/module/layernorm.py:30-70):
+//     xf = f32(x); mu = sum(xf)/D; d = xf - mu; var = sum(d*d)/D;
+//     y = narrow(((d * (1/sqrt(var + eps))) * f32(gamma)) + f32(beta))
+// softmax (mlir-tensorrt/compiler/lib/Dialect/StablehloExt/Utils/StablehloMatchers.cpp:311-335;
+//   tripy/nvtripy/frontend/ops/softmax.py:30-82):
+//     xf = f32(x); m = max(xf); e = exp(xf - m); s = sum(e); y = narrow(e / s)   [computed as e * (1/s)]
+//
+// The reference's code generator emits at least three (LayerNorm) or four (softmax)
+// kernels for these, each re-reading the tensor, with one thread walking a whole
+// row (mlir-tensorrt/kernel/lib/Utils/TilingUtils.cpp:669-677).  Here each row is
+// read from HBM exactly once: ONE WAVE OWNS ONE ROW, the row lives in that wave's
+// registers (NV 128-bit vectors per lane, lane l holding vectors l, l+64, ...: every
+// load instruction of the wave covers 1 KiB of contiguous HBM), and both row
+// reductions are cross-lane exchanges with no LDS and no barrier.  Rows that do not
+// fit that scheme (D not a multiple of the vector width, or D > 64*16 vectors) use
+// the workgroup-per-row "_any" kernels, which re-read the row from cache.
+//
+// All arithmetic is f32 with the operation order above; reductions are trees
+// rather than the host's left-to-right sums, which the float tolerance covers.
+#include "common.hpp"
+
+using namespace mtrt_dev;
+
+namespace norm_cluster {
+
+constexpr int kNormThreads = 256;
+constexpr int kRowsPerBlock = kNormThreads / kWave;
+
+template <typename X> struct Vec;     // one 128-bit vector <-> floats
+template <> struct Vec<F32> {
+  static constexpr int kElems = 4;
+  static __device__ __forceinline__ void unpack(u32x4 t, float* v) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = bits_to_f32(t[j]);
+  }
+  static __device__ __forceinline__ u32x4 pack(const float* v) {
+    u32x4 t;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) t[j] = f32_to_bits(v[j]);
+    return t;
+  }
+};
+template <> struct Vec<BF16> {
+  static constexpr int kElems = 8;
+  static __device__ __forceinline__ void unpack(u32x4 t, float* v) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { v[2 * j] = bits_to_f32(t[j] << 16); v[2 * j + 1] = bits_to_f32(t[j] & 0xFFFF0000u); }
+  }
+  static __device__ __forceinline__ u32x4 pack(const float* v) {
+    u32x4 t;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) t[j] = f32_to_bf16_bits(v[2 * j]) | (f32_to_bf16_bits(v[2 * j + 1]) << 16);
+    return t;
+  }
+};
+template <> struct Vec<F16> {
+  static constexpr int kElems = 8;
+  static __device__ __forceinline__ void unpack(u32x4 t, float* v) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { v[2 * j] = f16_bits_to_f32(t[j] & 0xFFFFu); v[2 * j + 1] = f16_bits_to_f32(t[j] >> 16); }
+  }
+  static __device__ __forceinline__ u32x4 pack(const float* v) {
+    u32x4 t;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) t[j] = f32_to_f16_bits(v[2 * j]) | (f32_to_f16_bits(v[2 * j + 1]) << 16);
+    return t;
+  }
+};
+
+// Load the wave's row into registers: NV vectors per lane, absent vectors zero/fill.
+template <typename X, int NV>
+__device__ __forceinline__ void load_row(const u32x4* __restrict__ row, int nvec, int lane, float fill,
+                                         float (&v)[NV * Vec<X>::kElems]) {
+  constexpr int E = Vec<X>::kElems;
+  u32x4 t[NV];
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int idx = lane + kWave * j;
+    if (idx < nvec) t[j] = __builtin_nontemporal_load(row + idx);
+  }
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int idx = lane + kWave * j;
+    if (idx < nvec) {
+      Vec<X>::unpack(t[j], &v[j * E]);
+    } else {
+#pragma unroll
+      for (int k = 0; k < E; ++k) v[j * E + k] = fill;
+    }
+  }
+}
+
+template <typename X, int NV>
+__device__ __forceinline__ void layernorm_rows(const typename X::storage* __restrict__ x,
+                                               const typename X::storage* __restrict__ gamma,
+                                               const typename X::storage* __restrict__ beta,
+                                               typename X::storage* __restrict__ y, int64_t rows, int64_t d, float eps) {
+  constexpr int E = Vec<X>::kElems;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t row = int64_t(blockIdx.x) * kRowsPerBlock + threadIdx.x / kWave;
+  if (row >= rows) return;                           // whole wave leaves together
+  const int nvec = int(d / E);
+  const u32x4* xr = reinterpret_cast<const u32x4*>(x + row * d);
+  float v[NV * E];
+  load_row<X, NV>(xr, nvec, lane, 0.0f, v);
+
+  const float fd = float(d);
+  float sum = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NV * E; ++i) sum = sum + v[i];
+  const float mu = wave_reduce(sum, SumF32()) / fd;
+  float sq = 0.0f;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const bool live = lane + kWave * j < nvec;
+#pragma unroll
+    for (int k = 0; k < E; ++k) {
+      const float dv = v[j * E + k] - mu;
+      v[j * E + k] = dv;
+      sq = sq + (live ? dv * dv : 0.0f);
+    }
+  }
+  const float var = wave_reduce(sq, SumF32()) / fd;
+  const float rstd = 1.0f / sqrtf(var + eps);
+
+  const u32x4* gv = reinterpret_cast<const u32x4*>(gamma);
+  const u32x4* bv = reinterpret_cast<const u32x4*>(beta);
+  u32x4* yr = reinterpret_cast<u32x4*>(y + row * d);
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int idx = lane + kWave * j;
+    if (idx < nvec) {
+      float g[E], b[E], o[E];
+      Vec<X>::unpack(gv[idx], g);
+      Vec<X>::unpack(bv[idx], b);
+#pragma unroll
+      for (int k = 0; k < E; ++k) o[k] = ((v[j * E + k] * rstd) * g[k]) + b[k];
+      __builtin_nontemporal_store(Vec<X>::pack(o), yr + idx);
+    }
+  }
+}
+
+template <typename X, int NV>
+__device__ __forceinline__ void softmax_rows(const typename X::storage* __restrict__ x, typename X::storage* __restrict__ y,
+                                             int64_t rows, int64_t d) {
+  constexpr int E = Vec<X>::kElems;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t row = int64_t(blockIdx.x) * kRowsPerBlock + threadIdx.x / kWave;
+  if (row >= rows) return;
+  const int nvec = int(d / E);
+  const u32x4* xr = reinterpret_cast<const u32x4*>(x + row * d);
+  float v[NV * E];
+  load_row<X, NV>(xr, nvec, lane, -INFINITY, v);
+
+  float mx = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < NV * E; ++i) mx = fmaxf(mx, v[i]);
+  mx = wave_reduce(mx, MaxF32());
+  float s = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NV * E; ++i) {
+    v[i] = __expf(v[i] - mx);                        // exp(-inf) = 0 for the fill lanes
+    s = s + v[i];
+  }
+  s = wave_reduce(s, SumF32());
+  // e / s as e * (1/s): one correctly rounded reciprocal per row instead of a
+  // divide per element; at most one f32 ulp from the quotient, far inside the
+  // float tolerance of this cluster.
+  const float inv = 1.0f / s;
+  u32x4* yr = reinterpret_cast<u32x4*>(y + row * d);
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int idx = lane + kWave * j;
+    if (idx < nvec) {
+      float o[E];
+#pragma unroll
+      for (int k = 0; k < E; ++k) o[k] = v[j * E + k] * inv;
+      __builtin_nontemporal_store(Vec<X>::pack(o), yr + idx);
+    }
+  }
+}
+
+// ---- any D, any alignment: one workgroup per row, row re-read from cache -------------
+template <typename Op>
+__device__ __forceinline__ float block_reduce(float v, Op op, float* lds) {
+  v = wave_reduce(v, op);
+  const int wave = threadIdx.x / kWave;
+  __syncthreads();                                   // lds may still be read from the previous round
+  if ((threadIdx.x & (kWave - 1)) == 0) lds[wave] = v;
+  __syncthreads();
+  float r = lds[0];
+#pragma unroll
+  for (int w = 1; w < kNormThreads / kWave; ++w) r = op(r, lds[w]);
+  return r;
+}
+
+template <typename X>
+__device__ __forceinline__ void layernorm_any(const typename X::storage* __restrict__ x,
+                                              const typename X::storage* __restrict__ gamma,
+                                              const typename X::storage* __restrict__ beta,
+                                              typename X::storage* __restrict__ y, int64_t rows, int64_t d, float eps) {
+  __shared__ float lds[kNormThreads / kWave];
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    const typename X::storage* xr = x + row * d;
+    float sum = 0.0f;
+    for (int64_t c = threadIdx.x; c < d; c += kNormThreads) sum = sum + Tile<X>::load1(xr + c);
+    const float mu = block_reduce(sum, SumF32(), lds) / float(d);
+    float sq = 0.0f;
+    for (int64_t c = threadIdx.x; c < d; c += kNormThreads) { const float dv = Tile<X>::load1(xr + c) - mu; sq = sq + dv * dv; }
+    const float var = block_reduce(sq, SumF32(), lds) / float(d);
+    const float rstd = 1.0f / sqrtf(var + eps);
+    for (int64_t c = threadIdx.x; c < d; c += kNormThreads) {
+      const float dv = Tile<X>::load1(xr + c) - mu;
+      Tile<X>::store1(y + row * d + c, ((dv * rstd) * Tile<X>::load1(gamma + c)) + Tile<X>::load1(beta + c));
+    }
+  }
+}
+
+template <typename X>
+__device__ __forceinline__ void softmax_any(const typename X::storage* __restrict__ x, typename X::storage* __restrict__ y,
+                                            int64_t rows, int64_t d) {
+  __shared__ float lds[kNormThreads / kWave];
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    const typename X::storage* xr = x + row * d;
+    float mx = -INFINITY;
+    for (int64_t c = threadIdx.x; c < d; c += kNormThreads) mx = fmaxf(mx, Tile<X>::load1(xr + c));
+    mx = block_reduce(mx, MaxF32(), lds);
+    float s = 0.0f;
+    for (int64_t c = threadIdx.x; c < d; c += kNormThreads) s = s + __expf(Tile<X>::load1(xr + c) - mx);
+    s = block_reduce(s, SumF32(), lds);
+    const float inv = 1.0f / s;
+    for (int64_t c = threadIdx.x; c < d; c += kNormThreads)
+      Tile<X>::store1(y + row * d + c, __expf(Tile<X>::load1(xr + c) - mx) * inv);
+  }
+}
+
+}  // namespace norm_cluster
+using namespace norm_cluster;
+
+// Entry points.  mtrt_layernorm_<t>_v<NV>(x, gamma, beta, y, rows, d, eps)
+//                mtrt_softmax_<t>_v<NV>(x, y, rows, d)         NV = vectors per lane
+#define MTRT_NORM_KERNELS(XN, XT, NV)                                                                         \
+  extern "C" __global__ void __launch_bounds__(kNormThreads) mtrt_layernorm_##XN##_v##NV(                      \
+      const XT::storage* x, const XT::storage* gamma, const XT::storage* beta, XT::storage* y, int64_t rows,  \
+      int64_t d, float eps) { layernorm_rows<XT, NV>(x, gamma, beta, y, rows, d, eps); }                      \
+  extern "C" __global__ void __launch_bounds__(kNormThreads) mtrt_softmax_##XN##_v##NV(                        \
+      const XT::storage* x, XT::storage* y, int64_t rows, int64_t d) { softmax_rows<XT, NV>(x, y, rows, d); }
+
+#define MTRT_NORM_FOR_TYPE(XN, XT)                                                                            \
+  MTRT_NORM_KERNELS(XN, XT, 1) MTRT_NORM_KERNELS(XN, XT, 2) MTRT_NORM_KERNELS(XN, XT, 4)                       \
+  MTRT_NORM_KERNELS(XN, XT, 8) MTRT_NORM_KERNELS(XN, XT, 16)                                                   \
+  extern "C" __global__ void __launch_bounds__(kNormThreads) mtrt_layernorm_##XN##_any(                        \
+      const XT::storage* x, const XT::storage* gamma, const XT::storage* beta, XT::storage* y, int64_t rows,  \
+      int64_t d, float eps) { layernorm_any<XT>(x, gamma, beta, y, rows, d, eps); }                           \
+  extern "C" __global__ void __launch_bounds__(kNormThreads) mtrt_softmax_##XN##_any(                          \
+      const XT::storage* x, XT::storage* y, int64_t rows, int64_t d) { softmax_any<XT>(x, y, rows, d); }
+
+MTRT_NORM_FOR_TYPE(f32, F32)
+MTRT_NORM_FOR_TYPE(f16, F16)
+MTRT_NORM_FOR_TYPE(bf16, BF16)

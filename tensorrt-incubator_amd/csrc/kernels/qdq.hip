@@ -1,0 +1,406 @@
+// Quantize / dequantize clusters for gfx950.
+//
+// Semantics (what each lane computes per element), following the reference's
+// canonical StableHLO forms
+//   quantize   : q = convert(clamp(lo, [round_nearest_even](f32(x) / scale), hi))
+//                mlir-tensorrt/compiler/lib/Dialect/StablehloExt/Transforms/StablehloRaiseQDQ.cpp:233-265
+//                mlir-tensorrt/tensorrt/include/mlir-tensorrt-dialect/TensorRT/IR/TensorRTOps.td:3133-3194
+//   dequantize : y = narrow(f32(q) * scale)
+//                StablehloRaiseQDQ.cpp:407-418 ; TensorRTOps.td:3408-3445
+// with lo/hi = -128/127 (i8), -448/448 (f8E4M3FN), -8/7 (i4).  The divide is the
+// correctly rounded IEEE f32 divide (no reciprocal shortcut): quantized codes must
+// be bit-identical to the host lowering.
+//
+// Scale addressing (the data tensor is viewed as row-major [d0, d1]):
+//   uniform : scale[0]                       per-tensor
+//   row     : scale[row % nscale]            per-channel on a non-last axis, blocks along the last axis
+//   col     : scale[(row / block) * d1 + c]  per-channel on the last axis (block = d0), blocks along axis 0
+//
+// Kernel arguments follow the reference's device ABI for generated kernels
+// (mlir-tensorrt/kernel/lib/Kernel/Transforms/ExpandMemRefArgs.cpp:65-120): one
+// bare pointer per buffer, then dynamic sizes as 64-bit integers, then scalars by
+// value.
+//
+// Data movement.  The unit is a GROUP: the G consecutive elements that fill one
+// 128-bit vector of the float operand (G = 4 for f32, 8 for f16/bf16).  In every
+// memory instruction lane l of a wave touches group (base + l), so one instruction
+// of a wave covers 64 consecutive groups: 1 KiB of the float operand and 256 or
+// 512 contiguous bytes of codes, all whole cache lines.  A lane carries J groups
+// per trip (16 elements), all loads issued before the first use.  The "_any"
+// variants take any shape and alignment, one element per lane.
+#include "common.hpp"
+
+using namespace mtrt_dev;
+
+namespace qdq_cluster {
+
+// ---- float operand: one 128-bit vector <-> G floats ----------------------------
+template <typename X> struct FloatGroup;
+template <> struct FloatGroup<F32> {
+  static constexpr int G = 4;
+  static __device__ __forceinline__ u32x4 load(const float* p) { return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p)); }
+  static __device__ __forceinline__ void unpack(u32x4 t, float (&v)[4]) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) v[k] = bits_to_f32(t[k]);
+  }
+  static __device__ __forceinline__ void store(float* p, const float (&v)[4]) {
+    u32x4 t = {f32_to_bits(v[0]), f32_to_bits(v[1]), f32_to_bits(v[2]), f32_to_bits(v[3])};
+    __builtin_nontemporal_store(t, reinterpret_cast<u32x4*>(p));
+  }
+};
+template <> struct FloatGroup<BF16> {
+  static constexpr int G = 8;
+  static __device__ __forceinline__ u32x4 load(const uint16_t* p) { return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p)); }
+  static __device__ __forceinline__ void unpack(u32x4 t, float (&v)[8]) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) { v[2 * k] = bits_to_f32(t[k] << 16); v[2 * k + 1] = bits_to_f32(t[k] & 0xFFFF0000u); }
+  }
+  static __device__ __forceinline__ void store(uint16_t* p, const float (&v)[8]) {
+    u32x4 t;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) t[k] = f32_to_bf16_bits(v[2 * k]) | (f32_to_bf16_bits(v[2 * k + 1]) << 16);
+    __builtin_nontemporal_store(t, reinterpret_cast<u32x4*>(p));
+  }
+};
+template <> struct FloatGroup<F16> {
+  static constexpr int G = 8;
+  static __device__ __forceinline__ u32x4 load(const uint16_t* p) { return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p)); }
+  static __device__ __forceinline__ void unpack(u32x4 t, float (&v)[8]) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) { v[2 * k] = f16_bits_to_f32(t[k] & 0xFFFFu); v[2 * k + 1] = f16_bits_to_f32(t[k] >> 16); }
+  }
+  static __device__ __forceinline__ void store(uint16_t* p, const float (&v)[8]) {
+    u32x4 t;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) t[k] = f32_to_f16_bits(v[2 * k]) | (f32_to_f16_bits(v[2 * k + 1]) << 16);
+    __builtin_nontemporal_store(t, reinterpret_cast<u32x4*>(p));
+  }
+};
+
+// ---- quantized codes ---------------------------------------------------------------
+// enc(v): code of an already divided / rounded / clamped value.  dec(code): f32 value.
+// A group of G codes travels as G/4 (bytes) or G/8 (nibbles) 32-bit words; the
+// 4-nibble group of an f32 operand is a single 16-bit access.
+template <typename Q> struct Codes;
+
+template <> struct Codes<I8> {
+  static constexpr float kLo = -128.0f, kHi = 127.0f;
+  static constexpr bool kAlwaysRound = true;
+  static __device__ __forceinline__ uint32_t enc(float v, int) { return uint32_t(int(v)) & 0xFFu; }
+  static __device__ __forceinline__ float dec(uint32_t c) { return float(int(c << 24) >> 24); }
+};
+template <> struct Codes<F8> {
+  static constexpr float kLo = -448.0f, kHi = 448.0f;
+  static constexpr bool kAlwaysRound = false;
+  static __device__ __forceinline__ uint32_t enc(float v, int flags) {
+    return (flags & kFlagF8RefHost) ? f32_to_f8_refhost(v) : (f32x2_to_f8_ieee(v, 0.0f) & 0xFFu);
+  }
+  static __device__ __forceinline__ float dec(uint32_t c) { return f8_to_f32<0>(c); }
+};
+// int4, one element per byte in the low nibble, upper nibble zero (host storage:
+// DataTypes.cpp:494-519 keeps `bits_ & 0xF`).
+template <> struct Codes<I4> {
+  static constexpr float kLo = -8.0f, kHi = 7.0f;
+  static constexpr bool kAlwaysRound = true;
+  static __device__ __forceinline__ uint32_t enc(float v, int) { return uint32_t(int(v)) & 0xFu; }
+  static __device__ __forceinline__ float dec(uint32_t c) { return float(int(c << 28) >> 28); }
+};
+// int4 packed two per byte over the flattened array, element 2i in the low nibble
+// (mlir-tensorrt/tensorrt/lib/Target/TensorRTEncodingOpInterface/NetworkEncoder.cpp:552-595).
+template <> struct Codes<I4P> {
+  static constexpr float kLo = -8.0f, kHi = 7.0f;
+  static constexpr bool kAlwaysRound = true;
+  static __device__ __forceinline__ uint32_t enc(float v, int) { return uint32_t(int(v)) & 0xFu; }
+  static __device__ __forceinline__ float dec(uint32_t c) { return float(int(c << 28) >> 28); }
+};
+
+// Four byte-wide codes <-> one 32-bit word.  The f8 IEEE path converts pairs in
+// hardware; everything else goes through enc/dec.
+template <typename Q>
+__device__ __forceinline__ uint32_t pack4(const float* v, int flags) {
+  return Codes<Q>::enc(v[0], flags) | (Codes<Q>::enc(v[1], flags) << 8) | (Codes<Q>::enc(v[2], flags) << 16) |
+         (Codes<Q>::enc(v[3], flags) << 24);
+}
+template <>
+__device__ __forceinline__ uint32_t pack4<F8>(const float* v, int flags) {
+  if (flags & kFlagF8RefHost)
+    return f32_to_f8_refhost(v[0]) | (f32_to_f8_refhost(v[1]) << 8) | (f32_to_f8_refhost(v[2]) << 16) |
+           (f32_to_f8_refhost(v[3]) << 24);
+  int w = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], 0, false);
+  return uint32_t(__builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], w, true));
+}
+template <typename Q>
+__device__ __forceinline__ void unpack4(uint32_t w, float* v) {
+#pragma unroll
+  for (int k = 0; k < 4; ++k) v[k] = Codes<Q>::dec((w >> (8 * k)) & 0xFFu);
+}
+template <>
+__device__ __forceinline__ void unpack4<F8>(uint32_t w, float* v) {
+  v[0] = f8_to_f32<0>(w); v[1] = f8_to_f32<1>(w); v[2] = f8_to_f32<2>(w); v[3] = f8_to_f32<3>(w);
+}
+
+// G codes of one group, at element offset `e` (a multiple of G) of the code array.
+// store() leaves f32(code) in v[]: the value a following dequantize multiplies by
+// the scale (this also turns the -0.0 a rounding can produce into the +0.0 that
+// reading the integer code back gives).
+template <typename Q, int G> struct CodeGroup {
+  static constexpr int kWords = G / 4;
+  static __device__ __forceinline__ void store(typename Q::storage* base, int64_t e, float (&v)[G], int flags) {
+    uint32_t w[kWords];
+#pragma unroll
+    for (int i = 0; i < kWords; ++i) { w[i] = pack4<Q>(&v[4 * i], flags); unpack4<Q>(w[i], &v[4 * i]); }
+    if (kWords == 1) {
+      __builtin_nontemporal_store(w[0], reinterpret_cast<uint32_t*>(base + e));
+    } else {
+      u32x2 t = {w[0], w[kWords - 1]};
+      __builtin_nontemporal_store(t, reinterpret_cast<u32x2*>(base + e));
+    }
+  }
+  static __device__ __forceinline__ void load_raw(const typename Q::storage* base, int64_t e, uint32_t (&w)[2]) {
+    if (kWords == 1) {
+      w[0] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(base + e));
+    } else {
+      const u32x2 t = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(base + e));
+      w[0] = t.x; w[1] = t.y;
+    }
+  }
+  static __device__ __forceinline__ void decode(const uint32_t (&w)[2], float (&v)[G]) {
+#pragma unroll
+    for (int i = 0; i < kWords; ++i) unpack4<Q>(w[i], &v[4 * i]);
+  }
+};
+template <int G> struct CodeGroup<I4P, G> {
+  static __device__ __forceinline__ void store(uint8_t* base, int64_t e, float (&v)[G], int) {
+    uint32_t w = 0;
+#pragma unroll
+    for (int k = 0; k < G; ++k) {
+      const int c = int(v[k]);
+      v[k] = float(c);
+      w |= (uint32_t(c) & 0xFu) << (4 * k);
+    }
+    if (G == 4) __builtin_nontemporal_store(uint16_t(w), reinterpret_cast<uint16_t*>(base + (e >> 1)));
+    else __builtin_nontemporal_store(w, reinterpret_cast<uint32_t*>(base + (e >> 1)));
+  }
+  static __device__ __forceinline__ void load_raw(const uint8_t* base, int64_t e, uint32_t (&w)[2]) {
+    if (G == 4) w[0] = __builtin_nontemporal_load(reinterpret_cast<const uint16_t*>(base + (e >> 1)));
+    else w[0] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(base + (e >> 1)));
+  }
+  static __device__ __forceinline__ void decode(const uint32_t (&w)[2], float (&v)[G]) {
+#pragma unroll
+    for (int k = 0; k < G; ++k) v[k] = float(int(w[0] << (28 - 4 * k)) >> 28);
+  }
+};
+
+template <typename Q>
+__device__ __forceinline__ float quant_value(float x, float s, int flags) {
+  float v = x / s;                                   // IEEE divide, bit-exact with the host
+  if (Codes<Q>::kAlwaysRound || (flags & kFlagRoundToInt))
+    v = __builtin_rintf(v);                          // v_rndne_f32: exact round-half-even
+  return fmaxf(fminf(v, Codes<Q>::kHi), Codes<Q>::kLo);
+}
+
+enum ScaleKind { kUniform = 0, kRow = 1, kCol = 2 };
+
+// MODE: 0 = quantize (write q), 1 = dequantize (read q, write y),
+//       2 = fused quantize->dequantize (read x, write q and y)
+// Host guarantees: n < 2^35; for row/col scales d1 % G == 0 (a group never
+// straddles rows); operands aligned for their group accesses.
+template <typename X, typename Q, int KIND, int MODE>
+__device__ __forceinline__ void qdq_groups(const typename X::storage* __restrict__ x, typename Q::storage* __restrict__ q,
+                                           typename X::storage* __restrict__ y, const float* __restrict__ scale,
+                                           int64_t n, int64_t d1, int64_t nb, int flags) {
+  using FG = FloatGroup<X>;
+  constexpr int G = FG::G;
+  constexpr int J = kTile / G;                       // groups per lane per trip
+  constexpr int SN = KIND == kCol ? G : 1;           // scale values a lane needs per group
+  using CG = CodeGroup<Q, G>;
+  const int64_t ngroups = n / G;
+  const uint32_t groups_per_row = KIND == kUniform ? 1u : uint32_t(d1 / G);
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t wave = (int64_t(blockIdx.x) * blockDim.x + threadIdx.x) / kWave;
+  const int64_t nwaves = int64_t(gridDim.x) * blockDim.x / kWave;
+  const float s_uniform = KIND == kUniform ? scale[0] : 0.0f;
+
+  for (int64_t base = wave * (kWave * J); base < ngroups; base += nwaves * (kWave * J)) {
+    float v[J][G];
+    float s[J][SN];
+    bool live[J];
+    u32x4 xin[J];
+    uint32_t qin[J][2];
+    // all loads of the trip first
+#pragma unroll
+    for (int j = 0; j < J; ++j) {
+      const int64_t g = base + j * kWave + lane;
+      live[j] = g < ngroups;
+      if (!live[j]) continue;
+      if (MODE == 1) CG::load_raw(q, g * G, qin[j]);
+      else xin[j] = FG::load(x + g * G);
+      if (KIND == kUniform) {
+        s[j][0] = s_uniform;
+      } else {
+        // group, row and scale indices are below 2^32 for anything that fits in HBM
+        const uint32_t row = uint32_t(g) / groups_per_row;
+        if (KIND == kRow) {
+          s[j][0] = scale[row % uint32_t(nb)];
+        } else {
+          const int64_t c0 = int64_t(uint32_t(g) - row * groups_per_row) * G;
+          const f32x4* sp = reinterpret_cast<const f32x4*>(scale + int64_t(row / uint32_t(nb)) * d1 + c0);
+#pragma unroll
+          for (int k = 0; k < SN / 4; ++k) {
+            const f32x4 t = sp[k];
+            s[j][(4 * k + 0) % SN] = t.x; s[j][(4 * k + 1) % SN] = t.y;
+            s[j][(4 * k + 2) % SN] = t.z; s[j][(4 * k + 3) % SN] = t.w;
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < J; ++j) {
+      if (!live[j]) continue;
+      const int64_t e = (base + j * kWave + lane) * G;
+      if (MODE == 1) {
+        CG::decode(qin[j], v[j]);
+      } else {
+        FG::unpack(xin[j], v[j]);
+#pragma unroll
+        for (int k = 0; k < G; ++k) v[j][k] = quant_value<Q>(v[j][k], s[j][k % SN], flags);
+        CG::store(q, e, v[j], flags);
+      }
+      if (MODE != 0) {
+#pragma unroll
+        for (int k = 0; k < G; ++k) v[j][k] = v[j][k] * s[j][k % SN];
+        FG::store(y + e, v[j]);
+      }
+    }
+  }
+
+  // Remainder (< G elements) of a per-tensor array, one lane each; row- and
+  // column-scaled launches have n % G == 0 by construction.  Packed nibbles: the
+  // lane of the even element writes the whole byte.
+  if (KIND == kUniform && blockIdx.x == 0 && threadIdx.x < G) {
+    const int64_t e = ngroups * G + threadIdx.x;
+    if (e < n) {
+      if (Q::kBits == 4) {
+        if ((e & 1) == 0) {
+          const bool has1 = e + 1 < n;
+          float v0, v1 = 0.0f;
+          if (MODE == 1) {
+            const uint32_t byte = uint32_t(uint8_t(q[e >> 1]));
+            v0 = Codes<Q>::dec(byte & 0xFu);
+            v1 = Codes<Q>::dec(byte >> 4);
+          } else {
+            v0 = quant_value<Q>(Tile<X>::load1(x + e), s_uniform, flags);
+            if (has1) v1 = quant_value<Q>(Tile<X>::load1(x + e + 1), s_uniform, flags);
+            const uint32_t c0 = Codes<Q>::enc(v0, flags), c1 = Codes<Q>::enc(v1, flags);
+            q[e >> 1] = typename Q::storage(c0 | (c1 << 4));
+            v0 = Codes<Q>::dec(c0); v1 = Codes<Q>::dec(c1);
+          }
+          if (MODE != 0) {
+            Tile<X>::store1(y + e, v0 * s_uniform);
+            if (has1) Tile<X>::store1(y + e + 1, v1 * s_uniform);
+          }
+        }
+      } else {
+        float v;
+        if (MODE == 1) {
+          v = Codes<Q>::dec(uint32_t(uint8_t(q[e])));
+        } else {
+          v = quant_value<Q>(Tile<X>::load1(x + e), s_uniform, flags);
+          const uint32_t c = Codes<Q>::enc(v, flags);
+          q[e] = typename Q::storage(c);
+          v = Codes<Q>::dec(c);
+        }
+        if (MODE != 0) Tile<X>::store1(y + e, v * s_uniform);
+      }
+    }
+  }
+}
+
+// Any shape, any alignment: one element per lane (packed int4: one byte = two
+// elements per lane), scale kind chosen at run time.
+template <typename X, typename Q, int MODE>
+__device__ __forceinline__ void qdq_any(const typename X::storage* __restrict__ x, typename Q::storage* __restrict__ q,
+                                        typename X::storage* __restrict__ y, const float* __restrict__ scale,
+                                        int64_t n, int64_t d1, int64_t nb, int kind, int flags) {
+  constexpr int kPer = (Q::kBits == 4) ? 2 : 1;
+  const int64_t units = (n + kPer - 1) / kPer;
+  const int64_t stride = int64_t(gridDim.x) * blockDim.x;
+  for (int64_t u = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; u < units; u += stride) {
+    uint32_t byte = (Q::kBits == 4 && MODE == 1) ? uint32_t(uint8_t(q[u])) : 0u;
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) {
+      const int64_t e = u * kPer + k;
+      if (e >= n) continue;
+      const int64_t row = e / d1;
+      const float s = kind == kUniform ? scale[0]
+                                       : (kind == kRow ? scale[row % nb] : scale[(row / nb) * d1 + (e - row * d1)]);
+      float v;
+      if (MODE == 1) {
+        v = Q::kBits == 4 ? Codes<Q>::dec((byte >> (4 * k)) & 0xFu) : Codes<Q>::dec(uint32_t(uint8_t(q[e])));
+      } else {
+        v = quant_value<Q>(Tile<X>::load1(x + e), s, flags);
+        const uint32_t c = Codes<Q>::enc(v, flags);
+        if (Q::kBits == 4) byte |= c << (4 * k);
+        else q[e] = typename Q::storage(c);
+        v = Codes<Q>::dec(c);
+      }
+      if (MODE != 0) Tile<X>::store1(y + e, v * s);
+    }
+    if (Q::kBits == 4 && MODE != 1) q[u] = typename Q::storage(byte);
+  }
+}
+
+}  // namespace qdq_cluster
+using namespace qdq_cluster;
+
+// ---- entry points -----------------------------------------------------------------
+// Names: mtrt_{q,dq,qdq}_{uniform,row,col,any}_<float type>_<code type>
+//   q   (x, q, scale, n, d1, nb, flags)        dq  (q, y, scale, n, d1, nb)
+//   qdq (x, q, y, scale, n, d1, nb, flags)     *_any add `kind` after nb
+#define MTRT_QDQ_KERNELS(XN, XT, QN, QT)                                                                          \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_q_uniform_##XN##_##QN(                                   \
+      const XT::storage* x, QT::storage* q, const float* scale, int64_t n, int64_t d1, int64_t nb, int32_t flags) { \
+    qdq_groups<XT, QT, kUniform, 0>(x, q, nullptr, scale, n, d1, nb, flags); }                                    \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_q_row_##XN##_##QN(                                       \
+      const XT::storage* x, QT::storage* q, const float* scale, int64_t n, int64_t d1, int64_t nb, int32_t flags) { \
+    qdq_groups<XT, QT, kRow, 0>(x, q, nullptr, scale, n, d1, nb, flags); }                                        \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_q_col_##XN##_##QN(                                       \
+      const XT::storage* x, QT::storage* q, const float* scale, int64_t n, int64_t d1, int64_t nb, int32_t flags) { \
+    qdq_groups<XT, QT, kCol, 0>(x, q, nullptr, scale, n, d1, nb, flags); }                                        \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_q_any_##XN##_##QN(                                       \
+      const XT::storage* x, QT::storage* q, const float* scale, int64_t n, int64_t d1, int64_t nb, int32_t kind,  \
+      int32_t flags) { qdq_any<XT, QT, 0>(x, q, nullptr, scale, n, d1, nb, kind, flags); }                        \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_dq_uniform_##XN##_##QN(                                  \
+      const QT::storage* q, XT::storage* y, const float* scale, int64_t n, int64_t d1, int64_t nb) {              \
+    qdq_groups<XT, QT, kUniform, 1>(nullptr, const_cast<QT::storage*>(q), y, scale, n, d1, nb, 0); }              \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_dq_row_##XN##_##QN(                                      \
+      const QT::storage* q, XT::storage* y, const float* scale, int64_t n, int64_t d1, int64_t nb) {              \
+    qdq_groups<XT, QT, kRow, 1>(nullptr, const_cast<QT::storage*>(q), y, scale, n, d1, nb, 0); }                  \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_dq_col_##XN##_##QN(                                      \
+      const QT::storage* q, XT::storage* y, const float* scale, int64_t n, int64_t d1, int64_t nb) {              \
+    qdq_groups<XT, QT, kCol, 1>(nullptr, const_cast<QT::storage*>(q), y, scale, n, d1, nb, 0); }                  \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_dq_any_##XN##_##QN(                                      \
+      const QT::storage* q, XT::storage* y, const float* scale, int64_t n, int64_t d1, int64_t nb, int32_t kind) { \
+    qdq_any<XT, QT, 1>(nullptr, const_cast<QT::storage*>(q), y, scale, n, d1, nb, kind, 0); }                     \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_qdq_uniform_##XN##_##QN(                                 \
+      const XT::storage* x, QT::storage* q, XT::storage* y, const float* scale, int64_t n, int64_t d1, int64_t nb, \
+      int32_t flags) { qdq_groups<XT, QT, kUniform, 2>(x, q, y, scale, n, d1, nb, flags); }                       \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_qdq_row_##XN##_##QN(                                     \
+      const XT::storage* x, QT::storage* q, XT::storage* y, const float* scale, int64_t n, int64_t d1, int64_t nb, \
+      int32_t flags) { qdq_groups<XT, QT, kRow, 2>(x, q, y, scale, n, d1, nb, flags); }                           \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_qdq_col_##XN##_##QN(                                     \
+      const XT::storage* x, QT::storage* q, XT::storage* y, const float* scale, int64_t n, int64_t d1, int64_t nb, \
+      int32_t flags) { qdq_groups<XT, QT, kCol, 2>(x, q, y, scale, n, d1, nb, flags); }                           \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_qdq_any_##XN##_##QN(                                     \
+      const XT::storage* x, QT::storage* q, XT::storage* y, const float* scale, int64_t n, int64_t d1, int64_t nb, \
+      int32_t kind, int32_t flags) { qdq_any<XT, QT, 2>(x, q, y, scale, n, d1, nb, kind, flags); }
+
+#define MTRT_QDQ_FOR_FLOAT(XN, XT)    \
+  MTRT_QDQ_KERNELS(XN, XT, i8, I8)    \
+  MTRT_QDQ_KERNELS(XN, XT, f8, F8)    \
+  MTRT_QDQ_KERNELS(XN, XT, i4, I4)    \
+  MTRT_QDQ_KERNELS(XN, XT, i4p, I4P)
+
+MTRT_QDQ_FOR_FLOAT(f32, F32)
+MTRT_QDQ_FOR_FLOAT(f16, F16)
+MTRT_QDQ_FOR_FLOAT(bf16, BF16)

@@ -1,0 +1,246 @@
+// Part 2 of the C ABI: one entry point per kernel cluster.  Each validates its
+// operands on the host (so that no launch can address memory outside them), picks
+// the kernel variant and launch shape for gfx950, builds the argument array in the
+// reference's kernelParams convention and launches from the built-in module.
+// This is the hand-written counterpart of the get-function + launch pairs the
+// reference compiler emits for its generated kernels
+// (mlir-tensorrt/compiler/lib/Passes/1_Core/KernelToCUDA/KernelToCUDA.cpp:151-186;
+//  mlir-tensorrt/compiler/lib/Passes/2_Host/HostToExecutor/CUDAToExecutor/CUDAToExecutor.cpp:355-413).
+#include "runtime_internal.hpp"
+
+#include <algorithm>
+#include <cstdlib>
+
+using namespace mtrt_rt;
+
+namespace {
+
+constexpr int kTile = 16;           // elements per lane per trip in qdq.hip
+constexpr uint32_t kBlock = 256;
+constexpr uint32_t kMaxGrid = 1u << 20;
+
+const char *float_name(int32_t dt) {
+  switch (dt) {
+  case MTRT_F32: return "f32";
+  case MTRT_F16: return "f16";
+  case MTRT_BF16: return "bf16";
+  }
+  return nullptr;
+}
+const char *code_name(int32_t dt) {
+  switch (dt) {
+  case MTRT_I8: return "i8";
+  case MTRT_F8E4M3FN: return "f8";
+  case MTRT_I4: return "i4";
+  case MTRT_I4_PACKED: return "i4p";
+  }
+  return nullptr;
+}
+int float_bytes(int32_t dt) { return dt == MTRT_F32 ? 4 : 2; }
+
+bool aligned(const void *p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+uint32_t blocks_for(int64_t units, uint32_t per_block) {
+  const int64_t b = (units + per_block - 1) / per_block;
+  return uint32_t(std::max<int64_t>(1, std::min<int64_t>(b, kMaxGrid)));
+}
+
+// mode: 0 quantize, 1 dequantize, 2 fused
+int32_t qdq_dispatch(int mode, hipStream_t stream, const void *x, int32_t x_dtype, void *q,
+                     int32_t q_dtype, void *y, const float *scale, int32_t kind, int64_t d0,
+                     int64_t d1, int64_t nb, int32_t flags) {
+  clear_error();
+  const char *xn = float_name(x_dtype);
+  const char *qn = code_name(q_dtype);
+  if (!xn)
+    return set_error(MTRT_INVALID_ARGUMENT, "float operand dtype %d is not one of f32/f16/bf16", x_dtype);
+  if (!qn)
+    return set_error(MTRT_INVALID_ARGUMENT, "quantized dtype %d is not one of i8/f8E4M3FN/i4/i4-packed", q_dtype);
+  if (d0 < 0 || d1 < 0)
+    return set_error(MTRT_INVALID_ARGUMENT, "negative extent [%lld, %lld]", (long long)d0, (long long)d1);
+  if (kind < MTRT_SCALE_UNIFORM || kind > MTRT_SCALE_COL)
+    return set_error(MTRT_INVALID_ARGUMENT, "unknown scale kind %d", kind);
+  if (kind != MTRT_SCALE_UNIFORM && nb <= 0)
+    return set_error(MTRT_INVALID_ARGUMENT, "scale kind %d needs a positive scale count / block size, got %lld",
+                     kind, (long long)nb);
+  if (kind == MTRT_SCALE_COL && d0 % nb != 0)
+    return set_error(MTRT_INVALID_ARGUMENT, "block size %lld does not divide the blocked extent %lld",
+                     (long long)nb, (long long)d0);
+  if (flags & ~(MTRT_Q_ROUND_TO_INT | MTRT_F8_REFHOST))
+    return set_error(MTRT_INVALID_ARGUMENT, "unknown flag bits 0x%x", flags);
+  const int64_t n = d0 * d1;
+  if (n == 0)
+    return MTRT_OK;
+  if (n >= (int64_t(1) << 35))
+    return set_error(MTRT_INVALID_ARGUMENT, "%lld elements exceed the supported 2^35", (long long)n);
+  if (!scale || !q || (mode != 1 && !x) || (mode != 0 && !y))
+    return set_error(MTRT_INVALID_ARGUMENT, "null operand");
+  if (!aligned(mode == 1 ? y : x, float_bytes(x_dtype)) || (mode == 2 && !aligned(y, float_bytes(x_dtype))))
+    return set_error(MTRT_INVALID_ARGUMENT, "float operand is not aligned to its element size");
+  if (d1 == 0)
+    return MTRT_OK;
+  if (kind == MTRT_SCALE_UNIFORM)
+    nb = 1;
+
+  DeviceState *st = device_state();
+  if (!st)
+    return MTRT_RUNTIME_ERROR;
+
+  // The group kernels move one 128-bit vector of the float operand (G elements)
+  // per lane per instruction: they need that operand 128-bit aligned, the codes
+  // aligned to the G codes a lane moves at once, and - whenever the scale changes
+  // along or across rows - rows that are whole groups.
+  const int group = x_dtype == MTRT_F32 ? 4 : 8;
+  const uintptr_t q_align = q_dtype == MTRT_I4_PACKED ? group / 2 : group;
+  bool tiles = aligned(q, q_align) && (mode == 1 || aligned(x, 16)) && (mode == 0 || aligned(y, 16));
+  if (kind != MTRT_SCALE_UNIFORM)
+    tiles = tiles && (d1 % group == 0);
+  if (kind == MTRT_SCALE_COL)
+    tiles = tiles && aligned(scale, 16);
+
+  static const char *kModeName[] = {"q", "dq", "qdq"};
+  static const char *kKindName[] = {"uniform", "row", "col"};
+  std::string name = std::string("mtrt_") + kModeName[mode] + "_" + (tiles ? kKindName[kind] : "any") + "_" + xn + "_" + qn;
+
+  int64_t n_arg = n, d1_arg = d1, nb_arg = nb;
+  int32_t kind_arg = kind, flags_arg = flags;
+  const void *x_arg = x;
+  void *q_arg = q, *y_arg = y;
+  const float *s_arg = scale;
+  void *args[9];
+  int na = 0;
+  if (mode != 1) args[na++] = &x_arg;
+  args[na++] = &q_arg;
+  if (mode != 0) args[na++] = &y_arg;
+  args[na++] = &s_arg;
+  args[na++] = &n_arg;
+  args[na++] = &d1_arg;
+  args[na++] = &nb_arg;
+  if (!tiles) args[na++] = &kind_arg;
+  if (mode != 1) args[na++] = &flags_arg;
+
+  const int64_t units = tiles ? (n + kTile - 1) / kTile : (q_dtype == MTRT_I4_PACKED ? (n + 1) / 2 : n);
+  return launch(st, name, blocks_for(units, kBlock), kBlock, stream, args);
+}
+
+int32_t pick_nv(int64_t nvec_per_row) {
+  for (int nv : {1, 2, 4, 8, 16})
+    if (nvec_per_row <= int64_t(64) * nv)
+      return nv;
+  return 0;
+}
+
+} // namespace
+
+extern "C" {
+
+int32_t mtrt_hip_amax(mtrt_stream_t stream, const void *x, int32_t dtype, int64_t n, float qmax,
+                      float *amax_out, float *scale_out) {
+  clear_error();
+  const char *xn = float_name(dtype);
+  if (!xn)
+    return set_error(MTRT_INVALID_ARGUMENT, "amax input dtype %d is not one of f32/f16/bf16", dtype);
+  if (n < 0)
+    return set_error(MTRT_INVALID_ARGUMENT, "negative element count %lld", (long long)n);
+  if (n > 0 && !x)
+    return set_error(MTRT_INVALID_ARGUMENT, "null input");
+  if (!aligned(x, float_bytes(dtype)))
+    return set_error(MTRT_INVALID_ARGUMENT, "input is not aligned to its element size");
+  DeviceState *st = device_state();
+  if (!st)
+    return MTRT_RUNTIME_ERROR;
+  uint32_t *slot = reduction_slot(st, as_hip(stream));
+  if (!slot)
+    return MTRT_RUNTIME_ERROR;
+  // Enough workgroups to occupy every CU with 8 of them (32 waves), each lane
+  // keeping four 128-bit loads in flight; fewer when the tensor is small.
+  const int per_vec = dtype == MTRT_F32 ? 4 : 8;
+  const int64_t nvec = n / per_vec;
+  const uint32_t grid = uint32_t(std::max<int64_t>(
+      1, std::min<int64_t>((nvec + int64_t(kBlock) * 4 - 1) / (int64_t(kBlock) * 4), int64_t(num_compute_units(st)) * 8)));
+  const void *x_arg = x;
+  int64_t n_arg = n;
+  float qmax_arg = qmax;
+  void *args[] = {&x_arg, &n_arg, &qmax_arg, &amax_out, &scale_out, &slot};
+  return launch(st, std::string("mtrt_amax_") + xn, grid, kBlock, as_hip(stream), args);
+}
+
+int32_t mtrt_hip_quantize(mtrt_stream_t stream, const void *x, int32_t x_dtype, void *q, int32_t q_dtype,
+                          const float *scale, int32_t scale_kind, int64_t d0, int64_t d1, int64_t nb,
+                          int32_t flags) {
+  return qdq_dispatch(0, as_hip(stream), x, x_dtype, q, q_dtype, nullptr, scale, scale_kind, d0, d1, nb, flags);
+}
+
+int32_t mtrt_hip_dequantize(mtrt_stream_t stream, const void *q, int32_t q_dtype, void *y, int32_t y_dtype,
+                            const float *scale, int32_t scale_kind, int64_t d0, int64_t d1, int64_t nb) {
+  return qdq_dispatch(1, as_hip(stream), nullptr, y_dtype, const_cast<void *>(q), q_dtype, y, scale, scale_kind,
+                      d0, d1, nb, 0);
+}
+
+int32_t mtrt_hip_quantize_dequantize(mtrt_stream_t stream, const void *x, int32_t x_dtype, void *q,
+                                     int32_t q_dtype, void *y, const float *scale, int32_t scale_kind,
+                                     int64_t d0, int64_t d1, int64_t nb, int32_t flags) {
+  return qdq_dispatch(2, as_hip(stream), x, x_dtype, q, q_dtype, y, scale, scale_kind, d0, d1, nb, flags);
+}
+
+int32_t mtrt_hip_layernorm(mtrt_stream_t stream, const void *x, const void *gamma, const void *beta, void *y,
+                           int32_t dtype, int64_t rows, int64_t d, float eps) {
+  clear_error();
+  const char *xn = float_name(dtype);
+  if (!xn)
+    return set_error(MTRT_INVALID_ARGUMENT, "layernorm dtype %d is not one of f32/f16/bf16", dtype);
+  if (rows < 0 || d < 0)
+    return set_error(MTRT_INVALID_ARGUMENT, "negative extent [%lld, %lld]", (long long)rows, (long long)d);
+  if (rows == 0 || d == 0)
+    return MTRT_OK;
+  if (!x || !gamma || !beta || !y)
+    return set_error(MTRT_INVALID_ARGUMENT, "null operand");
+  const int eb = float_bytes(dtype);
+  if (!aligned(x, eb) || !aligned(y, eb) || !aligned(gamma, eb) || !aligned(beta, eb))
+    return set_error(MTRT_INVALID_ARGUMENT, "operand is not aligned to its element size");
+  DeviceState *st = device_state();
+  if (!st)
+    return MTRT_RUNTIME_ERROR;
+  const int per_vec = 16 / eb;
+  const bool vec_ok = d % per_vec == 0 && aligned(x, 16) && aligned(y, 16) && aligned(gamma, 16) && aligned(beta, 16);
+  const int nv = vec_ok ? pick_nv(d / per_vec) : 0;
+  int64_t rows_arg = rows, d_arg = d;
+  float eps_arg = eps;
+  void *args[] = {&x, &gamma, &beta, &y, &rows_arg, &d_arg, &eps_arg};
+  if (nv)
+    return launch(st, std::string("mtrt_layernorm_") + xn + "_v" + std::to_string(nv),
+                  blocks_for(rows, kBlock / 64), kBlock, as_hip(stream), args);
+  return launch(st, std::string("mtrt_layernorm_") + xn + "_any",
+                uint32_t(std::min<int64_t>(rows, int64_t(num_compute_units(st)) * 8)), kBlock, as_hip(stream), args);
+}
+
+int32_t mtrt_hip_softmax(mtrt_stream_t stream, const void *x, void *y, int32_t dtype, int64_t rows, int64_t d) {
+  clear_error();
+  const char *xn = float_name(dtype);
+  if (!xn)
+    return set_error(MTRT_INVALID_ARGUMENT, "softmax dtype %d is not one of f32/f16/bf16", dtype);
+  if (rows < 0 || d < 0)
+    return set_error(MTRT_INVALID_ARGUMENT, "negative extent [%lld, %lld]", (long long)rows, (long long)d);
+  if (rows == 0 || d == 0)
+    return MTRT_OK;
+  if (!x || !y)
+    return set_error(MTRT_INVALID_ARGUMENT, "null operand");
+  const int eb = float_bytes(dtype);
+  if (!aligned(x, eb) || !aligned(y, eb))
+    return set_error(MTRT_INVALID_ARGUMENT, "operand is not aligned to its element size");
+  DeviceState *st = device_state();
+  if (!st)
+    return MTRT_RUNTIME_ERROR;
+  const int per_vec = 16 / eb;
+  const bool vec_ok = d % per_vec == 0 && aligned(x, 16) && aligned(y, 16);
+  const int nv = vec_ok ? pick_nv(d / per_vec) : 0;
+  int64_t rows_arg = rows, d_arg = d;
+  void *args[] = {&x, &y, &rows_arg, &d_arg};
+  if (nv)
+    return launch(st, std::string("mtrt_softmax_") + xn + "_v" + std::to_string(nv),
+                  blocks_for(rows, kBlock / 64), kBlock, as_hip(stream), args);
+  return launch(st, std::string("mtrt_softmax_") + xn + "_any",
+                uint32_t(std::min<int64_t>(rows, int64_t(num_compute_units(st)) * 8)), kBlock, as_hip(stream), args);
+}
+
+} // extern "C"

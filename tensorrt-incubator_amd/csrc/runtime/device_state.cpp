@@ -1,0 +1,221 @@
+// Per-device state of the cluster layer and the embedded kernel module.
+//
+// The gfx950 code object built from csrc/kernels/*.hip is linked into this
+// library as read-only data (the role PTX text plays inside a reference
+// executable's data segment,
+// mlir-tensorrt/compiler/lib/Passes/2_Host/HostToExecutor/CUDAToExecutor/CUDAToExecutor.cpp:858-905)
+// and loaded once per device, lazily, the way the reference initialises its module
+// and function globals on first use (CUDAToExecutor.cpp:797-905).
+#include "runtime_internal.hpp"
+
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <unordered_map>
+
+#ifndef MTRT_HSACO_PATH
+#error "MTRT_HSACO_PATH must name the code object to embed"
+#endif
+
+__asm__(".section .rodata\n"
+        ".balign 4096\n"
+        ".global mtrt_hip_hsaco_begin\n"
+        "mtrt_hip_hsaco_begin:\n"
+        ".incbin \"" MTRT_HSACO_PATH "\"\n"
+        ".global mtrt_hip_hsaco_end\n"
+        "mtrt_hip_hsaco_end:\n"
+        ".byte 0\n"
+        ".previous\n");
+extern "C" const char mtrt_hip_hsaco_begin[];
+extern "C" const char mtrt_hip_hsaco_end[];
+
+namespace mtrt_rt {
+
+namespace {
+thread_local char tl_error[1024] = {0};
+thread_local char tl_kernel[128] = {0};
+} // namespace
+
+int32_t set_error(int32_t code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  std::vsnprintf(tl_error, sizeof(tl_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+void clear_error() { tl_error[0] = '\0'; }
+const char *last_error() { return tl_error; }
+
+int32_t load_code_object(const char *data, size_t len, hipModule_t *out, std::string *err) {
+  static const char kBundle[] = "__CLANG_OFFLOAD_BUNDLE__";
+  const bool elf = len >= 4 && std::memcmp(data, "\x7f" "ELF", 4) == 0;
+  const bool bundle = len >= sizeof(kBundle) - 1 && std::memcmp(data, kBundle, sizeof(kBundle) - 1) == 0;
+  if (!data || (!elf && !bundle)) {
+    *err = "module data is not an AMDGPU code object (expected ELF or a clang offload bundle; "
+           "PTX is not accepted)";
+    return MTRT_INVALID_ARGUMENT;
+  }
+  // The loader reads sizes from the image's own headers; hand it a private copy so
+  // a caller's buffer that is not NUL-padded or is freed early cannot matter.
+  std::vector<char> copy(data, data + len);
+  copy.push_back('\0');
+  hipModule_t module = nullptr;
+  const hipError_t e = hipModuleLoadData(&module, copy.data());
+  if (e != hipSuccess) {
+    *err = std::string("hipModuleLoadData: ") + hipGetErrorString(e);
+    return MTRT_DRIVER_ERROR;
+  }
+  *out = module;
+  return MTRT_OK;
+}
+
+struct DeviceState {
+  int device = -1;
+  int num_cus = 0;
+  hipModule_t module = nullptr;
+  std::mutex mu;
+  std::unordered_map<std::string, hipFunction_t> funcs;
+  // Two zeroed 32-bit words per stream for single-launch grid reductions, each
+  // slot on its own 64-byte line.  Kernels return their slot to zero.
+  static constexpr int kSlots = 1024;
+  static constexpr int kSlotWords = 16;
+  uint32_t *slots = nullptr;
+  std::map<hipStream_t, int> slot_of;
+  int next_slot = 0;
+};
+
+namespace {
+std::mutex g_mu;
+std::map<int, DeviceState *> g_states;
+} // namespace
+
+DeviceState *device_state() {
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) {
+    set_error(MTRT_RUNTIME_ERROR, "no usable HIP device: %s", hipGetErrorString(e));
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_mu);
+  auto it = g_states.find(device);
+  if (it != g_states.end())
+    return it->second;
+
+  hipDeviceProp_t prop;
+  e = hipGetDeviceProperties(&prop, device);
+  if (e != hipSuccess) {
+    set_error(MTRT_RUNTIME_ERROR, "hipGetDeviceProperties: %s", hipGetErrorString(e));
+    return nullptr;
+  }
+  if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+    set_error(MTRT_RUNTIME_ERROR, "device %d is %s; this library carries gfx950 code only", device,
+              prop.gcnArchName);
+    return nullptr;
+  }
+  auto *st = new DeviceState();
+  st->device = device;
+  st->num_cus = prop.multiProcessorCount;
+  std::string err;
+  const size_t len = size_t(mtrt_hip_hsaco_end - mtrt_hip_hsaco_begin);
+  if (load_code_object(mtrt_hip_hsaco_begin, len, &st->module, &err) != MTRT_OK) {
+    set_error(MTRT_DRIVER_ERROR, "loading the built-in kernel module failed: %s", err.c_str());
+    delete st;
+    return nullptr;
+  }
+  const size_t bytes = size_t(DeviceState::kSlots) * DeviceState::kSlotWords * sizeof(uint32_t);
+  e = hipMalloc(reinterpret_cast<void **>(&st->slots), bytes);
+  if (e == hipSuccess)
+    e = hipMemset(st->slots, 0, bytes);
+  if (e != hipSuccess) {
+    set_error(MTRT_RUNTIME_ERROR, "allocating reduction slots: %s", hipGetErrorString(e));
+    (void)hipModuleUnload(st->module);
+    delete st;
+    return nullptr;
+  }
+  g_states[device] = st;
+  return st;
+}
+
+hipModule_t builtin_module(DeviceState *st) { return st->module; }
+int num_compute_units(DeviceState *st) { return st->num_cus; }
+
+hipFunction_t find_kernel(DeviceState *st, const std::string &name) {
+  std::lock_guard<std::mutex> lock(st->mu);
+  auto it = st->funcs.find(name);
+  if (it != st->funcs.end())
+    return it->second;
+  hipFunction_t f = nullptr;
+  const hipError_t e = hipModuleGetFunction(&f, st->module, name.c_str());
+  if (e != hipSuccess) {
+    set_error(MTRT_NOT_FOUND, "kernel '%s' is not in the built-in module: %s", name.c_str(),
+              hipGetErrorString(e));
+    return nullptr;
+  }
+  st->funcs.emplace(name, f);
+  return f;
+}
+
+uint32_t *reduction_slot(DeviceState *st, hipStream_t stream) {
+  std::lock_guard<std::mutex> lock(st->mu);
+  auto it = st->slot_of.find(stream);
+  int slot;
+  if (it != st->slot_of.end()) {
+    slot = it->second;
+  } else {
+    if (st->next_slot >= DeviceState::kSlots) {
+      set_error(MTRT_RUNTIME_ERROR, "more than %d live streams use grid reductions", DeviceState::kSlots);
+      return nullptr;
+    }
+    slot = st->next_slot++;
+    st->slot_of.emplace(stream, slot);
+  }
+  return st->slots + size_t(slot) * DeviceState::kSlotWords;
+}
+
+void forget_stream(hipStream_t) {
+  // Slots are never reused for a different stream: a destroyed stream's slot is
+  // zero again once its last kernel has finished, but handing it to another stream
+  // before that would race.  1024 slots outlive any realistic stream count.
+}
+
+int32_t launch(DeviceState *st, const std::string &kernel, uint32_t grid, uint32_t block,
+               hipStream_t stream, void **args) {
+  hipFunction_t f = find_kernel(st, kernel);
+  if (!f)
+    return MTRT_NOT_FOUND;
+  const hipError_t e =
+      hipModuleLaunchKernel(f, grid, 1, 1, block, 1, 1, /*sharedMemBytes=*/0, stream, args, nullptr);
+  if (e != hipSuccess)
+    return set_error(MTRT_DRIVER_ERROR, "launching '%s' grid %u block %u: %s", kernel.c_str(), grid,
+                     block, hipGetErrorString(e));
+  std::snprintf(tl_kernel, sizeof(tl_kernel), "%s", kernel.c_str());
+  return MTRT_OK;
+}
+
+const char *last_kernel_name() { return tl_kernel; }
+
+} // namespace mtrt_rt
+
+extern "C" {
+
+const char *mtrt_hip_last_error(void) { return mtrt_rt::last_error(); }
+const char *mtrt_hip_last_kernel(void) { return mtrt_rt::last_kernel_name(); }
+
+int32_t mtrt_hip_init(void) {
+  mtrt_rt::clear_error();
+  return mtrt_rt::device_state() ? MTRT_OK : MTRT_RUNTIME_ERROR;
+}
+
+mtrt_module_t mtrt_hip_builtin_module(void) {
+  mtrt_rt::DeviceState *st = mtrt_rt::device_state();
+  return st ? reinterpret_cast<mtrt_module_t>(mtrt_rt::builtin_module(st)) : nullptr;
+}
+
+const char *mtrt_hip_builtin_code_object(size_t *size) {
+  if (size)
+    *size = size_t(mtrt_hip_hsaco_end - mtrt_hip_hsaco_begin);
+  return mtrt_hip_hsaco_begin;
+}
+
+} // extern "C"

@@ -1,0 +1,43 @@
+// Internal helpers shared by the launch-ABI layer and the cluster layer.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <string>
+#include <vector>
+
+#include "mtrt_hip.h"
+
+namespace mtrt_rt {
+
+inline hipStream_t as_hip(mtrt_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+[[noreturn]] void fatal(const char *file, int line, const char *msg);
+bool read_file(const std::string &path, std::vector<char> &out);
+
+// Thread-local error text for the status-returning entry points.
+int32_t set_error(int32_t code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+void clear_error();
+const char *last_error();
+const char *last_kernel_name();
+
+// Validates that `data` looks like an AMDGPU code object (ELF or clang offload
+// bundle) and loads it on the current device.
+int32_t load_code_object(const char *data, size_t len, hipModule_t *out, std::string *err);
+
+// Per-device state of the cluster layer: the built-in module, a function cache and
+// the pool of two-word reduction slots handed out per stream.
+struct DeviceState;
+DeviceState *device_state();                 // nullptr + set_error on failure
+hipModule_t builtin_module(DeviceState *);
+int num_compute_units(DeviceState *);
+hipFunction_t find_kernel(DeviceState *, const std::string &name);   // nullptr + set_error
+uint32_t *reduction_slot(DeviceState *, hipStream_t stream);         // nullptr + set_error
+void forget_stream(hipStream_t stream);
+
+// Launch through the same driver call as mtrt_cuda_launch_kernel, returning a status.
+int32_t launch(DeviceState *, const std::string &kernel, uint32_t grid, uint32_t block,
+               hipStream_t stream, void **args);
+
+} // namespace mtrt_rt

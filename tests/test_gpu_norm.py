@@ -1,0 +1,165 @@
+"""Parity of the fused LayerNorm and softmax clusters with the CPU oracle.
+
+These are floating-point programs whose reductions the GPU evaluates as trees and
+the host evaluates left to right, so results are compared under a stated tolerance:
+
+  * against the float64 evaluation of the same formula:
+        |got - exact| <= 1e-3 * |exact| + 0.5 ulp_out(exact) + 2e-5 * cond
+    (1e-3 relative is the bar for fp16/bf16 outputs; the half ulp is the rounding every
+    implementation, the oracle included, must commit when it stores the narrow type;
+    `cond` is the magnitude of the terms whose f32 rounding errors the result inherits:
+    |d*rstd*gamma| + |beta| for LayerNorm, where the two can cancel to a result far
+    smaller than either, and 0 for softmax, which has no cancellation);
+  * against the oracle's stored output: at most 1 ulp of the output type (+ the same
+    cond term) apart on every element, and bit-identical on all but a small fraction
+    (a 1e-6 relative difference before the store flips the rounding of about
+    1e-6/2^-9 of bf16 values).  f32 outputs: 2e-5 relative to |exact| + cond.
+"""
+import numpy as np
+import pytest
+
+from helpers import float_storage, rng, to_device_float
+
+pytestmark = pytest.mark.gpu
+
+ULP_REL = {"f32": 2.0 ** -23, "f16": 2.0 ** -10, "bf16": 2.0 ** -7}
+MIN_NORMAL = {"f32": 2.0 ** -126, "f16": 2.0 ** -14, "bf16": 2.0 ** -126}
+
+
+def _x(pkg, orc, name):
+    return {"f32": (pkg.F32, orc.F32), "f16": (pkg.F16, orc.F16), "bf16": (pkg.BF16, orc.BF16)}[name]
+
+
+def _ulp(v, name):
+    """Spacing of the output type at magnitude |v| (subnormal spacing below the least normal)."""
+    a = np.maximum(np.abs(v), MIN_NORMAL[name])
+    return 2.0 ** np.floor(np.log2(a)) * ULP_REL[name]
+
+
+def _compare(orc, name, got_store, ref_store, exact, max_mismatch_frac, cond=None):
+    o = {"f32": orc.F32, "f16": orc.F16, "bf16": orc.BF16}[name]
+    got = orc.widen(got_store, o).astype(np.float64) if o != orc.F32 else got_store.astype(np.float64)
+    ref = orc.widen(ref_store, o).astype(np.float64) if o != orc.F32 else ref_store.astype(np.float64)
+    exact = exact.ravel()
+    slack = 2e-5 * (np.zeros_like(exact) if cond is None else cond.ravel())
+    err = np.abs(got - exact)
+    if name == "f32":
+        bound = 2e-5 * np.abs(exact) + slack + 1e-37
+        assert np.all(err <= bound), "vs float64: max excess %r" % (err - bound).max()
+        assert np.all(np.abs(got - ref) <= 2 * bound)
+        return 0.0
+    ulp = _ulp(exact, name)
+    bound = 1e-3 * np.abs(exact) + 0.5 * ulp * 1.0001 + slack + 1e-45
+    worst = np.argmax(err - bound)
+    assert np.all(err <= bound), "vs float64: element %d got %r exact %r" % (worst, got[worst], exact[worst])
+    d = np.abs(got - ref)
+    assert np.all(d <= _ulp(ref, name) * 1.0001 + 2 * slack), "more than 1 ulp from the oracle: max %r" % d.max()
+    frac = np.count_nonzero(got_store != ref_store) / got_store.size
+    assert frac <= max_mismatch_frac, "fraction of elements not bit-identical to the oracle: %g" % frac
+    return frac
+
+
+def _layernorm_f64(x, g, b, eps):
+    mu = x.mean(axis=1, keepdims=True)
+    d = x - mu
+    var = (d * d).mean(axis=1, keepdims=True)
+    t = d / np.sqrt(var + eps) * g
+    return t + b, np.abs(t) + np.abs(b)
+
+
+def _softmax_f64(x):
+    e = np.exp(x - x.max(axis=1, keepdims=True))
+    return e / e.sum(axis=1, keepdims=True)
+
+
+def _run_layernorm(pkg, orc, name, rows, d, seed, expect_kernel=None, frac=2e-3):
+    p, o = _x(pkg, orc, name)
+    g = rng(seed)
+    x = g.standard_normal((rows, d), dtype=np.float32)
+    gamma = g.uniform(0.5, 1.5, d).astype(np.float32)
+    beta = (g.standard_normal(d, dtype=np.float32) * np.float32(0.1))
+    xd, xs = to_device_float(orc, x, o, "cuda:0")
+    gd, gs = to_device_float(orc, gamma, o, "cuda:0")
+    bd, bs = to_device_float(orc, beta, o, "cuda:0")
+    y = pkg.layernorm(xd, gd, bd, 1e-5)
+    if expect_kernel:
+        assert pkg.last_kernel() == expect_kernel
+    y_ref = orc.layernorm(xs, gs, bs, o, rows, d, 1e-5)
+    w = (lambda a: orc.widen(a, o).astype(np.float64)) if o != orc.F32 else (lambda a: a.astype(np.float64))
+    exact, cond = _layernorm_f64(w(xs).reshape(rows, d), w(gs), w(bs), 1e-5)
+    return _compare(orc, name, float_storage(orc, y, o), y_ref, exact, frac, cond)
+
+
+def _run_softmax(pkg, orc, name, rows, d, seed, expect_kernel=None, frac=2e-2, sigma=2.0):
+    p, o = _x(pkg, orc, name)
+    x = rng(seed).standard_normal((rows, d), dtype=np.float32) * np.float32(sigma)
+    xd, xs = to_device_float(orc, x, o, "cuda:0")
+    y = pkg.softmax(xd)
+    if expect_kernel:
+        assert pkg.last_kernel() == expect_kernel
+    y_ref = orc.softmax(xs, o, rows, d)
+    w = (lambda a: orc.widen(a, o).astype(np.float64)) if o != orc.F32 else (lambda a: a.astype(np.float64))
+    exact = _softmax_f64(w(xs).reshape(rows, d))
+    got = float_storage(orc, y, o)
+    fr = _compare(orc, name, got, y_ref, exact, frac)
+    gotf = w(got).reshape(rows, d)
+    assert np.all(np.abs(gotf.sum(axis=1) - 1.0) < 2e-3 if name != "f32" else np.abs(gotf.sum(axis=1) - 1.0) < 1e-5)
+    return fr
+
+
+def test_c2a_layernorm_bf16_full_size(pkg, orc):
+    """BASELINE config 2a: bf16 [8192,4096], x~N(0,1), gamma~U(0.5,1.5), beta~N(0,0.1), eps 1e-5, seed 2."""
+    orc.set_threads(16)
+    _run_layernorm(pkg, orc, "bf16", 8192, 4096, 2, "mtrt_layernorm_bf16_v8")
+    orc.set_threads(1)
+
+
+def test_c2b_softmax_f16_full_size(pkg, orc):
+    """BASELINE config 2b: f16 [4096,4096], logits ~N(0,4) read as variance 4 (sigma 2), seed 2."""
+    orc.set_threads(16)
+    _run_softmax(pkg, orc, "f16", 4096, 4096, 2, "mtrt_softmax_f16_v8")
+    orc.set_threads(1)
+
+
+@pytest.mark.parametrize("name", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("shape", [(5, 8), (33, 512), (7, 1000), (3, 4104), (2, 8192), (9, 16384), (4, 331), (1, 1), (6, 40000)])
+def test_layernorm_shapes(pkg, orc, name, shape):
+    # Long rows: the host's left-to-right f32 sums drift from the tree sums by a few 1e-6
+    # relative, which moves proportionally more stored values across a rounding boundary.
+    frac = 2e-3 if shape[1] <= 8192 else 2e-2
+    _run_layernorm(pkg, orc, name, shape[0], shape[1], 20 + shape[1] % 97, frac=frac)
+
+
+@pytest.mark.parametrize("name", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("shape", [(5, 8), (33, 512), (7, 1000), (3, 4104), (2, 8192), (9, 16384), (4, 331), (1, 1), (6, 40000)])
+def test_softmax_shapes(pkg, orc, name, shape):
+    _run_softmax(pkg, orc, name, shape[0], shape[1], 40 + shape[1] % 97)
+
+
+def test_kernel_selection(pkg, orc):
+    import torch
+    for d, k in ((512, "v1"), (1024, "v2"), (2048, "v4"), (4096, "v8"), (8192, "v16"), (8200, "any"), (331, "any")):
+        x = torch.randn(4, d, device="cuda", dtype=torch.bfloat16)
+        pkg.softmax(x)
+        assert pkg.last_kernel() == "mtrt_softmax_bf16_" + k
+        pkg.layernorm(x, torch.ones(d, device="cuda", dtype=torch.bfloat16), torch.zeros(d, device="cuda", dtype=torch.bfloat16), 1e-5)
+        assert pkg.last_kernel() == "mtrt_layernorm_bf16_" + k
+    # a row pointer that is not 16-byte aligned falls back to the generic kernel
+    buf = torch.randn(4 * 512 + 1, device="cuda", dtype=torch.bfloat16)
+    pkg.softmax(buf[1:].view(4, 512))
+    assert pkg.last_kernel() == "mtrt_softmax_bf16_any"
+
+
+def test_softmax_extremes_and_empty(pkg, orc):
+    import torch
+    # widely spread logits: the largest entry dominates, tiny ones underflow to 0 or f16 subnormals
+    _run_softmax(pkg, orc, "f16", 16, 4096, 5, sigma=8.0)
+    _run_softmax(pkg, orc, "f32", 16, 1024, 6, sigma=30.0)
+    x = torch.full((3, 256), -7.0, device="cuda", dtype=torch.float32)
+    y = pkg.softmax(x)
+    assert torch.equal(y, torch.full_like(y, 1.0 / 256))
+    assert pkg.softmax(torch.empty((0, 64), device="cuda")).numel() == 0
+    z = torch.zeros((2, 128), device="cuda", dtype=torch.bfloat16)
+    out = pkg.layernorm(z, torch.ones(128, device="cuda", dtype=torch.bfloat16),
+                        torch.full((128,), 0.5, device="cuda", dtype=torch.bfloat16), 1e-5)
+    assert torch.equal(out, torch.full_like(out, 0.5))

@@ -1,0 +1,278 @@
+"""Parity of the amax / quantize / dequantize clusters with the CPU oracle, through
+the C ABI.  Bar: BIT-EXACT for amax, scale, every quantized code and every
+dequantized value (each is a single correctly-rounded f32 op chain followed by one
+narrowing, so there is nothing to tolerate)."""
+import numpy as np
+import pytest
+
+from helpers import bits16, f32_bits, float_storage, rng, to_device_float, torch_dtype_of
+
+pytestmark = pytest.mark.gpu
+
+QMAX = {"i8": 127.0, "f8": 448.0, "i4": 7.0, "i4p": 7.0}
+
+
+def _q(pkg, orc, name):
+    return {"i8": (pkg.I8, orc.I8), "f8": (pkg.F8E4M3FN, orc.F8E4M3FN), "i4": (pkg.I4, orc.I4),
+            "i4p": (pkg.I4_PACKED, orc.I4_PACKED)}[name]
+
+
+def _x(pkg, orc, name):
+    return {"f32": (pkg.F32, orc.F32), "f16": (pkg.F16, orc.F16), "bf16": (pkg.BF16, orc.BF16)}[name]
+
+
+def _codes_np(q):
+    return q.cpu().numpy().view(np.uint8).ravel()
+
+
+def _check_all(pkg, orc, x_f32, xname, qname, kind, d0, d1, nb, scale_np, flags=0, mode=None, misalign=0):
+    """Runs Q, DQ and fused Q+DQ on the GPU and compares all outputs with the oracle."""
+    import torch
+    p_x, o_x = _x(pkg, orc, xname)
+    p_q, o_q = _q(pkg, orc, qname)
+    mode = orc.IEEE if mode is None else mode
+    dev = torch.device("cuda:0")
+    n = d0 * d1
+    if misalign:
+        # place the data `misalign` elements into a larger buffer so no pointer is 16-byte aligned
+        pad = np.zeros(misalign, dtype=np.float32)
+        full, _ = to_device_float(orc, np.concatenate([pad, x_f32.ravel()]), o_x, dev)
+        x_dev = full[misalign:]
+        _, x_store = to_device_float(orc, x_f32.ravel(), o_x, "cpu")
+    else:
+        x_dev, x_store = to_device_float(orc, x_f32.reshape(d0, d1), o_x, dev)
+    scale_dev = torch.from_numpy(np.ascontiguousarray(scale_np, dtype=np.float32)).to(dev)
+    oflags = orc.Q_ROUND_TO_INT if (flags & pkg.Q_ROUND_TO_INT) else 0
+
+    q_ref = orc.quantize(x_store, o_x, o_q, scale_np, kind, d0, d1, nb, oflags, mode)
+    y_ref = orc.dequantize(q_ref, o_q, o_x, scale_np, kind, d0, d1, nb, mode)
+
+    if misalign:
+        qbuf = pkg.code_tensor(p_q, n + 2 * misalign + 2, dev)
+        q_out = qbuf[misalign:] if p_q != pkg.I4_PACKED else qbuf[1:]
+        ybuf = torch.zeros(n + misalign, dtype=torch_dtype_of(orc, o_x), device=dev)
+        y_out = ybuf[misalign:]
+    else:
+        q_out = y_out = None
+    nbytes = q_ref.size
+
+    q = pkg.quantize(x_dev, scale_dev, p_q, kind, d0, d1, nb, flags, out=q_out)
+    k_q = pkg.last_kernel()
+    assert np.array_equal(_codes_np(q)[:nbytes], q_ref.view(np.uint8)), "quantize codes (%s)" % k_q
+
+    y = pkg.dequantize(q, scale_dev, p_q, torch_dtype_of(orc, o_x), (n,), kind, d0, d1, nb, out=y_out)
+    k_dq = pkg.last_kernel()
+    got = float_storage(orc, y, o_x)[:n]
+    assert np.array_equal(got.view(np.uint8), y_ref.view(np.uint8)), "dequantize values (%s)" % k_dq
+
+    q2_out = None if q_out is None else torch.zeros_like(q_out)
+    y2_out = None if y_out is None else torch.zeros_like(y_out)
+    q2, y2 = pkg.quantize_dequantize(x_dev, scale_dev, p_q, kind, d0, d1, nb, flags, q_out=q2_out, y_out=y2_out)
+    k_f = pkg.last_kernel()
+    assert np.array_equal(_codes_np(q2)[:nbytes], q_ref.view(np.uint8)), "fused codes (%s)" % k_f
+    got2 = float_storage(orc, y2, o_x)[:n]
+    assert np.array_equal(got2.view(np.uint8), y_ref.view(np.uint8)), "fused values (%s)" % k_f
+    return k_q, k_dq, k_f
+
+
+def test_c1_per_tensor_int8_full_size(pkg, orc):
+    """BASELINE config 1: f32 [1024,4096] ~N(0,1) seed 1, scale = amax/127."""
+    import torch
+    x = rng(1).standard_normal((1024, 4096), dtype=np.float32)
+    xd = torch.from_numpy(x).cuda()
+    amax, scale = pkg.amax(xd, 127.0)
+    amax_ref = orc.amax(x, orc.F32)
+    scale_ref = orc.scale_from_amax(amax_ref, 127.0)
+    assert f32_bits(amax.cpu().numpy())[0] == f32_bits(amax_ref)[0]
+    assert f32_bits(scale.cpu().numpy())[0] == f32_bits(scale_ref)[0]
+    assert amax_ref == np.abs(x).max()      # closed form
+    kq, kdq, kf = _check_all(pkg, orc, x, "f32", "i8", pkg.SCALE_UNIFORM, 1024, 4096, 1, [scale_ref])
+    assert kq == "mtrt_q_uniform_f32_i8" and kdq == "mtrt_dq_uniform_f32_i8" and kf == "mtrt_qdq_uniform_f32_i8"
+    # the largest magnitude maps to +-127 exactly
+    q = pkg.quantize(xd, scale.reshape(1), pkg.I8)
+    assert int(q.abs().max()) == 127
+
+
+def test_c3_dynamic_fp8_full_size(pkg, orc):
+    """BASELINE config 3: bf16 [16384,8192] ~N(0,2) (variance 2), 0.1% of entries x50, seed 3."""
+    import torch
+    g = rng(3)
+    rows, cols = 16384, 8192
+    x = g.standard_normal((rows, cols), dtype=np.float32) * np.float32(np.sqrt(2.0))
+    x[g.random((rows, cols), dtype=np.float32) < 0.001] *= np.float32(50.0)
+    orc.set_threads(16)
+    xd, xs = to_device_float(orc, x, orc.BF16, "cuda:0")
+    del x
+    amax, scale = pkg.amax(xd, 448.0)
+    amax_ref = orc.amax(xs, orc.BF16)
+    scale_ref = orc.scale_from_amax(amax_ref, 448.0)
+    assert f32_bits(amax.cpu().numpy())[0] == f32_bits(amax_ref)[0]
+    assert f32_bits(scale.cpu().numpy())[0] == f32_bits(scale_ref)[0]
+    for flags, mode in ((0, orc.IEEE), (pkg.F8_REFHOST, orc.REFHOST)):
+        q, y = pkg.quantize_dequantize(xd, scale.reshape(1), pkg.F8E4M3FN, flags=flags)
+        assert pkg.last_kernel() == "mtrt_qdq_uniform_bf16_f8"
+        q_ref = orc.quantize(xs, orc.BF16, orc.F8E4M3FN, [scale_ref], orc.SCALE_UNIFORM, rows, cols, 1, 0, mode)
+        assert np.array_equal(_codes_np(q), q_ref), "fp8 codes, mode %d" % mode
+        y_ref = orc.dequantize(q_ref, orc.F8E4M3FN, orc.BF16, [scale_ref], orc.SCALE_UNIFORM, rows, cols, 1, mode)
+        assert np.array_equal(bits16(y), y_ref), "bf16 dequantized values, mode %d" % mode
+        del q, y, q_ref, y_ref
+    orc.set_threads(1)
+
+
+@pytest.mark.parametrize("xname", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("qname", ["i8", "f8", "i4", "i4p"])
+@pytest.mark.parametrize("shape", [(64, 1024), (37, 515), (1, 1), (1, 15), (3, 16)])
+def test_per_tensor_all_type_pairs(pkg, orc, xname, qname, shape):
+    d0, d1 = shape
+    g = rng(100 + d0 + d1)
+    x = g.standard_normal((d0, d1), dtype=np.float32) * np.float32(3.0)
+    _, o_x = _x(pkg, orc, xname)
+    xs = orc.narrow(x, o_x) if o_x != orc.F32 else x
+    scale = orc.scale_from_amax(orc.amax(xs, o_x), QMAX[qname])
+    _check_all(pkg, orc, x, xname, qname, pkg.SCALE_UNIFORM, d0, d1, 1, [scale])
+
+
+@pytest.mark.parametrize("xname", ["f32", "bf16"])
+@pytest.mark.parametrize("qname", ["i8", "f8", "i4p"])
+def test_misaligned_pointers_take_the_any_kernels(pkg, orc, xname, qname):
+    d0, d1 = 5, 333
+    x = rng(7).standard_normal((d0, d1), dtype=np.float32)
+    kq, kdq, kf = _check_all(pkg, orc, x, xname, qname, pkg.SCALE_UNIFORM, d0, d1, 1, [np.float32(0.05)], misalign=1)
+    assert "_any_" in kq and "_any_" in kdq and "_any_" in kf
+
+
+@pytest.mark.parametrize("xname", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("qname", ["i8", "f8"])
+def test_per_channel(pkg, orc, xname, qname):
+    g = rng(11)
+    # axis 0 of [48, 256]  -> rows carry the scale
+    x = g.standard_normal((48, 256), dtype=np.float32)
+    s = g.uniform(0.005, 0.05, 48).astype(np.float32)
+    k = _check_all(pkg, orc, x, xname, qname, pkg.SCALE_ROW, 48, 256, 48, s)
+    assert "_row_" in k[0]
+    # last axis of [48, 256] -> columns carry the scale (one block of d0 rows)
+    s = g.uniform(0.005, 0.05, 256).astype(np.float32)
+    k = _check_all(pkg, orc, x, xname, qname, pkg.SCALE_COL, 48, 256, 48, s)
+    assert "_col_" in k[0]
+    # middle axis of [4, 6, 128] -> d0 = 24 rows, scale index = row % 6
+    x = g.standard_normal((4, 6, 128), dtype=np.float32)
+    s = g.uniform(0.005, 0.05, 6).astype(np.float32)
+    _check_all(pkg, orc, x, xname, qname, pkg.SCALE_ROW, 24, 128, 6, s)
+    # ragged inner extent -> generic kernel
+    x = g.standard_normal((7, 5, 9), dtype=np.float32)
+    s = g.uniform(0.005, 0.05, 5).astype(np.float32)
+    k = _check_all(pkg, orc, x, xname, qname, pkg.SCALE_ROW, 35, 9, 5, s)
+    assert "_any_" in k[0]
+    s = g.uniform(0.005, 0.05, 9).astype(np.float32)
+    k = _check_all(pkg, orc, x, xname, qname, pkg.SCALE_COL, 35, 9, 35, s)
+    assert "_any_" in k[0]
+
+
+@pytest.mark.parametrize("xname", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("qname", ["i4", "i4p"])
+def test_int4_blockwise(pkg, orc, xname, qname):
+    g = rng(13)
+    # blocks of 128 rows along axis 0 (the weight layout of config 5: scale [K/128, N])
+    x = g.standard_normal((512, 192), dtype=np.float32) * np.float32(0.1)
+    s = g.uniform(0.005, 0.02, (4, 192)).astype(np.float32)
+    k = _check_all(pkg, orc, x, xname, qname, pkg.SCALE_COL, 512, 192, 128, s.ravel())
+    assert "_col_" in k[0]
+    # blocks of 128 along the last axis: [64, 512] with scale [64, 4] -> rows of one block each
+    x = g.standard_normal((64, 512), dtype=np.float32) * np.float32(0.1)
+    s = g.uniform(0.005, 0.02, (64, 4)).astype(np.float32)
+    k = _check_all(pkg, orc, x, xname, qname, pkg.SCALE_ROW, 64 * 4, 128, 64 * 4, s.ravel())
+    assert "_row_" in k[0]
+    # tiny blocks, odd column count -> generic kernel (pairs of nibbles straddle rows)
+    x = g.standard_normal((6, 7), dtype=np.float32)
+    s = g.uniform(0.1, 0.3, (3, 7)).astype(np.float32)
+    k = _check_all(pkg, orc, x, xname, qname, pkg.SCALE_COL, 6, 7, 2, s.ravel())
+    assert "_any_" in k[0]
+
+
+def test_ties_saturation_and_special_values(pkg, orc):
+    """Inputs that land exactly on k+0.5 after the divide, beyond the clamp, on signed
+    zeros and on subnormals; scale chosen so that x/scale is exact."""
+    s = np.float32(0.25)
+    ks = np.arange(-140, 141, dtype=np.float32)
+    x = np.concatenate([(ks + 0.5) * s, ks * s, (ks + 0.25) * s, np.float32([0.0, -0.0, 1e-40, -1e-40, 3e38, -3e38,
+                        np.nextafter(np.float32(0.125), np.float32(1)), np.nextafter(np.float32(0.125), np.float32(0))])])
+    x = np.resize(x, (1, 1024)).astype(np.float32)
+    for qname in ("i8", "i4", "i4p", "f8"):
+        _check_all(pkg, orc, x, "f32", qname, pkg.SCALE_UNIFORM, 1, 1024, 1, [s])
+    # closed form for the int8 codes: numpy's rint is round-half-even too
+    import torch
+    q = pkg.quantize(torch.from_numpy(x).cuda(), torch.tensor([s], device="cuda"), pkg.I8)
+    expect = np.clip(np.rint(x / s), -128, 127).astype(np.int8)
+    assert np.array_equal(q.cpu().numpy(), expect.ravel())
+
+
+@pytest.mark.parametrize("flags_mode", [(0, 0), (1, 0), (2, 1), (3, 1)])
+def test_fp8_every_f16_value_and_random_f32(pkg, orc, flags_mode):
+    """f32 -> f8E4M3FN through the quantize kernel with scale 1: every finite f16 value
+    (covers every tie and the whole subnormal range of f8) plus random f32 bit patterns,
+    in the IEEE and the reference-host behaviours, with and without the integer rounding."""
+    flags, mode = flags_mode
+    all_f16 = orc.widen(np.arange(65536, dtype=np.uint16), orc.F16)
+    all_f16 = all_f16[np.isfinite(all_f16)]
+    g = rng(17)
+    rnd = g.integers(0, 2**32, 1 << 20, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    rnd = rnd[np.isfinite(rnd)]
+    near = np.float32([0.0146484375, 0.015625, 0.01513671875, 247.99998, 248.0, 255.9, 256.0, 447.9, 448.0, 464.0, 1e9])
+    near = np.concatenate([near, -near, np.nextafter(near, np.float32(0)), np.nextafter(near, np.float32(np.inf))])
+    x = np.concatenate([all_f16, rnd, near]).astype(np.float32)
+    x = x[: (x.size // 16) * 16 + 5]
+    _check_all(pkg, orc, x, "f32", "f8", pkg.SCALE_UNIFORM, 1, x.size, 1, [np.float32(1.0)], flags=flags, mode=mode)
+
+
+def test_all_zero_tensor_and_empty(pkg, orc):
+    import torch
+    x = np.zeros((4, 64), dtype=np.float32)
+    xd = torch.from_numpy(x).cuda()
+    amax, scale = pkg.amax(xd, 127.0)
+    assert float(amax) == 0.0 and float(scale) == 0.0
+    # 0/0 is NaN on both sides; min/max drop the NaN and the code saturates the same way
+    _check_all(pkg, orc, x, "f32", "i8", pkg.SCALE_UNIFORM, 4, 64, 1, [np.float32(0.0)])
+    empty = torch.empty((0, 128), dtype=torch.float32, device="cuda")
+    q = pkg.quantize(empty, torch.ones(1, device="cuda"), pkg.I8)
+    assert q.numel() == 0
+    a, s = pkg.amax(empty, 127.0)
+    assert float(a) == 0.0
+
+
+@pytest.mark.parametrize("xname", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("n", [1, 7, 4096, 4099, 1 << 22, (1 << 22) + 13])
+def test_amax_sizes_alignments(pkg, orc, xname, n):
+    import torch
+    _, o_x = _x(pkg, orc, xname)
+    x = rng(n % 1000).standard_normal(n + 3, dtype=np.float32)
+    x[n // 2] = 77.25
+    for off in (0, 1, 3):
+        xd, xs = to_device_float(orc, x, o_x, "cuda:0")
+        amax, scale = pkg.amax(xd[off:off + n], 448.0)
+        ref = orc.amax(np.ascontiguousarray(xs[off:off + n]), o_x)
+        assert f32_bits(amax.cpu().numpy())[0] == f32_bits(ref)[0]
+        assert f32_bits(scale.cpu().numpy())[0] == f32_bits(orc.scale_from_amax(ref, 448.0))[0]
+    # back-to-back launches reuse the self-resetting reduction slot
+    a1, _ = pkg.amax(xd[:n], 1.0)
+    a2, _ = pkg.amax(xd[:n], 1.0)
+    assert float(a1) == float(a2)
+
+
+def test_invalid_arguments_are_reported(pkg):
+    import torch
+    L = pkg.lib()
+    x = torch.zeros(64, device="cuda")
+    q = torch.zeros(64, dtype=torch.int8, device="cuda")
+    s = torch.ones(1, device="cuda")
+    st = L.mtrt_hip_quantize(None, x.data_ptr(), pkg.I8, q.data_ptr(), pkg.I8, s.data_ptr(), 0, 1, 64, 1, 0)
+    assert st == 1 and b"f32/f16/bf16" in L.mtrt_hip_last_error()
+    st = L.mtrt_hip_quantize(None, x.data_ptr(), pkg.F32, q.data_ptr(), pkg.F32, s.data_ptr(), 0, 1, 64, 1, 0)
+    assert st == 1 and b"quantized dtype" in L.mtrt_hip_last_error()
+    st = L.mtrt_hip_quantize(None, x.data_ptr(), pkg.F32, q.data_ptr(), pkg.I8, s.data_ptr(), 2, 6, 8, 4, 0)
+    assert st == 1 and b"does not divide" in L.mtrt_hip_last_error()
+    st = L.mtrt_hip_quantize(None, x.data_ptr(), pkg.F32, None, pkg.I8, s.data_ptr(), 0, 1, 64, 1, 0)
+    assert st == 1 and b"null" in L.mtrt_hip_last_error()
+    st = L.mtrt_hip_quantize(None, x.data_ptr(), pkg.F32, q.data_ptr(), pkg.I8, s.data_ptr(), 0, 1, 64, 1, 64)
+    assert st == 1 and b"flag" in L.mtrt_hip_last_error()
+    st = L.mtrt_hip_amax(None, x.data_ptr(), pkg.I8, 64, 1.0, None, None)
+    assert st == 1
