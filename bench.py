@@ -1,0 +1,288 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantization / generated-kernel hot path on ONE MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|c1|c2a|c2b|c3|c4|c5]
+
+A STEP is one pass of the hot path over one batch of seeded synthetic input: the
+programs of BASELINE.json's configs run back to back through the C ABI
+(libmtrt_hip.so) on tensors already resident in HBM:
+    C1  amax + fused quantize->dequantize   f32 [1024,4096] -> i8          (per-tensor, amax/127)
+    C2a LayerNorm                           bf16 [8192,4096]
+    C2b softmax                             f16 [4096,4096]
+    C3  amax + fused quantize->dequantize   bf16 [16384,8192] -> f8E4M3FN  (amax/448)
+    C4  W8A8 GEMM                           M=2048 K=4096 N=11008          (when built)
+    C5  W4A16 GEMM                          M in {16,256,4096}             (when built)
+The metric is BASELINE.json's: achieved HBM GB/s (memory-bound kernels) and MFMA
+TOPS (GEMMs) as a percentage of MI355X peak.  For a step that mixes both, `value`
+is the time-weighted percentage: 100 * (sum over kernels of the time the kernel
+would take at its roofline peak, on its ALGORITHMIC bytes or ops) / (measured time
+of the step).  Peaks: HBM 8 TB/s, int8 MFMA 5 POP/s, f16 MFMA 2.5 PFLOP/s.
+Every kernel also gets its own line under "workloads" (achieved, peak, fraction),
+timed with HIP events on the launch stream over rotating buffers whose combined
+footprint exceeds the 256 MiB Infinity Cache, so cache hits do not count as HBM.
+"roofline" repeats the entry of the kernel with the largest share of the step.
+"cpu_baseline" times the CPU oracle (a C++ restatement of the reference's host
+lowering, NOT the reference binary) on a bounded sample, single-threaded like the
+reference interpreter, and extrapolates linearly to the step.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+import __graft_entry__ as entry  # noqa: E402
+
+HBM_PEAK = 8000.0       # GB/s
+INT8_PEAK = 5000.0      # TOP/s dense
+F16_PEAK = 2500.0       # TFLOP/s dense
+CACHE_BYTES = 512 << 20  # rotate buffers over at least this much
+
+
+def build_workloads(pkg, torch, which):
+    """Returns a list of kernel descriptors.  Each has: name (kernel symbol or short label),
+    config, bound ('hbm'|'mfma'), work (algorithmic bytes or ops per launch), peak, unit,
+    make(slot) -> zero-argument callable that enqueues one launch on buffer set `slot`, nslots."""
+    L = pkg.lib()
+    dev = torch.device("cuda:0")
+    out = []
+
+    def stream():
+        return torch.cuda.current_stream().cuda_stream
+
+    def gen(shape, dtype, seed, scale=1.0):
+        g = torch.Generator(device=dev)
+        g.manual_seed(seed)
+        return (torch.randn(shape, generator=g, device=dev, dtype=torch.float32) * scale).to(dtype)
+
+    def slots_for(bytes_per_set):
+        return max(2, int(np.ceil(CACHE_BYTES / bytes_per_set)))
+
+    if which in ("all", "c1"):
+        n = 1024 * 4096
+        ns = slots_for(n * 9)
+        x1 = [gen((1024, 4096), torch.float32, 1 + i) for i in range(ns)]
+        q1 = [torch.empty(n, dtype=torch.int8, device=dev) for _ in range(ns)]
+        y1 = [torch.empty_like(x) for x in x1]
+        s1 = [torch.empty(2, dtype=torch.float32, device=dev) for _ in range(ns)]
+
+        def amax(i, xs=x1, sc=s1, n=n):
+            a = (xs[i].data_ptr(), pkg.F32, n, 127.0, sc[i].data_ptr(), sc[i].data_ptr() + 4)
+            return lambda: pkg.check(L.mtrt_hip_amax(stream(), *a))
+
+        def qdq(i, xs=x1, qs=q1, ys=y1, sc=s1):
+            a = (xs[i].data_ptr(), pkg.F32, qs[i].data_ptr(), pkg.I8, ys[i].data_ptr(), sc[i].data_ptr() + 4,
+                 pkg.SCALE_UNIFORM, 1024, 4096, 1, 0)
+            return lambda: pkg.check(L.mtrt_hip_quantize_dequantize(stream(), *a))
+        xs, qs, ys, sc = x1, q1, y1, s1
+        out.append(dict(name="mtrt_amax_f32", config="C1", bound="hbm", work=4.0 * n, nslots=ns, make=amax, keep=(xs, sc)))
+        out.append(dict(name="mtrt_qdq_uniform_f32_i8", config="C1", bound="hbm", work=9.0 * n, nslots=ns, make=qdq,
+                        keep=(qs, ys)))
+
+    if which in ("all", "c2a"):
+        rows, d = 8192, 4096
+        ns = slots_for(rows * d * 4)
+        xs = [gen((rows, d), torch.bfloat16, 20 + i) for i in range(ns)]
+        ys = [torch.empty_like(x) for x in xs]
+        gamma = (torch.rand(d, device=dev) + 0.5).to(torch.bfloat16)
+        beta = (torch.randn(d, device=dev) * 0.1).to(torch.bfloat16)
+
+        def ln(i, xs=xs, ys=ys, rows=rows, d=d, gamma=gamma, beta=beta):
+            a = (xs[i].data_ptr(), gamma.data_ptr(), beta.data_ptr(), ys[i].data_ptr(), pkg.BF16, rows, d, 1e-5)
+            return lambda: pkg.check(L.mtrt_hip_layernorm(stream(), *a))
+        out.append(dict(name="mtrt_layernorm_bf16_v8", config="C2a", bound="hbm", work=4.0 * rows * d + 4.0 * d,
+                        nslots=ns, make=ln, keep=(xs, ys, gamma, beta)))
+
+    if which in ("all", "c2b"):
+        rows, d = 4096, 4096
+        ns = slots_for(rows * d * 4)
+        xs = [gen((rows, d), torch.float16, 40 + i, 2.0) for i in range(ns)]
+        ys = [torch.empty_like(x) for x in xs]
+
+        def sm(i, xs=xs, ys=ys, rows=rows, d=d):
+            a = (xs[i].data_ptr(), ys[i].data_ptr(), pkg.F16, rows, d)
+            return lambda: pkg.check(L.mtrt_hip_softmax(stream(), *a))
+        out.append(dict(name="mtrt_softmax_f16_v8", config="C2b", bound="hbm", work=4.0 * rows * d, nslots=ns, make=sm,
+                        keep=(xs, ys)))
+
+    if which in ("all", "c3"):
+        rows, cols = 16384, 8192
+        n = rows * cols
+        ns = 2
+        xs = []
+        for i in range(ns):
+            x = gen((rows, cols), torch.float32, 60 + i, float(np.sqrt(2.0)))
+            g = torch.Generator(device=dev)
+            g.manual_seed(600 + i)
+            x[torch.rand((rows, cols), generator=g, device=dev) < 0.001] *= 50.0
+            xs.append(x.to(torch.bfloat16))
+            del x
+        qs = [torch.empty(n, dtype=torch.uint8, device=dev) for _ in range(ns)]
+        ys = [torch.empty_like(x) for x in xs]
+        sc = [torch.empty(2, dtype=torch.float32, device=dev) for _ in range(ns)]
+
+        def amax(i, xs=xs, sc=sc, n=n):
+            a = (xs[i].data_ptr(), pkg.BF16, n, 448.0, sc[i].data_ptr(), sc[i].data_ptr() + 4)
+            return lambda: pkg.check(L.mtrt_hip_amax(stream(), *a))
+
+        def qdq(i, xs=xs, qs=qs, ys=ys, sc=sc, rows=rows, cols=cols):
+            a = (xs[i].data_ptr(), pkg.BF16, qs[i].data_ptr(), pkg.F8E4M3FN, ys[i].data_ptr(), sc[i].data_ptr() + 4,
+                 pkg.SCALE_UNIFORM, rows, cols, 1, 0)
+            return lambda: pkg.check(L.mtrt_hip_quantize_dequantize(stream(), *a))
+        out.append(dict(name="mtrt_amax_bf16", config="C3", bound="hbm", work=2.0 * n, nslots=ns, make=amax, keep=(xs, sc)))
+        out.append(dict(name="mtrt_qdq_uniform_bf16_f8", config="C3", bound="hbm", work=5.0 * n, nslots=ns, make=qdq,
+                        keep=(qs, ys)))
+
+    for w in out:
+        w["peak"] = HBM_PEAK if w["bound"] == "hbm" else w["peak"]
+        w["unit"] = "GB/s" if w["bound"] == "hbm" else w["unit"]
+    return out
+
+
+def time_kernel(pkg, torch, w, reps):
+    """Average launch duration in microseconds, HIP events on the launch stream."""
+    L = pkg.lib()
+    dev = L.mtrt_cuda_get_current_device()
+    calls = [w["make"](i) for i in range(w["nslots"])]
+    s = torch.cuda.current_stream().cuda_stream
+    for c in calls:
+        c()
+    e0, e1 = L.mtrt_cuda_event_create(dev), L.mtrt_cuda_event_create(dev)
+    L.mtrt_cuda_stream_sync(s)
+    L.mtrt_cuda_stream_record_event(s, e0)
+    for r in range(reps):
+        calls[r % len(calls)]()
+    L.mtrt_cuda_stream_record_event(s, e1)
+    L.mtrt_cuda_event_sync(e1)
+    us = L.mtrt_cuda_event_elapsed_msec(e0, e1) * 1e3 / reps
+    L.mtrt_cuda_event_release(e0)
+    L.mtrt_cuda_event_release(e1)
+    return us
+
+
+def cpu_baseline(which):
+    """Times the CPU oracle single-threaded on a bounded sample of each program and
+    extrapolates linearly to the full configuration; returns (seconds per step, description)."""
+    orc = entry.load_oracle()
+    orc.set_threads(1)
+    g = np.random.Generator(np.random.PCG64(1))
+    total = 0.0
+    parts = []
+
+    def timed(fn):
+        t0 = time.perf_counter()
+        fn()
+        return time.perf_counter() - t0
+
+    if which in ("all", "c1"):
+        x = g.standard_normal((1024, 4096), dtype=np.float32)
+        t = timed(lambda: orc.amax(x, orc.F32))
+        s = [orc.scale_from_amax(orc.amax(x, orc.F32), 127.0)]
+        q = orc.quantize(x, orc.F32, orc.I8, s, orc.SCALE_UNIFORM, 1024, 4096)
+        t += timed(lambda: orc.quantize(x, orc.F32, orc.I8, s, orc.SCALE_UNIFORM, 1024, 4096))
+        t += timed(lambda: orc.dequantize(q, orc.I8, orc.F32, s, orc.SCALE_UNIFORM, 1024, 4096))
+        total += t
+        parts.append("C1 full")
+    if which in ("all", "c2a"):
+        rows = 1024
+        x = orc.narrow(g.standard_normal((rows, 4096), dtype=np.float32), orc.BF16)
+        gm = orc.narrow(g.uniform(0.5, 1.5, 4096).astype(np.float32), orc.BF16)
+        bt = orc.narrow((g.standard_normal(4096) * 0.1).astype(np.float32), orc.BF16)
+        total += timed(lambda: orc.layernorm(x, gm, bt, orc.BF16, rows, 4096, 1e-5)) * (8192 / rows)
+        parts.append("C2a %d of 8192 rows" % rows)
+    if which in ("all", "c2b"):
+        rows = 512
+        x = orc.narrow(g.standard_normal((rows, 4096), dtype=np.float32) * 2, orc.F16)
+        total += timed(lambda: orc.softmax(x, orc.F16, rows, 4096)) * (4096 / rows)
+        parts.append("C2b %d of 4096 rows" % rows)
+    if which in ("all", "c3"):
+        rows = 1024
+        x = orc.narrow(g.standard_normal((rows, 8192), dtype=np.float32) * np.float32(1.414), orc.BF16)
+        t = timed(lambda: orc.amax(x, orc.BF16))
+        s = [orc.scale_from_amax(orc.amax(x, orc.BF16), 448.0)]
+        q = orc.quantize(x, orc.BF16, orc.F8E4M3FN, s, orc.SCALE_UNIFORM, rows, 8192)
+        t += timed(lambda: orc.quantize(x, orc.BF16, orc.F8E4M3FN, s, orc.SCALE_UNIFORM, rows, 8192))
+        t += timed(lambda: orc.dequantize(q, orc.F8E4M3FN, orc.BF16, s, orc.SCALE_UNIFORM, rows, 8192))
+        total += t * (16384 / rows)
+        parts.append("C3 %d of 16384 rows" % rows)
+    return total, ", ".join(parts)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="all", choices=["all", "c1", "c2a", "c2b", "c3"])
+    ap.add_argument("--kernel-reps", type=int, default=100, help="launches per kernel for the per-kernel timing")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: every box of this build has one, and the hot path has no "
+              "collective to time; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (there is no CPU fallback for the product path)", file=sys.stderr)
+        sys.exit(2)
+    pkg = entry.load_package()
+    pkg.check(pkg.lib().mtrt_hip_init())
+    torch.cuda.set_device(0)
+
+    wl = build_workloads(pkg, torch, args.workload)
+    # the step: every kernel once, in program order, on buffer set (step % nslots)
+    step_calls = [[w["make"](i) for i in range(w["nslots"])] for w in wl]
+
+    def run_step(k):
+        for calls in step_calls:
+            calls[k % len(calls)]()
+
+    for k in range(args.warmup):
+        run_step(k)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        run_step(k)
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    ideal_us = 0.0
+    kernels = []
+    for w in wl:
+        us = time_kernel(pkg, torch, w, args.kernel_reps)
+        achieved = w["work"] / us / 1e3 if w["bound"] == "hbm" else w["work"] / us / 1e6
+        ideal = w["work"] / (w["peak"] * 1e3) if w["bound"] == "hbm" else w["work"] / (w["peak"] * 1e6)
+        ideal_us += ideal
+        kernels.append(dict(kernel=w["name"], config=w["config"], bound=w["bound"], us=round(us, 2),
+                            achieved=round(achieved, 1), peak=w["peak"], unit=w["unit"], frac=round(achieved / w["peak"], 4),
+                            work=w["work"]))
+    value = 100.0 * (ideal_us / 1e3) / ms_per_step
+    dom = max(kernels, key=lambda k: k["us"])
+    line = {
+        "metric": "Q/DQ+reduce HBM GB/s and W8A8/W4A16 GEMM TOPS, as % of MI355X peak, 1 GPU",
+        "value": round(value, 2),
+        "unit": "% of MI355X peak (time-weighted over the step's kernels)",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32/bf16/f16 -> i8/f8e4m3fn (f32 arithmetic)", "data": "synthetic (seeded)",
+        "config": {"workload": {"all": "C1+C2a+C2b+C3 programs of BASELINE.json, one pass each per step"}.get(
+            args.workload, args.workload.upper()), "kernels_per_step": len(wl)},
+        "roofline": {"kernel": dom["kernel"], "bound": dom["bound"], "achieved": dom["achieved"], "peak": dom["peak"],
+                     "unit": dom["unit"], "frac": dom["frac"], "traffic": None},
+        "workloads": kernels,
+    }
+    if not args.no_cpu_baseline:
+        cpu_s, sample = cpu_baseline(args.workload)
+        line["cpu_baseline"] = {"value": round(100.0 * (ideal_us / 1e6) / cpu_s, 6),
+                                "unit": "% of MI355X peak (same definition)", "cores": 1, "kind": "port",
+                                "sample": sample + "; extrapolated linearly", "seconds_per_step": round(cpu_s, 3)}
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -10,7 +10,7 @@
 // (mlir-tensorrt/kernel/lib/Utils/TilingUtils.cpp:669-677); here the tensor is
 // streamed once with 128-bit loads by a grid sized to the chip, reduced per wave
 // with cross-lane exchanges, per workgroup through LDS, and across workgroups with
-// one device-scope atomic max per workgroup.  max is exact under any order, so the
+// a two-level tree of device-scope atomic max operations.  max is exact under any order, so the
 // result is bit-identical to the sequential host reduction.
 //
 // abs/max run on the BIT PATTERN: for non-NaN floats, |x| orders like the unsigned
@@ -19,9 +19,9 @@
 // (its pattern is the largest), unlike the host's std::max which would drop it
 // (CoreModule.cpp:540-551); the programs this serves are NaN-free.
 //
-// scratch: two 32-bit words owned by the caller's stream (running max, arrival
-// ticket), both zero on entry; the last workgroup to arrive publishes the results
-// and restores the zeros, so back-to-back launches on one stream need no memset.
+// scratch: (1 + 32) lines of 128 bytes owned by the caller's stream, each holding a
+// (running max, arrival ticket) pair, all zero on entry; whoever arrives last at a
+// pair restores its zeros, so back-to-back launches on one stream need no memset.
 #include "common.hpp"
 
 using namespace mtrt_dev;
@@ -30,6 +30,8 @@ namespace amax_cluster {
 
 constexpr int kAmaxThreads = 256;
 constexpr int kAmaxUnroll = 4;     // 128-bit loads in flight per lane per step
+constexpr uint32_t kAmaxFanIn = 32;     // first-level groups of the cross-workgroup arrival tree
+constexpr uint32_t kAmaxLineWords = 32; // one 128-byte line per (max, ticket) pair
 
 template <typename X> struct AbsBits;
 template <> struct AbsBits<F32> {  // returns max over the 4 floats, as f32 bit pattern
@@ -71,6 +73,26 @@ template <> struct AbsBits<F16> {  // 8 f16 per vector; result kept as f16 bit p
   static constexpr int kPerVec = 8;
 };
 
+// One arrival at a (max, ticket) pair.  Device-scope atomics execute at the memory
+// side, the one place all eight XCDs agree on, so no cache write-back or invalidate
+// is needed (an acquire/release pair at device scope would flush and invalidate the
+// XCD's L2 once per workgroup).  Ordering is by completion: the max RETURNS its old
+// value and the empty asm consumes it, so the wave waits for that value before it
+// issues the ticket; every max is therefore performed before the ticket of the same
+// arrival, and all of them before the last ticket.  Returns true for the last of
+// `expected` arrivals, with the combined max in `m`; that caller has also put the
+// pair back to zero.
+__device__ __forceinline__ bool arrive(uint32_t* pair, uint32_t expected, uint32_t& m) {
+  const uint32_t before = __hip_atomic_fetch_max(&pair[0], m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __asm__ volatile("" ::"v"(before) : "memory");
+  const uint32_t ticket = __hip_atomic_fetch_add(&pair[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (ticket != expected - 1) return false;
+  // read-modify-write, so the value comes from the memory side, not from a cache
+  m = __hip_atomic_exchange(&pair[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_exchange(&pair[1], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return true;
+}
+
 template <typename X>
 __device__ __forceinline__ void amax_body(const typename X::storage* __restrict__ x, int64_t n, float qmax,
                                           float* __restrict__ amax_out, float* __restrict__ scale_out,
@@ -78,24 +100,27 @@ __device__ __forceinline__ void amax_body(const typename X::storage* __restrict_
   using A = AbsBits<X>;
   // Elements before the first 16-byte boundary ("head") and after the last full
   // vector ("tail") are taken one per lane by workgroup 0; everything between is
-  // streamed as 128-bit vectors.
+  // streamed as 128-bit vectors, each workgroup owning one contiguous chunk.
   constexpr int kElemBytes = 16 / A::kPerVec;
+  constexpr int64_t kStep = int64_t(kAmaxThreads) * kAmaxUnroll;
   int64_t head = int64_t((16u - uint32_t(reinterpret_cast<uintptr_t>(x) & 15u)) & 15u) / kElemBytes;
   head = head < n ? head : n;
   const int64_t nvec = (n - head) / A::kPerVec;
   const u32x4* __restrict__ xv = reinterpret_cast<const u32x4*>(x + head);
-  const int64_t stride = int64_t(gridDim.x) * kAmaxThreads;
+  const int64_t per = ((nvec + gridDim.x - 1) / gridDim.x + kStep - 1) / kStep * kStep;   // chunk, whole steps
+  const int64_t c0 = int64_t(blockIdx.x) * per;
+  const int64_t c1 = c0 + per < nvec ? c0 + per : nvec;
   uint32_t m = 0;
-  int64_t i = int64_t(blockIdx.x) * kAmaxThreads + threadIdx.x;
-  // main loop: kAmaxUnroll independent 128-bit loads per lane per trip
-  for (; i + (kAmaxUnroll - 1) * stride < nvec; i += kAmaxUnroll * stride) {
+  int64_t i = c0 + threadIdx.x;
+  // kAmaxUnroll independent 128-bit loads per lane per trip
+  for (; i + (kAmaxUnroll - 1) * kAmaxThreads < c1; i += kStep) {
     u32x4 t[kAmaxUnroll];
 #pragma unroll
-    for (int u = 0; u < kAmaxUnroll; ++u) t[u] = __builtin_nontemporal_load(xv + i + u * stride);
+    for (int u = 0; u < kAmaxUnroll; ++u) t[u] = __builtin_nontemporal_load(xv + i + u * kAmaxThreads);
 #pragma unroll
     for (int u = 0; u < kAmaxUnroll; ++u) { const uint32_t a = A::of(t[u]); m = m > a ? m : a; }
   }
-  for (; i < nvec; i += stride) { const uint32_t a = A::of(__builtin_nontemporal_load(xv + i)); m = m > a ? m : a; }
+  for (; i < c1; i += kAmaxThreads) { const uint32_t a = A::of(__builtin_nontemporal_load(xv + i)); m = m > a ? m : a; }
   if (blockIdx.x == 0 && threadIdx.x < 2 * A::kPerVec) {
     const int64_t tail0 = head + nvec * A::kPerVec;
     const int64_t e = threadIdx.x < A::kPerVec ? int64_t(threadIdx.x) : tail0 + (threadIdx.x - A::kPerVec);
@@ -111,25 +136,16 @@ __device__ __forceinline__ void amax_body(const typename X::storage* __restrict_
   if (threadIdx.x == 0) {
 #pragma unroll
     for (int w = 1; w < kAmaxThreads / kWave; ++w) m = m > wave_max[w] ? m : wave_max[w];
-    // Cross-workgroup step.  Device-scope atomics execute at the memory side, the
-    // one place all eight XCDs agree on, so no cache write-back or invalidate is
-    // needed (an acquire/release pair at device scope would flush and invalidate this
-    // XCD's L2 once per workgroup, which costs more than the reduction itself).
-    // Ordering is by completion: the max RETURNS its old value and the empty asm
-    // consumes it, so the wave waits for that value before it issues the ticket;
-    // every max is therefore performed before the ticket of the same workgroup, and
-    // all of them before the last ticket.
-    const uint32_t before = __hip_atomic_fetch_max(&scratch[0], m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __asm__ volatile("" ::"v"(before) : "memory");
-    const uint32_t ticket = __hip_atomic_fetch_add(&scratch[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (ticket == gridDim.x - 1) {
-      // read-modify-write, so the value comes from the memory side, not from a cache
-      const uint32_t total = __hip_atomic_fetch_max(&scratch[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const float amax = A::finish(total);
+    // Two-level arrival tree: atomics on one address are served one after the other
+    // by the memory side, so workgroups first meet in kAmaxFanIn groups (one cache
+    // line each) and only the last of each group goes on to the root.
+    const uint32_t groups = gridDim.x < kAmaxFanIn ? gridDim.x : kAmaxFanIn;
+    const uint32_t g = blockIdx.x % groups;
+    const uint32_t members = (gridDim.x - g + groups - 1) / groups;
+    if (arrive(scratch + kAmaxLineWords * (1 + g), members, m) && arrive(scratch, groups, m)) {
+      const float amax = A::finish(m);
       if (amax_out) *amax_out = amax;
       if (scale_out) *scale_out = amax / qmax;         // one IEEE divide, as the host does it
-      __hip_atomic_exchange(&scratch[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_exchange(&scratch[1], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   }
 }

@@ -76,10 +76,11 @@ struct DeviceState {
   hipModule_t module = nullptr;
   std::mutex mu;
   std::unordered_map<std::string, hipFunction_t> funcs;
-  // Two zeroed 32-bit words per stream for single-launch grid reductions, each
-  // slot on its own 64-byte line.  Kernels return their slot to zero.
-  static constexpr int kSlots = 1024;
-  static constexpr int kSlotWords = 16;
+  // One zeroed block per stream for single-launch grid reductions: 33 lines of
+  // 128 bytes (root + 32 first-level groups, see amax.hip), rounded up to 40.
+  // Kernels return their block to zero.
+  static constexpr int kSlots = 256;
+  static constexpr int kSlotWords = 40 * 32;
   uint32_t *slots = nullptr;
   std::map<hipStream_t, int> slot_of;
   int next_slot = 0;
@@ -176,7 +177,7 @@ uint32_t *reduction_slot(DeviceState *st, hipStream_t stream) {
 void forget_stream(hipStream_t) {
   // Slots are never reused for a different stream: a destroyed stream's slot is
   // zero again once its last kernel has finished, but handing it to another stream
-  // before that would race.  1024 slots outlive any realistic stream count.
+  // before that would race.  256 slots outlive any realistic stream count.
 }
 
 int32_t launch(DeviceState *st, const std::string &kernel, uint32_t grid, uint32_t block,

@@ -27,7 +27,7 @@ const char *last_kernel_name();
 int32_t load_code_object(const char *data, size_t len, hipModule_t *out, std::string *err);
 
 // Per-device state of the cluster layer: the built-in module, a function cache and
-// the pool of two-word reduction slots handed out per stream.
+// the pool of zeroed reduction blocks handed out per stream.
 struct DeviceState;
 DeviceState *device_state();                 // nullptr + set_error on failure
 hipModule_t builtin_module(DeviceState *);

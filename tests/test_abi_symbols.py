@@ -1,0 +1,98 @@
+"""CPU-only checks of the drop-in boundary: the C-ABI library loads, exports exactly
+the entry points include/mtrt_hip.h declares, keeps the reference C backend's names,
+and carries a gfx950 code object with every kernel the cluster layer can ask for.
+No compute call is made here."""
+import ctypes
+import os
+import re
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "mtrt_hip.h")
+
+# names of the reference C backend, mlir-tensorrt/executor/lib/Runtime/Backend/C/CUDAModule.h:55-119
+REFERENCE_C_BACKEND = [
+    "mtrt_cuda_get_active_device", "mtrt_cuda_set_active_device", "mtrt_cuda_get_device",
+    "mtrt_cuda_stream_create", "mtrt_cuda_stream_destroy", "mtrt_cuda_stream_sync",
+    "mtrt_cuda_event_create", "mtrt_cuda_event_release", "mtrt_cuda_stream_record_event",
+    "mtrt_cuda_stream_wait_event", "mtrt_cuda_event_sync", "mtrt_cuda_event_elapsed_msec",
+    "mtrt_cuda_alloc_async", "mtrt_cuda_memcpy_async", "mtrt_cuda_free",
+    "mtrt_cuda_module_load_from_ptx", "mtrt_cuda_module_load_from_ptx_file", "mtrt_cuda_module_unload",
+    "mtrt_cuda_module_get_function", "mtrt_cuda_launch_kernel",
+    "mtrt_cuda_get_current_device", "mtrt_cuda_get_program_device",
+]
+
+
+def _declared():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return re.findall(r"MTRT_CAPI_EXPORTED[^;(]*?\b(mtrt_[a-z0-9_]+)\s*\(", text)
+
+
+def test_header_declares_the_reference_names():
+    declared = _declared()
+    assert len(declared) == len(set(declared))
+    for name in REFERENCE_C_BACKEND:
+        assert name in declared, name
+
+
+def test_library_exports_every_declared_symbol(pkg):
+    L = pkg.lib()
+    for name in _declared():
+        assert hasattr(L, name), "libmtrt_hip.so does not export %s" % name
+    assert set(pkg.PROTOTYPES) == set(_declared()), "python prototypes and header disagree"
+    out = subprocess.run(["nm", "-D", "--defined-only", pkg.LIB_PATH], capture_output=True, text=True).stdout
+    exported = set(re.findall(r" T (\w+)", out))
+    assert set(_declared()) <= exported
+    extra = {s for s in exported if s.startswith("mtrt_")} - set(_declared())
+    assert not extra, "exported but undeclared: %s" % sorted(extra)
+
+
+def test_embedded_code_object_is_gfx950_and_has_the_kernels(pkg):
+    L = pkg.lib()
+    size = ctypes.c_size_t(0)
+    ptr = L.mtrt_hip_builtin_code_object(ctypes.byref(size))
+    blob = ctypes.string_at(ptr, size.value)
+    assert blob == open(pkg.KERNEL_MODULE_PATH, "rb").read()
+    assert blob.startswith(b"__CLANG_OFFLOAD_BUNDLE__") and b"gfx950" in blob[:4096]
+    names = []
+    for mode in ("q", "dq", "qdq"):
+        for kind in ("uniform", "row", "col", "any"):
+            for x in ("f32", "f16", "bf16"):
+                for q in ("i8", "f8", "i4", "i4p"):
+                    names.append("mtrt_%s_%s_%s_%s" % (mode, kind, x, q))
+    for x in ("f32", "f16", "bf16"):
+        names.append("mtrt_amax_" + x)
+        for v in ("v1", "v2", "v4", "v8", "v16", "any"):
+            names += ["mtrt_layernorm_%s_%s" % (x, v), "mtrt_softmax_%s_%s" % (x, v)]
+    names.append("mtrt_copy_b128")
+    for n in names:
+        assert n.encode() + b"\x00" in blob, "kernel %s is not in the code object" % n
+
+
+def test_status_calls_fail_loudly_without_a_gpu(pkg):
+    """There is no CPU fallback: without a usable gfx950 device init reports an error."""
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    L = pkg.lib()
+    assert L.mtrt_hip_init() != 0
+    assert L.mtrt_hip_last_error()
+    assert L.mtrt_hip_builtin_module() is None
+    st = L.mtrt_hip_softmax(None, 16, 16, pkg.F32, 1, 4)
+    assert st != 0
+
+
+def test_argument_validation_needs_no_device(pkg):
+    L = pkg.lib()
+    assert L.mtrt_hip_quantize(None, 16, 9, 16, pkg.I8, 16, 0, 1, 4, 1, 0) == 1
+    assert b"f32/f16/bf16" in L.mtrt_hip_last_error()
+    assert L.mtrt_hip_quantize(None, 16, pkg.F32, 16, pkg.I8, 16, 5, 1, 4, 1, 0) == 1
+    assert L.mtrt_hip_quantize(None, 16, pkg.F32, 16, pkg.I8, 16, 0, -1, 4, 1, 0) == 1
+    assert L.mtrt_hip_layernorm(None, 16, 16, 16, 16, pkg.I8, 1, 4, 1e-5) == 1
+    assert L.mtrt_hip_amax(None, 16, pkg.F32, -5, 1.0, None, None) == 1
+    # zero-sized work is a no-op that needs no device either
+    assert L.mtrt_hip_quantize(None, 16, pkg.F32, 16, pkg.I8, 16, 0, 0, 4, 1, 0) == 0
+    assert L.mtrt_hip_softmax(None, 16, 16, pkg.F32, 0, 4) == 0

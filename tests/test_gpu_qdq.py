@@ -224,6 +224,35 @@ def test_fp8_every_f16_value_and_random_f32(pkg, orc, flags_mode):
     _check_all(pkg, orc, x, "f32", "f8", pkg.SCALE_UNIFORM, 1, x.size, 1, [np.float32(1.0)], flags=flags, mode=mode)
 
 
+@pytest.mark.parametrize("qname", ["i8", "f8"])
+def test_shared_scale_division_is_the_ieee_quotient(pkg, orc, qname):
+    """Per-tensor and per-row kernels divide through the reciprocal of the shared scale; the
+    quotient must still be the correctly rounded one for every input.  Scales with all-ones,
+    all-zero and alternating significands at exponents inside, at the edge of and outside the
+    fast range (outside, the kernels fall back to the divide itself), against inputs that are
+    random finite f32 bit patterns scaled into the representable range of the codes, plus
+    infinities, zeros and subnormals."""
+    g = rng(23)
+    mant = [0x7FFFFF, 0x7FFFFE, 0x000000, 0x000001, 0x400000, 0x3FFFFF, 0x2AAAAA, 0x555555, 0x6DB6DB]
+    expo = [127 - 70, 127 - 61, 127 - 60, 127 - 30, 127 - 7, 127, 127 + 9, 127 + 30, 127 + 60, 127 + 61]
+    n = 1 << 16
+    for e in expo:
+        for m in mant[: (len(mant) if e in (127 - 7, 127) else 3)]:
+            s = np.uint32((e << 23) | m).view(np.float32)
+            sig = (g.integers(0, 1 << 23, n, dtype=np.uint64).astype(np.uint32) | np.uint32(127 << 23)).view(np.float32)
+            x = (sig * np.float32(2.0) ** g.integers(-12, 10, n).astype(np.float32)) * s   # |x/s| in [2^-12, 2^10]
+            x *= np.where(g.random(n) < 0.5, np.float32(-1), np.float32(1))
+            x[:8] = np.float32([np.inf, -np.inf, 0.0, -0.0, 1e-45, -1e-45, 3e38, -3e38])
+            x = x.astype(np.float32)
+            _check_all(pkg, orc, x, "f32", qname, pkg.SCALE_UNIFORM, 1, n, 1, [s])
+    # one scale per row
+    rows = 64
+    sc = (g.integers(0, 1 << 23, rows, dtype=np.uint64).astype(np.uint32) | np.uint32(120 << 23)).view(np.float32)
+    sc[:4] = np.uint32([(120 << 23) | 0x7FFFFF, (50 << 23) | 1, (200 << 23) | 0x7FFFFF, 127 << 23]).view(np.float32)
+    x = (g.standard_normal((rows, 1024)).astype(np.float32) * np.float32(60.0)) * sc[:, None]
+    _check_all(pkg, orc, x.astype(np.float32), "f32", qname, pkg.SCALE_ROW, rows, 1024, rows, sc)
+
+
 def test_all_zero_tensor_and_empty(pkg, orc):
     import torch
     x = np.zeros((4, 64), dtype=np.float32)
