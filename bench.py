@@ -143,6 +143,40 @@ def build_workloads(pkg, torch, which):
     return out
 
 
+def calibration_copy(pkg, torch):
+    """One launch of the plain copy kernel over 128 MiB (reads 128 MiB, writes 128 MiB): the
+    yardstick that hardware byte counters of a profiled run are scaled by."""
+    import ctypes
+    L = pkg.lib()
+    nbytes = 128 << 20
+    src = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    dst = torch.empty_like(src)
+    src.fill_(1)
+    name = b"mtrt_copy_b128"
+    fn = L.mtrt_cuda_module_get_function(L.mtrt_hip_builtin_module(), name, len(name))
+    vals = (ctypes.c_void_p(src.data_ptr()), ctypes.c_void_p(dst.data_ptr()), ctypes.c_int64(nbytes // 16))
+    args = (ctypes.c_void_p * 3)(*[ctypes.cast(ctypes.pointer(v), ctypes.c_void_p) for v in vals])
+    nvec = nbytes // 16
+    L.mtrt_cuda_launch_kernel(fn, nvec // 256, 1, 1, 256, 1, 1, 0, torch.cuda.current_stream().cuda_stream, args)
+    torch.cuda.synchronize()
+
+
+def traffic_from_profile(kernel):
+    """HBM bytes per launch of `kernel` as measured by the committed counter profile
+    (profiles/hbm_traffic_bench_suite.md, table rows `| kernel | fetch | write | total |`), or None."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic_bench_suite.md")
+    if not os.path.exists(path):
+        return None
+    for line in open(path):
+        cells = [c.strip() for c in line.strip().strip("|").split("|")]
+        if len(cells) >= 4 and cells[0] == kernel:
+            try:
+                return float(cells[3])
+            except ValueError:
+                return None
+    return None
+
+
 def time_kernel(pkg, torch, w, reps):
     """Average launch duration in microseconds, HIP events on the launch stream."""
     L = pkg.lib()
@@ -234,6 +268,7 @@ def main():
     pkg.check(pkg.lib().mtrt_hip_init())
     torch.cuda.set_device(0)
 
+    calibration_copy(pkg, torch)
     wl = build_workloads(pkg, torch, args.workload)
     # the step: every kernel once, in program order, on buffer set (step % nslots)
     step_calls = [[w["make"](i) for i in range(w["nslots"])] for w in wl]
@@ -273,7 +308,7 @@ def main():
         "config": {"workload": {"all": "C1+C2a+C2b+C3 programs of BASELINE.json, one pass each per step"}.get(
             args.workload, args.workload.upper()), "kernels_per_step": len(wl)},
         "roofline": {"kernel": dom["kernel"], "bound": dom["bound"], "achieved": dom["achieved"], "peak": dom["peak"],
-                     "unit": dom["unit"], "frac": dom["frac"], "traffic": None},
+                     "unit": dom["unit"], "frac": dom["frac"], "traffic": traffic_from_profile(dom["kernel"])},
         "workloads": kernels,
     }
     if not args.no_cpu_baseline:

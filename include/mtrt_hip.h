@@ -198,6 +198,20 @@ MTRT_CAPI_EXPORTED int32_t mtrt_hip_layernorm(mtrt_stream_t stream, const void *
 MTRT_CAPI_EXPORTED int32_t mtrt_hip_softmax(mtrt_stream_t stream, const void *x, void *y,
                                             int32_t dtype, int64_t rows, int64_t d);
 
+/* W8A8 GEMM with fused dequantize epilogue:
+ *   acc[m,n] = sum_k i32(a[m,k]) * i32(w[k,n])   ;   y[m,n] = f16((f32(acc) * a_scale[m]) * w_scale[n])
+ * (the int8 form of the quantized Linear of tripy/nvtripy/frontend/module/linear.py:112-151; the
+ * reference's code generator emits an FMA loop nest for it, mlir-tensorrt/kernel/test/Kernel/
+ * TransformSchedules/fallback-schedule-matmul.mlir:24).  Weights are program constants: they are
+ * re-laid ONCE from the program's [K,N] into [N,K] (K contiguous, what the matrix cores read) by
+ * the prepack call; the GEMM takes the re-laid weights.  a: int8 [M,K]; a_scale: f32 [M];
+ * w_scale: f32 [N]; y: f16 [M,N]. */
+MTRT_CAPI_EXPORTED int32_t mtrt_hip_gemm_w8a8_prepack(mtrt_stream_t stream, const void *w_kn,
+                                                      void *w_nk, int64_t K, int64_t N);
+MTRT_CAPI_EXPORTED int32_t mtrt_hip_gemm_w8a8(mtrt_stream_t stream, const void *a, const void *w_nk,
+                                              const float *a_scale, const float *w_scale, void *y,
+                                              int64_t M, int64_t K, int64_t N);
+
 /* Name of the kernel that the most recent successful part-2 call on this thread
  * launched last (for profiles and tests). */
 MTRT_CAPI_EXPORTED const char *mtrt_hip_last_kernel(void);

@@ -63,6 +63,8 @@ PROTOTYPES = {
     "mtrt_hip_quantize_dequantize": (_i32, [_vp, _vp, _i32, _vp, _i32, _vp, _vp, _i32, _i64, _i64, _i64, _i32]),
     "mtrt_hip_layernorm": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i64, _i64, _f32]),
     "mtrt_hip_softmax": (_i32, [_vp, _vp, _vp, _i32, _i64, _i64]),
+    "mtrt_hip_gemm_w8a8_prepack": (_i32, [_vp, _vp, _vp, _i64, _i64]),
+    "mtrt_hip_gemm_w8a8": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64]),
 }
 
 _lib = None
@@ -190,6 +192,29 @@ def softmax(x, out=None):
     rows = x.numel() // d if d else 0
     y = torch.empty_like(x) if out is None else out
     check(lib().mtrt_hip_softmax(_stream(), x.data_ptr(), y.data_ptr(), float_dtype_of(x), rows, d))
+    return y
+
+
+def gemm_w8a8_prepack(w_kn):
+    """int8 weights [K,N] -> [N,K] (the layout the GEMM consumes)."""
+    torch = _torch()
+    assert w_kn.is_cuda and w_kn.is_contiguous() and w_kn.dtype == torch.int8 and w_kn.dim() == 2
+    K, N = w_kn.shape
+    w_nk = torch.empty((N, K), dtype=torch.int8, device=w_kn.device)
+    check(lib().mtrt_hip_gemm_w8a8_prepack(_stream(), w_kn.data_ptr(), w_nk.data_ptr(), K, N))
+    return w_nk
+
+
+def gemm_w8a8(a, w_nk, a_scale, w_scale, out=None):
+    torch = _torch()
+    assert a.is_cuda and a.is_contiguous() and a.dtype == torch.int8 and w_nk.is_contiguous() and w_nk.dtype == torch.int8
+    assert a_scale.dtype == torch.float32 and w_scale.dtype == torch.float32
+    M, K = a.shape
+    N = w_nk.shape[0]
+    assert w_nk.shape[1] == K and a_scale.numel() == M and w_scale.numel() == N
+    y = torch.empty((M, N), dtype=torch.float16, device=a.device) if out is None else out
+    check(lib().mtrt_hip_gemm_w8a8(_stream(), a.data_ptr(), w_nk.data_ptr(), a_scale.data_ptr(), w_scale.data_ptr(),
+                                   y.data_ptr(), M, K, N))
     return y
 
 

@@ -3,4 +3,5 @@
 #include "amax.hip"
 #include "qdq.hip"
 #include "norm.hip"
+#include "gemm_w8a8.hip"
 #include "util.hip"

@@ -243,4 +243,47 @@ int32_t mtrt_hip_softmax(mtrt_stream_t stream, const void *x, void *y, int32_t d
                 uint32_t(std::min<int64_t>(rows, int64_t(num_compute_units(st)) * 8)), kBlock, as_hip(stream), args);
 }
 
+int32_t mtrt_hip_gemm_w8a8_prepack(mtrt_stream_t stream, const void *w_kn, void *w_nk, int64_t K, int64_t N) {
+  clear_error();
+  if (K < 0 || N < 0)
+    return set_error(MTRT_INVALID_ARGUMENT, "negative extent [%lld, %lld]", (long long)K, (long long)N);
+  if (K == 0 || N == 0)
+    return MTRT_OK;
+  if (!w_kn || !w_nk)
+    return set_error(MTRT_INVALID_ARGUMENT, "null operand");
+  DeviceState *st = device_state();
+  if (!st)
+    return MTRT_RUNTIME_ERROR;
+  const int64_t tiles = ((K + 63) / 64) * ((N + 63) / 64);
+  if (tiles > int64_t(kMaxGrid) * 1024)
+    return set_error(MTRT_INVALID_ARGUMENT, "weight matrix [%lld, %lld] is too large", (long long)K, (long long)N);
+  void *args[] = {&w_kn, &w_nk, &K, &N};
+  return launch(st, "mtrt_w8_prepack_kn_to_nk", uint32_t(tiles), kBlock, as_hip(stream), args);
+}
+
+int32_t mtrt_hip_gemm_w8a8(mtrt_stream_t stream, const void *a, const void *w_nk, const float *a_scale,
+                           const float *w_scale, void *y, int64_t M, int64_t K, int64_t N) {
+  clear_error();
+  if (M < 0 || K < 0 || N < 0)
+    return set_error(MTRT_INVALID_ARGUMENT, "negative extent M=%lld K=%lld N=%lld", (long long)M, (long long)K,
+                     (long long)N);
+  if (M == 0 || N == 0)
+    return MTRT_OK;
+  if (!a_scale || !w_scale || !y || (K > 0 && (!a || !w_nk)))
+    return set_error(MTRT_INVALID_ARGUMENT, "null operand");
+  if (!aligned(y, 2))
+    return set_error(MTRT_INVALID_ARGUMENT, "output is not aligned to its element size");
+  DeviceState *st = device_state();
+  if (!st)
+    return MTRT_RUNTIME_ERROR;
+  void *args[] = {&a, &w_nk, &a_scale, &w_scale, &y, &M, &K, &N};
+  // The matrix-core kernel moves 128-byte K slices with 16-byte accesses.
+  if (K > 0 && K % 128 == 0 && aligned(a, 16) && aligned(w_nk, 16)) {
+    const int64_t tiles = ((M + 255) / 256) * ((N + 127) / 128);
+    if (tiles <= int64_t(kMaxGrid) * 1024)
+      return launch(st, "mtrt_gemm_w8a8_nk", uint32_t(tiles), kBlock, as_hip(stream), args);
+  }
+  return launch(st, "mtrt_gemm_w8a8_nk_any", blocks_for(M * N, kBlock), kBlock, as_hip(stream), args);
+}
+
 } // extern "C"
