@@ -212,6 +212,24 @@ MTRT_CAPI_EXPORTED int32_t mtrt_hip_gemm_w8a8(mtrt_stream_t stream, const void *
                                               const float *a_scale, const float *w_scale, void *y,
                                               int64_t M, int64_t K, int64_t N);
 
+/* W4A16 block-wise GEMM:
+ *   wd[k,n] = f16(f16(w[k,n]) * scale[k / block, n])   ;   y[m,n] = f16(sum_k f32(a[m,k]) * f32(wd[k,n]))
+ * (weight-only int4 Linear, linear.py:112-151; block dequantize TensorRTOps.td:3408-3445).
+ * a: f16 [M,K]; w_kn_packed: int4 [K,N] two per byte over the flattened array, element 2i in the
+ * low nibble (NetworkEncoder.cpp:552-595); scale: f16 [K/block, N]; y: f16 [M,N].
+ * The matrix-core kernels read the weights from a one-time re-layout (`w_prepacked`, made by the
+ * prepack call, mtrt_hip_gemm_w4a16_prepacked_bytes(K, N) bytes, needs K % 64 == 0); they are
+ * used when w_prepacked is given and K % 64 == 0, block % 64 == 0, K % block == 0.  Otherwise the
+ * generic kernel reads w_kn_packed directly (any shape, slow).  Either weight pointer may be NULL
+ * if the other path applies. */
+MTRT_CAPI_EXPORTED int64_t mtrt_hip_gemm_w4a16_prepacked_bytes(int64_t K, int64_t N);
+MTRT_CAPI_EXPORTED int32_t mtrt_hip_gemm_w4a16_prepack(mtrt_stream_t stream, const void *w_kn_packed,
+                                                       void *w_prepacked, int64_t K, int64_t N);
+MTRT_CAPI_EXPORTED int32_t mtrt_hip_gemm_w4a16(mtrt_stream_t stream, const void *a,
+                                               const void *w_kn_packed, const void *w_prepacked,
+                                               const void *scale, void *y, int64_t M, int64_t K,
+                                               int64_t N, int64_t block);
+
 /* Name of the kernel that the most recent successful part-2 call on this thread
  * launched last (for profiles and tests). */
 MTRT_CAPI_EXPORTED const char *mtrt_hip_last_kernel(void);

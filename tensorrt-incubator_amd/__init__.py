@@ -65,6 +65,9 @@ PROTOTYPES = {
     "mtrt_hip_softmax": (_i32, [_vp, _vp, _vp, _i32, _i64, _i64]),
     "mtrt_hip_gemm_w8a8_prepack": (_i32, [_vp, _vp, _vp, _i64, _i64]),
     "mtrt_hip_gemm_w8a8": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64]),
+    "mtrt_hip_gemm_w4a16_prepacked_bytes": (_i64, [_i64, _i64]),
+    "mtrt_hip_gemm_w4a16_prepack": (_i32, [_vp, _vp, _vp, _i64, _i64]),
+    "mtrt_hip_gemm_w4a16": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64]),
 }
 
 _lib = None
@@ -215,6 +218,27 @@ def gemm_w8a8(a, w_nk, a_scale, w_scale, out=None):
     y = torch.empty((M, N), dtype=torch.float16, device=a.device) if out is None else out
     check(lib().mtrt_hip_gemm_w8a8(_stream(), a.data_ptr(), w_nk.data_ptr(), a_scale.data_ptr(), w_scale.data_ptr(),
                                    y.data_ptr(), M, K, N))
+    return y
+
+
+def gemm_w4a16_prepack(w_kn_packed, K, N):
+    """packed int4 weights (uint8, K*N/2 bytes over the flattened [K,N]) -> fragment-order buffer."""
+    torch = _torch()
+    assert w_kn_packed.is_cuda and w_kn_packed.is_contiguous() and w_kn_packed.dtype == torch.uint8
+    nbytes = lib().mtrt_hip_gemm_w4a16_prepacked_bytes(K, N)
+    assert nbytes > 0, "prepack needs K % 64 == 0"
+    wp = torch.empty(nbytes, dtype=torch.uint8, device=w_kn_packed.device)
+    check(lib().mtrt_hip_gemm_w4a16_prepack(_stream(), w_kn_packed.data_ptr(), wp.data_ptr(), K, N))
+    return wp
+
+
+def gemm_w4a16(a, scale, K, N, block, w_kn_packed=None, w_prepacked=None, out=None):
+    torch = _torch()
+    assert a.is_cuda and a.is_contiguous() and a.dtype == torch.float16 and scale.dtype == torch.float16
+    M = a.shape[0]
+    y = torch.empty((M, N), dtype=torch.float16, device=a.device) if out is None else out
+    check(lib().mtrt_hip_gemm_w4a16(_stream(), a.data_ptr(), _ptr(w_kn_packed), _ptr(w_prepacked), scale.data_ptr(),
+                                    y.data_ptr(), M, K, N, block))
     return y
 
 

@@ -4,4 +4,5 @@
 #include "qdq.hip"
 #include "norm.hip"
 #include "gemm_w8a8.hip"
+#include "gemm_w4a16.hip"
 #include "util.hip"

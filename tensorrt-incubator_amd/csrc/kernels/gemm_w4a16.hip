@@ -1,0 +1,279 @@
+// W4A16 block-wise GEMM cluster for gfx950:
+//     wd[k,n] = f16( f16(w_i4[k,n]) * s[k / block, n] )          (one f16 rounding)
+//     y[m,n]  = f16( sum_k f32(a[m,k]) * f32(wd[k,n]) )            (f32 accumulation)
+// the weight-only int4 form of the quantized Linear
+// (tripy/nvtripy/frontend/module/linear.py:112-151, block dequantize as in
+//  mlir-tensorrt/tensorrt/include/mlir-tensorrt-dialect/TensorRT/IR/TensorRTOps.td:3408-3445).
+//
+// Weights are program constants.  They arrive packed two per byte over the flattened
+// [K,N] array (element 2i in the low nibble,
+// mlir-tensorrt/tensorrt/lib/Target/TensorRTEncodingOpInterface/NetworkEncoder.cpp:552-595)
+// and are re-laid ONCE by mtrt_w4_prepack into the order the matrix cores read:
+//   for each tile of 32 columns and each block of 64 k, 64 lanes x 4 dwords, where
+//   lane = 32*h + (n % 32) and dword j of that lane holds the 8 weights
+//   k = 64*kb + 8*(2j + h) + [0..7] of column n.  Inside a dword nibble p (p < 4) is
+//   weight 2p and nibble p + 4 is weight 2p + 1, each stored as (value + 8).
+// A wave therefore loads 1 KiB of contiguous memory and every lane gets exactly its
+// B-fragments for four v_mfma_f32_32x32x16_f16 steps; (w >> 4p) & 0x000F000F isolates
+// the pair (2p, 2p+1) in the two halves of a register, OR-ing 0x6400 into each half
+// makes the f16 numbers 1024 + (value + 8), a packed subtract of 1032 gives the exact
+// integer value and a packed f16 multiply by the scale gives wd with the single
+// rounding the program asks for.
+//
+// Large M: dequantisation happens in registers on the way INTO LDS; the multiply loop
+// is the plain f16 loop over 128-byte LDS rows (same swizzle as the int8 GEMM).
+// Small M (<= 32): the GEMM is bound by reading the weights once.  One workgroup per
+// 32 columns, its four waves split K, fragments go straight from global memory into
+// registers (no LDS on the way in), partial tiles are added through LDS at the end.
+#include "common.hpp"
+
+using namespace mtrt_dev;
+
+namespace gemm_w4a16_cluster {
+
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+
+constexpr int BKH = 64;                              // k per slice (f16 elements): 128-byte LDS rows
+constexpr int THREADS = 256;
+
+__device__ __forceinline__ int lds_off(int row, int chunk) { return row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4); }
+
+union H2Bits { uint32_t u; h2 h; };
+
+// One prepacked dword -> 8 dequantised f16 weights (k order 0..7), as a 16-byte chunk.
+__device__ __forceinline__ u4 dequant8(uint32_t w, h2 scale2) {
+  u4 out;
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    H2Bits t;
+    t.u = ((w >> (4 * p)) & 0x000F000Fu) | 0x64006400u;   // {1024 + u(2p), 1024 + u(2p+1)}
+    const h2 bias = {(_Float16)1032.0f, (_Float16)1032.0f};
+    t.h = (t.h - bias) * scale2;                            // exact integer, then one f16 rounding
+    out[p] = t.u;
+  }
+  return out;
+}
+
+__device__ __forceinline__ h2 load_scale2(const uint16_t* __restrict__ scale, int64_t idx) {
+  union { uint16_t u; _Float16 h; } c;
+  c.u = scale[idx];
+  h2 r = {c.h, c.h};
+  return r;
+}
+
+// ---- large-M kernel ----------------------------------------------------------------
+// IT x JT MFMA tiles per wave, 2 x 2 waves: BM = 64*IT, BN = 64*JT.
+template <int IT, int JT>
+__device__ __forceinline__ void gemm_tiles(const uint16_t* __restrict__ a, const uint32_t* __restrict__ wp,
+                                           const uint16_t* __restrict__ scale, uint16_t* __restrict__ y, int64_t M,
+                                           int64_t K, int64_t N, int64_t block, int8_t* lds) {
+  constexpr int BM = 64 * IT, BN = 64 * JT;
+  constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
+  constexpr int A_CHUNKS = BM * 8 / THREADS;         // 16-byte loads per thread per slice
+  constexpr int B_LOADERS = BN * 2;                  // threads that fetch weights (16 B each)
+
+  const int64_t tiles_m = (M + BM - 1) / BM;
+  const int64_t m0 = int64_t(blockIdx.x % tiles_m) * BM;
+  const int64_t n0 = int64_t(blockIdx.x / tiles_m) * BN;
+  const int64_t kblocks = K / BKH;
+
+  const int t = threadIdx.x;
+  const int lane = t & 63, wave = t >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int frow = lane & 31, fhalf = lane >> 5;
+  // weight loader role: n-tile (t >> 6) of this workgroup's columns, fragment lane (t & 63)
+  const bool loads_b = t < B_LOADERS;
+  const int64_t b_tile = n0 / 32 + (t >> 6);
+  const int64_t b_col = b_tile * 32 + frow;          // column whose weights this thread dequantises
+  const bool b_live = loads_b && b_col < N;
+
+  v16f acc[IT][JT];
+#pragma unroll
+  for (int i = 0; i < IT; ++i)
+#pragma unroll
+    for (int j = 0; j < JT; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  u4 sa[A_CHUNKS];
+  u4 sb;
+  h2 sscale;
+
+  auto load_slice = [&](int64_t kb) {
+#pragma unroll
+    for (int i = 0; i < A_CHUNKS; ++i) {
+      int64_t row = m0 + (t >> 3) + 32 * i;
+      row = row < M ? row : M - 1;
+      sa[i] = *reinterpret_cast<const u4*>(a + row * K + kb * BKH + (t & 7) * 8);
+    }
+    if (loads_b) {
+      sb = b_live ? *reinterpret_cast<const u4*>(wp + ((b_tile * kblocks + kb) * 64 + lane) * 4) : (u4){0x88888888u, 0x88888888u, 0x88888888u, 0x88888888u};
+      sscale = b_live ? load_scale2(scale, ((kb * BKH) / block) * N + b_col) : (h2){(_Float16)0.0f, (_Float16)0.0f};
+    }
+  };
+  auto store_slice = [&](int8_t* pa, int8_t* pb) {
+#pragma unroll
+    for (int i = 0; i < A_CHUNKS; ++i) *reinterpret_cast<u4*>(pa + lds_off((t >> 3) + 32 * i, t & 7)) = sa[i];
+    if (loads_b) {
+      const int row = (t >> 6) * 32 + frow;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) *reinterpret_cast<u4*>(pb + lds_off(row, 2 * j + fhalf)) = dequant8(sb[j], sscale);
+    }
+  };
+
+  load_slice(0);
+  store_slice(lds, lds + A_BYTES);
+  __syncthreads();
+  for (int64_t kb = 0; kb < kblocks; ++kb) {
+    const int cur = int(kb & 1);
+    const int8_t* pa = lds + cur * STAGE;
+    const int8_t* pb = pa + A_BYTES;
+    if (kb + 1 < kblocks) load_slice(kb + 1);
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      v8h fa[IT], fb[JT];
+      const int chunk = ks * 2 + fhalf;
+#pragma unroll
+      for (int i = 0; i < IT; ++i) fa[i] = *reinterpret_cast<const v8h*>(pa + lds_off(wm * (32 * IT) + i * 32 + frow, chunk));
+#pragma unroll
+      for (int j = 0; j < JT; ++j) fb[j] = *reinterpret_cast<const v8h*>(pb + lds_off(wn * (32 * JT) + j * 32 + frow, chunk));
+#pragma unroll
+      for (int i = 0; i < IT; ++i)
+#pragma unroll
+        for (int j = 0; j < JT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    }
+    if (kb + 1 < kblocks) store_slice(lds + (cur ^ 1) * STAGE, lds + (cur ^ 1) * STAGE + A_BYTES);
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int j = 0; j < JT; ++j) {
+    const int64_t col = n0 + wn * (32 * JT) + j * 32 + frow;
+    if (col >= N) continue;
+#pragma unroll
+    for (int i = 0; i < IT; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int64_t row = m0 + wm * (32 * IT) + i * 32 + (r >> 2) * 8 + fhalf * 4 + (r & 3);
+        if (row < M) y[row * N + col] = uint16_t(f32_to_f16_bits(acc[i][j][r]));
+      }
+  }
+}
+
+// The entry points below have C linkage; they sit inside the namespace only so that
+// its helper names do not meet those of the other clusters in the one-module build.
+
+// (a [M,K] f16, w_prepacked, scale [K/block, N] f16, y [M,N] f16, M, K, N, block) ; K % 64 == 0, block % 64 == 0.
+extern "C" __global__ void __launch_bounds__(THREADS) mtrt_gemm_w4a16_t256x128(
+    const uint16_t* __restrict__ a, const uint32_t* __restrict__ wp, const uint16_t* __restrict__ scale,
+    uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t block) {
+  __shared__ __attribute__((aligned(16))) int8_t lds[2 * (256 + 128) * 128];
+  gemm_tiles<4, 2>(a, wp, scale, y, M, K, N, block, lds);
+}
+extern "C" __global__ void __launch_bounds__(THREADS) mtrt_gemm_w4a16_t128x64(
+    const uint16_t* __restrict__ a, const uint32_t* __restrict__ wp, const uint16_t* __restrict__ scale,
+    uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t block) {
+  __shared__ __attribute__((aligned(16))) int8_t lds[2 * (128 + 64) * 128];
+  gemm_tiles<2, 1>(a, wp, scale, y, M, K, N, block, lds);
+}
+
+// Small M (<= 32): one workgroup per 32 columns, four waves split K.
+extern "C" __global__ void __launch_bounds__(THREADS) mtrt_gemm_w4a16_skinny(
+    const uint16_t* __restrict__ a, const uint32_t* __restrict__ wp, const uint16_t* __restrict__ scale,
+    uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t block) {
+  __shared__ float partial[4][16][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int frow = lane & 31, fhalf = lane >> 5;
+  const int64_t tile = blockIdx.x;
+  const int64_t col = tile * 32 + frow;
+  const int64_t kblocks = K / BKH;
+  const int64_t kb0 = kblocks * wave / 4, kb1 = kblocks * (wave + 1) / 4;
+  const bool live_b = col < N;
+  const int64_t arow = frow < M ? frow : M - 1;      // rows past M repeat the last row; never stored
+  const uint16_t* ap = a + arow * K + fhalf * 8;
+  const u4* bp = reinterpret_cast<const u4*>(wp) + (tile * kblocks) * 64 + lane;
+
+  v16f acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+
+  for (int64_t kb = kb0; kb < kb1; ++kb) {
+    const u4 wq = live_b ? __builtin_nontemporal_load(bp + kb * 64) : (u4){0x88888888u, 0x88888888u, 0x88888888u, 0x88888888u};
+    const h2 s2 = live_b ? load_scale2(scale, ((kb * BKH) / block) * N + col) : (h2){(_Float16)0.0f, (_Float16)0.0f};
+    v8h fa[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) fa[ks] = *reinterpret_cast<const v8h*>(ap + kb * BKH + ks * 16);
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      union { u4 u; v8h h; } fb;
+      fb.u = dequant8(wq[ks], s2);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[ks], fb.h, acc, 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < 16; ++r) partial[wave][r][lane] = acc[r];
+  __syncthreads();
+  // 32 x 32 outputs, 256 threads: 4 each
+  for (int e = threadIdx.x; e < 16 * 64; e += THREADS) {
+    const int r = e >> 6, l = e & 63;
+    const float v = ((partial[0][r][l] + partial[1][r][l]) + partial[2][r][l]) + partial[3][r][l];
+    const int64_t row = (r >> 2) * 8 + (l >> 5) * 4 + (r & 3);
+    const int64_t c = tile * 32 + (l & 31);
+    if (row < M && c < N) y[row * N + c] = uint16_t(f32_to_f16_bits(v));
+  }
+}
+
+// Any shape: one output per lane, reading the ORIGINAL packed [K,N] nibbles; not a fast path.
+extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w4a16_any(
+    const uint16_t* __restrict__ a, const uint8_t* __restrict__ w_kn_packed, const uint16_t* __restrict__ scale,
+    uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t block) {
+  const int64_t total = M * N;
+  for (int64_t e = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; e < total; e += int64_t(gridDim.x) * blockDim.x) {
+    const int64_t m = e / N, n = e - m * N;
+    float acc = 0.0f;
+    for (int64_t k = 0; k < K; ++k) {
+      const int64_t i = k * N + n;
+      const uint32_t byte = w_kn_packed[i >> 1];
+      const uint32_t nib = (i & 1) ? (byte >> 4) : (byte & 0xFu);
+      const float wv = float(int(nib << 28) >> 28);
+      const float wd = f16_bits_to_f32(f32_to_f16_bits(wv * f16_bits_to_f32(scale[(k / block) * N + n])));
+      acc = acc + f16_bits_to_f32(a[m * K + k]) * wd;
+    }
+    y[e] = uint16_t(f32_to_f16_bits(acc));
+  }
+}
+
+// Weight re-layout: packed [K,N] nibbles -> fragment order described at the top.
+// One thread per output dword.  (w_kn_packed, wp, K, N) ; K % 64 == 0.
+extern "C" __global__ void __launch_bounds__(256) mtrt_w4_prepack(const uint8_t* __restrict__ w_kn_packed,
+                                                                uint32_t* __restrict__ wp, int64_t K, int64_t N) {
+  const int64_t kblocks = K / BKH;
+  const int64_t ntiles = (N + 31) / 32;
+  const int64_t total = ntiles * kblocks * 256;
+  for (int64_t d = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; d < total; d += int64_t(gridDim.x) * blockDim.x) {
+    const int j = int(d & 3), lane = int((d >> 2) & 63);
+    const int64_t kb = (d >> 8) % kblocks, tile = (d >> 8) / kblocks;
+    const int h = lane >> 5;
+    const int64_t n = tile * 32 + (lane & 31);
+    const int64_t k0 = kb * BKH + 8 * (2 * j + h);
+    uint32_t w = 0;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      uint32_t nib = 0;                                 // columns past N: value 0
+      if (n < N) {
+        const int64_t i = (k0 + q) * N + n;
+        const uint32_t byte = w_kn_packed[i >> 1];
+        nib = (i & 1) ? (byte >> 4) : (byte & 0xFu);
+      }
+      const uint32_t u = (nib ^ 8u) & 0xFu;             // value + 8
+      const int pos = (q & 1) ? (q >> 1) + 4 : (q >> 1);
+      w |= u << (4 * pos);
+    }
+    wp[d] = w;
+  }
+}
+
+}  // namespace gemm_w4a16_cluster

@@ -68,8 +68,8 @@ __device__ __forceinline__ void store_slice(const Staging& st, int8_t* lds_a, in
   for (int i = 0; i < B_CHUNKS; ++i) *reinterpret_cast<v4i*>(lds_b + lds_off((t >> 3) + 32 * i, ch)) = st.b[i];
 }
 
-}  // namespace gemm_w8a8_cluster
-using namespace gemm_w8a8_cluster;
+// The entry points below have C linkage; they sit inside the namespace only so that
+// its helper names do not meet those of the other clusters in the one-module build.
 
 // (a [M,K] i8, w_nk [N,K] i8, a_scale [M] f32, w_scale [N] f32, y [M,N] f16, M, K, N) ; K % 128 == 0,
 // a and w_nk 16-byte aligned.  grid = ceil(M/256) * ceil(N/128), block = 256.
@@ -178,3 +178,5 @@ extern "C" __global__ void __launch_bounds__(256) mtrt_w8_prepack_kn_to_nk(const
     if (k < K && n < N) w_nk[n * K + k] = tile[tx][ty + 4 * i];
   }
 }
+
+}  // namespace gemm_w8a8_cluster

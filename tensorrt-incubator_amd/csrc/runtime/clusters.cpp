@@ -286,4 +286,64 @@ int32_t mtrt_hip_gemm_w8a8(mtrt_stream_t stream, const void *a, const void *w_nk
   return launch(st, "mtrt_gemm_w8a8_nk_any", blocks_for(M * N, kBlock), kBlock, as_hip(stream), args);
 }
 
+int64_t mtrt_hip_gemm_w4a16_prepacked_bytes(int64_t K, int64_t N) {
+  if (K <= 0 || N <= 0 || K % 64 != 0)
+    return 0;
+  return ((N + 31) / 32) * (K / 64) * 1024;   // per 32 columns and 64 k: 64 lanes x 16 bytes
+}
+
+int32_t mtrt_hip_gemm_w4a16_prepack(mtrt_stream_t stream, const void *w_kn_packed, void *w_prepacked, int64_t K,
+                                    int64_t N) {
+  clear_error();
+  if (K <= 0 || N <= 0 || K % 64 != 0)
+    return set_error(MTRT_INVALID_ARGUMENT, "prepack needs positive extents and K %% 64 == 0, got K=%lld N=%lld",
+                     (long long)K, (long long)N);
+  if (!w_kn_packed || !w_prepacked)
+    return set_error(MTRT_INVALID_ARGUMENT, "null operand");
+  if (!aligned(w_prepacked, 16))
+    return set_error(MTRT_INVALID_ARGUMENT, "prepacked buffer must be 16-byte aligned");
+  DeviceState *st = device_state();
+  if (!st)
+    return MTRT_RUNTIME_ERROR;
+  const int64_t dwords = mtrt_hip_gemm_w4a16_prepacked_bytes(K, N) / 4;
+  void *args[] = {&w_kn_packed, &w_prepacked, &K, &N};
+  return launch(st, "mtrt_w4_prepack", blocks_for(dwords, kBlock), kBlock, as_hip(stream), args);
+}
+
+int32_t mtrt_hip_gemm_w4a16(mtrt_stream_t stream, const void *a, const void *w_kn_packed, const void *w_prepacked,
+                            const void *scale, void *y, int64_t M, int64_t K, int64_t N, int64_t block) {
+  clear_error();
+  if (M < 0 || K < 0 || N < 0)
+    return set_error(MTRT_INVALID_ARGUMENT, "negative extent M=%lld K=%lld N=%lld", (long long)M, (long long)K,
+                     (long long)N);
+  if (M == 0 || N == 0)
+    return MTRT_OK;
+  if (block <= 0 || (K > 0 && K % block != 0))
+    return set_error(MTRT_INVALID_ARGUMENT, "block size %lld does not divide K=%lld", (long long)block, (long long)K);
+  if (!y || (K > 0 && (!a || !scale)) || (!w_kn_packed && !w_prepacked && K > 0))
+    return set_error(MTRT_INVALID_ARGUMENT, "null operand");
+  if (!aligned(a, 2) || !aligned(y, 2) || !aligned(scale, 2))
+    return set_error(MTRT_INVALID_ARGUMENT, "operand is not aligned to its element size");
+  DeviceState *st = device_state();
+  if (!st)
+    return MTRT_RUNTIME_ERROR;
+  const bool fast = w_prepacked && K > 0 && K % 64 == 0 && block % 64 == 0 && aligned(a, 16) && aligned(w_prepacked, 16);
+  if (fast) {
+    void *args[] = {&a, &w_prepacked, &scale, &y, &M, &K, &N, &block};
+    if (M <= 32)
+      return launch(st, "mtrt_gemm_w4a16_skinny", uint32_t((N + 31) / 32), kBlock, as_hip(stream), args);
+    // Big tiles once they still fill the chip; smaller tiles otherwise.
+    const int64_t big = ((M + 255) / 256) * ((N + 127) / 128);
+    if (big >= int64_t(num_compute_units(st)) * 2)
+      return launch(st, "mtrt_gemm_w4a16_t256x128", uint32_t(big), kBlock, as_hip(stream), args);
+    const int64_t small = ((M + 127) / 128) * ((N + 63) / 64);
+    return launch(st, "mtrt_gemm_w4a16_t128x64", uint32_t(small), kBlock, as_hip(stream), args);
+  }
+  if (!w_kn_packed)
+    return set_error(MTRT_INVALID_ARGUMENT, "this shape needs the original packed weights (K=%lld block=%lld)",
+                     (long long)K, (long long)block);
+  void *args[] = {&a, &w_kn_packed, &scale, &y, &M, &K, &N, &block};
+  return launch(st, "mtrt_gemm_w4a16_any", blocks_for(M * N, kBlock), kBlock, as_hip(stream), args);
+}
+
 } // extern "C"

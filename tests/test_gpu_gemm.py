@@ -3,6 +3,14 @@
 W8A8: the int32 accumulators are exact under any summation order and the epilogue is a
 fixed chain of correctly rounded f32 operations followed by one f16 narrowing, so the
 f16 outputs must be BIT-IDENTICAL to the oracle's.
+
+W4A16: the dequantised weights are bit-exact (one f16 rounding, checked by reading them
+back through one-hot activations); the f32 accumulation runs in the matrix cores' order,
+not the host's left-to-right order, so outputs are compared under a tolerance:
+    |got - ref| <= 1e-3 * |ref| + 1 ulp_f16(ref) + 1e-3 * sqrt(K) * rms(a_row) * rms(wd_col)
+The last term is the scale of the rounding noise of a length-K f32 dot product whose terms
+cancel; without it results near zero could not be compared relatively at all.  The same bound
+is applied against a float64 evaluation.
 """
 import numpy as np
 import pytest
@@ -90,3 +98,93 @@ def test_w8a8_argument_checks(pkg):
     assert L.mtrt_hip_gemm_w8a8(None, t.data_ptr(), t.data_ptr(), t.data_ptr(), t.data_ptr(), t.data_ptr(), -1, 128, 4) == 1
     assert L.mtrt_hip_gemm_w8a8(None, None, t.data_ptr(), t.data_ptr(), t.data_ptr(), t.data_ptr(), 4, 128, 4) == 1
     assert L.mtrt_hip_gemm_w8a8(None, t.data_ptr(), t.data_ptr(), t.data_ptr(), t.data_ptr(), t.data_ptr(), 0, 128, 4) == 0
+
+
+# ---------------------------------------------------------------------------------------
+# W4A16
+# ---------------------------------------------------------------------------------------
+
+def _w4a16_inputs(orc, g, M, K, N, B):
+    a = orc.narrow(g.standard_normal((M, K), dtype=np.float32), orc.F16)
+    w = g.integers(-8, 8, (K, N)).astype(np.int8)
+    s = orc.narrow(g.uniform(0.005, 0.02, (K // B, N)).astype(np.float32), orc.F16)
+    return a, w, orc.pack_int4(w), s
+
+
+def _run_w4a16(pkg, a, wp_host, s, K, N, B, prepack=True):
+    import torch
+    ad = torch.from_numpy(a.view(np.int16)).view(torch.float16).cuda()
+    wd = torch.from_numpy(wp_host).cuda()
+    sd = torch.from_numpy(s.view(np.int16)).view(torch.float16).cuda()
+    pre = pkg.gemm_w4a16_prepack(wd, K, N) if prepack else None
+    y = pkg.gemm_w4a16(ad, sd, K, N, B, w_kn_packed=wd, w_prepacked=pre)
+    return y, pkg.last_kernel()
+
+
+def _check_w4a16(orc, y, a, w, s, K, N, B, ref_bits):
+    got = bits16(y).reshape(-1, N).view(np.float16).astype(np.float64)
+    ref = ref_bits.view(np.float16).astype(np.float64)
+    af = a.view(np.float16).astype(np.float64)
+    wdf = (w.astype(np.float16) * np.repeat(s.view(np.float16), B, axis=0)).astype(np.float64)
+    exact = af @ wdf
+    noise = 1e-3 * np.sqrt(K) * np.sqrt((af ** 2).mean(axis=1))[:, None] * np.sqrt((wdf ** 2).mean(axis=0))[None, :]
+    def ulp(v):
+        return 2.0 ** np.floor(np.log2(np.maximum(np.abs(v), 2.0 ** -14))) * 2.0 ** -10
+    for name, target in (("oracle", ref), ("float64", exact)):
+        bound = 1e-3 * np.abs(target) + ulp(target) + noise
+        err = np.abs(got - target)
+        assert np.all(err <= bound), "%s: worst excess %g at %s" % (name, (err - bound).max(), np.unravel_index(np.argmax(err - bound), err.shape))
+    return np.count_nonzero(got != ref) / got.size
+
+
+@pytest.mark.parametrize("shape", [(16, 256, 64), (1, 128, 32), (32, 1024, 96), (7, 512, 40), (33, 256, 64), (128, 512, 64),
+                                   (200, 384, 100), (300, 1024, 256), (512, 256, 384)])
+def test_w4a16_small_shapes(pkg, orc, shape):
+    M, K, N = shape
+    B = 128
+    a, w, wp, s = _w4a16_inputs(orc, rng(M + K + N), M, K, N, B)
+    y, kernel = _run_w4a16(pkg, a, wp, s, K, N, B)
+    assert kernel == ("mtrt_gemm_w4a16_skinny" if M <= 32 else "mtrt_gemm_w4a16_t128x64")
+    _check_w4a16(orc, y, a, w, s, K, N, B, orc.gemm_w4a16(a, wp, s, K, N, B))
+
+
+def test_w4a16_dequantised_weights_are_bit_exact(pkg, orc):
+    """One-hot activations read the dequantised weights back unchanged: pins the prepack order,
+    the nibble decoding, the block index of the scale and the single f16 rounding."""
+    K, N, B = 512, 160, 128
+    g = rng(31)
+    w = g.integers(-8, 8, (K, N)).astype(np.int8)
+    s = orc.narrow(g.uniform(0.005, 0.02, (K // B, N)).astype(np.float32), orc.F16)
+    eye = np.zeros((K, K), np.float32)
+    np.fill_diagonal(eye, 1.0)
+    wd = (w.astype(np.float16) * np.repeat(s.view(np.float16), B, axis=0)).view(np.uint16)
+    for rows in (slice(0, K), slice(0, 32), slice(100, 116)):        # big-tile, skinny (32 rows), skinny (16 rows)
+        a = orc.narrow(eye[rows], orc.F16)
+        y, kernel = _run_w4a16(pkg, a, orc.pack_int4(w), s, K, N, B)
+        assert np.array_equal(bits16(y).reshape(-1, N), wd[rows]), kernel
+
+
+def test_w4a16_generic_kernel(pkg, orc):
+    for (M, K, N, B) in ((5, 48, 7, 16), (9, 100, 33, 20), (3, 128, 6, 128)):
+        a, w, wp, s = _w4a16_inputs(orc, rng(M * K + N), M, K, N, B)
+        y, kernel = _run_w4a16(pkg, a, wp, s, K, N, B, prepack=False)
+        assert kernel == "mtrt_gemm_w4a16_any"
+        # same left-to-right f32 accumulation as the host: bit-identical
+        assert np.array_equal(bits16(y).reshape(M, N), orc.gemm_w4a16(a, wp, s, K, N, B))
+
+
+@pytest.mark.parametrize("M", [16, 256, 4096])
+def test_c5_w4a16_full_size(pkg, orc, M):
+    """BASELINE config 5: K=4096, N=11008, block 128, M in {16, 256, 4096}, seed 5.  The oracle
+    evaluates up to 40 rows spread over the tiles; all N columns of those rows are compared."""
+    K, N, B = 4096, 11008, 128
+    a, w, wp, s = _w4a16_inputs(orc, rng(5), M, K, N, B)
+    y, kernel = _run_w4a16(pkg, a, wp, s, K, N, B)
+    assert kernel == {16: "mtrt_gemm_w4a16_skinny", 256: "mtrt_gemm_w4a16_t128x64", 4096: "mtrt_gemm_w4a16_t256x128"}[M]
+    rows = sorted(set([0, M - 1] + list(range(0, M, max(1, M // 38)))))[:40]
+    orc.set_threads(16)
+    import torch
+    got = y[rows].contiguous()
+    ref = np.concatenate([orc.gemm_w4a16(a, wp, s, K, N, B, m0=r, mcount=1) for r in rows])
+    orc.set_threads(1)
+    _check_w4a16(orc, got, a[rows], w, s, K, N, B, ref)
