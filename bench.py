@@ -10,8 +10,8 @@ programs of BASELINE.json's configs run back to back through the C ABI
     C2a LayerNorm                           bf16 [8192,4096]
     C2b softmax                             f16 [4096,4096]
     C3  amax + fused quantize->dequantize   bf16 [16384,8192] -> f8E4M3FN  (amax/448)
-    C4  W8A8 GEMM                           M=2048 K=4096 N=11008          (when built)
-    C5  W4A16 GEMM                          M in {16,256,4096}             (when built)
+    C4  W8A8 GEMM + dequantize epilogue     M=2048 K=4096 N=11008          (weights re-laid once, untimed)
+    C5  W4A16 block-wise GEMM               M in {16,256,4096} K=4096 N=11008 block 128
 The metric is BASELINE.json's: achieved HBM GB/s (memory-bound kernels) and MFMA
 TOPS (GEMMs) as a percentage of MI355X peak.  For a step that mixes both, `value`
 is the time-weighted percentage: 100 * (sum over kernels of the time the kernel
@@ -137,6 +137,49 @@ def build_workloads(pkg, torch, which):
         out.append(dict(name="mtrt_qdq_uniform_bf16_f8", config="C3", bound="hbm", work=5.0 * n, nslots=ns, make=qdq,
                         keep=(qs, ys)))
 
+    if which in ("all", "c4"):
+        M, K, N = 2048, 4096, 11008
+        ns = slots_for(M * K + K * N + 2 * M * N)
+        g = torch.Generator(device=dev)
+        g.manual_seed(4)
+
+        def q8(shape):
+            return torch.clamp(torch.round(torch.randn(shape, generator=g, device=dev) * 40.0), -128, 127).to(torch.int8)
+        a4 = [q8((M, K)) for _ in range(ns)]
+        w4 = [pkg.gemm_w8a8_prepack(q8((K, N))) for _ in range(ns)]       # weights are constants: re-laid once, untimed
+        as4 = (torch.rand(M, generator=g, device=dev) * 0.015 + 0.005)
+        ws4 = (torch.rand(N, generator=g, device=dev) * 0.015 + 0.005)
+        y4 = [torch.empty((M, N), dtype=torch.float16, device=dev) for _ in range(ns)]
+
+        def gemm8(i, a4=a4, w4=w4, y4=y4, as4=as4, ws4=ws4, M=M, K=K, N=N):
+            a = (a4[i].data_ptr(), w4[i].data_ptr(), as4.data_ptr(), ws4.data_ptr(), y4[i].data_ptr(), M, K, N)
+            return lambda: pkg.check(L.mtrt_hip_gemm_w8a8(stream(), *a))
+        out.append(dict(name="mtrt_gemm_w8a8_nk", config="C4", bound="mfma", work=2.0 * M * K * N, peak=INT8_PEAK,
+                        unit="TOP/s", nslots=ns, make=gemm8, keep=(a4, w4, y4, as4, ws4)))
+
+    if which in ("all", "c5"):
+        K, N, B = 4096, 11008, 128
+        g = torch.Generator(device=dev)
+        g.manual_seed(5)
+        for M, kname in ((16, "mtrt_gemm_w4a16_skinny"), (256, "mtrt_gemm_w4a16_t128x64"), (4096, "mtrt_gemm_w4a16_t256x128")):
+            nbytes = K * N // 2 + (K // B) * N * 2 + M * K * 2 + M * N * 2
+            ns = min(slots_for(nbytes), 24)
+            a5 = [torch.randn((M, K), generator=g, device=dev).half() for _ in range(ns)]
+            w5 = [pkg.gemm_w4a16_prepack(torch.randint(0, 256, (K * N // 2,), generator=g, device=dev, dtype=torch.uint8), K, N)
+                  for _ in range(ns)]                                      # re-laid once, untimed
+            s5 = [(torch.rand((K // B, N), generator=g, device=dev) * 0.015 + 0.005).half() for _ in range(ns)]
+            y5 = [torch.empty((M, N), dtype=torch.float16, device=dev) for _ in range(ns)]
+
+            def gemm4(i, a5=a5, w5=w5, s5=s5, y5=y5, M=M):
+                a = (a5[i].data_ptr(), None, w5[i].data_ptr(), s5[i].data_ptr(), y5[i].data_ptr(), M, K, N, B)
+                return lambda: pkg.check(L.mtrt_hip_gemm_w4a16(stream(), *a))
+            if M == 16:      # arithmetic intensity ~61 FLOP/B: bound by reading the weights once
+                out.append(dict(name=kname, config="C5 M=16", bound="hbm", work=float(nbytes), nslots=ns, make=gemm4,
+                                keep=(a5, w5, s5, y5)))
+            else:
+                out.append(dict(name=kname, config="C5 M=%d" % M, bound="mfma", work=2.0 * M * K * N, peak=F16_PEAK,
+                                unit="TFLOP/s", nslots=ns, make=gemm4, keep=(a5, w5, s5, y5)))
+
     for w in out:
         w["peak"] = HBM_PEAK if w["bound"] == "hbm" else w["peak"]
         w["unit"] = "GB/s" if w["bound"] == "hbm" else w["unit"]
@@ -243,6 +286,24 @@ def cpu_baseline(which):
         t += timed(lambda: orc.dequantize(q, orc.F8E4M3FN, orc.BF16, s, orc.SCALE_UNIFORM, rows, 8192))
         total += t * (16384 / rows)
         parts.append("C3 %d of 16384 rows" % rows)
+    if which in ("all", "c4"):
+        M, K, N, rows = 2048, 4096, 11008, 8
+        a = np.clip(np.rint(g.standard_normal((rows, K)) * 40), -128, 127).astype(np.int8)
+        w = np.clip(np.rint(g.standard_normal((K, N)) * 40), -128, 127).astype(np.int8)
+        a_s = g.uniform(0.005, 0.02, rows).astype(np.float32)
+        w_s = g.uniform(0.005, 0.02, N).astype(np.float32)
+        total += timed(lambda: orc.gemm_w8a8(a, w, a_s, w_s)) * (M / rows)
+        parts.append("C4 %d of 2048 rows" % rows)
+    if which in ("all", "c5"):
+        K, N, B, rows = 4096, 11008, 128, 4
+        a = orc.narrow(g.standard_normal((rows, K), dtype=np.float32), orc.F16)
+        wp = orc.pack_int4(g.integers(-8, 8, (K, N)).astype(np.int8))
+        sc = orc.narrow(g.uniform(0.005, 0.02, (K // B, N)).astype(np.float32), orc.F16)
+        orc.gemm_w4a16(a, wp, sc, K, N, B, mcount=0)                      # dequantised weights built once per call: time it apart
+        t_deq = timed(lambda: orc.gemm_w4a16(a, wp, sc, K, N, B, mcount=0))
+        t_rows = timed(lambda: orc.gemm_w4a16(a, wp, sc, K, N, B)) - t_deq
+        total += 3 * t_deq + max(t_rows, 0.0) / rows * (16 + 256 + 4096)
+        parts.append("C5 weight dequantisation in full + %d rows, scaled to M=16,256,4096" % rows)
     return total, ", ".join(parts)
 
 
@@ -251,7 +312,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="all", choices=["all", "c1", "c2a", "c2b", "c3"])
+    ap.add_argument("--workload", default="all", choices=["all", "c1", "c2a", "c2b", "c3", "c4", "c5"])
     ap.add_argument("--kernel-reps", type=int, default=100, help="launches per kernel for the per-kernel timing")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -304,8 +365,8 @@ def main():
         "unit": "% of MI355X peak (time-weighted over the step's kernels)",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32/bf16/f16 -> i8/f8e4m3fn (f32 arithmetic)", "data": "synthetic (seeded)",
-        "config": {"workload": {"all": "C1+C2a+C2b+C3 programs of BASELINE.json, one pass each per step"}.get(
+        "dtype": "f32 (Q/DQ, LayerNorm, softmax), int8->int32 (W8A8), f16->f32 (W4A16)", "data": "synthetic (seeded)",
+        "config": {"workload": {"all": "C1+C2a+C2b+C3+C4+C5 programs of BASELINE.json, one pass each per step"}.get(
             args.workload, args.workload.upper()), "kernels_per_step": len(wl)},
         "roofline": {"kernel": dom["kernel"], "bound": dom["bound"], "achieved": dom["achieved"], "peak": dom["peak"],
                      "unit": dom["unit"], "frac": dom["frac"], "traffic": traffic_from_profile(dom["kernel"])},
