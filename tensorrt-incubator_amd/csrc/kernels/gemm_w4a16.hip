@@ -21,11 +21,13 @@
 // rounding the program asks for.
 //
 // Large M: dequantisation happens in registers on the way INTO LDS; the multiply loop
-// is the plain f16 loop over 128-byte LDS rows (same swizzle as the int8 GEMM).
+// is the shared one of gemm_core.hpp (256 x 256 tiles, activations by direct-to-LDS
+// loads, v_mfma_f32_32x32x16_f16).  Medium M uses a 128 x 64 tile variant of the same
+// idea so that the grid still fills the chip.
 // Small M (<= 32): the GEMM is bound by reading the weights once.  One workgroup per
 // 32 columns, its four waves split K, fragments go straight from global memory into
 // registers (no LDS on the way in), partial tiles are added through LDS at the end.
-#include "common.hpp"
+#include "gemm_core.hpp"
 
 using namespace mtrt_dev;
 
@@ -166,12 +168,76 @@ __device__ __forceinline__ void gemm_tiles(const uint16_t* __restrict__ a, const
 // The entry points below have C linkage; they sit inside the namespace only so that
 // its helper names do not meet those of the other clusters in the one-module build.
 
-// (a [M,K] f16, w_prepacked, scale [K/block, N] f16, y [M,N] f16, M, K, N, block) ; K % 64 == 0, block % 64 == 0.
-extern "C" __global__ void __launch_bounds__(THREADS) mtrt_gemm_w4a16_t256x128(
+struct F16Traits {
+  using Acc = v16f;
+  static __device__ __forceinline__ Acc zero() {
+    Acc z;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) z[r] = 0.0f;
+    return z;
+  }
+  static __device__ __forceinline__ Acc mfma(gemm_core::v4i a, gemm_core::v4i b, Acc c) {
+    union { gemm_core::v4i i; v8h h; } ua, ub;
+    ua.i = a; ub.i = b;
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(ua.h, ub.h, c, 0, 0, 0);
+  }
+};
+
+// int4 weights of a 256-column panel: 8 column tiles x (64 lanes x 16 B) per 64-k slice.
+// Thread t fetches fragment lane (t & 63) of column tiles (t >> 6) and (t >> 6) + 4, keeps the
+// raw nibbles and the scales in registers while the slice before is multiplied, then
+// dequantises into the LDS panel.
+struct Int4Loader {
+  const uint32_t* wp;
+  const uint16_t* scale;
+  int64_t kblocks, N, block, tile0;
+  u4 raw[2];
+  h2 sc[2];
+  __device__ __forceinline__ void issue(int64_t slice, int8_t*) {
+    const int lane = threadIdx.x & 63;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int64_t tile = tile0 + (threadIdx.x >> 6) + 4 * i;
+      const int64_t col = tile * 32 + (lane & 31);
+      const bool live = col < N;
+      raw[i] = live ? *reinterpret_cast<const u4*>(wp + ((tile * kblocks + slice) * 64 + lane) * 4)
+                    : (u4){0x88888888u, 0x88888888u, 0x88888888u, 0x88888888u};
+      sc[i] = live ? load_scale2(scale, ((slice * BKH) / block) * N + col) : (h2){(_Float16)0.0f, (_Float16)0.0f};
+    }
+  }
+  __device__ __forceinline__ void commit(int8_t* panel) {
+    const int lane = threadIdx.x & 63;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int row = ((threadIdx.x >> 6) + 4 * i) * 32 + (lane & 31);
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        *reinterpret_cast<u4*>(panel + gemm_core::lds_off(row, 2 * j + (lane >> 5))) = dequant8(raw[i][j], sc[i]);
+    }
+  }
+};
+
+struct PlainEpilogue {
+  __device__ __forceinline__ void setup(int8_t*, int64_t, int64_t) {}
+  __device__ __forceinline__ void column(int64_t, int64_t) {}
+  __device__ __forceinline__ void convert4(const v16f& acc, int q, int, uint32_t (&bits)[4]) const {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) bits[e] = f32_to_f16_bits(acc[4 * q + e]);
+  }
+};
+
+// (a [M,K] f16, w_prepacked, scale [K/block, N] f16, y [M,N] f16, M, K, N, block) ; K % 64 == 0, block % 64 == 0,
+// a 16-byte aligned and below 4 GiB.  grid = 8 * ceil(ceil(N/256) / 8) * ceil(M/256), block = 256.
+extern "C" __global__ void __launch_bounds__(gemm_core::THREADS, 1) mtrt_gemm_w4a16_t256x256(
     const uint16_t* __restrict__ a, const uint32_t* __restrict__ wp, const uint16_t* __restrict__ scale,
     uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t block) {
-  __shared__ __attribute__((aligned(16))) int8_t lds[2 * (256 + 128) * 128];
-  gemm_tiles<4, 2>(a, wp, scale, y, M, K, N, block, lds);
+  __shared__ __attribute__((aligned(16))) int8_t lds[gemm_core::LDS_BYTES];
+  int64_t m0, n0;
+  if (!gemm_core::tile_origin(M, N, m0, n0)) return;
+  Int4Loader bl;
+  bl.wp = wp; bl.scale = scale; bl.kblocks = K / BKH; bl.N = N; bl.block = block; bl.tile0 = n0 / 32;
+  PlainEpilogue epi;
+  gemm_core::run<F16Traits>(reinterpret_cast<const int8_t*>(a), 2 * K, bl, epi, y, M, N, K / BKH, m0, n0, lds);
 }
 extern "C" __global__ void __launch_bounds__(THREADS) mtrt_gemm_w4a16_t128x64(
     const uint16_t* __restrict__ a, const uint32_t* __restrict__ wp, const uint16_t* __restrict__ scale,

@@ -278,8 +278,11 @@ int32_t mtrt_hip_gemm_w8a8(mtrt_stream_t stream, const void *a, const void *w_nk
     return MTRT_RUNTIME_ERROR;
   void *args[] = {&a, &w_nk, &a_scale, &w_scale, &y, &M, &K, &N};
   // The matrix-core kernel moves 128-byte K slices with 16-byte accesses.
-  if (K > 0 && K % 128 == 0 && aligned(a, 16) && aligned(w_nk, 16)) {
-    const int64_t tiles = ((M + 255) / 256) * ((N + 127) / 128);
+  if (K > 0 && K % 128 == 0 && aligned(a, 16) && aligned(w_nk, 16) && M * K < (int64_t(1) << 32) &&
+      N * K < (int64_t(1) << 32)) {
+    // 256 x 256 tiles; N panels are dealt round-robin to the 8 XCDs (see gemm_core.hpp): the
+    // grid is padded to 8 * ceil(panels / 8) * tiles_m workgroups.
+    const int64_t tiles = 8 * ((((N + 255) / 256) + 7) / 8) * ((M + 255) / 256);
     if (tiles <= int64_t(kMaxGrid) * 1024)
       return launch(st, "mtrt_gemm_w8a8_nk", uint32_t(tiles), kBlock, as_hip(stream), args);
   }
@@ -332,10 +335,12 @@ int32_t mtrt_hip_gemm_w4a16(mtrt_stream_t stream, const void *a, const void *w_k
     void *args[] = {&a, &w_prepacked, &scale, &y, &M, &K, &N, &block};
     if (M <= 32)
       return launch(st, "mtrt_gemm_w4a16_skinny", uint32_t((N + 31) / 32), kBlock, as_hip(stream), args);
-    // Big tiles once they still fill the chip; smaller tiles otherwise.
-    const int64_t big = ((M + 255) / 256) * ((N + 127) / 128);
-    if (big >= int64_t(num_compute_units(st)) * 2)
-      return launch(st, "mtrt_gemm_w4a16_t256x128", uint32_t(big), kBlock, as_hip(stream), args);
+    // 256 x 256 tiles once they still fill the chip twice over (and the activations stay
+    // inside 32-bit byte offsets); 128 x 64 tiles otherwise.
+    const int64_t panels = (N + 255) / 256, tiles_m = (M + 255) / 256;
+    if (panels * tiles_m >= int64_t(num_compute_units(st)) * 2 && M * K * 2 < (int64_t(1) << 32))
+      return launch(st, "mtrt_gemm_w4a16_t256x256", uint32_t(8 * ((panels + 7) / 8) * tiles_m), kBlock, as_hip(stream),
+                    args);
     const int64_t small = ((M + 127) / 128) * ((N + 63) / 64);
     return launch(st, "mtrt_gemm_w4a16_t128x64", uint32_t(small), kBlock, as_hip(stream), args);
   }

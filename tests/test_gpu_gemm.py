@@ -180,7 +180,7 @@ def test_c5_w4a16_full_size(pkg, orc, M):
     K, N, B = 4096, 11008, 128
     a, w, wp, s = _w4a16_inputs(orc, rng(5), M, K, N, B)
     y, kernel = _run_w4a16(pkg, a, wp, s, K, N, B)
-    assert kernel == {16: "mtrt_gemm_w4a16_skinny", 256: "mtrt_gemm_w4a16_t128x64", 4096: "mtrt_gemm_w4a16_t256x128"}[M]
+    assert kernel == {16: "mtrt_gemm_w4a16_skinny", 256: "mtrt_gemm_w4a16_t128x64", 4096: "mtrt_gemm_w4a16_t256x256"}[M]
     rows = sorted(set([0, M - 1] + list(range(0, M, max(1, M // 38)))))[:40]
     orc.set_threads(16)
     import torch
@@ -188,3 +188,17 @@ def test_c5_w4a16_full_size(pkg, orc, M):
     ref = np.concatenate([orc.gemm_w4a16(a, wp, s, K, N, B, m0=r, mcount=1) for r in rows])
     orc.set_threads(1)
     _check_w4a16(orc, got, a[rows], w, s, K, N, B, ref)
+
+
+def test_w4a16_big_tile_kernel_ragged_edges(pkg, orc):
+    """The 256 x 256-tile kernel on a shape whose M and N are not multiples of the tile
+    (M = 2000, N = 16416 = 513 column tiles of 32), K = 256 so the oracle stays cheap."""
+    M, K, N, B = 2000, 256, 16416, 128
+    a, w, wp, s = _w4a16_inputs(orc, rng(77), M, K, N, B)
+    y, kernel = _run_w4a16(pkg, a, wp, s, K, N, B)
+    assert kernel == "mtrt_gemm_w4a16_t256x256"
+    rows = sorted(set([0, 1, 127, 128, 255, 256, 1023, 1791, 1792, 1998, 1999] + list(range(5, M, 97))))
+    orc.set_threads(16)
+    ref = np.concatenate([orc.gemm_w4a16(a, wp, s, K, N, B, m0=r, mcount=1) for r in rows])
+    orc.set_threads(1)
+    _check_w4a16(orc, y[rows].contiguous(), a[rows], w, s, K, N, B, ref)
