@@ -55,12 +55,17 @@ constexpr int THREADS = 256;
 constexpr int A_BYTES = BM * BKB, B_BYTES = BN * BKB, STAGE = A_BYTES + B_BYTES;
 constexpr int kOutRow = 144;                           // bytes per LDS row of the output staging (64 f16 + pad)
 constexpr int kOutWave = 128 * kOutRow;
-constexpr int LDS_BYTES = 2 * STAGE;                   // 128 KiB (output staging needs 4 * kOutWave + 1 KiB, less)
+constexpr int LDS_BYTES = 2 * STAGE;                   // 128 KiB (output staging needs 4 * kOutWave + 2 KiB, less)
 
 __device__ __forceinline__ int lds_off(int row, int chunk) { return row * BKB + ((chunk ^ ((row >> 1) & 7)) << 4); }
 
 typedef __attribute__((address_space(3))) void lds_void_t;
 typedef __attribute__((address_space(1))) const void global_void_t;
+
+template <int V>
+struct IntC {
+  static constexpr int value = V;
+};
 
 // Byte operand [rows, row_bytes] -> one 256-row LDS panel per slice, by direct-to-LDS loads.
 // A panel is 32 groups of 8 rows (1 KiB each); wave w moves groups 8w .. 8w+7.  In a group
@@ -69,30 +74,42 @@ typedef __attribute__((address_space(1))) const void global_void_t;
 struct DmaLoader {
   uint32_t off[8];
   const int8_t* base;
+  int wave_u;                                          // wave index as a scalar: the LDS base of a load must be uniform
   __device__ __forceinline__ void init(const int8_t* operand, int64_t rows, int64_t row_bytes, int64_t r0) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    wave_u = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     base = operand;
 #pragma unroll
     for (int g = 0; g < 8; ++g) {
-      const int lrow = (wave * 8 + g) * 8 + (lane >> 3);
+      const int lrow = (wave_u * 8 + g) * 8 + (lane >> 3);
       int64_t row = r0 + lrow;
       row = row < rows ? row : rows - 1;               // rows past the edge re-read the last row; never stored
       off[g] = uint32_t(row * row_bytes + (((lane & 7) ^ ((lrow >> 1) & 7)) << 4));
     }
   }
-  __device__ __forceinline__ void issue(int64_t slice, int8_t* panel) {
-    const int wave = threadIdx.x >> 6;
-    const int8_t* src = base + slice * BKB;
-#pragma unroll
-    for (int g = 0; g < 8; ++g)
-      __builtin_amdgcn_global_load_lds((global_void_t*)(src + off[g]), (lds_void_t*)(panel + (wave * 8 + g) * 1024), 16, 0, 0);
+  // group g (of 8) of this wave's share of slice `slice`
+  __device__ __forceinline__ void dma(int64_t slice, int8_t* panel, int g) const {
+    __builtin_amdgcn_global_load_lds((global_void_t*)(base + slice * BKB + off[g]), (lds_void_t*)(panel + (wave_u * 8 + g) * 1024), 16, 0, 0);
   }
-  __device__ __forceinline__ void commit(int8_t*) {}
+};
+
+// B operand that is plain bytes in [N, K] order: same transport as A.
+struct DmaB {
+  DmaLoader l;
+  __device__ __forceinline__ void prologue(int8_t* panel0, int64_t) {
+#pragma unroll
+    for (int g = 0; g < 8; ++g) l.dma(0, panel0, g);
+  }
+  template <int PAR, int P>
+  __device__ __forceinline__ void chunk(int c, int64_t s1, int64_t, int8_t* nb) {
+    if (P == 0) l.dma(s1, nb, c);
+  }
 };
 
 // all of this wave's outstanding loads and LDS accesses are done; then meet the other waves
 __device__ __forceinline__ void drain_and_barrier() {
-  __asm__ volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  __builtin_amdgcn_s_waitcnt(0x0070);                  // vmcnt(0) lgkmcnt(0), visible to the compiler's wait-count pass
+  __asm__ volatile("s_barrier" ::: "memory");
 }
 
 struct Frags {
@@ -100,17 +117,12 @@ struct Frags {
   v4i b[4];
 };
 
-__device__ __forceinline__ void read_frags(Frags& f, const int8_t* pa, const int8_t* pb, int wm, int wn, int frow, int chunk) {
-#pragma unroll
-  for (int i = 0; i < 4; ++i) f.a[i] = *reinterpret_cast<const v4i*>(pa + lds_off(wm * 128 + i * 32 + frow, chunk));
-#pragma unroll
-  for (int j = 0; j < 4; ++j) f.b[j] = *reinterpret_cast<const v4i*>(pb + lds_off(wn * 128 + j * 32 + frow, chunk));
-}
-
-// Traits: Acc (16-wide accumulator vector), mfma(a, b, acc), zero().
-// BLoader: issue(slice, lds panel) starts the fetch of a 256-row B panel, commit(lds panel)
-//          finishes it (nothing for direct-to-LDS loads; dequantise + ds_write for int4).
-// Epilogue: setup(lds scratch, m0, M), column(col, N), convert4(acc, q, row in tile, bits).
+// Traits: Acc (16-wide accumulator vector), mfma(first, second, acc), zero().
+// BLoader: prologue(panel of slice 0, last slice) starts slice 0 and whatever it keeps in flight;
+//          chunk<PAR, P>(c, s1, s2, panel of slice s1) is its share of the work that rides with
+//          chunk c (0..7) of k-step P (0..3) while a slice of parity PAR is multiplied; whatever
+//          goes to the panel must be issued in k-steps 0..2.
+// Epilogue: setup(lds scratch, m0, M, n0, N), row(row in tile), convert4(acc, q, col in tile, bits).
 template <class Traits, class BLoader, class Epilogue>
 __device__ __forceinline__ void run(const int8_t* __restrict__ a, int64_t a_row_bytes, BLoader& bl, Epilogue& epi,
                                     uint16_t* __restrict__ y, int64_t M, int64_t N, int64_t slices, int64_t m0,
@@ -121,6 +133,8 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, int64_t a_row_
   const int wm = wave >> 1, wn = wave & 1;             // 2 x 2 waves: 128 x 128 each
   const int frow = lane & 31, fhalf = lane >> 5;
 
+  // acc[i][j] holds the TRANSPOSED 32 x 32 tile (B fragment first): lane l <-> output row
+  // i*32 + (l & 31), register r <-> output column j*32 + 8*(r/4) + 4*(l >> 5) + (r % 4).
   Acc acc[4][4];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
@@ -131,61 +145,95 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, int64_t a_row_
   DmaLoader al;
   al.init(a, M, a_row_bytes, m0);
   Frags f0, f1;
-  al.issue(0, lds);
-  bl.issue(0, lds + A_BYTES);
-  bl.commit(lds + A_BYTES);
-  drain_and_barrier();
-  read_frags(f0, lds, lds + A_BYTES, wm, wn, frow, fhalf);
 
-  auto mfma_all = [&](const Frags& f) {
+  auto read_a = [&](Frags& f, const int8_t* pa, int chunk, int i) {
+    f.a[i] = *reinterpret_cast<const v4i*>(pa + lds_off(wm * 128 + i * 32 + frow, chunk));
+  };
+  auto read_b = [&](Frags& f, const int8_t* pb, int chunk, int j) {
+    f.b[j] = *reinterpret_cast<const v4i*>(pb + lds_off(wn * 128 + j * 32 + frow, chunk));
+  };
+  auto read_frags = [&](Frags& f, const int8_t* pa, const int8_t* pb, int chunk) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 4; ++i) read_a(f, pa, chunk, i);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc[i][j] = Traits::mfma(f.a[i], f.b[j], acc[i][j]);
+    for (int j = 0; j < 4; ++j) read_b(f, pb, chunk, j);
   };
 
-  for (int64_t s = 0; s < slices; ++s) {
-    const int cur = int(s & 1);
-    const int8_t* pa = lds + cur * STAGE;
+#pragma unroll
+  for (int g = 0; g < 8; ++g) al.dma(0, lds, g);
+  bl.prologue(lds + A_BYTES, last);
+  drain_and_barrier();
+  read_frags(f0, lds, lds + A_BYTES, fhalf);
+
+  // One K slice = 4 k-steps = 4 x 8 chunks.  A chunk is two MFMAs, one fragment read for the
+  // next k-step and a small share of the loaders' work, fenced so that the compiler keeps the
+  // interleave as written (left alone it gathers the LDS reads in front of the MFMAs that
+  // need them and the matrix cores idle for an LDS round trip every k-step).
+  auto kstep = [&](auto par, auto step, const Frags& cur, Frags& nxt, const int8_t* ra, const int8_t* rb, int chunk,
+                   int64_t s1, int64_t s2, int8_t* na, int8_t* nb) {
+    constexpr int PAR = decltype(par)::value, P = decltype(step)::value;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      const int i = c >> 1, j = (c & 1) * 2;
+      acc[i][j] = Traits::mfma(cur.b[j], cur.a[i], acc[i][j]);
+      acc[i][j + 1] = Traits::mfma(cur.b[j + 1], cur.a[i], acc[i][j + 1]);
+      if (c == 0) {                                    // in the order the next k-step consumes them;
+        read_a(nxt, ra, chunk, 0);                     // none in the last chunk, so the wait in front
+        read_b(nxt, rb, chunk, 0);                     // of the next k-step finds them done
+      } else if (c < 4) {
+        read_b(nxt, rb, chunk, c);
+      } else if (c < 7) {
+        read_a(nxt, ra, chunk, c - 3);
+      }
+      if (P == 0) al.dma(s1, na, c);
+      bl.template chunk<PAR, P>(c, s1, s2, nb);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  auto slice_body = [&](auto par, int64_t s) {
+    constexpr int PAR = decltype(par)::value;
+    const int8_t* pa = lds + PAR * STAGE;
     const int8_t* pb = pa + A_BYTES;
-    int8_t* na = lds + (cur ^ 1) * STAGE;
+    int8_t* na = lds + (PAR ^ 1) * STAGE;
+    int8_t* nb = na + A_BYTES;
     const int64_t s1 = s + 1 < last ? s + 1 : last;
-    al.issue(s1, na);
-    bl.issue(s1, na + A_BYTES);
-    read_frags(f1, pa, pb, wm, wn, frow, 2 + fhalf);
-    mfma_all(f0);
-    read_frags(f0, pa, pb, wm, wn, frow, 4 + fhalf);
-    mfma_all(f1);
-    read_frags(f1, pa, pb, wm, wn, frow, 6 + fhalf);
-    mfma_all(f0);
-    bl.commit(na + A_BYTES);
+    const int64_t s2 = s + 2 < last ? s + 2 : last;
+    kstep(par, IntC<0>{}, f0, f1, pa, pb, 2 + fhalf, s1, s2, na, nb);
+    kstep(par, IntC<1>{}, f1, f0, pa, pb, 4 + fhalf, s1, s2, na, nb);
+    kstep(par, IntC<2>{}, f0, f1, pa, pb, 6 + fhalf, s1, s2, na, nb);
     drain_and_barrier();                                 // slice s+1 is in LDS for everybody
-    read_frags(f0, na, na + A_BYTES, wm, wn, frow, fhalf);
-    mfma_all(f1);
+    kstep(par, IntC<3>{}, f1, f0, na, nb, fhalf, s1, s2, na, nb);
+  };
+
+  int64_t s = 0;
+  for (; s + 1 < slices; s += 2) {                     // no branch inside: the loop body stays one basic block
+    slice_body(IntC<0>{}, s);
+    slice_body(IntC<1>{}, s + 1);
   }
+  if (s < slices) slice_body(IntC<0>{}, s);
 
   __syncthreads();                                     // every wave is done with the operand stages
-  epi.setup(lds + 4 * kOutWave, m0, M);
+  epi.setup(lds + 4 * kOutWave, m0, M, n0, N);
   __syncthreads();
   int8_t* out = lds + wave * kOutWave;
   const bool vec_ok = (N % 8 == 0) && ((reinterpret_cast<uintptr_t>(y) & 15) == 0);
 #pragma unroll
   for (int half = 0; half < 2; ++half) {
 #pragma unroll
-    for (int jj = 0; jj < 2; ++jj) {
-      const int j = half * 2 + jj;
-      const int64_t col = n0 + wn * 128 + j * 32 + frow;
-      epi.column(col, N);
+    for (int i = 0; i < 4; ++i) {
+      const int lrow = i * 32 + frow;
+      epi.row(wm * 128 + lrow);
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int jj = 0; jj < 2; ++jj)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const int lrow = i * 32 + q * 8 + fhalf * 4;   // rows lrow .. lrow+3 <-> r = 4q .. 4q+3
+          const int lcol = jj * 32 + q * 8 + fhalf * 4;  // columns lcol .. lcol+3 of this half <-> r = 4q .. 4q+3
           uint32_t bits[4];
-          epi.convert4(acc[i][j], q, wm * 128 + lrow, bits);
-#pragma unroll
-          for (int e = 0; e < 4; ++e)
-            *reinterpret_cast<uint16_t*>(out + (lrow + e) * kOutRow + (jj * 32 + frow) * 2) = uint16_t(bits[e]);
+          epi.convert4(acc[i][half * 2 + jj], q, wn * 128 + half * 64 + lcol, bits);
+          u32x2 packed;
+          packed[0] = bits[0] | (bits[1] << 16);
+          packed[1] = bits[2] | (bits[3] << 16);
+          *reinterpret_cast<u32x2*>(out + lrow * kOutRow + lcol * 2) = packed;
         }
     }
     // each wave reads back only what it wrote itself: no workgroup barrier needed

@@ -59,6 +59,18 @@ __device__ __forceinline__ u4 dequant8(uint32_t w, h2 scale2) {
   return out;
 }
 
+// Half of dequant8: dwords 2*part and 2*part + 1 of the chunk.
+__device__ __forceinline__ void dequant4(uint32_t w, h2 scale2, int part, u4& out) {
+#pragma unroll
+  for (int p = 2 * part; p < 2 * part + 2; ++p) {
+    H2Bits t;
+    t.u = ((w >> (4 * p)) & 0x000F000Fu) | 0x64006400u;
+    const h2 bias = {(_Float16)1032.0f, (_Float16)1032.0f};
+    t.h = (t.h - bias) * scale2;
+    out[p] = t.u;
+  }
+}
+
 __device__ __forceinline__ h2 load_scale2(const uint16_t* __restrict__ scale, int64_t idx) {
   union { uint16_t u; _Float16 h; } c;
   c.u = scale[idx];
@@ -184,42 +196,78 @@ struct F16Traits {
 };
 
 // int4 weights of a 256-column panel: 8 column tiles x (64 lanes x 16 B) per 64-k slice.
-// Thread t fetches fragment lane (t & 63) of column tiles (t >> 6) and (t >> 6) + 4, keeps the
-// raw nibbles and the scales in registers while the slice before is multiplied, then
-// dequantises into the LDS panel.
-struct Int4Loader {
+// Thread t fetches fragment lane (t & 63) of column tiles (t >> 6) and (t >> 6) + 4.  The raw
+// nibbles and scales of a slice are fetched two slices ahead into one of two register sets
+// and dequantised into the LDS panel one slice ahead, in eight units (one prepacked dword ->
+// 8 f16 -> one 16-byte LDS store) that are spread over the first three k-steps of a slice.
+struct Int4B {
   const uint32_t* wp;
   const uint16_t* scale;
-  int64_t kblocks, N, block, tile0;
-  u4 raw[2];
-  h2 sc[2];
-  __device__ __forceinline__ void issue(int64_t slice, int8_t*) {
+  int64_t kblocks, N, tile0;
+  uint32_t slices_per_block;                         // block / 64: slices that share one row of scales
+  u4 raw[2][2];
+  uint32_t sc_bits[2][2];                            // scales as loaded; widened to a pair where they are used,
+                                                     // so that nothing waits for the load where it is issued
+  // No branch here: a conditional load inside the K loop splits its basic block and the
+  // accumulators get shuffled around the split.  Columns past N read the last column's
+  // scales and the last tile's nibbles instead; their results are never stored.
+  template <int SET>
+  __device__ __forceinline__ void fetch(int64_t slice) {
     const int lane = threadIdx.x & 63;
+    const int64_t last_tile = (N + 31) / 32 - 1;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      const int64_t tile = tile0 + (threadIdx.x >> 6) + 4 * i;
-      const int64_t col = tile * 32 + (lane & 31);
-      const bool live = col < N;
-      raw[i] = live ? *reinterpret_cast<const u4*>(wp + ((tile * kblocks + slice) * 64 + lane) * 4)
-                    : (u4){0x88888888u, 0x88888888u, 0x88888888u, 0x88888888u};
-      sc[i] = live ? load_scale2(scale, ((slice * BKH) / block) * N + col) : (h2){(_Float16)0.0f, (_Float16)0.0f};
+      int64_t tile = tile0 + (threadIdx.x >> 6) + 4 * i;
+      tile = tile < last_tile ? tile : last_tile;
+      int64_t col = tile * 32 + (lane & 31);
+      col = col < N ? col : N - 1;
+      raw[SET][i] = *reinterpret_cast<const u4*>(wp + ((tile * kblocks + slice) * 64 + lane) * 4);
+      const int64_t srow = int64_t(uint32_t(slice) / slices_per_block);   // 32-bit: no division loop in the K loop
+      sc_bits[SET][i] = scale[srow * N + col];
     }
   }
-  __device__ __forceinline__ void commit(int8_t* panel) {
+  template <int SET>
+  __device__ __forceinline__ h2 scale_pair(int i) const {
+    H2Bits t;
+    t.u = sc_bits[SET][i] * 0x00010001u;
+    return t.h;
+  }
+  template <int SET>
+  __device__ __forceinline__ void commit_unit(int u, int8_t* panel) {
     const int lane = threadIdx.x & 63;
+    const int i = u >> 2, j = u & 3;
+    const int row = ((threadIdx.x >> 6) + 4 * i) * 32 + (lane & 31);
+    *reinterpret_cast<u4*>(panel + gemm_core::lds_off(row, 2 * j + (lane >> 5))) = dequant8(raw[SET][i][j], scale_pair<SET>(i));
+  }
+  __device__ __forceinline__ void prologue(int8_t* panel0, int64_t last) {
+    fetch<0>(0);
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int u = 0; u < 8; ++u) commit_unit<0>(u, panel0);
+    fetch<1>(1 < last ? 1 : last);
+  }
+  // While slice s (parity PAR) is multiplied, set PAR is free (its slice went to LDS during
+  // s-1) and takes slice s+2; set PAR^1 holds slice s+1 and goes to LDS in 24 steps, three per
+  // unit (two halves of the dequantisation, then the store), one step per chunk of k-steps 0..2.
+  u4 pending;
+  template <int PAR, int P>
+  __device__ __forceinline__ void chunk(int c, int64_t, int64_t s2, int8_t* nb) {
+    if (P == 3) return;
+    const int step = P * 8 + c, u = step / 3, part = step % 3;
+    if (step == 0) fetch<PAR>(s2);
+    const int i = u >> 2, j = u & 3;
+    if (part < 2) {
+      dequant4(raw[PAR ^ 1][i][j], scale_pair<PAR ^ 1>(i), part, pending);
+    } else {
+      const int lane = threadIdx.x & 63;
       const int row = ((threadIdx.x >> 6) + 4 * i) * 32 + (lane & 31);
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        *reinterpret_cast<u4*>(panel + gemm_core::lds_off(row, 2 * j + (lane >> 5))) = dequant8(raw[i][j], sc[i]);
+      *reinterpret_cast<u4*>(nb + gemm_core::lds_off(row, 2 * j + (lane >> 5))) = pending;
     }
   }
 };
 
 struct PlainEpilogue {
-  __device__ __forceinline__ void setup(int8_t*, int64_t, int64_t) {}
-  __device__ __forceinline__ void column(int64_t, int64_t) {}
+  __device__ __forceinline__ void setup(int8_t*, int64_t, int64_t, int64_t, int64_t) {}
+  __device__ __forceinline__ void row(int) {}
   __device__ __forceinline__ void convert4(const v16f& acc, int q, int, uint32_t (&bits)[4]) const {
 #pragma unroll
     for (int e = 0; e < 4; ++e) bits[e] = f32_to_f16_bits(acc[4 * q + e]);
@@ -234,8 +282,8 @@ extern "C" __global__ void __launch_bounds__(gemm_core::THREADS, 1) mtrt_gemm_w4
   __shared__ __attribute__((aligned(16))) int8_t lds[gemm_core::LDS_BYTES];
   int64_t m0, n0;
   if (!gemm_core::tile_origin(M, N, m0, n0)) return;
-  Int4Loader bl;
-  bl.wp = wp; bl.scale = scale; bl.kblocks = K / BKH; bl.N = N; bl.block = block; bl.tile0 = n0 / 32;
+  Int4B bl;
+  bl.wp = wp; bl.scale = scale; bl.kblocks = K / BKH; bl.N = N; bl.slices_per_block = uint32_t(block / BKH); bl.tile0 = n0 / 32;
   PlainEpilogue epi;
   gemm_core::run<F16Traits>(reinterpret_cast<const int8_t*>(a), 2 * K, bl, epi, y, M, N, K / BKH, m0, n0, lds);
 }

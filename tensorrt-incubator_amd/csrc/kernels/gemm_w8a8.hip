@@ -34,18 +34,21 @@ struct ScaleEpilogue {
   const float* a_scale;
   const float* w_scale;
   const float* sa;                                   // a_scale of this tile's 256 rows, in LDS
-  float ws;
-  __device__ __forceinline__ void setup(int8_t* scratch, int64_t m0, int64_t M) {
+  const float* sw;                                   // w_scale of this tile's 256 columns, in LDS
+  float as;
+  __device__ __forceinline__ void setup(int8_t* scratch, int64_t m0, int64_t M, int64_t n0, int64_t N) {
     float* dst = reinterpret_cast<float*>(scratch);
-    const int64_t row = m0 + threadIdx.x;              // 256 threads, 256 rows
+    const int64_t row = m0 + threadIdx.x, col = n0 + threadIdx.x;   // 256 threads: 256 rows, 256 columns
     dst[threadIdx.x] = row < M ? a_scale[row] : 0.0f;
+    dst[256 + threadIdx.x] = col < N ? w_scale[col] : 0.0f;
     sa = dst;
+    sw = dst + 256;
   }
-  __device__ __forceinline__ void column(int64_t col, int64_t N) { ws = col < N ? w_scale[col] : 0.0f; }
-  __device__ __forceinline__ void convert4(const v16i& acc, int q, int row_in_tile, uint32_t (&bits)[4]) const {
-    const f32x4 as = *reinterpret_cast<const f32x4*>(sa + row_in_tile);
+  __device__ __forceinline__ void row(int row_in_tile) { as = sa[row_in_tile]; }
+  __device__ __forceinline__ void convert4(const v16i& acc, int q, int col_in_tile, uint32_t (&bits)[4]) const {
+    const f32x4 ws = *reinterpret_cast<const f32x4*>(sw + col_in_tile);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) bits[e] = f32_to_f16_bits((float(acc[4 * q + e]) * as[e]) * ws);
+    for (int e = 0; e < 4; ++e) bits[e] = f32_to_f16_bits((float(acc[4 * q + e]) * as) * ws[e]);
   }
 };
 
@@ -60,9 +63,9 @@ extern "C" __global__ void __launch_bounds__(gemm_core::THREADS, 1) mtrt_gemm_w8
   __shared__ __attribute__((aligned(16))) int8_t lds[gemm_core::LDS_BYTES];
   int64_t m0, n0;
   if (!gemm_core::tile_origin(M, N, m0, n0)) return;
-  gemm_core::DmaLoader wl;                           // W [N,K] bytes: same access pattern as the A operand
-  wl.init(w, N, K, n0);
-  ScaleEpilogue epi{a_scale, w_scale, nullptr, 0.0f};
+  gemm_core::DmaB wl;                                // W [N,K] bytes: same transport as the A operand
+  wl.l.init(w, N, K, n0);
+  ScaleEpilogue epi{a_scale, w_scale, nullptr, nullptr, 0.0f};
   gemm_core::run<I8Traits>(a, K, wl, epi, y, M, N, K / gemm_core::BKB, m0, n0, lds);
 }
 
