@@ -55,7 +55,8 @@ constexpr int THREADS = 256;
 constexpr int A_BYTES = BM * BKB, B_BYTES = BN * BKB, STAGE = A_BYTES + B_BYTES;
 constexpr int kOutRow = 144;                           // bytes per LDS row of the output staging (64 f16 + pad)
 constexpr int kOutWave = 128 * kOutRow;
-constexpr int LDS_BYTES = 2 * STAGE;                   // 128 KiB (output staging needs 4 * kOutWave + 2 KiB, less)
+constexpr int LDS_BYTES = 2 * STAGE;                   // 128 KiB (output staging of 4 waves needs 4 * kOutWave + 2 KiB, less)
+constexpr int LDS_BYTES_8WAVES = 8 * kOutWave + 2048;  // 146 KiB: output staging of 8 waves (the A ring needs 128 KiB)
 
 __device__ __forceinline__ int lds_off(int row, int chunk) { return row * BKB + ((chunk ^ ((row >> 1) & 7)) << 4); }
 
@@ -71,8 +72,9 @@ struct IntC {
 // A panel is 32 groups of 8 rows (1 KiB each); wave w moves groups 8w .. 8w+7.  In a group
 // lane l owns LDS slot l = (row l >> 3, chunk position l & 7) and therefore fetches chunk
 // (l & 7) ^ swizzle(row) of that row.
-struct DmaLoader {
-  uint32_t off[8];
+template <int G>                                       // G = 32 / waves: groups each wave moves
+struct DmaLoaderT {
+  uint32_t off[G];
   const int8_t* base;
   int wave_u;                                          // wave index as a scalar: the LDS base of a load must be uniform
   __device__ __forceinline__ void init(const int8_t* operand, int64_t rows, int64_t row_bytes, int64_t r0) {
@@ -80,18 +82,19 @@ struct DmaLoader {
     wave_u = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     base = operand;
 #pragma unroll
-    for (int g = 0; g < 8; ++g) {
-      const int lrow = (wave_u * 8 + g) * 8 + (lane >> 3);
+    for (int g = 0; g < G; ++g) {
+      const int lrow = (wave_u * G + g) * 8 + (lane >> 3);
       int64_t row = r0 + lrow;
       row = row < rows ? row : rows - 1;               // rows past the edge re-read the last row; never stored
       off[g] = uint32_t(row * row_bytes + (((lane & 7) ^ ((lrow >> 1) & 7)) << 4));
     }
   }
-  // group g (of 8) of this wave's share of slice `slice`
+  // group g (of G) of this wave's share of slice `slice`
   __device__ __forceinline__ void dma(int64_t slice, int8_t* panel, int g) const {
-    __builtin_amdgcn_global_load_lds((global_void_t*)(base + slice * BKB + off[g]), (lds_void_t*)(panel + (wave_u * 8 + g) * 1024), 16, 0, 0);
+    __builtin_amdgcn_global_load_lds((global_void_t*)(base + slice * BKB + off[g]), (lds_void_t*)(panel + (wave_u * G + g) * 1024), 16, 0, 0);
   }
 };
+using DmaLoader = DmaLoaderT<8>;
 
 // B operand that is plain bytes in [N, K] order: same transport as A.
 struct DmaB {
@@ -116,6 +119,63 @@ struct Frags {
   v4i a[4];
   v4i b[4];
 };
+
+// Accumulators -> y.  acc[i][j] holds the TRANSPOSED 32 x 32 tile (B fragment first): lane l
+// <-> output row i*32 + (l & 31), register r <-> output column j*32 + 8*(r/4) + 4*(l >> 5) + (r % 4),
+// so a lane owns runs of 4 consecutive outputs of a row.  Each wave parks its converted 128 x 128
+// sub-tile (in two halves of 64 columns) in LDS with 8-byte stores, rows padded to 144 B, and
+// writes it out as whole 128-byte row segments, 16 bytes per lane.
+template <int JT, class Acc, class Epilogue>          // JT column tiles per wave: 4 (4 waves, 2 x 2) or 2 (8 waves, 2 x 4)
+__device__ __forceinline__ void write_tile(Acc (&acc)[4][JT], Epilogue& epi, uint16_t* __restrict__ y, int64_t M, int64_t N,
+                                           int64_t m0, int64_t n0, int8_t* lds) {
+  constexpr int NWN = 8 / JT, WAVES = 2 * NWN, WCOLS = 32 * JT;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int wm = wave / NWN, wn = wave % NWN;
+  const int frow = lane & 31, fhalf = lane >> 5;
+  __syncthreads();                                     // every wave is done with the operand stages
+  epi.setup(lds + WAVES * kOutWave, m0, M, n0, N);
+  __syncthreads();
+  int8_t* out = lds + wave * kOutWave;
+  const bool vec_ok = (N % 8 == 0) && ((reinterpret_cast<uintptr_t>(y) & 15) == 0);
+#pragma unroll
+  for (int half = 0; half < JT / 2; ++half) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int lrow = i * 32 + frow;
+      epi.row(wm * 128 + lrow);
+#pragma unroll
+      for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int lcol = jj * 32 + q * 8 + fhalf * 4;  // columns lcol .. lcol+3 of this half <-> r = 4q .. 4q+3
+          uint32_t bits[4];
+          epi.convert4(acc[i][half * 2 + jj], q, wn * WCOLS + half * 64 + lcol, bits);
+          u32x2 packed;
+          packed[0] = bits[0] | (bits[1] << 16);
+          packed[1] = bits[2] | (bits[3] << 16);
+          *reinterpret_cast<u32x2*>(out + lrow * kOutRow + lcol * 2) = packed;
+        }
+    }
+    // each wave reads back only what it wrote itself: no workgroup barrier needed
+#pragma unroll
+    for (int it = 0; it < 16; ++it) {
+      const int lrow = it * 8 + (lane >> 3), ch = lane & 7;
+      const int64_t row = m0 + wm * 128 + lrow;
+      const int64_t col = n0 + wn * WCOLS + half * 64 + ch * 8;
+      const u32x4 v = *reinterpret_cast<const u32x4*>(out + lrow * kOutRow + ch * 16);
+      if (row < M) {
+        if (vec_ok) {
+          if (col < N) *reinterpret_cast<u32x4*>(y + row * N + col) = v;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (col + e < N) y[row * N + col + e] = uint16_t(v[e >> 1] >> (16 * (e & 1)));
+        }
+      }
+    }
+  }
+}
 
 // Traits: Acc (16-wide accumulator vector), mfma(first, second, acc), zero().
 // BLoader: prologue(panel of slice 0, last slice) starts slice 0 and whatever it keeps in flight;
@@ -212,48 +272,7 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, int64_t a_row_
   }
   if (s < slices) slice_body(IntC<0>{}, s);
 
-  __syncthreads();                                     // every wave is done with the operand stages
-  epi.setup(lds + 4 * kOutWave, m0, M, n0, N);
-  __syncthreads();
-  int8_t* out = lds + wave * kOutWave;
-  const bool vec_ok = (N % 8 == 0) && ((reinterpret_cast<uintptr_t>(y) & 15) == 0);
-#pragma unroll
-  for (int half = 0; half < 2; ++half) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int lrow = i * 32 + frow;
-      epi.row(wm * 128 + lrow);
-#pragma unroll
-      for (int jj = 0; jj < 2; ++jj)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int lcol = jj * 32 + q * 8 + fhalf * 4;  // columns lcol .. lcol+3 of this half <-> r = 4q .. 4q+3
-          uint32_t bits[4];
-          epi.convert4(acc[i][half * 2 + jj], q, wn * 128 + half * 64 + lcol, bits);
-          u32x2 packed;
-          packed[0] = bits[0] | (bits[1] << 16);
-          packed[1] = bits[2] | (bits[3] << 16);
-          *reinterpret_cast<u32x2*>(out + lrow * kOutRow + lcol * 2) = packed;
-        }
-    }
-    // each wave reads back only what it wrote itself: no workgroup barrier needed
-#pragma unroll
-    for (int it = 0; it < 16; ++it) {
-      const int lrow = it * 8 + (lane >> 3), ch = lane & 7;
-      const int64_t row = m0 + wm * 128 + lrow;
-      const int64_t col = n0 + wn * 128 + half * 64 + ch * 8;
-      const u32x4 v = *reinterpret_cast<const u32x4*>(out + lrow * kOutRow + ch * 16);
-      if (row < M) {
-        if (vec_ok) {
-          if (col < N) *reinterpret_cast<u32x4*>(y + row * N + col) = v;
-        } else {
-#pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (col + e < N) y[row * N + col + e] = uint16_t(v[e >> 1] >> (16 * (e & 1)));
-        }
-      }
-    }
-  }
+  write_tile<4>(acc, epi, y, M, N, m0, n0, lds);
 }
 
 // Workgroup id -> tile origin with the XCD-aware order described above; false = no tile.

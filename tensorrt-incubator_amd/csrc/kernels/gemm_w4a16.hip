@@ -59,16 +59,23 @@ __device__ __forceinline__ u4 dequant8(uint32_t w, h2 scale2) {
   return out;
 }
 
-// Half of dequant8: dwords 2*part and 2*part + 1 of the chunk.
-__device__ __forceinline__ void dequant4(uint32_t w, h2 scale2, int part, u4& out) {
+// Half of dequant8: dwords 2*part and 2*part + 1 of the chunk.  `mask` is 0x000F000F held in a
+// vector register: the and-or then is ONE instruction (it may name a single scalar or literal
+// operand, and 0x64006400 is that one).
+__device__ __forceinline__ void dequant4(uint32_t w, h2 scale2, int part, uint32_t mask, u4& out) {
 #pragma unroll
   for (int p = 2 * part; p < 2 * part + 2; ++p) {
     H2Bits t;
-    t.u = ((w >> (4 * p)) & 0x000F000Fu) | 0x64006400u;
+    t.u = ((w >> (4 * p)) & mask) | 0x64006400u;
     const h2 bias = {(_Float16)1032.0f, (_Float16)1032.0f};
     t.h = (t.h - bias) * scale2;
     out[p] = t.u;
   }
+}
+__device__ __forceinline__ uint32_t nibble_pair_mask() {
+  uint32_t m = 0x000F000Fu;
+  __asm__ volatile("" : "+v"(m));                     // opaque to the compiler: stays in a vector register
+  return m;
 }
 
 __device__ __forceinline__ h2 load_scale2(const uint16_t* __restrict__ scale, int64_t idx) {
@@ -249,6 +256,7 @@ struct Int4B {
   // s-1) and takes slice s+2; set PAR^1 holds slice s+1 and goes to LDS in 24 steps, three per
   // unit (two halves of the dequantisation, then the store), one step per chunk of k-steps 0..2.
   u4 pending;
+  uint32_t mask = nibble_pair_mask();
   template <int PAR, int P>
   __device__ __forceinline__ void chunk(int c, int64_t, int64_t s2, int8_t* nb) {
     if (P == 3) return;
@@ -256,7 +264,7 @@ struct Int4B {
     if (step == 0) fetch<PAR>(s2);
     const int i = u >> 2, j = u & 3;
     if (part < 2) {
-      dequant4(raw[PAR ^ 1][i][j], scale_pair<PAR ^ 1>(i), part, pending);
+      dequant4(raw[PAR ^ 1][i][j], scale_pair<PAR ^ 1>(i), part, mask, pending);
     } else {
       const int lane = threadIdx.x & 63;
       const int row = ((threadIdx.x >> 6) + 4 * i) * 32 + (lane & 31);
@@ -274,18 +282,159 @@ struct PlainEpilogue {
   }
 };
 
+// ---- large M, weights straight into registers -------------------------------------------
+// The prepacked stream is already in fragment order, so a wave can load the raw nibbles of
+// its own 128 columns (4 column tiles x 16 B per lane and slice) straight into registers and
+// dequantise dword p of each into the B fragment of k-step p: the weights never touch LDS.
+// LDS then carries the activations only (direct-to-LDS loads into a ring of four 32 KiB
+// stages, fetched two slices ahead), which takes the fragment reads, the panel stores and
+// half of the direct-to-LDS traffic of the shared loop off the LDS port; the price is that
+// the two waves of a column half dequantise the same weights.
+// Per k-step a wave issues 16 MFMAs in 8 fenced chunks; each chunk also carries half of one
+// dequantisation (8 VALU instructions) for the next k-step, every other chunk an A fragment
+// read, and in k-step 0 one direct-to-LDS load.  Raw nibbles and scales of slice s+2 are
+// fetched in the last k-step of slice s into the register set that k-step 2 finished with.
+template <int JT>
+struct WeightRegs {
+  const uint32_t* wp;
+  const uint16_t* scale;
+  int64_t kblocks, N, tile0;                         // tile0: first 32-column tile of this wave
+  uint32_t slices_per_block;
+  u4 raw[2][JT];
+  uint32_t sc_bits[2][JT];
+  uint32_t mask = nibble_pair_mask();
+  template <int SET>
+  __device__ __forceinline__ void fetch(int64_t slice) {
+    const int lane = threadIdx.x & 63;
+    const int64_t last_tile = (N + 31) / 32 - 1;
+    const int64_t srow = int64_t(uint32_t(slice) / slices_per_block);
+#pragma unroll
+    for (int j = 0; j < JT; ++j) {
+      int64_t tile = tile0 + j;
+      tile = tile < last_tile ? tile : last_tile;      // columns past N: some valid data, never stored
+      int64_t col = tile * 32 + (lane & 31);
+      col = col < N ? col : N - 1;
+      raw[SET][j] = *reinterpret_cast<const u4*>(wp + ((tile * kblocks + slice) * 64 + lane) * 4);
+      sc_bits[SET][j] = scale[srow * N + col];
+    }
+  }
+  template <int SET, int P>
+  __device__ __forceinline__ void half(int j, int part, u4& frag) const {
+    H2Bits t;
+    t.u = sc_bits[SET][j] * 0x00010001u;
+    dequant4(raw[SET][j][P], t.h, part, mask, frag);
+  }
+};
+
+// JT = 4: 4 waves (2 x 2), one per SIMD, 128 x 128 each.  JT = 2: 8 waves (2 x 4), two per SIMD,
+// 128 x 64 each.  A wave's own VALU, LDS and memory instructions do not overlap its MFMAs (each
+// takes its issue cycles out of the MFMA stream), only another wave's do, so with the
+// dequantisation in the loop two waves per SIMD are the faster shape.
+template <int JT, class Epilogue>
+__device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, int64_t a_row_bytes, WeightRegs<JT>& wr, Epilogue& epi,
+                                                uint16_t* __restrict__ y, int64_t M, int64_t N, int64_t slices, int64_t m0,
+                                                int64_t n0, int8_t* lds) {
+  using namespace gemm_core;
+  constexpr int NWN = 8 / JT, WAVES = 2 * NWN, G = 32 / WAVES;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int wm = wave / NWN;
+  const int frow = lane & 31, fhalf = lane >> 5;
+
+  v16f acc[4][JT];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < JT; ++j) acc[i][j] = F16Traits::zero();
+
+  const int64_t last = slices - 1;
+  DmaLoaderT<G> al;
+  al.init(a, M, a_row_bytes, m0);
+  struct FragSet {
+    v4i a[4];
+    u4 b[JT];
+  } f0, f1;
+  auto read_a = [&](FragSet& f, const int8_t* pa, int chunk, int i) {
+    f.a[i] = *reinterpret_cast<const v4i*>(pa + lds_off(wm * 128 + i * 32 + frow, chunk));
+  };
+  auto stage = [&](int64_t slice) { return lds + int(slice & 3) * A_BYTES; };
+
+#pragma unroll
+  for (int g = 0; g < G; ++g) al.dma(0, stage(0), g);
+#pragma unroll
+  for (int g = 0; g < G; ++g) al.dma(1 < last ? 1 : last, stage(1), g);
+  wr.template fetch<0>(0);
+  wr.template fetch<1>(1 < last ? 1 : last);
+  drain_and_barrier();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) read_a(f0, stage(0), fhalf, i);
+#pragma unroll
+  for (int j = 0; j < JT; ++j) {
+    wr.template half<0, 0>(j, 0, f0.b[j]);
+    wr.template half<0, 0>(j, 1, f0.b[j]);
+  }
+
+  // k-step P of a slice of parity PAR: MFMAs on `cur`, everything for the next k-step into `nxt`.
+  // Four fenced chunks; chunk c multiplies row tile c and carries one A fragment read, JT/2
+  // halves of the next weights' dequantisation and, in k-step 0, G/4 direct-to-LDS loads.
+  auto kstep = [&](auto par, auto step, const FragSet& cur, FragSet& nxt, const int8_t* ra, int chunk, int64_t s2, int8_t* nd) {
+    constexpr int PAR = decltype(par)::value, P = decltype(step)::value;
+    constexpr int NSET = P == 3 ? (PAR ^ 1) : PAR;     // register set and dword the next k-step's weights come from
+    constexpr int NP = P == 3 ? 0 : P + 1;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+#pragma unroll
+      for (int j = 0; j < JT; ++j) acc[c][j] = F16Traits::mfma(__builtin_bit_cast(v4i, cur.b[j]), cur.a[c], acc[c][j]);
+      read_a(nxt, ra, chunk, c);
+#pragma unroll
+      for (int h = 0; h < JT / 2; ++h) {
+        const int unit = c * (JT / 2) + h;               // 2 * JT halves per k-step
+        wr.template half<NSET, NP>(unit >> 1, unit & 1, nxt.b[unit >> 1]);
+      }
+      if (P == 0) {
+#pragma unroll
+        for (int g = 0; g < G / 4; ++g) al.dma(s2, nd, c * (G / 4) + g);
+      }
+      if (P == 3 && c == 0) wr.template fetch<PAR>(s2);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  auto slice_body = [&](auto par, int64_t s) {
+    const int8_t* pa = stage(s);
+    const int64_t s2 = s + 2 < last ? s + 2 : last;
+    int8_t* nd = stage(s + 2);
+    kstep(par, IntC<0>{}, f0, f1, pa, 2 + fhalf, s2, nd);
+    kstep(par, IntC<1>{}, f1, f0, pa, 4 + fhalf, s2, nd);
+    kstep(par, IntC<2>{}, f0, f1, pa, 6 + fhalf, s2, nd);
+    // slice s+1 and the registers of slice s+1 have landed; only this slice's G loads may still fly
+    __builtin_amdgcn_s_waitcnt(0x0070 | G);            // vmcnt(G) lgkmcnt(0)
+    __asm__ volatile("s_barrier" ::: "memory");
+    kstep(par, IntC<3>{}, f1, f0, stage(s + 1), fhalf, s2, nd);
+  };
+
+  int64_t s = 0;
+  for (; s + 1 < slices; s += 2) {
+    slice_body(IntC<0>{}, s);
+    slice_body(IntC<1>{}, s + 1);
+  }
+  if (s < slices) slice_body(IntC<0>{}, s);
+  __builtin_amdgcn_s_waitcnt(0x0070);                  // the surplus loads of the last slices have landed
+  write_tile<JT>(acc, epi, y, M, N, m0, n0, lds);
+}
+
 // (a [M,K] f16, w_prepacked, scale [K/block, N] f16, y [M,N] f16, M, K, N, block) ; K % 64 == 0, block % 64 == 0,
 // a 16-byte aligned and below 4 GiB.  grid = 8 * ceil(ceil(N/256) / 8) * ceil(M/256), block = 256.
-extern "C" __global__ void __launch_bounds__(gemm_core::THREADS, 1) mtrt_gemm_w4a16_t256x256(
+extern "C" __global__ void __launch_bounds__(512, 1) mtrt_gemm_w4a16_t256x256(
     const uint16_t* __restrict__ a, const uint32_t* __restrict__ wp, const uint16_t* __restrict__ scale,
     uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t block) {
-  __shared__ __attribute__((aligned(16))) int8_t lds[gemm_core::LDS_BYTES];
+  __shared__ __attribute__((aligned(16))) int8_t lds[gemm_core::LDS_BYTES_8WAVES];
   int64_t m0, n0;
   if (!gemm_core::tile_origin(M, N, m0, n0)) return;
-  Int4B bl;
-  bl.wp = wp; bl.scale = scale; bl.kblocks = K / BKH; bl.N = N; bl.slices_per_block = uint32_t(block / BKH); bl.tile0 = n0 / 32;
+  WeightRegs<2> wr;
+  wr.wp = wp; wr.scale = scale; wr.kblocks = K / BKH; wr.N = N; wr.slices_per_block = uint32_t(block / BKH);
+  wr.tile0 = n0 / 32 + ((threadIdx.x >> 6) & 3) * 2;
   PlainEpilogue epi;
-  gemm_core::run<F16Traits>(reinterpret_cast<const int8_t*>(a), 2 * K, bl, epi, y, M, N, K / BKH, m0, n0, lds);
+  run_weight_regs<2>(reinterpret_cast<const int8_t*>(a), 2 * K, wr, epi, y, M, N, K / BKH, m0, n0, lds);
 }
 extern "C" __global__ void __launch_bounds__(THREADS) mtrt_gemm_w4a16_t128x64(
     const uint16_t* __restrict__ a, const uint32_t* __restrict__ wp, const uint16_t* __restrict__ scale,

@@ -335,11 +335,12 @@ int32_t mtrt_hip_gemm_w4a16(mtrt_stream_t stream, const void *a, const void *w_k
     void *args[] = {&a, &w_prepacked, &scale, &y, &M, &K, &N, &block};
     if (M <= 32)
       return launch(st, "mtrt_gemm_w4a16_skinny", uint32_t((N + 31) / 32), kBlock, as_hip(stream), args);
-    // 256 x 256 tiles once they still fill the chip twice over (and the activations stay
-    // inside 32-bit byte offsets); 128 x 64 tiles otherwise.
+    // 256 x 256 tiles (512 threads) once they cover at least half of the compute units (measured:
+    // from M = 1024 on at N = 11008 they beat the small tiles) and the activations stay inside
+    // 32-bit byte offsets; 128 x 64 tiles otherwise.
     const int64_t panels = (N + 255) / 256, tiles_m = (M + 255) / 256;
-    if (panels * tiles_m >= int64_t(num_compute_units(st)) * 2 && M * K * 2 < (int64_t(1) << 32))
-      return launch(st, "mtrt_gemm_w4a16_t256x256", uint32_t(8 * ((panels + 7) / 8) * tiles_m), kBlock, as_hip(stream),
+    if (panels * tiles_m * 2 >= int64_t(num_compute_units(st)) && M * K * 2 < (int64_t(1) << 32))
+      return launch(st, "mtrt_gemm_w4a16_t256x256", uint32_t(8 * ((panels + 7) / 8) * tiles_m), 512, as_hip(stream),
                     args);
     const int64_t small = ((M + 127) / 128) * ((N + 63) / 64);
     return launch(st, "mtrt_gemm_w4a16_t128x64", uint32_t(small), kBlock, as_hip(stream), args);
