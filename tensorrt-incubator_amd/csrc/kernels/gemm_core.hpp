@@ -96,28 +96,16 @@ struct DmaLoaderT {
 };
 using DmaLoader = DmaLoaderT<8>;
 
-// B operand that is plain bytes in [N, K] order: same transport as A.
-struct DmaB {
-  DmaLoader l;
-  __device__ __forceinline__ void prologue(int8_t* panel0, int64_t) {
-#pragma unroll
-    for (int g = 0; g < 8; ++g) l.dma(0, panel0, g);
-  }
-  template <int PAR, int P>
-  __device__ __forceinline__ void chunk(int c, int64_t s1, int64_t, int8_t* nb) {
-    if (P == 0) l.dma(s1, nb, c);
-  }
-};
-
 // all of this wave's outstanding loads and LDS accesses are done; then meet the other waves
 __device__ __forceinline__ void drain_and_barrier() {
   __builtin_amdgcn_s_waitcnt(0x0070);                  // vmcnt(0) lgkmcnt(0), visible to the compiler's wait-count pass
   __asm__ volatile("s_barrier" ::: "memory");
 }
 
+template <int JT>
 struct Frags {
   v4i a[4];
-  v4i b[4];
+  v4i b[JT];
 };
 
 // Accumulators -> y.  acc[i][j] holds the TRANSPOSED 32 x 32 tile (B fragment first): lane l
@@ -125,10 +113,10 @@ struct Frags {
 // so a lane owns runs of 4 consecutive outputs of a row.  Each wave parks its converted 128 x 128
 // sub-tile (in two halves of 64 columns) in LDS with 8-byte stores, rows padded to 144 B, and
 // writes it out as whole 128-byte row segments, 16 bytes per lane.
-template <int JT, class Acc, class Epilogue>          // JT column tiles per wave: 4 (4 waves, 2 x 2) or 2 (8 waves, 2 x 4)
+template <int JT, int NWN, class Acc, class Epilogue>  // 2 x NWN waves, JT column tiles (32 wide) per wave
 __device__ __forceinline__ void write_tile(Acc (&acc)[4][JT], Epilogue& epi, uint16_t* __restrict__ y, int64_t M, int64_t N,
                                            int64_t m0, int64_t n0, int8_t* lds) {
-  constexpr int NWN = 8 / JT, WAVES = 2 * NWN, WCOLS = 32 * JT;
+  constexpr int WAVES = 2 * NWN, WCOLS = 32 * JT;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int wm = wave / NWN, wn = wave % NWN;
@@ -177,76 +165,81 @@ __device__ __forceinline__ void write_tile(Acc (&acc)[4][JT], Epilogue& epi, uin
   }
 }
 
+// Both operands as bytes, K-contiguous per row / per column: a [M, a_row_bytes], b [N, a_row_bytes].
+// 4 waves (2 x 2) compute a 256 x (64 * JT) tile: JT = 4 is the full tile, JT = 2 the half-width
+// tile that fills the last, partial round of a launch.
 // Traits: Acc (16-wide accumulator vector), mfma(first, second, acc), zero().
-// BLoader: prologue(panel of slice 0, last slice) starts slice 0 and whatever it keeps in flight;
-//          chunk<PAR, P>(c, s1, s2, panel of slice s1) is its share of the work that rides with
-//          chunk c (0..7) of k-step P (0..3) while a slice of parity PAR is multiplied; whatever
-//          goes to the panel must be issued in k-steps 0..2.
 // Epilogue: setup(lds scratch, m0, M, n0, N), row(row in tile), convert4(acc, q, col in tile, bits).
-template <class Traits, class BLoader, class Epilogue>
-__device__ __forceinline__ void run(const int8_t* __restrict__ a, int64_t a_row_bytes, BLoader& bl, Epilogue& epi,
+template <class Traits, int JT, class Epilogue>
+__device__ __forceinline__ void run(const int8_t* __restrict__ a, const int8_t* __restrict__ b, int64_t row_bytes, Epilogue& epi,
                                     uint16_t* __restrict__ y, int64_t M, int64_t N, int64_t slices, int64_t m0,
                                     int64_t n0, int8_t* lds) {
   using Acc = typename Traits::Acc;
+  constexpr int GB = 2 * JT;                           // direct-to-LDS loads per wave and slice for the B panel
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int wm = wave >> 1, wn = wave & 1;             // 2 x 2 waves: 128 x 128 each
+  const int wm = wave >> 1, wn = wave & 1;             // 2 x 2 waves: 128 x (32 * JT) each
   const int frow = lane & 31, fhalf = lane >> 5;
 
-  // acc[i][j] holds the TRANSPOSED 32 x 32 tile (B fragment first): lane l <-> output row
-  // i*32 + (l & 31), register r <-> output column j*32 + 8*(r/4) + 4*(l >> 5) + (r % 4).
-  Acc acc[4][4];
+  Acc acc[4][JT];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = Traits::zero();
+    for (int j = 0; j < JT; ++j) acc[i][j] = Traits::zero();
 
   const int64_t last = slices - 1;
-  DmaLoader al;
-  al.init(a, M, a_row_bytes, m0);
-  Frags f0, f1;
+  DmaLoaderT<8> al;
+  al.init(a, M, row_bytes, m0);
+  DmaLoaderT<GB> bl;
+  bl.init(b, N, row_bytes, n0);
+  Frags<JT> f0, f1;
 
-  auto read_a = [&](Frags& f, const int8_t* pa, int chunk, int i) {
+  auto read_a = [&](Frags<JT>& f, const int8_t* pa, int chunk, int i) {
     f.a[i] = *reinterpret_cast<const v4i*>(pa + lds_off(wm * 128 + i * 32 + frow, chunk));
   };
-  auto read_b = [&](Frags& f, const int8_t* pb, int chunk, int j) {
-    f.b[j] = *reinterpret_cast<const v4i*>(pb + lds_off(wn * 128 + j * 32 + frow, chunk));
+  auto read_b = [&](Frags<JT>& f, const int8_t* pb, int chunk, int j) {
+    f.b[j] = *reinterpret_cast<const v4i*>(pb + lds_off(wn * (32 * JT) + j * 32 + frow, chunk));
   };
-  auto read_frags = [&](Frags& f, const int8_t* pa, const int8_t* pb, int chunk) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) read_a(f, pa, chunk, i);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) read_b(f, pb, chunk, j);
+  // fragment n of a k-step in the order the MFMAs consume them: a0, b0 .. b(JT-1), a1, a2, a3
+  auto read_nth = [&](Frags<JT>& f, const int8_t* pa, const int8_t* pb, int chunk, int n) {
+    if (n == 0) read_a(f, pa, chunk, 0);
+    else if (n <= JT) read_b(f, pb, chunk, n - 1);
+    else read_a(f, pa, chunk, n - JT);
   };
 
 #pragma unroll
   for (int g = 0; g < 8; ++g) al.dma(0, lds, g);
-  bl.prologue(lds + A_BYTES, last);
+#pragma unroll
+  for (int g = 0; g < GB; ++g) bl.dma(0, lds + A_BYTES, g);
   drain_and_barrier();
-  read_frags(f0, lds, lds + A_BYTES, fhalf);
+#pragma unroll
+  for (int n = 0; n < 4 + JT; ++n) read_nth(f0, lds, lds + A_BYTES, fhalf, n);
 
-  // One K slice = 4 k-steps = 4 x 8 chunks.  A chunk is two MFMAs, one fragment read for the
-  // next k-step and a small share of the loaders' work, fenced so that the compiler keeps the
-  // interleave as written (left alone it gathers the LDS reads in front of the MFMAs that
-  // need them and the matrix cores idle for an LDS round trip every k-step).
-  auto kstep = [&](auto par, auto step, const Frags& cur, Frags& nxt, const int8_t* ra, const int8_t* rb, int chunk,
-                   int64_t s1, int64_t s2, int8_t* na, int8_t* nb) {
-    constexpr int PAR = decltype(par)::value, P = decltype(step)::value;
+  // One K slice = 4 k-steps = 4 x 8 chunks.  A chunk is JT/2 MFMAs, one fragment read for the
+  // next k-step (two in chunk 0, none in the last ones, so that the wait in front of the next
+  // k-step finds them done) and in k-step 0 its share of the loads of the next slice, fenced so
+  // that the compiler keeps the interleave as written (left alone it gathers the LDS reads in
+  // front of the MFMAs that need them and the matrix cores idle for an LDS round trip every
+  // k-step).  A wave's own LDS and memory instructions take their issue cycles out of its MFMA
+  // stream, so there are as few of them as the tile shape allows.
+  auto kstep = [&](auto step, const Frags<JT>& cur, Frags<JT>& nxt, const int8_t* ra, const int8_t* rb, int chunk,
+                   int64_t s1, int8_t* na, int8_t* nb) {
+    constexpr int P = decltype(step)::value;
 #pragma unroll
     for (int c = 0; c < 8; ++c) {
-      const int i = c >> 1, j = (c & 1) * 2;
-      acc[i][j] = Traits::mfma(cur.b[j], cur.a[i], acc[i][j]);
-      acc[i][j + 1] = Traits::mfma(cur.b[j + 1], cur.a[i], acc[i][j + 1]);
-      if (c == 0) {                                    // in the order the next k-step consumes them;
-        read_a(nxt, ra, chunk, 0);                     // none in the last chunk, so the wait in front
-        read_b(nxt, rb, chunk, 0);                     // of the next k-step finds them done
-      } else if (c < 4) {
-        read_b(nxt, rb, chunk, c);
-      } else if (c < 7) {
-        read_a(nxt, ra, chunk, c - 3);
+      const int i = c >> 1, j = (c & 1) * (JT / 2);
+#pragma unroll
+      for (int jj = 0; jj < JT / 2; ++jj) acc[i][j + jj] = Traits::mfma(cur.b[j + jj], cur.a[i], acc[i][j + jj]);
+      if (c == 0) {
+        read_nth(nxt, ra, rb, chunk, 0);
+        read_nth(nxt, ra, rb, chunk, 1);
+      } else if (c + 1 < 4 + JT) {
+        read_nth(nxt, ra, rb, chunk, c + 1);
       }
-      if (P == 0) al.dma(s1, na, c);
-      bl.template chunk<PAR, P>(c, s1, s2, nb);
+      if (P == 0) {
+        al.dma(s1, na, c);
+        if (c < GB) bl.dma(s1, nb, c);
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -257,12 +250,11 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, int64_t a_row_
     int8_t* na = lds + (PAR ^ 1) * STAGE;
     int8_t* nb = na + A_BYTES;
     const int64_t s1 = s + 1 < last ? s + 1 : last;
-    const int64_t s2 = s + 2 < last ? s + 2 : last;
-    kstep(par, IntC<0>{}, f0, f1, pa, pb, 2 + fhalf, s1, s2, na, nb);
-    kstep(par, IntC<1>{}, f1, f0, pa, pb, 4 + fhalf, s1, s2, na, nb);
-    kstep(par, IntC<2>{}, f0, f1, pa, pb, 6 + fhalf, s1, s2, na, nb);
+    kstep(IntC<0>{}, f0, f1, pa, pb, 2 + fhalf, s1, na, nb);
+    kstep(IntC<1>{}, f1, f0, pa, pb, 4 + fhalf, s1, na, nb);
+    kstep(IntC<2>{}, f0, f1, pa, pb, 6 + fhalf, s1, na, nb);
     drain_and_barrier();                                 // slice s+1 is in LDS for everybody
-    kstep(par, IntC<3>{}, f1, f0, na, nb, fhalf, s1, s2, na, nb);
+    kstep(IntC<3>{}, f1, f0, na, nb, fhalf, s1, na, nb);
   };
 
   int64_t s = 0;
@@ -272,17 +264,24 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, int64_t a_row_
   }
   if (s < slices) slice_body(IntC<0>{}, s);
 
-  write_tile<4>(acc, epi, y, M, N, m0, n0, lds);
+  write_tile<JT, 2>(acc, epi, y, M, N, m0, n0, lds);
 }
 
-// Workgroup id -> tile origin with the XCD-aware order described above; false = no tile.
+// Tile order: the hardware deals consecutive workgroup ids round-robin to the 8 XCDs, each with
+// its own L2.  XCD x is given the N panels x, x+8, ... and walks down all M tiles of a panel
+// before the next, so a B panel is fetched into one L2 only.  A set of `panels` panels takes
+// padded_blocks(panels, tiles_m) ids; surplus ids get no tile.
+__device__ __host__ __forceinline__ int64_t padded_blocks(int64_t panels, int64_t tiles_m) { return 8 * ((panels + 7) / 8) * tiles_m; }
+__device__ __forceinline__ bool tile_of(int64_t id, int64_t tiles_m, int64_t panels, int64_t& tile_m, int64_t& panel) {
+  const int64_t xcd = id & 7, local = id >> 3;
+  panel = (local / tiles_m) * 8 + xcd;
+  tile_m = local % tiles_m;
+  return panel < panels;
+}
 __device__ __forceinline__ bool tile_origin(int64_t M, int64_t N, int64_t& m0, int64_t& n0) {
-  const int64_t tiles_m = (M + BM - 1) / BM;
-  const int64_t panels = (N + BN - 1) / BN;
-  const int64_t xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
-  const int64_t panel = (local / tiles_m) * 8 + xcd;
-  if (panel >= panels) return false;
-  m0 = (local % tiles_m) * BM;
+  int64_t tile_m, panel;
+  if (!tile_of(blockIdx.x, (M + BM - 1) / BM, (N + BN - 1) / BN, tile_m, panel)) return false;
+  m0 = tile_m * BM;
   n0 = panel * BN;
   return true;
 }

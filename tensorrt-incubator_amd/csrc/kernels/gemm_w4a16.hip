@@ -202,77 +202,6 @@ struct F16Traits {
   }
 };
 
-// int4 weights of a 256-column panel: 8 column tiles x (64 lanes x 16 B) per 64-k slice.
-// Thread t fetches fragment lane (t & 63) of column tiles (t >> 6) and (t >> 6) + 4.  The raw
-// nibbles and scales of a slice are fetched two slices ahead into one of two register sets
-// and dequantised into the LDS panel one slice ahead, in eight units (one prepacked dword ->
-// 8 f16 -> one 16-byte LDS store) that are spread over the first three k-steps of a slice.
-struct Int4B {
-  const uint32_t* wp;
-  const uint16_t* scale;
-  int64_t kblocks, N, tile0;
-  uint32_t slices_per_block;                         // block / 64: slices that share one row of scales
-  u4 raw[2][2];
-  uint32_t sc_bits[2][2];                            // scales as loaded; widened to a pair where they are used,
-                                                     // so that nothing waits for the load where it is issued
-  // No branch here: a conditional load inside the K loop splits its basic block and the
-  // accumulators get shuffled around the split.  Columns past N read the last column's
-  // scales and the last tile's nibbles instead; their results are never stored.
-  template <int SET>
-  __device__ __forceinline__ void fetch(int64_t slice) {
-    const int lane = threadIdx.x & 63;
-    const int64_t last_tile = (N + 31) / 32 - 1;
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      int64_t tile = tile0 + (threadIdx.x >> 6) + 4 * i;
-      tile = tile < last_tile ? tile : last_tile;
-      int64_t col = tile * 32 + (lane & 31);
-      col = col < N ? col : N - 1;
-      raw[SET][i] = *reinterpret_cast<const u4*>(wp + ((tile * kblocks + slice) * 64 + lane) * 4);
-      const int64_t srow = int64_t(uint32_t(slice) / slices_per_block);   // 32-bit: no division loop in the K loop
-      sc_bits[SET][i] = scale[srow * N + col];
-    }
-  }
-  template <int SET>
-  __device__ __forceinline__ h2 scale_pair(int i) const {
-    H2Bits t;
-    t.u = sc_bits[SET][i] * 0x00010001u;
-    return t.h;
-  }
-  template <int SET>
-  __device__ __forceinline__ void commit_unit(int u, int8_t* panel) {
-    const int lane = threadIdx.x & 63;
-    const int i = u >> 2, j = u & 3;
-    const int row = ((threadIdx.x >> 6) + 4 * i) * 32 + (lane & 31);
-    *reinterpret_cast<u4*>(panel + gemm_core::lds_off(row, 2 * j + (lane >> 5))) = dequant8(raw[SET][i][j], scale_pair<SET>(i));
-  }
-  __device__ __forceinline__ void prologue(int8_t* panel0, int64_t last) {
-    fetch<0>(0);
-#pragma unroll
-    for (int u = 0; u < 8; ++u) commit_unit<0>(u, panel0);
-    fetch<1>(1 < last ? 1 : last);
-  }
-  // While slice s (parity PAR) is multiplied, set PAR is free (its slice went to LDS during
-  // s-1) and takes slice s+2; set PAR^1 holds slice s+1 and goes to LDS in 24 steps, three per
-  // unit (two halves of the dequantisation, then the store), one step per chunk of k-steps 0..2.
-  u4 pending;
-  uint32_t mask = nibble_pair_mask();
-  template <int PAR, int P>
-  __device__ __forceinline__ void chunk(int c, int64_t, int64_t s2, int8_t* nb) {
-    if (P == 3) return;
-    const int step = P * 8 + c, u = step / 3, part = step % 3;
-    if (step == 0) fetch<PAR>(s2);
-    const int i = u >> 2, j = u & 3;
-    if (part < 2) {
-      dequant4(raw[PAR ^ 1][i][j], scale_pair<PAR ^ 1>(i), part, mask, pending);
-    } else {
-      const int lane = threadIdx.x & 63;
-      const int row = ((threadIdx.x >> 6) + 4 * i) * 32 + (lane & 31);
-      *reinterpret_cast<u4*>(nb + gemm_core::lds_off(row, 2 * j + (lane >> 5))) = pending;
-    }
-  }
-};
-
 struct PlainEpilogue {
   __device__ __forceinline__ void setup(int8_t*, int64_t, int64_t, int64_t, int64_t) {}
   __device__ __forceinline__ void row(int) {}
@@ -419,7 +348,7 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
   }
   if (s < slices) slice_body(IntC<0>{}, s);
   __builtin_amdgcn_s_waitcnt(0x0070);                  // the surplus loads of the last slices have landed
-  write_tile<JT>(acc, epi, y, M, N, m0, n0, lds);
+  write_tile<JT, NWN>(acc, epi, y, M, N, m0, n0, lds);
 }
 
 // (a [M,K] f16, w_prepacked, scale [K/block, N] f16, y [M,N] f16, M, K, N, block) ; K % 64 == 0, block % 64 == 0,

@@ -55,18 +55,27 @@ struct ScaleEpilogue {
 // The entry points below have C linkage; they sit inside the namespace only so that
 // its helper names do not meet those of the other clusters in the one-module build.
 
-// (a [M,K] i8, w_nk [N,K] i8, a_scale [M] f32, w_scale [N] f32, y [M,N] f16, M, K, N) ; K % 128 == 0,
-// a and w_nk 16-byte aligned, both below 4 GiB.  grid = 8 * ceil(ceil(N/256) / 8) * ceil(M/256), block = 256.
+// (a [M,K] i8, w_nk [N,K] i8, a_scale [M] f32, w_scale [N] f32, y [M,N] f16, M, K, N, full_panels) ; K % 128 == 0,
+// a and w_nk 16-byte aligned, both below 4 GiB.  The first full_panels * 256 columns are computed in
+// 256 x 256 tiles, the rest in 256 x 128 tiles: with one workgroup per compute unit a launch runs in
+// rounds, and a last round that would use few of the units is cut into twice as many tiles of half
+// the length.  grid = padded_blocks(full_panels, tiles_m) + padded_blocks(half panels, tiles_m), block = 256.
 extern "C" __global__ void __launch_bounds__(gemm_core::THREADS, 1) mtrt_gemm_w8a8_nk(
     const int8_t* __restrict__ a, const int8_t* __restrict__ w, const float* __restrict__ a_scale,
-    const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N) {
+    const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t full_panels) {
   __shared__ __attribute__((aligned(16))) int8_t lds[gemm_core::LDS_BYTES];
-  int64_t m0, n0;
-  if (!gemm_core::tile_origin(M, N, m0, n0)) return;
-  gemm_core::DmaB wl;                                // W [N,K] bytes: same transport as the A operand
-  wl.l.init(w, N, K, n0);
+  const int64_t tiles_m = (M + gemm_core::BM - 1) / gemm_core::BM;
+  const int64_t full_blocks = gemm_core::padded_blocks(full_panels, tiles_m);
   ScaleEpilogue epi{a_scale, w_scale, nullptr, nullptr, 0.0f};
-  gemm_core::run<I8Traits>(a, K, wl, epi, y, M, N, K / gemm_core::BKB, m0, n0, lds);
+  int64_t tile_m, panel;
+  if (int64_t(blockIdx.x) < full_blocks) {
+    if (!gemm_core::tile_of(blockIdx.x, tiles_m, full_panels, tile_m, panel)) return;
+    gemm_core::run<I8Traits, 4>(a, w, K, epi, y, M, N, K / gemm_core::BKB, tile_m * 256, panel * 256, lds);
+  } else {
+    const int64_t n_full = full_panels * 256;
+    if (!gemm_core::tile_of(blockIdx.x - full_blocks, tiles_m, (N - n_full + 127) / 128, tile_m, panel)) return;
+    gemm_core::run<I8Traits, 2>(a, w, K, epi, y, M, N, K / gemm_core::BKB, tile_m * 256, n_full + panel * 128, lds);
+  }
 }
 
 // Any K (no alignment needs): one output element per lane, plain loops.  Serves

@@ -280,11 +280,23 @@ int32_t mtrt_hip_gemm_w8a8(mtrt_stream_t stream, const void *a, const void *w_nk
   // The matrix-core kernel moves 128-byte K slices with 16-byte accesses.
   if (K > 0 && K % 128 == 0 && aligned(a, 16) && aligned(w_nk, 16) && M * K < (int64_t(1) << 32) &&
       N * K < (int64_t(1) << 32)) {
-    // 256 x 256 tiles; N panels are dealt round-robin to the 8 XCDs (see gemm_core.hpp): the
-    // grid is padded to 8 * ceil(panels / 8) * tiles_m workgroups.
-    const int64_t tiles = 8 * ((((N + 255) / 256) + 7) / 8) * ((M + 255) / 256);
-    if (tiles <= int64_t(kMaxGrid) * 1024)
-      return launch(st, "mtrt_gemm_w8a8_nk", uint32_t(tiles), kBlock, as_hip(stream), args);
+    // 256 x 256 tiles, one workgroup per compute unit at a time, N panels dealt round-robin to the
+    // 8 XCDs (gemm_core.hpp), so each set of panels takes 8 * ceil(panels / 8) * tiles_m workgroup
+    // ids.  The launch runs in rounds of one tile per unit; when the last round would use at most
+    // half of the units (or the whole launch does), its panels are cut into 128-wide halves.
+    const int64_t panels = (N + 255) / 256, tiles_m = (M + 255) / 256, units = num_compute_units(st);
+    const int64_t tiles = panels * tiles_m, rest = tiles % units;
+    int64_t full_panels = panels;
+    if (tiles * 2 <= units)
+      full_panels = 0;
+    else if (rest > 0 && rest * 2 <= units)
+      full_panels = panels - (rest + tiles_m - 1) / tiles_m;
+    const int64_t half_panels = (N - full_panels * 256 + 127) / 128;
+    const int64_t grid = 8 * ((full_panels + 7) / 8) * tiles_m + 8 * ((half_panels + 7) / 8) * tiles_m;
+    if (grid <= int64_t(kMaxGrid) * 1024) {
+      void *fast_args[] = {&a, &w_nk, &a_scale, &w_scale, &y, &M, &K, &N, &full_panels};
+      return launch(st, "mtrt_gemm_w8a8_nk", uint32_t(grid), kBlock, as_hip(stream), fast_args);
+    }
   }
   return launch(st, "mtrt_gemm_w8a8_nk_any", blocks_for(M * N, kBlock), kBlock, as_hip(stream), args);
 }
