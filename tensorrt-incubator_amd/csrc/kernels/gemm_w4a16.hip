@@ -376,35 +376,115 @@ extern "C" __global__ void __launch_bounds__(THREADS) mtrt_gemm_w4a16_t128x64(
 extern "C" __global__ void __launch_bounds__(THREADS) mtrt_gemm_w4a16_skinny(
     const uint16_t* __restrict__ a, const uint32_t* __restrict__ wp, const uint16_t* __restrict__ scale,
     uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t block) {
-  __shared__ float partial[4][16][64];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // Per wave a ring of four 4 KiB stages (32 rows x 64 k of activations each), filled by
+  // direct-to-LDS loads three slices ahead: a fragment read straight from global memory would
+  // touch 64 different cache lines per instruction (32 rows 8 KiB apart), the ring is filled
+  // with whole 128-byte row segments.  The waves never touch each other's ring: no barriers.
+  constexpr int kStages = 4, kStageBytes = 32 * 128;
+  __shared__ __attribute__((aligned(16))) int8_t lds[4 * kStages * kStageBytes];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int frow = lane & 31, fhalf = lane >> 5;
   const int64_t tile = blockIdx.x;
-  const int64_t col = tile * 32 + frow;
   const int64_t kblocks = K / BKH;
   const int64_t kb0 = kblocks * wave / 4, kb1 = kblocks * (wave + 1) / 4;
-  const bool live_b = col < N;
-  const int64_t arow = frow < M ? frow : M - 1;      // rows past M repeat the last row; never stored
-  const uint16_t* ap = a + arow * K + fhalf * 8;
+  const int64_t klast = kb1 - 1;
+  int64_t col = tile * 32 + frow;
+  col = col < N ? col : N - 1;                       // columns past N: the last column's scales, never stored
+  const uint32_t slices_per_block = uint32_t(block / BKH);
   const u4* bp = reinterpret_cast<const u4*>(wp) + (tile * kblocks) * 64 + lane;
+  int8_t* ring = lds + wave * (kStages * kStageBytes);
+
+  // direct-to-LDS load g (of 4) of a slice: rows 8g .. 8g+7, lane l <-> (row l >> 3, LDS chunk l & 7)
+  uint32_t aoff[4];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const int lrow = g * 8 + (lane >> 3);
+    const int64_t row = lrow < M ? lrow : M - 1;     // rows past M repeat the last row; never stored
+    aoff[g] = uint32_t(row * K * 2 + (((lane & 7) ^ ((lrow >> 1) & 7)) << 4));
+  }
+  const int8_t* abase = reinterpret_cast<const int8_t*>(a);
+  struct Slice {
+    u4 w;
+    uint32_t sc;
+  };
+  // everything slice kb needs from memory: 4 + 2 loads, always, so that the waits can count
+  auto fetch = [&](int64_t kb, int64_t clamp, Slice& dst) {
+    kb = kb < clamp ? kb : clamp;
+    int8_t* st = ring + int(kb & (kStages - 1)) * kStageBytes;
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+      __builtin_amdgcn_global_load_lds((gemm_core::global_void_t*)(abase + kb * (BKH * 2) + aoff[g]),
+                                       (gemm_core::lds_void_t*)(st + g * 1024), 16, 0, 0);
+    // Register loads issued as opaque instructions: the compiler's own wait-count bookkeeping
+    // gives up on loads carried around a loop and drains everything (vmcnt(0)) before their first
+    // use, which would leave nothing in flight.  The waits are placed by hand in `landed`.
+    const u4* wsrc = bp + kb * 64;
+    const uint16_t* ssrc = scale + int64_t(uint32_t(kb) / slices_per_block) * N + col;
+    __asm__ volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(dst.w) : "v"(wsrc) : "memory");
+    __asm__ volatile("global_load_ushort %0, %1, off" : "=v"(dst.sc) : "v"(ssrc) : "memory");
+  };
+  // ties the registers of a slice to the wait, so that no use can be scheduled in front of it:
+  // 24 loads issued, 18 may fly -> the 6 of the oldest slice have landed
+  auto landed = [&](Slice& sl) { __asm__ volatile("s_waitcnt vmcnt(18)" : "+v"(sl.w), "+v"(sl.sc)::"memory"); };
+  auto landed_all = [&](Slice& sl) { __asm__ volatile("s_waitcnt vmcnt(0)" : "+v"(sl.w), "+v"(sl.sc)::"memory"); };
 
   v16f acc;
 #pragma unroll
   for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
-
-  for (int64_t kb = kb0; kb < kb1; ++kb) {
-    const u4 wq = live_b ? __builtin_nontemporal_load(bp + kb * 64) : (u4){0x88888888u, 0x88888888u, 0x88888888u, 0x88888888u};
-    const h2 s2 = live_b ? load_scale2(scale, ((kb * BKH) / block) * N + col) : (h2){(_Float16)0.0f, (_Float16)0.0f};
-    v8h fa[4];
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) fa[ks] = *reinterpret_cast<const v8h*>(ap + kb * BKH + ks * 16);
+  const uint32_t mask = nibble_pair_mask();
+  auto multiply = [&](int64_t kb, const Slice& sl) {
+    const int8_t* st = ring + int(kb & (kStages - 1)) * kStageBytes;
+    H2Bits sp;
+    sp.u = sl.sc * 0x00010001u;
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
+      const v8h fa = *reinterpret_cast<const v8h*>(st + gemm_core::lds_off(frow, 2 * ks + fhalf));
       union { u4 u; v8h h; } fb;
-      fb.u = dequant8(wq[ks], s2);
-      acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[ks], fb.h, acc, 0, 0, 0);
+      dequant4(sl.w[ks], sp.h, 0, mask, fb.u);
+      dequant4(sl.w[ks], sp.h, 1, mask, fb.u);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, fb.h, acc, 0, 0, 0);
     }
+  };
+
+  // Main part: groups of four slices with four register sets, so that nothing is copied (a copy
+  // would have to wait for the load) and the loop has no branch; three slices stay in flight.
+  const int64_t kmain = kb0 + ((kb1 - kb0) & ~int64_t(3));
+  if (kb0 < kmain) {
+    const int64_t clamp = kmain - 1;                   // past the end: the last slice again, into a stage nobody reads
+    Slice s0, s1, s2, s3;
+    fetch(kb0, clamp, s0);
+    fetch(kb0 + 1, clamp, s1);
+    fetch(kb0 + 2, clamp, s2);
+    for (int64_t kb = kb0; kb < kmain; kb += 4) {
+      fetch(kb + 3, clamp, s3);
+      landed(s0);
+      multiply(kb, s0);
+      fetch(kb + 4, clamp, s0);
+      landed(s1);
+      multiply(kb + 1, s1);
+      fetch(kb + 5, clamp, s1);
+      landed(s2);
+      multiply(kb + 2, s2);
+      fetch(kb + 6, clamp, s2);
+      landed(s3);
+      multiply(kb + 3, s3);
+    }
+    // the surplus loads of the last group still target these registers: keep them until they land
+    landed_all(s0);
+    landed_all(s1);
+    landed_all(s2);
   }
+  for (int64_t kb = kmain; kb < kb1; ++kb) {           // at most three slices, one at a time
+    Slice sl;
+    __builtin_amdgcn_s_waitcnt(0x0070);
+    fetch(kb, kb, sl);
+    landed_all(sl);
+    multiply(kb, sl);
+  }
+  __builtin_amdgcn_s_waitcnt(0x0070);                  // surplus loads have landed before the ring is reused
+  __syncthreads();
+  float (*partial)[16][64] = reinterpret_cast<float (*)[16][64]>(lds);
 #pragma unroll
   for (int r = 0; r < 16; ++r) partial[wave][r][lane] = acc[r];
   __syncthreads();
