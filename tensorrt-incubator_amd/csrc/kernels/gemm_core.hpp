@@ -113,32 +113,36 @@ struct Frags {
 // so a lane owns runs of 4 consecutive outputs of a row.  Each wave parks its converted 128 x 128
 // sub-tile (in two halves of 64 columns) in LDS with 8-byte stores, rows padded to 144 B, and
 // writes it out as whole 128-byte row segments, 16 bytes per lane.
-template <int JT, int NWN, class Acc, class Epilogue>  // 2 x NWN waves, JT column tiles (32 wide) per wave
+// SLOTS waves own a sub-tile each (slot = wm * NWN + wn, 128 rows x 32*JT columns); `active` is
+// false for waves that only take part in the barriers.
+template <int JT, int NWN, int SLOTS, class Acc, class Epilogue>
 __device__ __forceinline__ void write_tile(Acc (&acc)[4][JT], Epilogue& epi, uint16_t* __restrict__ y, int64_t M, int64_t N,
-                                           int64_t m0, int64_t n0, int8_t* lds) {
-  constexpr int WAVES = 2 * NWN, WCOLS = 32 * JT;
+                                           int64_t m0, int64_t n0, int8_t* lds, int slot, bool active) {
+  constexpr int WCOLS = 32 * JT;
+  constexpr int HC = JT >= 2 ? 2 : 1;                  // column tiles staged at a time: 64 or 32 columns
+  constexpr int CHUNKS = HC * 4;                       // 16-byte chunks per staged row
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int wm = wave / NWN, wn = wave % NWN;
+  const int wm = slot / NWN, wn = slot % NWN;
   const int frow = lane & 31, fhalf = lane >> 5;
   __syncthreads();                                     // every wave is done with the operand stages
-  epi.setup(lds + WAVES * kOutWave, m0, M, n0, N);
+  epi.setup(lds + SLOTS * kOutWave, m0, M, n0, N);
   __syncthreads();
-  int8_t* out = lds + wave * kOutWave;
+  if (!active) return;
+  int8_t* out = lds + slot * kOutWave;
   const bool vec_ok = (N % 8 == 0) && ((reinterpret_cast<uintptr_t>(y) & 15) == 0);
 #pragma unroll
-  for (int half = 0; half < JT / 2; ++half) {
+  for (int half = 0; half < JT / HC; ++half) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int lrow = i * 32 + frow;
       epi.row(wm * 128 + lrow);
 #pragma unroll
-      for (int jj = 0; jj < 2; ++jj)
+      for (int jj = 0; jj < HC; ++jj)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const int lcol = jj * 32 + q * 8 + fhalf * 4;  // columns lcol .. lcol+3 of this half <-> r = 4q .. 4q+3
+          const int lcol = jj * 32 + q * 8 + fhalf * 4;  // columns lcol .. lcol+3 of this group <-> r = 4q .. 4q+3
           uint32_t bits[4];
-          epi.convert4(acc[i][half * 2 + jj], q, wn * WCOLS + half * 64 + lcol, bits);
+          epi.convert4(acc[i][half * HC + jj], q, wn * WCOLS + half * (32 * HC) + lcol, bits);
           u32x2 packed;
           packed[0] = bits[0] | (bits[1] << 16);
           packed[1] = bits[2] | (bits[3] << 16);
@@ -147,10 +151,10 @@ __device__ __forceinline__ void write_tile(Acc (&acc)[4][JT], Epilogue& epi, uin
     }
     // each wave reads back only what it wrote itself: no workgroup barrier needed
 #pragma unroll
-    for (int it = 0; it < 16; ++it) {
-      const int lrow = it * 8 + (lane >> 3), ch = lane & 7;
+    for (int it = 0; it < 128 * CHUNKS / 64; ++it) {
+      const int lrow = it * (64 / CHUNKS) + lane / CHUNKS, ch = lane % CHUNKS;
       const int64_t row = m0 + wm * 128 + lrow;
-      const int64_t col = n0 + wn * WCOLS + half * 64 + ch * 8;
+      const int64_t col = n0 + wn * WCOLS + half * (32 * HC) + ch * 8;
       const u32x4 v = *reinterpret_cast<const u32x4*>(out + lrow * kOutRow + ch * 16);
       if (row < M) {
         if (vec_ok) {
@@ -264,7 +268,7 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, const int8_t* 
   }
   if (s < slices) slice_body(IntC<0>{}, s);
 
-  write_tile<JT, 2>(acc, epi, y, M, N, m0, n0, lds);
+  write_tile<JT, 2, 4>(acc, epi, y, M, N, m0, n0, lds, wave, true);
 }
 
 // Tile order: the hardware deals consecutive workgroup ids round-robin to the 8 XCDs, each with

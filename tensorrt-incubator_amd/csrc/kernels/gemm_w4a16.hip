@@ -20,13 +20,12 @@
 // integer value and a packed f16 multiply by the scale gives wd with the single
 // rounding the program asks for.
 //
-// Large M: dequantisation happens in registers on the way INTO LDS; the multiply loop
-// is the shared one of gemm_core.hpp (256 x 256 tiles, activations by direct-to-LDS
-// loads, v_mfma_f32_32x32x16_f16).  Medium M uses a 128 x 64 tile variant of the same
-// idea so that the grid still fills the chip.
+// All kernels take the weight fragments straight from global memory into registers and
+// dequantise them there; only the activations go through LDS (direct-to-LDS loads).
+// Large M: 256 x 256 tiles, 8 waves.  Medium M: 128 x 64 tiles so that the grid still fills
+// the chip, 4 waves in two sets that split each K slice.
 // Small M (<= 32): the GEMM is bound by reading the weights once.  One workgroup per
-// 32 columns, its four waves split K, fragments go straight from global memory into
-// registers (no LDS on the way in), partial tiles are added through LDS at the end.
+// 32 columns, its four waves split K, partial tiles are added through LDS at the end.
 #include "gemm_core.hpp"
 
 using namespace mtrt_dev;
@@ -83,105 +82,6 @@ __device__ __forceinline__ h2 load_scale2(const uint16_t* __restrict__ scale, in
   c.u = scale[idx];
   h2 r = {c.h, c.h};
   return r;
-}
-
-// ---- large-M kernel ----------------------------------------------------------------
-// IT x JT MFMA tiles per wave, 2 x 2 waves: BM = 64*IT, BN = 64*JT.
-template <int IT, int JT>
-__device__ __forceinline__ void gemm_tiles(const uint16_t* __restrict__ a, const uint32_t* __restrict__ wp,
-                                           const uint16_t* __restrict__ scale, uint16_t* __restrict__ y, int64_t M,
-                                           int64_t K, int64_t N, int64_t block, int8_t* lds) {
-  constexpr int BM = 64 * IT, BN = 64 * JT;
-  constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
-  constexpr int A_CHUNKS = BM * 8 / THREADS;         // 16-byte loads per thread per slice
-  constexpr int B_LOADERS = BN * 2;                  // threads that fetch weights (16 B each)
-
-  const int64_t tiles_m = (M + BM - 1) / BM;
-  const int64_t m0 = int64_t(blockIdx.x % tiles_m) * BM;
-  const int64_t n0 = int64_t(blockIdx.x / tiles_m) * BN;
-  const int64_t kblocks = K / BKH;
-
-  const int t = threadIdx.x;
-  const int lane = t & 63, wave = t >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
-  const int frow = lane & 31, fhalf = lane >> 5;
-  // weight loader role: n-tile (t >> 6) of this workgroup's columns, fragment lane (t & 63)
-  const bool loads_b = t < B_LOADERS;
-  const int64_t b_tile = n0 / 32 + (t >> 6);
-  const int64_t b_col = b_tile * 32 + frow;          // column whose weights this thread dequantises
-  const bool b_live = loads_b && b_col < N;
-
-  v16f acc[IT][JT];
-#pragma unroll
-  for (int i = 0; i < IT; ++i)
-#pragma unroll
-    for (int j = 0; j < JT; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-
-  u4 sa[A_CHUNKS];
-  u4 sb;
-  h2 sscale;
-
-  auto load_slice = [&](int64_t kb) {
-#pragma unroll
-    for (int i = 0; i < A_CHUNKS; ++i) {
-      int64_t row = m0 + (t >> 3) + 32 * i;
-      row = row < M ? row : M - 1;
-      sa[i] = *reinterpret_cast<const u4*>(a + row * K + kb * BKH + (t & 7) * 8);
-    }
-    if (loads_b) {
-      sb = b_live ? *reinterpret_cast<const u4*>(wp + ((b_tile * kblocks + kb) * 64 + lane) * 4) : (u4){0x88888888u, 0x88888888u, 0x88888888u, 0x88888888u};
-      sscale = b_live ? load_scale2(scale, ((kb * BKH) / block) * N + b_col) : (h2){(_Float16)0.0f, (_Float16)0.0f};
-    }
-  };
-  auto store_slice = [&](int8_t* pa, int8_t* pb) {
-#pragma unroll
-    for (int i = 0; i < A_CHUNKS; ++i) *reinterpret_cast<u4*>(pa + lds_off((t >> 3) + 32 * i, t & 7)) = sa[i];
-    if (loads_b) {
-      const int row = (t >> 6) * 32 + frow;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) *reinterpret_cast<u4*>(pb + lds_off(row, 2 * j + fhalf)) = dequant8(sb[j], sscale);
-    }
-  };
-
-  load_slice(0);
-  store_slice(lds, lds + A_BYTES);
-  __syncthreads();
-  for (int64_t kb = 0; kb < kblocks; ++kb) {
-    const int cur = int(kb & 1);
-    const int8_t* pa = lds + cur * STAGE;
-    const int8_t* pb = pa + A_BYTES;
-    if (kb + 1 < kblocks) load_slice(kb + 1);
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      v8h fa[IT], fb[JT];
-      const int chunk = ks * 2 + fhalf;
-#pragma unroll
-      for (int i = 0; i < IT; ++i) fa[i] = *reinterpret_cast<const v8h*>(pa + lds_off(wm * (32 * IT) + i * 32 + frow, chunk));
-#pragma unroll
-      for (int j = 0; j < JT; ++j) fb[j] = *reinterpret_cast<const v8h*>(pb + lds_off(wn * (32 * JT) + j * 32 + frow, chunk));
-#pragma unroll
-      for (int i = 0; i < IT; ++i)
-#pragma unroll
-        for (int j = 0; j < JT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
-    }
-    if (kb + 1 < kblocks) store_slice(lds + (cur ^ 1) * STAGE, lds + (cur ^ 1) * STAGE + A_BYTES);
-    __syncthreads();
-  }
-
-#pragma unroll
-  for (int j = 0; j < JT; ++j) {
-    const int64_t col = n0 + wn * (32 * JT) + j * 32 + frow;
-    if (col >= N) continue;
-#pragma unroll
-    for (int i = 0; i < IT; ++i)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int64_t row = m0 + wm * (32 * IT) + i * 32 + (r >> 2) * 8 + fhalf * 4 + (r & 3);
-        if (row < M) y[row * N + col] = uint16_t(f32_to_f16_bits(acc[i][j][r]));
-      }
-  }
 }
 
 // The entry points below have C linkage; they sit inside the namespace only so that
@@ -255,19 +155,34 @@ struct WeightRegs {
   }
 };
 
-// JT = 4: 4 waves (2 x 2), one per SIMD, 128 x 128 each.  JT = 2: 8 waves (2 x 4), two per SIMD,
-// 128 x 64 each.  A wave's own VALU, LDS and memory instructions do not overlap its MFMAs (each
-// takes its issue cycles out of the MFMA stream), only another wave's do, so with the
-// dequantisation in the loop two waves per SIMD are the faster shape.
-template <int JT, class Epilogue>
-__device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, int64_t a_row_bytes, WeightRegs<JT>& wr, Epilogue& epi,
-                                                uint16_t* __restrict__ y, int64_t M, int64_t N, int64_t slices, int64_t m0,
-                                                int64_t n0, int8_t* lds) {
+// Shape of a workgroup: KW x MW x NWN waves.  MW x NWN waves tile the output, each 128 rows x
+// 32*JT columns; with KW = 2 two such sets split every slice between them (k-steps KH and KH + 2
+// of the four) and their accumulators are added at the end, which doubles the waves of a small
+// tile without making the tile smaller.  A wave's own VALU, LDS and memory instructions do not
+// overlap its MFMAs (each takes its issue cycles out of the MFMA stream), only another wave's
+// do, so with the dequantisation in the loop two waves per SIMD are the faster shape.
+template <int MW, int NWN, int JT, int KW>
+struct Shape {
+  static constexpr int kMW = MW, kNWN = NWN, kJT = JT, kKW = KW;
+  static constexpr int kSlots = MW * NWN, kWaves = KW * kSlots;
+  static constexpr int kBM = 128 * MW, kBN = 32 * JT * NWN;
+  static constexpr int kStageBytes = kBM * 128;        // one slice of the activation panel
+  static constexpr int kRingBytes = 4 * kStageBytes;
+  static constexpr int kOutBytes = kSlots * gemm_core::kOutWave + 2048;
+  static constexpr int kSumBytes = KW == 2 ? kSlots * 128 * 32 * JT * 4 : 0;
+  static constexpr int kLds = kRingBytes > kOutBytes ? (kRingBytes > kSumBytes ? kRingBytes : kSumBytes)
+                                                     : (kOutBytes > kSumBytes ? kOutBytes : kSumBytes);
+};
+
+template <class S, int KH, class Epilogue>
+__device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, int64_t a_row_bytes, WeightRegs<S::kJT>& wr,
+                                                Epilogue& epi, uint16_t* __restrict__ y, int64_t M, int64_t N, int64_t slices,
+                                                int64_t m0, int64_t n0, int8_t* lds, int slot) {
   using namespace gemm_core;
-  constexpr int NWN = 8 / JT, WAVES = 2 * NWN, G = 32 / WAVES;
+  constexpr int JT = S::kJT, NWN = S::kNWN, KW = S::kKW, G = (16 * S::kMW) / S::kWaves, NK = 4 / KW;
+  static_assert(G >= 4 && G % 4 == 0 && G <= 15, "direct-to-LDS loads per wave and slice");
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int wm = wave / NWN;
+  const int wm = slot / NWN;
   const int frow = lane & 31, fhalf = lane >> 5;
 
   v16f acc[4][JT];
@@ -286,7 +201,7 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
   auto read_a = [&](FragSet& f, const int8_t* pa, int chunk, int i) {
     f.a[i] = *reinterpret_cast<const v4i*>(pa + lds_off(wm * 128 + i * 32 + frow, chunk));
   };
-  auto stage = [&](int64_t slice) { return lds + int(slice & 3) * A_BYTES; };
+  auto stage = [&](int64_t slice) { return lds + int(slice & 3) * S::kStageBytes; };
 
 #pragma unroll
   for (int g = 0; g < G; ++g) al.dma(0, stage(0), g);
@@ -296,35 +211,37 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
   wr.template fetch<1>(1 < last ? 1 : last);
   drain_and_barrier();
 #pragma unroll
-  for (int i = 0; i < 4; ++i) read_a(f0, stage(0), fhalf, i);
+  for (int i = 0; i < 4; ++i) read_a(f0, stage(0), 2 * KH + fhalf, i);
 #pragma unroll
   for (int j = 0; j < JT; ++j) {
-    wr.template half<0, 0>(j, 0, f0.b[j]);
-    wr.template half<0, 0>(j, 1, f0.b[j]);
+    wr.template half<0, KH>(j, 0, f0.b[j]);
+    wr.template half<0, KH>(j, 1, f0.b[j]);
   }
 
-  // k-step P of a slice of parity PAR: MFMAs on `cur`, everything for the next k-step into `nxt`.
-  // Four fenced chunks; chunk c multiplies row tile c and carries one A fragment read, JT/2
-  // halves of the next weights' dequantisation and, in k-step 0, G/4 direct-to-LDS loads.
-  auto kstep = [&](auto par, auto step, const FragSet& cur, FragSet& nxt, const int8_t* ra, int chunk, int64_t s2, int8_t* nd) {
-    constexpr int PAR = decltype(par)::value, P = decltype(step)::value;
-    constexpr int NSET = P == 3 ? (PAR ^ 1) : PAR;     // register set and dword the next k-step's weights come from
-    constexpr int NP = P == 3 ? 0 : P + 1;
+  // Step T (of NK) of a slice of parity PAR: MFMAs on `cur`, everything for this wave's next
+  // k-step into `nxt`.  Four fenced chunks; chunk c multiplies row tile c and carries one A
+  // fragment read, its share of the 2 * JT halves of the next weights' dequantisation and, in
+  // step 0, G/4 direct-to-LDS loads.  Raw nibbles and scales of slice s+2 are fetched in the
+  // last step into the register set that the step before finished with.
+  auto kstep = [&](auto par, auto step, const FragSet& cur, FragSet& nxt, const int8_t* ra, int64_t s2, int8_t* nd) {
+    constexpr int PAR = decltype(par)::value, T = decltype(step)::value;
+    constexpr bool kLast = T == NK - 1;
+    constexpr int NSET = kLast ? (PAR ^ 1) : PAR;      // register set and dword the next k-step's weights come from
+    constexpr int NP = kLast ? KH : KH + (T + 1) * KW;
+    const int chunk = 2 * NP + fhalf;
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
 #pragma unroll
       for (int j = 0; j < JT; ++j) acc[c][j] = F16Traits::mfma(__builtin_bit_cast(v4i, cur.b[j]), cur.a[c], acc[c][j]);
       read_a(nxt, ra, chunk, c);
 #pragma unroll
-      for (int h = 0; h < JT / 2; ++h) {
-        const int unit = c * (JT / 2) + h;               // 2 * JT halves per k-step
-        wr.template half<NSET, NP>(unit >> 1, unit & 1, nxt.b[unit >> 1]);
-      }
-      if (P == 0) {
+      for (int u = 0; u < 2 * JT; ++u)
+        if ((u * 4) / (2 * JT) == c) wr.template half<NSET, NP>(u >> 1, u & 1, nxt.b[u >> 1]);
+      if (T == 0) {
 #pragma unroll
         for (int g = 0; g < G / 4; ++g) al.dma(s2, nd, c * (G / 4) + g);
       }
-      if (P == 3 && c == 0) wr.template fetch<PAR>(s2);
+      if (kLast && c == 0) wr.template fetch<PAR>(s2);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -332,13 +249,17 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
     const int8_t* pa = stage(s);
     const int64_t s2 = s + 2 < last ? s + 2 : last;
     int8_t* nd = stage(s + 2);
-    kstep(par, IntC<0>{}, f0, f1, pa, 2 + fhalf, s2, nd);
-    kstep(par, IntC<1>{}, f1, f0, pa, 4 + fhalf, s2, nd);
-    kstep(par, IntC<2>{}, f0, f1, pa, 6 + fhalf, s2, nd);
+    if (NK == 4) {
+      kstep(par, IntC<0>{}, f0, f1, pa, s2, nd);
+      kstep(par, IntC<1>{}, f1, f0, pa, s2, nd);
+      kstep(par, IntC<NK == 4 ? 2 : 0>{}, f0, f1, pa, s2, nd);
+    } else {
+      kstep(par, IntC<0>{}, f0, f1, pa, s2, nd);
+    }
     // slice s+1 and the registers of slice s+1 have landed; only this slice's G loads may still fly
     __builtin_amdgcn_s_waitcnt(0x0070 | G);            // vmcnt(G) lgkmcnt(0)
     __asm__ volatile("s_barrier" ::: "memory");
-    kstep(par, IntC<3>{}, f1, f0, stage(s + 1), fhalf, s2, nd);
+    kstep(par, IntC<NK - 1>{}, f1, f0, stage(s + 1), s2, nd);
   };
 
   int64_t s = 0;
@@ -348,46 +269,93 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
   }
   if (s < slices) slice_body(IntC<0>{}, s);
   __builtin_amdgcn_s_waitcnt(0x0070);                  // the surplus loads of the last slices have landed
-  write_tile<JT, NWN>(acc, epi, y, M, N, m0, n0, lds);
+
+  if (KW == 2) {                                       // second set hands its sums to the first through LDS
+    __syncthreads();
+    float* sum = reinterpret_cast<float*>(lds) + slot * (128 * 32 * JT);
+    if (KH == 1) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < JT; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            *reinterpret_cast<f32x4*>(sum + (((i * JT + j) * 4 + q) * 64 + lane) * 4) =
+                (f32x4){acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+    }
+    __syncthreads();
+    if (KH == 0) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < JT; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const f32x4 o = *reinterpret_cast<const f32x4*>(sum + (((i * JT + j) * 4 + q) * 64 + lane) * 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] = acc[i][j][4 * q + e] + o[e];
+          }
+    }
+  }
+  write_tile<JT, NWN, S::kSlots>(acc, epi, y, M, N, m0, n0, lds, slot, KH == 0);
+}
+
+// Common body of the weight-in-register kernels: which tile, which wave does what.
+template <class S>
+__device__ __forceinline__ void weight_regs_kernel(const uint16_t* __restrict__ a, const uint32_t* __restrict__ wp,
+                                                   const uint16_t* __restrict__ scale, uint16_t* __restrict__ y, int64_t M,
+                                                   int64_t K, int64_t N, int64_t block, int8_t* lds) {
+  int64_t tile_m, panel;
+  if (!gemm_core::tile_of(blockIdx.x, (M + S::kBM - 1) / S::kBM, (N + S::kBN - 1) / S::kBN, tile_m, panel)) return;
+  const int64_t m0 = tile_m * S::kBM, n0 = panel * S::kBN;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int slot = wave % S::kSlots;
+  WeightRegs<S::kJT> wr;
+  wr.wp = wp; wr.scale = scale; wr.kblocks = K / BKH; wr.N = N; wr.slices_per_block = uint32_t(block / BKH);
+  wr.tile0 = n0 / 32 + (slot % S::kNWN) * S::kJT;
+  PlainEpilogue epi;
+  const int8_t* ab = reinterpret_cast<const int8_t*>(a);
+  if (S::kKW == 1 || wave < S::kSlots) run_weight_regs<S, 0>(ab, 2 * K, wr, epi, y, M, N, K / BKH, m0, n0, lds, slot);
+  else run_weight_regs<S, S::kKW - 1>(ab, 2 * K, wr, epi, y, M, N, K / BKH, m0, n0, lds, slot);
 }
 
 // (a [M,K] f16, w_prepacked, scale [K/block, N] f16, y [M,N] f16, M, K, N, block) ; K % 64 == 0, block % 64 == 0,
 // a 16-byte aligned and below 4 GiB.  grid = 8 * ceil(ceil(N/256) / 8) * ceil(M/256), block = 256.
+using BigShape = Shape<2, 4, 2, 1>;                    // 256 x 256, 8 waves
 extern "C" __global__ void __launch_bounds__(512, 1) mtrt_gemm_w4a16_t256x256(
     const uint16_t* __restrict__ a, const uint32_t* __restrict__ wp, const uint16_t* __restrict__ scale,
     uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t block) {
-  __shared__ __attribute__((aligned(16))) int8_t lds[gemm_core::LDS_BYTES_8WAVES];
-  int64_t m0, n0;
-  if (!gemm_core::tile_origin(M, N, m0, n0)) return;
-  WeightRegs<2> wr;
-  wr.wp = wp; wr.scale = scale; wr.kblocks = K / BKH; wr.N = N; wr.slices_per_block = uint32_t(block / BKH);
-  wr.tile0 = n0 / 32 + ((threadIdx.x >> 6) & 3) * 2;
-  PlainEpilogue epi;
-  run_weight_regs<2>(reinterpret_cast<const int8_t*>(a), 2 * K, wr, epi, y, M, N, K / BKH, m0, n0, lds);
+  __shared__ __attribute__((aligned(16))) int8_t lds[BigShape::kLds];
+  weight_regs_kernel<BigShape>(a, wp, scale, y, M, K, N, block, lds);
 }
-extern "C" __global__ void __launch_bounds__(THREADS) mtrt_gemm_w4a16_t128x64(
+// Medium M: 128 x 64 tiles so that the grid still fills the chip, two wave sets splitting each slice.
+// Same argument list.  grid = 8 * ceil(ceil(N/64) / 8) * ceil(M/128), block = 256.
+using MidShape = Shape<1, 2, 1, 2>;                    // 128 x 64, 4 waves
+extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w4a16_t128x64(
     const uint16_t* __restrict__ a, const uint32_t* __restrict__ wp, const uint16_t* __restrict__ scale,
     uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t block) {
-  __shared__ __attribute__((aligned(16))) int8_t lds[2 * (128 + 64) * 128];
-  gemm_tiles<2, 1>(a, wp, scale, y, M, K, N, block, lds);
+  __shared__ __attribute__((aligned(16))) int8_t lds[MidShape::kLds];
+  weight_regs_kernel<MidShape>(a, wp, scale, y, M, K, N, block, lds);
 }
 
 // Small M (<= 32): one workgroup per 32 columns, four waves split K.
-extern "C" __global__ void __launch_bounds__(THREADS) mtrt_gemm_w4a16_skinny(
-    const uint16_t* __restrict__ a, const uint32_t* __restrict__ wp, const uint16_t* __restrict__ scale,
-    uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t block) {
-  // Per wave a ring of four 4 KiB stages (32 rows x 64 k of activations each), filled by
+// G: groups of 8 activation rows kept per stage (M <= 8 * G); WAVES: waves that split K.
+template <int G, int WAVES>
+__device__ __forceinline__ void skinny(const uint16_t* __restrict__ a, const uint32_t* __restrict__ wp,
+                                       const uint16_t* __restrict__ scale, uint16_t* __restrict__ y, int64_t M, int64_t K,
+                                       int64_t N, int64_t block, int8_t* lds) {
+  // Per wave a ring of four stages (8 * G rows x 64 k of activations each), filled by
   // direct-to-LDS loads three slices ahead: a fragment read straight from global memory would
   // touch 64 different cache lines per instruction (32 rows 8 KiB apart), the ring is filled
   // with whole 128-byte row segments.  The waves never touch each other's ring: no barriers.
-  constexpr int kStages = 4, kStageBytes = 32 * 128;
-  __shared__ __attribute__((aligned(16))) int8_t lds[4 * kStages * kStageBytes];
+  constexpr int kStages = 4, kStageBytes = 8 * G * 128;
+  constexpr int kLoads = G + 2;                      // memory instructions per slice and wave
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int frow = lane & 31, fhalf = lane >> 5;
   const int64_t tile = blockIdx.x;
   const int64_t kblocks = K / BKH;
-  const int64_t kb0 = kblocks * wave / 4, kb1 = kblocks * (wave + 1) / 4;
+  const int64_t kb0 = kblocks * wave / WAVES, kb1 = kblocks * (wave + 1) / WAVES;
   const int64_t klast = kb1 - 1;
   int64_t col = tile * 32 + frow;
   col = col < N ? col : N - 1;                       // columns past N: the last column's scales, never stored
@@ -395,10 +363,10 @@ extern "C" __global__ void __launch_bounds__(THREADS) mtrt_gemm_w4a16_skinny(
   const u4* bp = reinterpret_cast<const u4*>(wp) + (tile * kblocks) * 64 + lane;
   int8_t* ring = lds + wave * (kStages * kStageBytes);
 
-  // direct-to-LDS load g (of 4) of a slice: rows 8g .. 8g+7, lane l <-> (row l >> 3, LDS chunk l & 7)
-  uint32_t aoff[4];
+  // direct-to-LDS load g (of G) of a slice: rows 8g .. 8g+7, lane l <-> (row l >> 3, LDS chunk l & 7)
+  uint32_t aoff[G];
 #pragma unroll
-  for (int g = 0; g < 4; ++g) {
+  for (int g = 0; g < G; ++g) {
     const int lrow = g * 8 + (lane >> 3);
     const int64_t row = lrow < M ? lrow : M - 1;     // rows past M repeat the last row; never stored
     aoff[g] = uint32_t(row * K * 2 + (((lane & 7) ^ ((lrow >> 1) & 7)) << 4));
@@ -408,12 +376,12 @@ extern "C" __global__ void __launch_bounds__(THREADS) mtrt_gemm_w4a16_skinny(
     u4 w;
     uint32_t sc;
   };
-  // everything slice kb needs from memory: 4 + 2 loads, always, so that the waits can count
+  // everything slice kb needs from memory: G + 2 loads, always, so that the waits can count
   auto fetch = [&](int64_t kb, int64_t clamp, Slice& dst) {
     kb = kb < clamp ? kb : clamp;
     int8_t* st = ring + int(kb & (kStages - 1)) * kStageBytes;
 #pragma unroll
-    for (int g = 0; g < 4; ++g)
+    for (int g = 0; g < G; ++g)
       __builtin_amdgcn_global_load_lds((gemm_core::global_void_t*)(abase + kb * (BKH * 2) + aoff[g]),
                                        (gemm_core::lds_void_t*)(st + g * 1024), 16, 0, 0);
     // Register loads issued as opaque instructions: the compiler's own wait-count bookkeeping
@@ -425,8 +393,8 @@ extern "C" __global__ void __launch_bounds__(THREADS) mtrt_gemm_w4a16_skinny(
     __asm__ volatile("global_load_ushort %0, %1, off" : "=v"(dst.sc) : "v"(ssrc) : "memory");
   };
   // ties the registers of a slice to the wait, so that no use can be scheduled in front of it:
-  // 24 loads issued, 18 may fly -> the 6 of the oldest slice have landed
-  auto landed = [&](Slice& sl) { __asm__ volatile("s_waitcnt vmcnt(18)" : "+v"(sl.w), "+v"(sl.sc)::"memory"); };
+  // four slices issued, the loads of three may fly -> those of the oldest slice have landed
+  auto landed = [&](Slice& sl) { __asm__ volatile("s_waitcnt vmcnt(%2)" : "+v"(sl.w), "+v"(sl.sc) : "n"(3 * kLoads) : "memory"); };
   auto landed_all = [&](Slice& sl) { __asm__ volatile("s_waitcnt vmcnt(0)" : "+v"(sl.w), "+v"(sl.sc)::"memory"); };
 
   v16f acc;
@@ -439,7 +407,8 @@ extern "C" __global__ void __launch_bounds__(THREADS) mtrt_gemm_w4a16_skinny(
     sp.u = sl.sc * 0x00010001u;
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
-      const v8h fa = *reinterpret_cast<const v8h*>(st + gemm_core::lds_off(frow, 2 * ks + fhalf));
+      const int arow = frow < 8 * G ? frow : 8 * G - 1;   // rows past the ring: any valid data, never stored
+      const v8h fa = *reinterpret_cast<const v8h*>(st + gemm_core::lds_off(arow, 2 * ks + fhalf));
       union { u4 u; v8h h; } fb;
       dequant4(sl.w[ks], sp.h, 0, mask, fb.u);
       dequant4(sl.w[ks], sp.h, 1, mask, fb.u);
@@ -488,14 +457,30 @@ extern "C" __global__ void __launch_bounds__(THREADS) mtrt_gemm_w4a16_skinny(
 #pragma unroll
   for (int r = 0; r < 16; ++r) partial[wave][r][lane] = acc[r];
   __syncthreads();
-  // 32 x 32 outputs, 256 threads: 4 each
-  for (int e = threadIdx.x; e < 16 * 64; e += THREADS) {
+  for (int e = threadIdx.x; e < 16 * 64; e += 64 * WAVES) {
     const int r = e >> 6, l = e & 63;
-    const float v = ((partial[0][r][l] + partial[1][r][l]) + partial[2][r][l]) + partial[3][r][l];
+    float v = partial[0][r][l];
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) v = v + partial[w][r][l];
     const int64_t row = (r >> 2) * 8 + (l >> 5) * 4 + (r & 3);
     const int64_t c = tile * 32 + (l & 31);
     if (row < M && c < N) y[row * N + c] = uint16_t(f32_to_f16_bits(v));
   }
+}
+
+// M <= 16: half the activation rows per stage (8 waves splitting K were no faster than 4).
+extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w4a16_skinny16(
+    const uint16_t* __restrict__ a, const uint32_t* __restrict__ wp, const uint16_t* __restrict__ scale,
+    uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t block) {
+  __shared__ __attribute__((aligned(16))) int8_t lds[4 * 4 * 2 * 1024];
+  skinny<2, 4>(a, wp, scale, y, M, K, N, block, lds);
+}
+// M <= 32: 4 waves split K.
+extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w4a16_skinny(
+    const uint16_t* __restrict__ a, const uint32_t* __restrict__ wp, const uint16_t* __restrict__ scale,
+    uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t block) {
+  __shared__ __attribute__((aligned(16))) int8_t lds[4 * 4 * 4 * 1024];
+  skinny<4, 4>(a, wp, scale, y, M, K, N, block, lds);
 }
 
 // Any shape: one output per lane, reading the ORIGINAL packed [K,N] nibbles; not a fast path.

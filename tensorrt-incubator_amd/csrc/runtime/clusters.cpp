@@ -345,6 +345,8 @@ int32_t mtrt_hip_gemm_w4a16(mtrt_stream_t stream, const void *a, const void *w_k
   const bool fast = w_prepacked && K > 0 && K % 64 == 0 && block % 64 == 0 && aligned(a, 16) && aligned(w_prepacked, 16);
   if (fast) {
     void *args[] = {&a, &w_prepacked, &scale, &y, &M, &K, &N, &block};
+    if (M <= 16)
+      return launch(st, "mtrt_gemm_w4a16_skinny16", uint32_t((N + 31) / 32), kBlock, as_hip(stream), args);
     if (M <= 32)
       return launch(st, "mtrt_gemm_w4a16_skinny", uint32_t((N + 31) / 32), kBlock, as_hip(stream), args);
     // 256 x 256 tiles (512 threads) once they cover at least half of the compute units (measured:
@@ -354,8 +356,10 @@ int32_t mtrt_hip_gemm_w4a16(mtrt_stream_t stream, const void *a, const void *w_k
     if (panels * tiles_m * 2 >= int64_t(num_compute_units(st)) && M * K * 2 < (int64_t(1) << 32))
       return launch(st, "mtrt_gemm_w4a16_t256x256", uint32_t(8 * ((panels + 7) / 8) * tiles_m), 512, as_hip(stream),
                     args);
-    const int64_t small = ((M + 127) / 128) * ((N + 63) / 64);
-    return launch(st, "mtrt_gemm_w4a16_t128x64", uint32_t(small), kBlock, as_hip(stream), args);
+    if (M * K * 2 < (int64_t(1) << 32)) {
+      const int64_t small = 8 * ((((N + 63) / 64) + 7) / 8) * ((M + 127) / 128);
+      return launch(st, "mtrt_gemm_w4a16_t128x64", uint32_t(small), kBlock, as_hip(stream), args);
+    }
   }
   if (!w_kn_packed)
     return set_error(MTRT_INVALID_ARGUMENT, "this shape needs the original packed weights (K=%lld block=%lld)",

@@ -144,7 +144,7 @@ def test_w4a16_small_shapes(pkg, orc, shape):
     B = 128
     a, w, wp, s = _w4a16_inputs(orc, rng(M + K + N), M, K, N, B)
     y, kernel = _run_w4a16(pkg, a, wp, s, K, N, B)
-    assert kernel == ("mtrt_gemm_w4a16_skinny" if M <= 32 else "mtrt_gemm_w4a16_t128x64")
+    assert kernel == ("mtrt_gemm_w4a16_skinny16" if M <= 16 else "mtrt_gemm_w4a16_skinny" if M <= 32 else "mtrt_gemm_w4a16_t128x64")
     _check_w4a16(orc, y, a, w, s, K, N, B, orc.gemm_w4a16(a, wp, s, K, N, B))
 
 
@@ -180,7 +180,7 @@ def test_c5_w4a16_full_size(pkg, orc, M):
     K, N, B = 4096, 11008, 128
     a, w, wp, s = _w4a16_inputs(orc, rng(5), M, K, N, B)
     y, kernel = _run_w4a16(pkg, a, wp, s, K, N, B)
-    assert kernel == {16: "mtrt_gemm_w4a16_skinny", 256: "mtrt_gemm_w4a16_t128x64", 4096: "mtrt_gemm_w4a16_t256x256"}[M]
+    assert kernel == {16: "mtrt_gemm_w4a16_skinny16", 256: "mtrt_gemm_w4a16_t128x64", 4096: "mtrt_gemm_w4a16_t256x256"}[M]
     rows = sorted(set([0, M - 1] + list(range(0, M, max(1, M // 38)))))[:40]
     orc.set_threads(16)
     import torch
