@@ -21,6 +21,9 @@ Every kernel also gets its own line under "workloads" (achieved, peak, fraction)
 timed with HIP events on the launch stream over rotating buffers whose combined
 footprint exceeds the 256 MiB Infinity Cache, so cache hits do not count as HBM.
 "roofline" repeats the entry of the kernel with the largest share of the step.
+"mfma_sustained" is the matrix-core rate a loop of nothing but MFMAs reaches on the bench's
+own operand data (the published dense peaks hold for idle data only: the clock drops under
+the board's power limit); GEMM entries carry "frac_of_sustained" beside "frac".
 "cpu_baseline" times the CPU oracle (a C++ restatement of the reference's host
 lowering, NOT the reference binary) on a bounded sample, single-threaded like the
 reference interpreter, and extrapolates linearly to the step.
@@ -155,7 +158,8 @@ def build_workloads(pkg, torch, which):
             a = (a4[i].data_ptr(), w4[i].data_ptr(), as4.data_ptr(), ws4.data_ptr(), y4[i].data_ptr(), M, K, N)
             return lambda: pkg.check(L.mtrt_hip_gemm_w8a8(stream(), *a))
         out.append(dict(name="mtrt_gemm_w8a8_nk", config="C4", bound="mfma", work=2.0 * M * K * N, peak=INT8_PEAK,
-                        unit="TOP/s", nslots=ns, make=gemm8, keep=(a4, w4, y4, as4, ws4)))
+                        unit="TOP/s", nslots=ns, make=gemm8, keep=(a4, w4, y4, as4, ws4),
+                        probe=("mtrt_mfma_probe_i8", w4[0], 65536.0)))
 
     if which in ("all", "c5"):
         K, N, B = 4096, 11008, 128
@@ -178,7 +182,8 @@ def build_workloads(pkg, torch, which):
                                 keep=(a5, w5, s5, y5)))
             else:
                 out.append(dict(name=kname, config="C5 M=%d" % M, bound="mfma", work=2.0 * M * K * N, peak=F16_PEAK,
-                                unit="TFLOP/s", nslots=ns, make=gemm4, keep=(a5, w5, s5, y5)))
+                                unit="TFLOP/s", nslots=ns, make=gemm4, keep=(a5, w5, s5, y5),
+                                probe=("mtrt_mfma_probe_f16", a5[0], 32768.0) if M == 4096 else None))
 
     for w in out:
         w["peak"] = HBM_PEAK if w["bound"] == "hbm" else w["peak"]
@@ -202,6 +207,39 @@ def calibration_copy(pkg, torch):
     nvec = nbytes // 16
     L.mtrt_cuda_launch_kernel(fn, nvec // 256, 1, 1, 256, 1, 1, 0, torch.cuda.current_stream().cuda_stream, args)
     torch.cuda.synchronize()
+
+
+def mfma_sustained(pkg, torch, kernel, operand, ops_per_mfma):
+    """Rate (T ops/s) of the matrix-core yardstick kernel on `operand`'s bytes: 16 independent
+    MFMAs per round and wave, one wave per SIMD, no memory traffic in the loop."""
+    import ctypes
+    L = pkg.lib()
+    dev = L.mtrt_cuda_get_current_device()
+    units = torch.cuda.get_device_properties(0).multi_processor_count
+    ksteps = 2048
+    out = torch.empty(units * 256, dtype=torch.int32, device="cuda")
+    assert operand.numel() * operand.element_size() >= (1 << 24)
+    name = kernel.encode()
+    fn = L.mtrt_cuda_module_get_function(L.mtrt_hip_builtin_module(), name, len(name))
+    vals = (ctypes.c_void_p(operand.data_ptr()), ctypes.c_void_p(out.data_ptr()), ctypes.c_int32(ksteps))
+    args = (ctypes.c_void_p * 3)(*[ctypes.cast(ctypes.pointer(v), ctypes.c_void_p) for v in vals])
+    s = torch.cuda.current_stream().cuda_stream
+
+    def launch():
+        L.mtrt_cuda_launch_kernel(fn, units, 1, 1, 256, 1, 1, 0, s, args)
+    for _ in range(2):
+        launch()
+    e0, e1 = L.mtrt_cuda_event_create(dev), L.mtrt_cuda_event_create(dev)
+    L.mtrt_cuda_stream_record_event(s, e0)
+    reps = 5
+    for _ in range(reps):
+        launch()
+    L.mtrt_cuda_stream_record_event(s, e1)
+    L.mtrt_cuda_event_sync(e1)
+    us = L.mtrt_cuda_event_elapsed_msec(e0, e1) * 1e3 / reps
+    L.mtrt_cuda_event_release(e0)
+    L.mtrt_cuda_event_release(e1)
+    return ksteps * 16.0 * units * 4 * ops_per_mfma / us / 1e6
 
 
 def traffic_from_profile(kernel):
@@ -357,6 +395,15 @@ def main():
         kernels.append(dict(kernel=w["name"], config=w["config"], bound=w["bound"], us=round(us, 2),
                             achieved=round(achieved, 1), peak=w["peak"], unit=w["unit"], frac=round(achieved / w["peak"], 4),
                             work=w["work"]))
+    # what the matrix cores sustain on this very data with nothing else going on (power-limited)
+    sustained = {}
+    for w in wl:
+        if w.get("probe"):
+            kname, operand, ops = w["probe"]
+            sustained[w["unit"]] = round(mfma_sustained(pkg, torch, kname, operand, ops), 1)
+    for k in kernels:
+        if k["bound"] == "mfma" and k["unit"] in sustained:
+            k["frac_of_sustained"] = round(k["achieved"] / sustained[k["unit"]], 4)
     value = 100.0 * (ideal_us / 1e3) / ms_per_step
     dom = max(kernels, key=lambda k: k["us"])
     line = {
@@ -370,6 +417,9 @@ def main():
             args.workload, args.workload.upper()), "kernels_per_step": len(wl)},
         "roofline": {"kernel": dom["kernel"], "bound": dom["bound"], "achieved": dom["achieved"], "peak": dom["peak"],
                      "unit": dom["unit"], "frac": dom["frac"], "traffic": traffic_from_profile(dom["kernel"])},
+        "mfma_sustained": {"rates": sustained, "method": "mtrt_mfma_probe_*: 16 independent MFMAs per round and wave, one wave "
+                           "per SIMD, operands = this bench's own data, no memory traffic; published dense peaks are "
+                           "not reached on non-zero data (power limit)"},
         "workloads": kernels,
     }
     if not args.no_cpu_baseline:
