@@ -1,0 +1,373 @@
+"""Host-side mirror of the Tripy quantization surface over libmtrt_hip.so.
+
+What is mirrored (names, argument meaning, validation order and error text):
+
+  quantize(input, scale, dtype, dim=None)    tripy/nvtripy/frontend/ops/quantize.py:32-119
+  dequantize(input, scale, dtype, dim=None)  tripy/nvtripy/frontend/ops/dequantize.py:32-114
+  check_qdq_args                             tripy/nvtripy/frontend/ops/utils.py:179-256
+  cast (the float8 / int4 routes)            tripy/nvtripy/frontend/ops/cast.py:67-84
+  Linear (fake-quant forward)                tripy/nvtripy/frontend/module/linear.py:112-151
+  scale from calibration amax                tripy/examples/nanogpt/weight_loader.py:67-68
+
+Tripy builds a trace and hands `tensorrt.quantize` / `tensorrt.dequantize` to TensorRT
+(tripy/nvtripy/trace/ops/quantize.py:27-46).  Here every call runs at once: the wrapper
+maps (input shape, scale shape, dim) to the scale addressing of the C ABI and launches
+the gfx950 cluster on the current stream.  torch owns the device memory; nothing else of
+it is used on the quantization path.  Without the library or a gfx950 device the calls
+raise: there is no other path.
+
+Storage of the quantized types: int8 as int8; float8 as the e4m3fn byte; int4 one code per
+byte in the low nibble (the executor's buffer form,
+mlir-tensorrt/executor/lib/Runtime/Backend/Common/DataTypes.cpp:494-519).
+"""
+import numbers
+
+import numpy as np
+
+from . import (BF16, F16, F32, F8E4M3FN, I4, I8, SCALE_COL, SCALE_ROW, SCALE_UNIFORM, check, lib)
+
+
+class TripyException(Exception):
+    """tripy/nvtripy/common/exception.py:26-31"""
+
+
+def raise_error(summary, details=None):
+    """Summary first, then the details joined, as tripy/nvtripy/common/exception.py:123-170 prints them
+    (source-code excerpts of the reference's message are left out)."""
+    raise TripyException(summary + "".join("\n    " + str(d) if i == 0 else str(d) for i, d in enumerate(details or [])))
+
+
+class dtype:
+    def __init__(self, name, code, itemsize, np_dtype=None):
+        self.name, self.code, self.itemsize, self.np_dtype = name, code, itemsize, np_dtype
+
+    def __repr__(self):
+        return self.name
+
+    __str__ = __repr__
+
+
+float32 = dtype("float32", F32, 4, np.float32)
+float16 = dtype("float16", F16, 2, np.float16)
+bfloat16 = dtype("bfloat16", BF16, 2)
+int8 = dtype("int8", I8, 1, np.int8)
+int4 = dtype("int4", I4, 1)
+float8 = dtype("float8", F8E4M3FN, 1)
+int32 = dtype("int32", None, 4, np.int32)
+
+# tripy/nvtripy/frontend/ops/utils.py:183-184
+QUANTIZABLE_DTYPES = (float32, float16, bfloat16)
+QUANTIZED_DTYPES = (int8, int4, float8)
+
+
+def is_quantized_dtype(d):
+    return d in QUANTIZED_DTYPES
+
+
+def _torch():
+    import torch
+    return torch
+
+
+def _torch_dtype(d):
+    torch = _torch()
+    return {float32: torch.float32, float16: torch.float16, bfloat16: torch.bfloat16, int8: torch.int8,
+            int4: torch.int8, float8: torch.uint8, int32: torch.int32}[d]
+
+
+def _from_torch_dtype(td):
+    torch = _torch()
+    table = {torch.float32: float32, torch.float16: float16, torch.bfloat16: bfloat16, torch.int8: int8,
+             torch.int32: int32, torch.int64: int32, torch.float64: float32}
+    if td not in table:
+        raise_error("Unsupported data type.", ["Got: %s" % td])
+    return table[td]
+
+
+class Tensor:
+    """A value with a Tripy dtype.  `is_cpu_constant` is what the reference reads off the trace:
+    the tensor was made from host data and has not gone through an operation
+    (`isinstance(scale.trace_tensor.producer, Constant) and producer.device.kind == "cpu"`,
+    utils.py:246)."""
+
+    def __init__(self, data, dtype=None, _produced=False, _tp_dtype=None):
+        torch = _torch()
+        if isinstance(data, Tensor):
+            self._t, self.dtype, self.is_cpu_constant = data._t, data.dtype, data.is_cpu_constant
+            return
+        if _produced:
+            self._t, self.dtype, self.is_cpu_constant = data, _tp_dtype, False
+            return
+        if isinstance(data, np.ndarray):
+            t = torch.from_numpy(data if data.flags.c_contiguous else data.copy(order="C"))
+        elif isinstance(data, torch.Tensor):
+            t = data
+        else:
+            t = torch.tensor(data)
+        want = dtype if dtype is not None else _from_torch_dtype(t.dtype)
+        if want in (int4, float8):
+            raise_error("Tensors of a quantized type are made with cast or quantize.", ["Got dtype=%s" % want])
+        t = t.to(_torch_dtype(want))
+        self.is_cpu_constant = not t.is_cuda
+        self._t, self.dtype = t, want
+
+    @property
+    def shape(self):
+        return tuple(self._t.shape)
+
+    @property
+    def rank(self):
+        return self._t.dim()
+
+    def device_data(self):
+        """The values in device memory (uploaded once)."""
+        if not self._t.is_cuda:
+            self._t = self._t.cuda()
+        return self._t
+
+    def torch(self):
+        """A torch view of the stored values (codes for int4 / float8)."""
+        return self._t
+
+    def __repr__(self):
+        return "tensor(shape=%s, dtype=%s)" % (self.shape, self.dtype)
+
+
+def _produced(t, d):
+    return Tensor(t, _produced=True, _tp_dtype=d)
+
+
+def ones(shape, dtype=float32):
+    """An operation result, hence not a constant (tripy/tests/frontend/ops/test_quantize.py:76-84 relies on it).
+    Values are made on the host and uploaded on first use by a kernel."""
+    return _produced(_torch().ones(tuple(shape), dtype=_torch_dtype(dtype)), dtype)
+
+
+def iota(shape, dim=0, dtype=float32):
+    torch = _torch()
+    shape = tuple(shape)
+    idx = torch.arange(shape[dim], dtype=torch.float32)
+    view = [1] * len(shape)
+    view[dim] = shape[dim]
+    return _produced(idx.reshape(view).expand(shape).contiguous().to(_torch_dtype(dtype)), dtype)
+
+
+def _convert_scale(scale, want):
+    """`convert_to_tensors={"scale"}` of the reference's interface decorator: numbers and sequences
+    become constants in the dtype the input requirements ask for (wrappers.py:364-370)."""
+    if isinstance(scale, Tensor):
+        return scale
+    if isinstance(scale, (numbers.Number, list, tuple)):
+        return Tensor(np.asarray(scale, dtype=np.float64).astype(np.float32), dtype=want if want in QUANTIZABLE_DTYPES else float32)
+    return Tensor(scale)
+
+
+def _invalid_inputs(func, expected):
+    raise_error("Invalid inputs for function: '%s'." % func, ["Expected: ", expected])
+
+
+def check_qdq_args(input, scale, dtype, dim, is_quantize):
+    """tripy/nvtripy/frontend/ops/utils.py:191-256, same order, same text."""
+    valid_input_dtypes = QUANTIZABLE_DTYPES if is_quantize else QUANTIZED_DTYPES
+    valid_target_dtypes = QUANTIZED_DTYPES if is_quantize else QUANTIZABLE_DTYPES
+    op_str = "quantize op" if is_quantize else "dequantize op"
+
+    if input.dtype not in valid_input_dtypes:
+        raise_error(f"Input does not have a valid dtype in {op_str}.",
+                    [f"input.dtype must be one of {valid_input_dtypes}, ", f"Got dtype={input.dtype}"])
+    if dtype not in valid_target_dtypes:
+        raise_error(f"Unsupported data type in {op_str}.",
+                    [f"Supported data types are: {valid_target_dtypes}. ", f"Got dtype={dtype}"])
+
+    quantizable_dtype, quantized_dtype = (input.dtype, dtype) if is_quantize else (dtype, input.dtype)
+    if scale.dtype != quantizable_dtype:
+        raise_error(f"Scale dtype does not match expected dtype in {op_str}.",
+                    [f"scale should have dtype={quantizable_dtype}, got {scale.dtype}"])
+
+    if dim is not None:
+        if scale.rank != 1:
+            raise_error(f"If dim is given, scale must be a 1-D tensor in per-channel {op_str}.",
+                        [f"scale has rank={scale.rank}."])
+    elif scale.rank == 2:
+        if input.rank != 2:
+            raise_error(f"Input must be a 2-D tensor in block-wise {op_str}.", [f"input has rank={input.rank}."])
+        if quantized_dtype != int4:
+            raise_error(f"Unsupported data type in block-wise {op_str}.",
+                        [f"Only `tp.int4` is supported, got {quantized_dtype}"])
+    elif scale.rank != 0:
+        raise_error(f"Scale must be a scalar tensor in per-tensor {op_str}.", [f"scale has rank={scale.rank}."])
+
+    if not scale.is_cpu_constant:
+        raise_error("`scale` argument must be a constant in CPU memory.",
+                    ["Hint: Use `scale = tp.copy(scale, tp.device('cpu'))` to copy the scale to CPU memory. "])
+
+
+def _scale_addressing(shape, scale, dim, op_str):
+    """(scale kind, d0, d1, nb) of the C ABI for the three modes of the op
+    (mlir-tensorrt/tensorrt/include/mlir-tensorrt-dialect/TensorRT/IR/TensorRTOps.td:3133-3194;
+    shape rules of mlir-tensorrt/tensorrt/lib/TensorRT/IR/Verification.cpp:1182-1265)."""
+    numel = int(np.prod(shape)) if len(shape) else 1
+    if dim is not None:
+        rank = len(shape)
+        if not -rank <= dim < rank:
+            raise_error(f"Dimension argument is out of bounds in {op_str}.", [f"dim={dim}, input rank={rank}"])
+        dim %= rank
+        c = shape[dim]
+        if scale.shape[0] != c:
+            raise_error(f"Scale size must match the size of the quantization axis in per-channel {op_str}.",
+                        [f"scale has {scale.shape[0]} elements, input.shape[{dim}]={c}"])
+        inner = int(np.prod(shape[dim + 1:])) if dim + 1 < rank else 1
+        if inner == 1:
+            return SCALE_COL, numel // c if c else 0, c, max(numel // c, 1) if c else 1
+        return SCALE_ROW, numel // inner, inner, c
+    if scale.rank == 2:
+        d0, d1 = shape
+        s0, s1 = scale.shape
+        if s1 != d1 or s0 == 0 or d0 % s0 != 0:
+            raise_error(f"Scale shape does not divide the input in block-wise {op_str}.",
+                        [f"input.shape={list(shape)}, scale.shape={list(scale.shape)}"])
+        return SCALE_COL, d0, d1, d0 // s0
+    d1 = shape[-1] if len(shape) else 1
+    return SCALE_UNIFORM, numel // d1 if d1 else 0, d1, 1
+
+
+def _scale_on_device(scale):
+    """The device ABI takes f32 scales; f16 / bf16 constants widen exactly."""
+    cached = getattr(scale, "_f32_dev", None)
+    if cached is None:
+        cached = scale.torch().to(_torch().float32).contiguous().cuda().reshape(-1)
+        scale._f32_dev = cached
+    return cached
+
+
+def _stream():
+    return _torch().cuda.current_stream().cuda_stream
+
+
+def quantize(input, scale, dtype, dim=None):
+    """tp.quantize: clamp(round_half_even(input / scale)) in `dtype` (int8, int4 or float8)."""
+    if not isinstance(input, Tensor):
+        input = Tensor(input)
+    scale = _convert_scale(scale, input.dtype)
+    # the interface decorator's input requirements are checked first (quantize.py:33-39)
+    if input.dtype not in QUANTIZABLE_DTYPES or scale.dtype != input.dtype or dtype not in QUANTIZED_DTYPES:
+        _invalid_inputs("quantize", "input.dtype to be one of [float32, float16, bfloat16], scale.dtype == input.dtype "
+                                    "and dtype to be one of [int4, int8, float8]")
+    check_qdq_args(input, scale, dtype, dim, True)
+    kind, d0, d1, nb = _scale_addressing(input.shape, scale, dim, "quantize op")
+    torch = _torch()
+    x = input.device_data().contiguous()
+    q = torch.empty(input.shape, dtype=_torch_dtype(dtype), device=x.device)
+    if x.numel():
+        check(lib().mtrt_hip_quantize(_stream(), x.data_ptr(), input.dtype.code, q.data_ptr(), dtype.code,
+                                      _scale_on_device(scale).data_ptr(), kind, d0, d1, nb, 0))
+    return _produced(q, dtype)
+
+
+def dequantize(input, scale, dtype, dim=None):
+    """tp.dequantize: input * scale in `dtype` (float32, float16 or bfloat16)."""
+    if not isinstance(input, Tensor):
+        input = Tensor(input)
+    scale = _convert_scale(scale, dtype)
+    if input.dtype not in QUANTIZED_DTYPES or dtype not in QUANTIZABLE_DTYPES or scale.dtype != dtype:
+        _invalid_inputs("dequantize", "input.dtype to be one of [int4, int8, float8], dtype to be one of "
+                                      "[float32, float16, bfloat16] and scale.dtype == dtype")
+    check_qdq_args(input, scale, dtype, dim, False)
+    kind, d0, d1, nb = _scale_addressing(input.shape, scale, dim, "dequantize op")
+    torch = _torch()
+    q = input.device_data().contiguous()
+    y = torch.empty(input.shape, dtype=_torch_dtype(dtype), device=q.device)
+    if q.numel():
+        check(lib().mtrt_hip_dequantize(_stream(), q.data_ptr(), input.dtype.code, y.data_ptr(), dtype.code,
+                                        _scale_on_device(scale).data_ptr(), kind, d0, d1, nb))
+    return _produced(y, dtype)
+
+
+def cast(input, dtype):
+    """tripy/nvtripy/frontend/ops/cast.py:67-84: quantized types other than int8 convert through
+    quantize / dequantize with scale 1."""
+    if not isinstance(input, Tensor):
+        input = Tensor(input)
+    if input.dtype == dtype:
+        return input
+    if is_quantized_dtype(input.dtype) and input.dtype != int8:
+        input = dequantize(input, 1.0, float32)
+        if dtype == float32:
+            return input
+    if is_quantized_dtype(dtype) and dtype != int8:
+        if input.dtype != float32:
+            input = _produced(input.device_data().to(_torch().float32), float32)
+        return quantize(input, 1.0, dtype)
+    return _produced(input.device_data().to(_torch_dtype(dtype)), dtype)
+
+
+def scale_from_amax(input, dtype):
+    """`scale = amax / maxbound` of the calibration flow (weight_loader.py:67-68; maxbound 127, 448 or 7),
+    computed on the device in one launch; returns (amax, scale) as 0-d f32 device tensors."""
+    from . import amax
+    qmax = {int8: 127.0, float8: 448.0, int4: 7.0}[dtype]
+    return amax(input.device_data().contiguous(), qmax)
+
+
+class Linear:
+    """tp.Linear (linear.py:30-151): out = x @ W^T + b, with the fake-quant pair on the input and on the
+    weight when `quant_dtype` is set.  weight: [out_features, in_features].
+
+    With int8, an input scale and a per-output-channel (dim 0) or per-tensor weight scale the product of
+    the two dequantized operands equals (q_x . q_W^T) * s_x * s_w[n] exactly in real arithmetic; `fused=True`
+    runs that form on the integer matrix cores (W8A8 cluster, int32 accumulation, f16 result) instead of
+    a float matmul of the dequantized operands."""
+
+    def __init__(self, in_features, out_features, bias=True, dtype=float32, quant_dtype=None, weight_quant_dim=None,
+                 fused=False):
+        torch = _torch()
+        self.dtype = dtype
+        self.weight = _produced(torch.zeros((out_features, in_features), dtype=_torch_dtype(dtype)), dtype)
+        self.bias = _produced(torch.zeros((out_features,), dtype=_torch_dtype(dtype)), dtype) if bias else None
+        self.quant_dtype = quant_dtype
+        self.weight_quant_dim = weight_quant_dim
+        self.weight_scale = None
+        self.input_scale = None
+        self.fused = fused
+
+    def __call__(self, x):
+        return self.forward(x)
+
+    def forward(self, x):
+        torch = _torch()
+        if not isinstance(x, Tensor):
+            x = Tensor(x)
+        if self.quant_dtype is not None:
+            q_x = None
+            if isinstance(self.input_scale, Tensor):
+                if self.weight_quant_dim == 1:
+                    raise_error("Unsupported quantization parameters for Linear module.",
+                                ["weight_quant_dim cannot be 1 when input_scale is provided. ",
+                                 f"input_scale={self.input_scale}, weight_quant_dim={self.weight_quant_dim}"])
+                q_x = quantize(x, self.input_scale, self.quant_dtype)
+            q_weight = quantize(self.weight, self.weight_scale, self.quant_dtype, self.weight_quant_dim)
+            if self.fused and q_x is not None and self.quant_dtype == int8 and x.rank == 2 and self.weight_scale.rank < 2:
+                return self._forward_w8a8(q_x, q_weight)
+            if q_x is not None:
+                x = dequantize(q_x, self.input_scale, self.dtype)
+            weight = dequantize(q_weight, self.weight_scale, self.dtype, self.weight_quant_dim)
+        else:
+            weight = self.weight
+        out = x.device_data() @ weight.device_data().transpose(1, 0)
+        if self.bias is not None:
+            out = out + self.bias.device_data().unsqueeze(0)
+        return _produced(out, self.dtype)
+
+    def _forward_w8a8(self, q_x, q_weight):
+        from . import gemm_w8a8
+        torch = _torch()
+        M = q_x.shape[0]
+        N = q_weight.shape[0]
+        s_x = _scale_on_device(self.input_scale).expand(M).contiguous()
+        s_w = _scale_on_device(self.weight_scale).expand(N).contiguous()
+        # Tripy's weight is [out, in] = [N, K] with K contiguous: already the layout the int8 cluster reads.
+        y = gemm_w8a8(q_x.device_data(), q_weight.device_data().contiguous(), s_x, s_w)
+        out = y.to(_torch_dtype(self.dtype))
+        if self.bias is not None:
+            out = out + self.bias.device_data().unsqueeze(0)
+        return _produced(out, self.dtype)

@@ -1,0 +1,243 @@
+"""Values of the Tripy-compatible mirror on the GPU.
+
+Known answers are those of the reference's integration tests:
+  tripy/tests/integration/test_quantize.py:32-43, 58-69, 72-114, 121-145
+  tripy/tests/integration/test_dequantize.py:30-79
+  tripy/tests/integration/test_linear.py:54-130
+  mlir-tensorrt/integrations/PJRT/test/JAX/CustomPrimitives/test_quantize.py:60-83
+and, on seeded random data, the CPU oracle addressed independently of the mirror (the scale is
+broadcast to the full shape with numpy and the oracle runs per-element on a flat view).
+Bar: bit-exact codes and dequantized values; Linear within 1e-3 relative of a float64 product of
+the oracle's dequantized operands.
+"""
+import importlib
+
+import numpy as np
+import pytest
+
+from helpers import rng
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def tp(pkg):
+    return importlib.import_module(pkg.__name__ + ".tp")
+
+
+def _torch_dtypes(tp):
+    import torch
+    return {tp.float32: torch.float32, tp.float16: torch.float16, tp.bfloat16: torch.bfloat16}
+
+
+def _all_float(tp):
+    return [tp.float32, tp.float16, tp.bfloat16]
+
+
+def test_quantize_int8_per_tensor(tp):
+    import torch
+    for d in _all_float(tp):
+        td = _torch_dtypes(tp)[d]
+        x = torch.tensor([1.0, 2.0], dtype=td)
+        scale = torch.tensor(0.5, dtype=td)
+        q = tp.quantize(tp.Tensor(x), tp.Tensor(scale), tp.int8)
+        assert q.dtype == tp.int8
+        assert torch.equal((x / scale).to(torch.int8), q.torch().cpu())
+
+
+def test_quantize_int8_per_channel(tp):
+    import torch
+    for d in (tp.float32, tp.bfloat16):
+        td = _torch_dtypes(tp)[d]
+        x = torch.tensor([[1.0, 2.0], [3.0, 4.0]], dtype=td)
+        scale = torch.tensor([0.2, 0.1], dtype=td)
+        q = tp.quantize(tp.Tensor(x), tp.Tensor(scale), tp.int8, dim=0)
+        # the reference test truncates ((x/scale).to(int8)); the op rounds half to even
+        # (TensorRTOps.td:3145-3185), which differs when the f32 quotient is not integral
+        expected = torch.clamp(torch.round(x.float() / scale.float().reshape(2, 1)), -128, 127).to(torch.int8)
+        assert torch.equal(expected, q.torch().cpu())
+
+
+def test_quantize_float8(tp):
+    import torch
+    for d in _all_float(tp):
+        td = _torch_dtypes(tp)[d]
+        x = torch.tensor([1.0, 2.0], dtype=td)
+        q = tp.quantize(tp.Tensor(x), tp.Tensor(torch.tensor(0.5, dtype=td)), tp.float8)
+        assert q.dtype == tp.float8
+        assert torch.equal(torch.tensor([2.0, 4.0]), tp.cast(q, tp.float32).torch().cpu())
+        x2 = torch.tensor([[1.0, 2.0], [3.0, 4.0]], dtype=td)
+        s2 = torch.tensor([0.5, 0.25], dtype=td)
+        q2 = tp.quantize(tp.Tensor(x2), tp.Tensor(s2), tp.float8, dim=0)
+        assert torch.equal(x2.float() / s2.float().reshape(2, 1), tp.cast(q2, tp.float32).torch().cpu())
+
+
+@pytest.mark.parametrize("quant_mode", ["block-wise", "per-tensor", "per-channel-0", "per-channel-1"])
+def test_qdq_int4(tp, quant_mode):
+    import torch
+    for d in _all_float(tp):
+        td = _torch_dtypes(tp)[d]
+        dim = None
+        if quant_mode == "block-wise":
+            scale = torch.ones((2, 4), dtype=td)
+        elif quant_mode == "per-tensor":
+            scale = torch.tensor(1.0, dtype=td)
+        else:
+            dim = int(quant_mode[-1])
+            scale = torch.ones((4,), dtype=td)
+        x = torch.ones((4, 4), dtype=td)
+        s = tp.Tensor(scale)
+        q = tp.quantize(tp.Tensor(x), s, tp.int4, dim)
+        y = tp.dequantize(q, s, d, dim)
+        assert y.dtype == d and torch.equal(x, y.torch().cpu())
+
+
+def test_dequantize_int8(tp):
+    import torch
+    for d in _all_float(tp):
+        td = _torch_dtypes(tp)[d]
+        q = tp.cast(tp.Tensor([4, 8]), tp.int8)
+        scale = torch.tensor(0.5, dtype=td)
+        y = tp.dequantize(q, tp.Tensor(scale), d)
+        assert torch.allclose(torch.tensor([4, 8]) * scale, y.torch().cpu())
+        q2 = tp.cast(tp.Tensor([[4, 8], [4, 8]]), tp.int8)
+        s2 = torch.tensor([0.8, 0.9], dtype=td)
+        y2 = tp.dequantize(q2, tp.Tensor(s2), d, dim=0)
+        assert torch.allclose(torch.tensor([[4, 8], [4, 8]]) * s2.reshape(2, 1), y2.torch().cpu())
+
+
+def test_dequantize_float8_per_tensor(tp):
+    import torch
+    for d in _all_float(tp):
+        td = _torch_dtypes(tp)[d]
+        q = tp.cast(tp.Tensor([1.0, 1.0]), tp.float8)
+        y = tp.dequantize(q, tp.Tensor(torch.tensor(0.5, dtype=td)), d)
+        assert y.dtype == d
+        assert torch.allclose(torch.tensor([0.5, 0.5]), y.torch().float().cpu())
+
+
+def test_jax_custom_primitive_known_answers(tp):
+    x = np.array([[10.0, 20.0, 30.0, 40.0], [50.0, 60.0, 70.0, 80.0]], dtype=np.float32)
+    q = tp.quantize(tp.Tensor(x), 1.0, tp.int8)
+    assert np.array_equal(q.torch().cpu().numpy(), x.astype(np.int8))
+    q = tp.quantize(tp.Tensor(x), [2.0, 10.0], tp.int8, dim=0)
+    assert np.array_equal(q.torch().cpu().numpy(), np.array([[5, 10, 15, 20], [5, 6, 7, 8]], dtype=np.int8))
+
+
+def _oracle_elementwise(orc, x_f32, scale_full_f32, o_x, o_q):
+    """Oracle result with the scale already broadcast: one row per element."""
+    n = x_f32.size
+    xs = orc.narrow(x_f32.ravel(), o_x)
+    q = orc.quantize(xs, o_x, o_q, scale_full_f32.ravel(), orc.SCALE_ROW, n, 1, n)
+    y = orc.dequantize(q, o_q, o_x, scale_full_f32.ravel(), orc.SCALE_ROW, n, 1, n)
+    return xs, q, y
+
+
+@pytest.mark.parametrize("case", [
+    ("f32", "i8", (3, 5, 7), 1), ("bf16", "f8", (4, 6, 10), 2), ("f16", "i8", (6, 33), 0), ("f32", "i4", (5, 9, 4), 0),
+    ("f32", "i8", (17, 64), None), ("bf16", "i4", (256, 48), "block"), ("f16", "f8", (2, 3, 4, 5), -1),
+])
+def test_modes_against_oracle(tp, orc, case):
+    import torch
+    xname, qname, shape, dim = case
+    r = rng(1000 + sum(shape) * 7 + len(xname) + 3 * len(qname))
+    d = {"f32": tp.float32, "f16": tp.float16, "bf16": tp.bfloat16}[xname]
+    o_x = {"f32": orc.F32, "f16": orc.F16, "bf16": orc.BF16}[xname]
+    qd, o_q, qmax = {"i8": (tp.int8, orc.I8, 127.0), "f8": (tp.float8, orc.F8E4M3FN, 448.0),
+                     "i4": (tp.int4, orc.I4, 7.0)}[qname]
+    x = (r.standard_normal(shape) * 3).astype(np.float32)
+    if dim == "block":
+        s = r.uniform(0.2, 1.5, (shape[0] // 64, shape[1])).astype(np.float32)
+        full = np.repeat(s, 64, axis=0)
+        dim_arg = None
+    elif dim is None:
+        s = np.float32(np.abs(x).max() / qmax)
+        full = np.full(shape, s, dtype=np.float32)
+        dim_arg = None
+    else:
+        c = shape[dim]
+        s = r.uniform(0.01, 0.2, (c,)).astype(np.float32)
+        view = [1] * len(shape)
+        view[dim] = c
+        full = np.broadcast_to(s.reshape(view), shape).astype(np.float32)
+        dim_arg = dim
+    # scale constants live in the input's type (the op requires scale.dtype == input.dtype)
+    s_store = orc.widen(orc.narrow(np.asarray(s, dtype=np.float32).ravel(), o_x), o_x).reshape(np.shape(s))
+    full_store = orc.widen(orc.narrow(full.ravel(), o_x), o_x).reshape(shape)
+    xs, q_ref, y_ref = _oracle_elementwise(orc, x, full_store, o_x, o_q)
+
+    td = _torch_dtypes(tp)[d]
+    x_t = torch.from_numpy(orc.widen(xs, o_x).reshape(shape)).to(td)      # exact: values are representable
+    s_t = torch.from_numpy(np.asarray(s_store, dtype=np.float32)).to(td)
+    scale = tp.Tensor(s_t)
+    q = tp.quantize(tp.Tensor(x_t), scale, qd, dim_arg)
+    assert np.array_equal(q.torch().cpu().numpy().view(np.uint8).ravel(), q_ref.view(np.uint8).ravel())
+    y = tp.dequantize(q, scale, d, dim_arg)
+    got = y.torch().cpu()
+    got_f32 = got.float().numpy().ravel()
+    assert np.array_equal(got_f32.view(np.uint32), orc.widen(y_ref, o_x).view(np.uint32))
+
+
+def test_quant_linear_reference_cases(tp):
+    """tripy/tests/integration/test_linear.py:88-130: unit scales, small integers: exact."""
+    import torch
+    for quant_dtype in (tp.int8, tp.float8):
+        for use_input_scale in (False, True):
+            for wqd in (None, 0, 1):
+                if use_input_scale and wqd == 1:
+                    continue
+                lin = tp.Linear(4, 2, quant_dtype=quant_dtype, weight_quant_dim=wqd)
+                lin.weight = tp.iota((2, 4))
+                lin.bias = tp.iota((2,))
+                lin.weight_scale = tp.Tensor(1.0 if wqd is None else [1.0] * (2 if wqd == 0 else 4))
+                if use_input_scale:
+                    lin.input_scale = tp.Tensor(1.0)
+                out = lin(tp.Tensor(np.ones((3, 4), dtype=np.float32)))
+                w = lin.weight.torch().cpu().numpy()
+                expect = np.ones((3, 4), dtype=np.float32) @ w.T + lin.bias.torch().cpu().numpy()
+                assert np.array_equal(out.torch().cpu().numpy(), expect)
+    for wqd, scale in [(None, np.ones((2, 4), dtype=np.float32)), (None, 1.0), (0, np.ones((8,), dtype=np.float32)),
+                       (1, np.ones((4,), dtype=np.float32))]:
+        lin = tp.Linear(4, 8, quant_dtype=tp.int4, weight_quant_dim=wqd)
+        lin.weight_scale = tp.Tensor(scale)
+        lin.weight = tp.Tensor(np.ones((8, 4), dtype=np.float32))
+        lin.bias = tp.Tensor(np.ones((8,), dtype=np.float32))
+        out = lin(tp.Tensor(np.ones((4, 4), dtype=np.float32)))
+        assert np.array_equal(out.torch().cpu().numpy(), np.full((4, 8), 5.0, dtype=np.float32))
+
+
+def test_quant_linear_fused_w8a8_matches_fake_quant(tp, orc):
+    """int8 Linear with an input scale and per-output-channel weight scales: the fused integer form
+    against a float64 product of the oracle's dequantized operands, 1e-3 relative (f16 result)."""
+    import torch
+    r = rng(77)
+    M, K, N = 96, 256, 160
+    x = r.standard_normal((M, K)).astype(np.float32)
+    w = (r.standard_normal((N, K)) * 0.05).astype(np.float32)
+    s_x = np.float32(np.abs(x).max() / 127.0)
+    s_w = (np.abs(w).max(axis=1) / 127.0).astype(np.float32)
+    lin = tp.Linear(K, N, bias=False, quant_dtype=tp.int8, weight_quant_dim=0, fused=True)
+    lin.weight = tp.Tensor(w)
+    lin.weight_scale = tp.Tensor(s_w)
+    lin.input_scale = tp.Tensor(s_x)
+    out = lin(tp.Tensor(x)).torch().cpu().numpy().astype(np.float64)
+
+    qx = orc.quantize(x.ravel(), orc.F32, orc.I8, np.array([s_x]), orc.SCALE_UNIFORM, M, K)
+    qw = orc.quantize(w.ravel(), orc.F32, orc.I8, s_w, orc.SCALE_ROW, N, K, N)
+    xd = qx.astype(np.float64).reshape(M, K) * np.float64(s_x)
+    wd = qw.astype(np.float64).reshape(N, K) * s_w.astype(np.float64)[:, None]
+    ref = xd @ wd.T
+    tol = 1e-3 * np.abs(ref) + 2.0 ** -10 * np.abs(ref) + 1e-6     # 1e-3 relative + one f16 rounding
+    assert np.all(np.abs(out - ref) <= tol), float(np.max(np.abs(out - ref) / (np.abs(ref) + 1e-9)))
+    lin.fused = False
+    out2 = lin(tp.Tensor(x)).torch().cpu().numpy().astype(np.float64)
+    assert np.all(np.abs(out2 - ref) <= 1e-3 * np.abs(ref) + 1e-4)
+
+
+def test_scale_from_amax(tp, orc):
+    r = rng(5)
+    x = r.standard_normal((64, 512)).astype(np.float32)
+    amax, scale = tp.scale_from_amax(tp.Tensor(x), tp.float8)
+    a_ref = orc.amax(x, orc.F32)
+    assert np.float32(amax.item()).tobytes() == a_ref.tobytes()
+    assert np.float32(scale.item()).tobytes() == orc.scale_from_amax(a_ref, 448.0).tobytes()
