@@ -230,6 +230,58 @@ MTRT_CAPI_EXPORTED int32_t mtrt_hip_gemm_w4a16(mtrt_stream_t stream, const void 
                                                const void *scale, void *y, int64_t M, int64_t K,
                                                int64_t N, int64_t block);
 
+/* ------------------------------------------------------------------------- */
+/* Part 3 — the interpreter's builtin set, status-returning                    */
+/* (mlir-tensorrt/executor/lib/Runtime/Backend/Lua/Modules/CUDA/CUDAModule.cpp) */
+/* ------------------------------------------------------------------------- */
+
+/* The reference registers `__cuda_*` builtins in the Lua state as lambdas over the driver API;
+ * handles travel as uintptr_t and a failure becomes a Lua error (SET_LUA_ERROR_IF_ERROR).  These
+ * are the bodies of those lambdas over HIP: same value conventions (handles as uintptr_t, i32
+ * launch dimensions), a status as the return value and mtrt_hip_last_error() as the text a
+ * binding raises.  Nothing aborts. */
+
+/* __cuda_load_module(u32 device, uptr data, u64 nbytes) -> uptr (CUDAModule.cpp:297-327).
+ * `data` / `nbytes`: a gfx950 code object in host memory (the executable's data segment that
+ * holds PTX in the reference); no JIT.  `device` must be the current device. */
+MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_load_module(uint32_t device, uintptr_t data, uint64_t nbytes,
+                                                     uintptr_t *out_module);
+/* __cuda_get_function(uptr module, string name) -> uptr (CUDAModule.cpp:287-295); NUL-terminated name. */
+MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_get_function(uintptr_t module, const char *name,
+                                                      uintptr_t *out_function);
+/* __cuda_launch(uptr func, i32 grid x,y,z, i32 block x,y,z, i32 smem, uptr stream, uptr argPtrArray)
+ * (CUDAModule.cpp:329-342).  The reference asserts func, stream and the argument array non-null;
+ * here a null func or argument array is MTRT_INVALID_ARGUMENT and a null stream is the default stream. */
+MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_launch(uintptr_t func, int32_t gridX, int32_t gridY, int32_t gridZ,
+                                                int32_t blockX, int32_t blockY, int32_t blockZ,
+                                                int32_t dynamicSharedMemory, uintptr_t stream,
+                                                uintptr_t argPtrArray);
+/* __cuda_stream_create / _sync / _destroy (CUDAModule.cpp:269-285) */
+MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_stream_create(uintptr_t *out_stream);
+MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_stream_sync(uintptr_t stream);
+MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_stream_destroy(uintptr_t stream);
+/* __cuda_alloc_device(stream, nbytes) / __cuda_free_device (CUDAModule.cpp:344-352, 413-421) */
+MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_alloc_device(uintptr_t stream, uint64_t nbytes, uintptr_t *out_ptr);
+MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_free_device(uintptr_t stream, uintptr_t ptr);
+/* __cuda_memcpy_{host2device,device2host,device2device}(stream, src, srcOffset, dst, dstOffset, nbytes)
+ * (CUDAModule.cpp:423-549): one entry point, the direction is found from the pointers. */
+MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_memcpy(uintptr_t stream, uintptr_t src, uint64_t srcOffset,
+                                                uintptr_t dst, uint64_t dstOffset, uint64_t nbytes);
+/* __cuda_memset_{8,16,32}(ptr, offset, nbytes, fill) (CUDAModule.cpp:170-205); width in {1,2,4}, runs a
+ * fill kernel on `stream` (no memset node, so it can be captured into a graph). */
+MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_memset(uintptr_t stream, uintptr_t ptr, uint64_t offset,
+                                                uint64_t nbytes, uint32_t fill, int32_t width);
+/* __cuda_num_devices (CUDAModule.cpp:86-90) and __cuda_get_program_device(logicalId) (:560-571) */
+MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_num_devices(int32_t *out_count);
+MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_get_program_device(int32_t logicalId, int32_t *out_device);
+
+/* Name table for a binding to register in a loop: Lua builtin name -> entry point of this part. */
+struct mtrt_lua_builtin {
+  const char *lua_name;
+  const char *symbol;
+};
+MTRT_CAPI_EXPORTED const struct mtrt_lua_builtin *mtrt_lua_cuda_builtins(size_t *count);
+
 /* Name of the kernel that the most recent successful part-2 call on this thread
  * launched last (for profiles and tests). */
 MTRT_CAPI_EXPORTED const char *mtrt_hip_last_kernel(void);

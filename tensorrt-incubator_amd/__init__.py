@@ -52,6 +52,20 @@ PROTOTYPES = {
     "mtrt_cuda_launch_kernel": (None, [_vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp, _c.POINTER(_vp)]),
     "mtrt_cuda_get_current_device": (_i32, []),
     "mtrt_cuda_get_program_device": (_i32, [_i32]),
+    # interpreter builtin bodies: handles travel as uintptr_t
+    "mtrt_lua_cuda_load_module": (_i32, [_c.c_uint32, _sz, _c.c_uint64, _c.POINTER(_sz)]),
+    "mtrt_lua_cuda_get_function": (_i32, [_sz, _c.c_char_p, _c.POINTER(_sz)]),
+    "mtrt_lua_cuda_launch": (_i32, [_sz, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _sz, _sz]),
+    "mtrt_lua_cuda_stream_create": (_i32, [_c.POINTER(_sz)]),
+    "mtrt_lua_cuda_stream_sync": (_i32, [_sz]),
+    "mtrt_lua_cuda_stream_destroy": (_i32, [_sz]),
+    "mtrt_lua_cuda_alloc_device": (_i32, [_sz, _c.c_uint64, _c.POINTER(_sz)]),
+    "mtrt_lua_cuda_free_device": (_i32, [_sz, _sz]),
+    "mtrt_lua_cuda_memcpy": (_i32, [_sz, _sz, _c.c_uint64, _sz, _c.c_uint64, _c.c_uint64]),
+    "mtrt_lua_cuda_memset": (_i32, [_sz, _sz, _c.c_uint64, _c.c_uint64, _c.c_uint32, _i32]),
+    "mtrt_lua_cuda_num_devices": (_i32, [_c.POINTER(_i32)]),
+    "mtrt_lua_cuda_get_program_device": (_i32, [_i32, _c.POINTER(_i32)]),
+    "mtrt_lua_cuda_builtins": (_vp, [_c.POINTER(_sz)]),
     "mtrt_hip_last_error": (_c.c_char_p, []),
     "mtrt_hip_last_kernel": (_c.c_char_p, []),
     "mtrt_hip_init": (_i32, []),

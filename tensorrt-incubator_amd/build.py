@@ -4,6 +4,8 @@
   lib/mtrt_test_fixtures.hsaco  the two launch-ABI test kernels, as a separate module
   lib/libmtrt_hip.so            C ABI (launch layer + cluster layer) with the kernel
                                 module embedded as read-only data
+  lib/mtrt_standalone_selftest  host program in the style of EmitC-generated C++ that calls the
+                                `namespace mtrt` flavour of the launch layer (run by the tests)
 
 hipcc cross-compiles for gfx950 without a GPU present.  Run as
 `python tensorrt-incubator_amd/build.py` or through `__graft_entry__.build()`.
@@ -67,6 +69,13 @@ def build_runtime():
           "-o", os.path.join(LIB, "libmtrt_hip.so")])
 
 
+def build_selftest():
+    src = os.path.join(CSRC, "selftest", "standalone_selftest.cpp")
+    _run(["g++", "-O1", "-std=c++17", "-Wall", "-Wextra", "-I" + os.path.join(ROOT, "include"), src,
+          "-L" + LIB, "-lmtrt_hip", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + os.path.join(ROCM, "lib"),
+          "-o", os.path.join(LIB, "mtrt_standalone_selftest")])
+
+
 def build_oracle():
     """The CPU oracle is test infrastructure; building it here keeps one build entry point."""
     _run(["make", "-C", os.path.join(ROOT, "oracle")])
@@ -75,6 +84,7 @@ def build_oracle():
 def build_all():
     build_kernels()
     build_runtime()
+    build_selftest()
     build_oracle()
 
 

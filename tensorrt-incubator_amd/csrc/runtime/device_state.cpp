@@ -187,9 +187,11 @@ int32_t launch(DeviceState *st, const std::string &kernel, uint32_t grid, uint32
     return MTRT_NOT_FOUND;
   const hipError_t e =
       hipModuleLaunchKernel(f, grid, 1, 1, block, 1, 1, /*sharedMemBytes=*/0, stream, args, nullptr);
-  if (e != hipSuccess)
+  if (e != hipSuccess) {
+    (void)hipGetLastError(); // reported through the status; do not leave it for the caller's next HIP call
     return set_error(MTRT_DRIVER_ERROR, "launching '%s' grid %u block %u: %s", kernel.c_str(), grid,
                      block, hipGetErrorString(e));
+  }
   std::snprintf(tl_kernel, sizeof(tl_kernel), "%s", kernel.c_str());
   return MTRT_OK;
 }

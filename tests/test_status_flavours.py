@@ -1,0 +1,145 @@
+"""The two status-returning flavours of the launch layer.
+
+  * `namespace mtrt` (include/mtrt_hip_standalone.h), the functions EmitC-generated host code calls in
+    the reference (mlir-tensorrt/executor/lib/Runtime/StandaloneCPP/MTRTRuntimeCuda.h:36-110): exercised
+    by a C++ host program linked against the library, built by build.py.
+  * `mtrt_lua_cuda_*`, the bodies of the interpreter's `__cuda_*` builtins
+    (mlir-tensorrt/executor/lib/Runtime/Backend/Lua/Modules/CUDA/CUDAModule.cpp:86-571): called through ctypes.
+
+CPU tests cover exports and argument validation (no device call); GPU tests replay the reference's launch
+known answers (mlir-tensorrt/compiler/test/IntegrationTests/EmitC/cuda-launch-argpack.mlir:84-130,
+IntegrationTests/CUDA/cuda-launch-kernel.mlir:60-99)."""
+import ctypes
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+STANDALONE_HEADER = os.path.join(ROOT, "include", "mtrt_hip_standalone.h")
+
+# MTRTRuntimeCuda.h:36-110 and MTRTRuntimeStatus.h:48-53
+REFERENCE_STANDALONE = [
+    "cuda_get_current_device", "cuda_get_program_device", "cuda_stream_sync", "cuda_alloc", "cuda_free", "cuda_copy",
+    "cuda_module_create_from_ptx_file", "cuda_module_destroy", "cuda_module_get_func", "cuda_launch_kernel",
+    "cuda_event_create", "cuda_event_release", "cuda_stream_record_event", "cuda_stream_wait_event",
+    "cuda_event_sync", "cuda_event_elapsed_msec", "get_last_error_message", "clear_last_error_message",
+]
+
+
+def _selftest(pkg):
+    return os.path.join(pkg.LIB_DIR, "mtrt_standalone_selftest")
+
+
+def test_standalone_header_and_exports(pkg):
+    text = re.sub(r"/\*.*?\*/", "", open(STANDALONE_HEADER).read(), flags=re.S)
+    declared = re.findall(r"MTRT_CAPI_EXPORTED[^;(]*?\b([a-z_]+)\s*\(", text)
+    assert sorted(declared) == sorted(REFERENCE_STANDALONE)
+    out = subprocess.run(["nm", "-DC", "--defined-only", pkg.LIB_PATH], capture_output=True, text=True).stdout
+    exported = set(re.findall(r" T mtrt::(\w+)\(", out))
+    assert exported == set(REFERENCE_STANDALONE)
+
+
+def test_standalone_argument_validation(pkg):
+    """null out-parameters, empty names, negative sizes, missing files: status + message, no device needed."""
+    res = subprocess.run([_selftest(pkg), "--validate"], capture_output=True, text=True, timeout=60)
+    assert res.returncode == 0, res.stdout + res.stderr
+    assert "standalone selftest ok" in res.stdout
+
+
+def test_builtin_name_table(pkg):
+    L = pkg.lib()
+    n = ctypes.c_size_t(0)
+    table = L.mtrt_lua_cuda_builtins(ctypes.byref(n))
+    entries = ctypes.cast(table, ctypes.POINTER(ctypes.c_char_p * 2 * n.value)).contents
+    names = {bytes(e[0]).decode(): bytes(e[1]).decode() for e in entries}
+    for lua_name in ("__cuda_load_module", "__cuda_get_function", "__cuda_launch", "__cuda_stream_create",
+                     "__cuda_alloc_device", "__cuda_memcpy_host2device", "__cuda_memset_32",
+                     "__cuda_get_program_device"):
+        assert lua_name in names
+    for sym in names.values():
+        assert hasattr(L, sym), sym
+
+
+def test_builtin_argument_validation(pkg):
+    L = pkg.lib()
+    out = ctypes.c_size_t(7)
+    assert L.mtrt_lua_cuda_load_module(0, 0, 0, ctypes.byref(out)) == 1 and out.value == 0
+    assert b"must not be empty" in L.mtrt_hip_last_error()
+    assert L.mtrt_lua_cuda_load_module(0, 16, 16, None) == 1
+    assert L.mtrt_lua_cuda_get_function(0, b"k", ctypes.byref(out)) == 1
+    assert L.mtrt_lua_cuda_get_function(16, b"", ctypes.byref(out)) == 1
+    assert L.mtrt_lua_cuda_launch(0, 1, 1, 1, 1, 1, 1, 0, 0, 16) == 1
+    assert L.mtrt_lua_cuda_launch(16, 1, 1, 1, 1, 1, 1, 0, 0, 0) == 1
+    assert L.mtrt_lua_cuda_memset(0, 16, 0, 16, 0, 3) == 1
+    assert b"fill width" in L.mtrt_hip_last_error()
+    assert L.mtrt_lua_cuda_memset(0, 16, 1, 16, 0, 4) == 1          # misaligned for a 32-bit pattern
+    assert L.mtrt_lua_cuda_memset(0, 16, 0, 3, 0, 4) == 0           # fewer bytes than one element: nothing to do
+    assert L.mtrt_lua_cuda_memcpy(0, 0, 0, 16, 0, 8) == 1
+    assert L.mtrt_lua_cuda_memcpy(0, 0, 0, 0, 0, 0) == 0
+    dev = ctypes.c_int32(-1)
+    assert L.mtrt_lua_cuda_get_program_device(3, ctypes.byref(dev)) == 7
+    assert b"out of range" in L.mtrt_hip_last_error()
+    assert L.mtrt_lua_cuda_stream_destroy(0) == 1
+
+
+@pytest.mark.gpu
+def test_standalone_launch_known_answer(pkg):
+    print("case: standalone selftest on", pkg.FIXTURE_MODULE_PATH, flush=True)
+    res = subprocess.run([_selftest(pkg), pkg.FIXTURE_MODULE_PATH], capture_output=True, text=True, timeout=100)
+    assert res.returncode == 0, res.stdout + res.stderr
+    assert "standalone selftest ok" in res.stdout
+
+
+@pytest.mark.gpu
+def test_builtin_bodies_known_answers(pkg):
+    """load_module from host bytes -> get_function -> launch with an argument-pointer array; memset, memcpy."""
+    L = pkg.lib()
+    sz = ctypes.c_size_t
+    blob = open(pkg.FIXTURE_MODULE_PATH, "rb").read()
+    buf = ctypes.create_string_buffer(blob, len(blob))
+    mod, fn, stream = sz(0), sz(0), sz(0)
+    dev = ctypes.c_int32(-1)
+    assert L.mtrt_lua_cuda_get_program_device(0, ctypes.byref(dev)) == 0
+    ndev = ctypes.c_int32(0)
+    assert L.mtrt_lua_cuda_num_devices(ctypes.byref(ndev)) == 0 and ndev.value >= 1
+    # PTX text is refused with a status, not an abort
+    ptx = ctypes.create_string_buffer(b".version 7.0\n.target sm_80\n")
+    assert L.mtrt_lua_cuda_load_module(dev.value, ctypes.addressof(ptx), len(ptx), ctypes.byref(mod)) == 1
+    assert b"PTX is not accepted" in L.mtrt_hip_last_error()
+    assert L.mtrt_lua_cuda_load_module(dev.value + 1, ctypes.addressof(buf), len(blob), ctypes.byref(mod)) == 1
+    assert L.mtrt_lua_cuda_load_module(dev.value, ctypes.addressof(buf), len(blob), ctypes.byref(mod)) == 0, \
+        L.mtrt_hip_last_error()
+    assert L.mtrt_lua_cuda_get_function(mod.value, b"missing_kernel", ctypes.byref(fn)) == 4
+    assert L.mtrt_lua_cuda_get_function(mod.value, b"binary_shift_right", ctypes.byref(fn)) == 0 and fn.value
+    assert L.mtrt_lua_cuda_stream_create(ctypes.byref(stream)) == 0 and stream.value
+
+    nbytes = 32 * 4 * 4
+    a, b = sz(0), sz(0)
+    assert L.mtrt_lua_cuda_alloc_device(stream.value, nbytes, ctypes.byref(a)) == 0 and a.value
+    assert L.mtrt_lua_cuda_alloc_device(stream.value, nbytes, ctypes.byref(b)) == 0 and b.value
+    # memset_32 with all ones, memset_8 zero (cuda-launch-kernel.mlir fills -1 and 0)
+    assert L.mtrt_lua_cuda_memset(stream.value, a.value, 0, nbytes, 0xFFFFFFFF, 4) == 0
+    assert L.mtrt_lua_cuda_memset(stream.value, b.value, 0, nbytes, 0, 1) == 0
+    src, shift_i, dst = ctypes.c_void_p(a.value), ctypes.c_int32(7), ctypes.c_void_p(b.value)
+    shift_f = ctypes.c_float(np.array([1], dtype=np.int32).view(np.float32)[0])
+    slots = (src, shift_i, shift_f, dst)
+    argv = (ctypes.c_void_p * 4)(*[ctypes.cast(ctypes.pointer(s), ctypes.c_void_p) for s in slots])
+    assert L.mtrt_lua_cuda_launch(fn.value, 1, 1, 1, 32, 1, 1, 0, stream.value, ctypes.addressof(argv)) == 0
+    host = np.zeros(32 * 4, dtype=np.int32)
+    assert L.mtrt_lua_cuda_memcpy(stream.value, b.value, 0, host.ctypes.data, 0, nbytes) == 0
+    assert L.mtrt_lua_cuda_stream_sync(stream.value) == 0
+    assert np.all(host == 16777215)
+    # 16-bit pattern on the second half only, through the offset argument
+    assert L.mtrt_lua_cuda_memset(stream.value, b.value, nbytes // 2, nbytes // 2, 0xABCD, 2) == 0
+    assert L.mtrt_lua_cuda_memcpy(stream.value, b.value, 0, host.ctypes.data, 0, nbytes) == 0
+    assert L.mtrt_lua_cuda_stream_sync(stream.value) == 0
+    assert np.all(host[:64] == 16777215) and np.all(host[64:].view(np.uint16) == 0xABCD)
+    # a launch shape the device cannot run is a status
+    assert L.mtrt_lua_cuda_launch(fn.value, 1, 1, 1, 4096, 1, 1, 0, stream.value, ctypes.addressof(argv)) == 4
+    assert L.mtrt_lua_cuda_free_device(stream.value, a.value) == 0
+    assert L.mtrt_lua_cuda_free_device(stream.value, b.value) == 0
+    assert L.mtrt_lua_cuda_stream_sync(stream.value) == 0
+    assert L.mtrt_lua_cuda_stream_destroy(stream.value) == 0
