@@ -71,8 +71,11 @@ template <> struct Vec<F16> {
   }
 };
 
-// Load the wave's row into registers: NV vectors per lane, absent vectors zero/fill.
-template <typename X, int NV>
+// Load the wave's row into registers: NV vectors per lane.  Every lane always loads (vectors past
+// the end of the row re-read the row's last vector and are replaced by `fill` afterwards), so the
+// loads are issued back to back with no branches between them; with FULL (the row fills all
+// 64 * NV vectors) the replacement disappears as well.
+template <typename X, int NV, bool FULL>
 __device__ __forceinline__ void load_row(const u32x4* __restrict__ row, int nvec, int lane, float fill,
                                          float (&v)[NV * Vec<X>::kElems]) {
   constexpr int E = Vec<X>::kElems;
@@ -80,47 +83,63 @@ __device__ __forceinline__ void load_row(const u32x4* __restrict__ row, int nvec
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
     const int idx = lane + kWave * j;
-    if (idx < nvec) t[j] = __builtin_nontemporal_load(row + idx);
+    t[j] = __builtin_nontemporal_load(row + (FULL ? idx : min(idx, nvec - 1)));
   }
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
-    const int idx = lane + kWave * j;
-    if (idx < nvec) {
-      Vec<X>::unpack(t[j], &v[j * E]);
-    } else {
+    Vec<X>::unpack(t[j], &v[j * E]);
+    if (!FULL) {
+      const bool live = lane + kWave * j < nvec;
 #pragma unroll
-      for (int k = 0; k < E; ++k) v[j * E + k] = fill;
+      for (int k = 0; k < E; ++k) v[j * E + k] = live ? v[j * E + k] : fill;
     }
   }
 }
 
-template <typename X, int NV>
-__device__ __forceinline__ void layernorm_rows(const typename X::storage* __restrict__ x,
-                                               const typename X::storage* __restrict__ gamma,
-                                               const typename X::storage* __restrict__ beta,
-                                               typename X::storage* __restrict__ y, int64_t rows, int64_t d, float eps) {
+// Hides a vector's provenance from the optimiser (no instruction is emitted).
+__device__ __forceinline__ void opaque(u32x4& t) { __asm__ volatile("" : "+v"(t)); }
+
+// The row stays in registers in its STORAGE form (NV 128-bit vectors per lane) and is widened
+// again in each of the three passes: for 16-bit types that halves the live registers compared
+// with keeping f32 values (a widening is one shift or mask per element), and the higher
+// occupancy it buys is worth more to this memory-bound kernel than the extra VALU work.
+template <typename X, int NV, bool FULL>
+__device__ __forceinline__ void layernorm_row(const typename X::storage* __restrict__ x,
+                                              const typename X::storage* __restrict__ gamma,
+                                              const typename X::storage* __restrict__ beta,
+                                              typename X::storage* __restrict__ y, int64_t row, int64_t d, float eps) {
   constexpr int E = Vec<X>::kElems;
   const int lane = threadIdx.x & (kWave - 1);
-  const int64_t row = int64_t(blockIdx.x) * kRowsPerBlock + threadIdx.x / kWave;
-  if (row >= rows) return;                           // whole wave leaves together
   const int nvec = int(d / E);
   const u32x4* xr = reinterpret_cast<const u32x4*>(x + row * d);
-  float v[NV * E];
-  load_row<X, NV>(xr, nvec, lane, 0.0f, v);
+  u32x4 t[NV];
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int idx = lane + kWave * j;
+    t[j] = __builtin_nontemporal_load(xr + (FULL ? idx : min(idx, nvec - 1)));
+  }
 
   const float fd = float(d);
   float sum = 0.0f;
 #pragma unroll
-  for (int i = 0; i < NV * E; ++i) sum = sum + v[i];
+  for (int j = 0; j < NV; ++j) {
+    const bool live = FULL || lane + kWave * j < nvec;
+    float v[E];
+    Vec<X>::unpack(t[j], v);
+#pragma unroll
+    for (int k = 0; k < E; ++k) sum = sum + (live ? v[k] : 0.0f);
+  }
   const float mu = wave_reduce(sum, SumF32()) / fd;
   float sq = 0.0f;
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
-    const bool live = lane + kWave * j < nvec;
+    const bool live = FULL || lane + kWave * j < nvec;
+    float v[E];
+    opaque(t[j]);                                    // widen again instead of keeping pass 1's values live
+    Vec<X>::unpack(t[j], v);
 #pragma unroll
     for (int k = 0; k < E; ++k) {
-      const float dv = v[j * E + k] - mu;
-      v[j * E + k] = dv;
+      const float dv = v[k] - mu;
       sq = sq + (live ? dv * dv : 0.0f);
     }
   }
@@ -133,28 +152,40 @@ __device__ __forceinline__ void layernorm_rows(const typename X::storage* __rest
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
     const int idx = lane + kWave * j;
-    if (idx < nvec) {
-      float g[E], b[E], o[E];
-      Vec<X>::unpack(gv[idx], g);
-      Vec<X>::unpack(bv[idx], b);
+    const int idc = FULL ? idx : min(idx, nvec - 1);
+    float v[E], g[E], b[E], o[E];
+    opaque(t[j]);
+    Vec<X>::unpack(t[j], v);
+    Vec<X>::unpack(gv[idc], g);
+    Vec<X>::unpack(bv[idc], b);
 #pragma unroll
-      for (int k = 0; k < E; ++k) o[k] = ((v[j * E + k] * rstd) * g[k]) + b[k];
-      __builtin_nontemporal_store(Vec<X>::pack(o), yr + idx);
-    }
+    for (int k = 0; k < E; ++k) o[k] = (((v[k] - mu) * rstd) * g[k]) + b[k];
+    if (FULL || idx < nvec) __builtin_nontemporal_store(Vec<X>::pack(o), yr + idx);
   }
 }
 
 template <typename X, int NV>
-__device__ __forceinline__ void softmax_rows(const typename X::storage* __restrict__ x, typename X::storage* __restrict__ y,
-                                             int64_t rows, int64_t d) {
+__device__ __forceinline__ void layernorm_rows(const typename X::storage* __restrict__ x,
+                                               const typename X::storage* __restrict__ gamma,
+                                               const typename X::storage* __restrict__ beta,
+                                               typename X::storage* __restrict__ y, int64_t rows, int64_t d, float eps) {
+  const int64_t row = int64_t(blockIdx.x) * kRowsPerBlock + threadIdx.x / kWave;
+  if (row >= rows) return;                           // whole wave leaves together
+  if (d == int64_t(Vec<X>::kElems) * kWave * NV)
+    layernorm_row<X, NV, true>(x, gamma, beta, y, row, d, eps);
+  else
+    layernorm_row<X, NV, false>(x, gamma, beta, y, row, d, eps);
+}
+
+template <typename X, int NV, bool FULL>
+__device__ __forceinline__ void softmax_row(const typename X::storage* __restrict__ x, typename X::storage* __restrict__ y,
+                                            int64_t row, int64_t d) {
   constexpr int E = Vec<X>::kElems;
   const int lane = threadIdx.x & (kWave - 1);
-  const int64_t row = int64_t(blockIdx.x) * kRowsPerBlock + threadIdx.x / kWave;
-  if (row >= rows) return;
   const int nvec = int(d / E);
   const u32x4* xr = reinterpret_cast<const u32x4*>(x + row * d);
   float v[NV * E];
-  load_row<X, NV>(xr, nvec, lane, -INFINITY, v);
+  load_row<X, NV, FULL>(xr, nvec, lane, -INFINITY, v);
 
   float mx = -INFINITY;
 #pragma unroll
@@ -175,13 +206,22 @@ __device__ __forceinline__ void softmax_rows(const typename X::storage* __restri
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
     const int idx = lane + kWave * j;
-    if (idx < nvec) {
-      float o[E];
+    float o[E];
 #pragma unroll
-      for (int k = 0; k < E; ++k) o[k] = v[j * E + k] * inv;
-      __builtin_nontemporal_store(Vec<X>::pack(o), yr + idx);
-    }
+    for (int k = 0; k < E; ++k) o[k] = v[j * E + k] * inv;
+    if (FULL || idx < nvec) __builtin_nontemporal_store(Vec<X>::pack(o), yr + idx);
   }
+}
+
+template <typename X, int NV>
+__device__ __forceinline__ void softmax_rows(const typename X::storage* __restrict__ x, typename X::storage* __restrict__ y,
+                                             int64_t rows, int64_t d) {
+  const int64_t row = int64_t(blockIdx.x) * kRowsPerBlock + threadIdx.x / kWave;
+  if (row >= rows) return;
+  if (d == int64_t(Vec<X>::kElems) * kWave * NV)
+    softmax_row<X, NV, true>(x, y, row, d);
+  else
+    softmax_row<X, NV, false>(x, y, row, d);
 }
 
 // ---- any D, any alignment: one workgroup per row, row re-read from cache -------------
