@@ -149,15 +149,15 @@ def build_workloads(pkg, torch, which):
         def q8(shape):
             return torch.clamp(torch.round(torch.randn(shape, generator=g, device=dev) * 40.0), -128, 127).to(torch.int8)
         a4 = [q8((M, K)) for _ in range(ns)]
-        w4 = [pkg.gemm_w8a8_prepack(q8((K, N))) for _ in range(ns)]       # weights are constants: re-laid once, untimed
+        w4 = [pkg.gemm_w8a8_prepack_fragments(q8((K, N))) for _ in range(ns)]   # weights are constants: re-laid once, untimed
         as4 = (torch.rand(M, generator=g, device=dev) * 0.015 + 0.005)
         ws4 = (torch.rand(N, generator=g, device=dev) * 0.015 + 0.005)
         y4 = [torch.empty((M, N), dtype=torch.float16, device=dev) for _ in range(ns)]
 
         def gemm8(i, a4=a4, w4=w4, y4=y4, as4=as4, ws4=ws4, M=M, K=K, N=N):
             a = (a4[i].data_ptr(), w4[i].data_ptr(), as4.data_ptr(), ws4.data_ptr(), y4[i].data_ptr(), M, K, N)
-            return lambda: pkg.check(L.mtrt_hip_gemm_w8a8(stream(), *a))
-        out.append(dict(name="mtrt_gemm_w8a8_nk", config="C4", bound="mfma", work=2.0 * M * K * N, peak=INT8_PEAK,
+            return lambda: pkg.check(L.mtrt_hip_gemm_w8a8_fragments(stream(), *a))
+        out.append(dict(name="mtrt_gemm_w8a8_frag", config="C4", bound="mfma", work=2.0 * M * K * N, peak=INT8_PEAK,
                         unit="TOP/s", nslots=ns, make=gemm8, keep=(a4, w4, y4, as4, ws4),
                         probe=("mtrt_mfma_probe_i8", w4[0], 65536.0)))
 

@@ -212,6 +212,20 @@ MTRT_CAPI_EXPORTED int32_t mtrt_hip_gemm_w8a8(mtrt_stream_t stream, const void *
                                               const float *a_scale, const float *w_scale, void *y,
                                               int64_t M, int64_t K, int64_t N);
 
+/* The same GEMM on the faster kernel that takes the weights from a FRAGMENT-ORDER re-layout straight
+ * into registers (the [N,K] form above goes through LDS and is kept for callers that hold the weights
+ * in that form only).  `w` is the program's [K,N] constant (w_is_nk = 0) or an [N,K] array (w_is_nk = 1);
+ * w_frag holds mtrt_hip_gemm_w8a8_fragments_bytes(K, N) bytes (0 = shape not supported: K % 128 != 0)
+ * and must be 16-byte aligned.  Same results, bit for bit. */
+MTRT_CAPI_EXPORTED int64_t mtrt_hip_gemm_w8a8_fragments_bytes(int64_t K, int64_t N);
+MTRT_CAPI_EXPORTED int32_t mtrt_hip_gemm_w8a8_prepack_fragments(mtrt_stream_t stream, const void *w,
+                                                                int32_t w_is_nk, void *w_frag, int64_t K,
+                                                                int64_t N);
+MTRT_CAPI_EXPORTED int32_t mtrt_hip_gemm_w8a8_fragments(mtrt_stream_t stream, const void *a,
+                                                        const void *w_frag, const float *a_scale,
+                                                        const float *w_scale, void *y, int64_t M, int64_t K,
+                                                        int64_t N);
+
 /* W4A16 block-wise GEMM:
  *   wd[k,n] = f16(f16(w[k,n]) * scale[k / block, n])   ;   y[m,n] = f16(sum_k f32(a[m,k]) * f32(wd[k,n]))
  * (weight-only int4 Linear, linear.py:112-151; block dequantize TensorRTOps.td:3408-3445).

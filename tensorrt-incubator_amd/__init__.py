@@ -79,6 +79,9 @@ PROTOTYPES = {
     "mtrt_hip_softmax": (_i32, [_vp, _vp, _vp, _i32, _i64, _i64]),
     "mtrt_hip_gemm_w8a8_prepack": (_i32, [_vp, _vp, _vp, _i64, _i64]),
     "mtrt_hip_gemm_w8a8": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64]),
+    "mtrt_hip_gemm_w8a8_fragments_bytes": (_i64, [_i64, _i64]),
+    "mtrt_hip_gemm_w8a8_prepack_fragments": (_i32, [_vp, _vp, _i32, _vp, _i64, _i64]),
+    "mtrt_hip_gemm_w8a8_fragments": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64]),
     "mtrt_hip_gemm_w4a16_prepacked_bytes": (_i64, [_i64, _i64]),
     "mtrt_hip_gemm_w4a16_prepack": (_i32, [_vp, _vp, _vp, _i64, _i64]),
     "mtrt_hip_gemm_w4a16": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64]),
@@ -232,6 +235,31 @@ def gemm_w8a8(a, w_nk, a_scale, w_scale, out=None):
     y = torch.empty((M, N), dtype=torch.float16, device=a.device) if out is None else out
     check(lib().mtrt_hip_gemm_w8a8(_stream(), a.data_ptr(), w_nk.data_ptr(), a_scale.data_ptr(), w_scale.data_ptr(),
                                    y.data_ptr(), M, K, N))
+    return y
+
+
+def gemm_w8a8_prepack_fragments(w, is_nk=False):
+    """int8 weights [K,N] (or [N,K] with is_nk) -> fragment-order buffer of the weights-in-registers kernel."""
+    torch = _torch()
+    assert w.is_cuda and w.is_contiguous() and w.dtype == torch.int8 and w.dim() == 2
+    N, K = w.shape if is_nk else (w.shape[1], w.shape[0])
+    nbytes = lib().mtrt_hip_gemm_w8a8_fragments_bytes(K, N)
+    assert nbytes > 0, "fragment order needs K % 128 == 0"
+    wf = torch.empty(nbytes, dtype=torch.int8, device=w.device)
+    check(lib().mtrt_hip_gemm_w8a8_prepack_fragments(_stream(), w.data_ptr(), 1 if is_nk else 0, wf.data_ptr(), K, N))
+    return wf
+
+
+def gemm_w8a8_fragments(a, w_frag, a_scale, w_scale, N, out=None):
+    torch = _torch()
+    assert a.is_cuda and a.is_contiguous() and a.dtype == torch.int8 and w_frag.dtype == torch.int8
+    assert a_scale.dtype == torch.float32 and w_scale.dtype == torch.float32
+    M, K = a.shape
+    assert a_scale.numel() == M and w_scale.numel() == N
+    assert w_frag.numel() == lib().mtrt_hip_gemm_w8a8_fragments_bytes(K, N)
+    y = torch.empty((M, N), dtype=torch.float16, device=a.device) if out is None else out
+    check(lib().mtrt_hip_gemm_w8a8_fragments(_stream(), a.data_ptr(), w_frag.data_ptr(), a_scale.data_ptr(),
+                                             w_scale.data_ptr(), y.data_ptr(), M, K, N))
     return y
 
 

@@ -38,9 +38,11 @@ struct ScaleEpilogue {
   float as;
   __device__ __forceinline__ void setup(int8_t* scratch, int64_t m0, int64_t M, int64_t n0, int64_t N) {
     float* dst = reinterpret_cast<float*>(scratch);
-    const int64_t row = m0 + threadIdx.x, col = n0 + threadIdx.x;   // 256 threads: 256 rows, 256 columns
-    dst[threadIdx.x] = row < M ? a_scale[row] : 0.0f;
-    dst[256 + threadIdx.x] = col < N ? w_scale[col] : 0.0f;
+    const int64_t row = m0 + threadIdx.x, col = n0 + threadIdx.x;   // the first 256 threads: 256 rows, 256 columns
+    if (threadIdx.x < 256) {
+      dst[threadIdx.x] = row < M ? a_scale[row] : 0.0f;
+      dst[256 + threadIdx.x] = col < N ? w_scale[col] : 0.0f;
+    }
     sa = dst;
     sw = dst + 256;
   }
@@ -75,6 +77,184 @@ extern "C" __global__ void __launch_bounds__(gemm_core::THREADS, 1) mtrt_gemm_w8
     const int64_t n_full = full_panels * 256;
     if (!gemm_core::tile_of(blockIdx.x - full_blocks, tiles_m, (N - n_full + 127) / 128, tile_m, panel)) return;
     gemm_core::run<I8Traits, 2>(a, w, K, epi, y, M, N, K / gemm_core::BKB, tile_m * 256, n_full + panel * 128, lds);
+  }
+}
+
+// ---- weights straight into registers ---------------------------------------------------
+// The loop above moves both operands through LDS with two 64 KiB stages, so the loads of a slice
+// are issued only three k-steps before they are needed.  This kernel takes the WEIGHTS from a
+// fragment-order re-layout straight into registers (two register sets, each k-step's registers
+// re-filled seven k-steps before their next use) and leaves LDS to the activations alone: a ring
+// of four 32 KiB stages filled by direct-to-LDS loads two slices ahead.  8 waves (2 x 4, two per
+// SIMD), each 128 rows x 64 columns (JT = 2) or x 32 columns (JT = 1, the half-width tile of a last
+// partial round).
+//
+// What bounds it (measured on one MI355X at M=2048 K=4096 N=11008, counters per launch):
+//   * with every load and LDS read taken out of the loop the launch still needs 164 k cycles per
+//     XCD (ideal for its MFMAs: 98 k), with them 220 k; removing only the LDS reads or only the
+//     barrier changes nothing, removing either operand's loads saves ~13 k, both ~56 k;
+//   * making all workgroups load the same tile (everything L2-resident) changes nothing, making
+//     all lanes of a load hit ONE cache line saves 36 k: the cost is per cache line requested by
+//     the L1, not per byte, instruction or miss further out; the L1 reports "pending request"
+//     stalls for 30 % of the launch (TCP_PENDING_STALL_CYCLES) at 24 B/clk/CU, less than half of
+//     what the same L1 streams (60 B/clk/CU) when nothing else runs;
+//   * the two waves that share a column half load the same weight lines; cacheable (not
+//     nontemporal) weight loads let the second one hit and are 3 % faster.
+// The tile already is as large as the register file allows, so the lines per MFMA cannot drop.
+//
+// Fragment order (mtrt_w8_prepack_frag): for each tile of 32 columns and each slice of 128 k, four
+// 1 KiB blocks, one per k-step p; in a block lane l = 32*h + (n % 32) owns the 16 bytes
+// k = 128*slice + 32*p + 16*h + [0..15] of column n: exactly the B operand of
+// v_mfma_i32_32x32x32_i8 for that k-step, and every load instruction of a wave reads 1 KiB of
+// contiguous memory.  Columns past N hold zeros.
+namespace frag {
+
+constexpr int kThreads = 512, kWaves = 8, kMW = 2, kNWN = 4;
+constexpr int kStageBytes = 256 * 128;                 // one slice of the activation panel
+constexpr int kG = 16 * kMW / kWaves;                  // direct-to-LDS loads per wave and slice
+constexpr int kLds = gemm_core::LDS_BYTES_8WAVES;      // output staging of 8 waves; the ring needs 128 KiB
+
+template <int JT, class Epilogue>
+__device__ __forceinline__ void run(const int8_t* __restrict__ a, int64_t a_row_bytes, const v4i* __restrict__ wfrag,
+                                    int64_t ntiles, Epilogue& epi, uint16_t* __restrict__ y, int64_t M, int64_t N,
+                                    int64_t slices, int64_t m0, int64_t n0, int8_t* lds) {
+  using namespace gemm_core;
+  const int lane = threadIdx.x & 63;
+  const int slot = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = slot / kNWN, wn = slot % kNWN;
+  const int frow = lane & 31, fhalf = lane >> 5;
+
+  v16i acc[4][JT];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < JT; ++j) acc[i][j] = I8Traits::zero();
+
+  const int64_t last = slices - 1;
+  DmaLoaderT<kG> al;
+  al.init(a, M, a_row_bytes, m0);
+  v4i fa0[4], fa1[4];
+  v4i raw[2][JT][4];
+  const v4i* wsrc[JT];                                 // this lane's chunk of slice 0, k-step 0 of each column tile
+#pragma unroll
+  for (int j = 0; j < JT; ++j) {
+    int64_t tile = n0 / 32 + wn * JT + j;
+    tile = tile < ntiles ? tile : ntiles - 1;          // tiles past N: some valid data, never stored
+    wsrc[j] = wfrag + tile * slices * 256 + lane;
+  }
+  auto fetch_one = [&](auto set, int j, int64_t slice, int p) {
+    constexpr int SET = decltype(set)::value;
+    raw[SET][j][p] = wsrc[j][slice * 256 + p * 64];
+  };
+  auto read_a = [&](v4i (&f)[4], const int8_t* pa, int chunk, int i) {
+    f[i] = *reinterpret_cast<const v4i*>(pa + lds_off(wm * 128 + i * 32 + frow, chunk));
+  };
+  auto stage = [&](int64_t slice) { return lds + int(slice & 3) * kStageBytes; };
+
+  const int64_t one = 1 < last ? 1 : last;
+#pragma unroll
+  for (int g = 0; g < kG; ++g) al.dma(0, stage(0), g);
+#pragma unroll
+  for (int g = 0; g < kG; ++g) al.dma(one, stage(1), g);
+#pragma unroll
+  for (int p = 0; p < 4; ++p)
+#pragma unroll
+    for (int j = 0; j < JT; ++j) fetch_one(IntC<0>{}, j, 0, p);
+#pragma unroll
+  for (int p = 0; p < 3; ++p)                          // k-step 3 of slice 1 is fetched in k-step 0 of slice 0
+#pragma unroll
+    for (int j = 0; j < JT; ++j) fetch_one(IntC<1>{}, j, one, p);
+  drain_and_barrier();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) read_a(fa0, stage(0), fhalf, i);
+
+  // k-step T of slice s (parity PAR): four fenced chunks; chunk c multiplies row tile c by the JT
+  // weight fragments of this k-step and carries one A fragment read for the next k-step.  The
+  // memory instructions are spread EVENLY over the k-steps (issued in bursts they queue up in
+  // front of the L1, whose 64 B/clk this loop uses to three quarters, and the waves behind them
+  // stall): each k-step issues one direct-to-LDS load of slice s+2 and JT weight loads into the
+  // registers the PREVIOUS k-step finished with: k-step T >= 1 re-fills k-step T-1's registers
+  // of this parity for slice s+2, k-step 0 re-fills k-step 3's registers of the other parity for
+  // slice s+1.
+  auto kstep = [&](auto par, auto step, const v4i (&cur)[4], v4i (&nxt)[4], const int8_t* ra, int64_t s1, int64_t s2,
+                   int8_t* nd) {
+    constexpr int PAR = decltype(par)::value, T = decltype(step)::value;
+    const int chunk = 2 * ((T + 1) & 3) + fhalf;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+#pragma unroll
+      for (int j = 0; j < JT; ++j) acc[c][j] = I8Traits::mfma(raw[PAR][j][T], cur[c], acc[c][j]);
+      read_a(nxt, ra, chunk, c);
+      if (c == 0) al.dma(s2, nd, T);
+      if (c >= 1 && c - 1 < JT) {
+        if (T == 0) fetch_one(IntC<PAR ^ 1>{}, c - 1, s1, 3);
+        else fetch_one(par, c - 1, s2, T - 1);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  auto slice_body = [&](auto par, int64_t s) {
+    const int8_t* pa = stage(s);
+    const int64_t s1 = s + 1 < last ? s + 1 : last, s2 = s + 2 < last ? s + 2 : last;
+    int8_t* nd = stage(s + 2);
+    kstep(par, IntC<0>{}, fa0, fa1, pa, s1, s2, nd);
+    kstep(par, IntC<1>{}, fa1, fa0, pa, s1, s2, nd);
+    kstep(par, IntC<2>{}, fa0, fa1, pa, s1, s2, nd);
+    // everything issued before this slice has landed (the panel of slice s+1 and its weights for
+    // k-steps 0..2); the 3 + 3 * JT loads of this slice's first three k-steps may still fly
+    __builtin_amdgcn_s_waitcnt(0x0070 | (3 + 3 * JT));   // vmcnt(3 + 3 JT) lgkmcnt(0)
+    __asm__ volatile("s_barrier" ::: "memory");
+    kstep(par, IntC<3>{}, fa1, fa0, stage(s + 1), s1, s2, nd);
+  };
+
+  int64_t s = 0;
+  for (; s + 1 < slices; s += 2) {
+    slice_body(IntC<0>{}, s);
+    slice_body(IntC<1>{}, s + 1);
+  }
+  if (s < slices) slice_body(IntC<0>{}, s);
+  __builtin_amdgcn_s_waitcnt(0x0070);                  // the surplus loads of the last slices have landed
+
+  write_tile<JT, kNWN, kWaves>(acc, epi, y, M, N, m0, n0, lds, slot, true);
+}
+
+}  // namespace frag
+
+// (a [M,K] i8, w_frag (fragment order), a_scale [M] f32, w_scale [N] f32, y [M,N] f16, M, K, N, full_panels) ;
+// K % 128 == 0, a and w_frag 16-byte aligned, a below 4 GiB.  Tiles and grid as mtrt_gemm_w8a8_nk
+// (256 x 256 for the first full_panels * 256 columns, 256 x 128 after), block = 512.
+extern "C" __global__ void __launch_bounds__(frag::kThreads, 1) mtrt_gemm_w8a8_frag(
+    const int8_t* __restrict__ a, const v4i* __restrict__ w_frag, const float* __restrict__ a_scale,
+    const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t full_panels) {
+  __shared__ __attribute__((aligned(16))) int8_t lds[frag::kLds];
+  const int64_t tiles_m = (M + 255) / 256, ntiles = (N + 31) / 32;
+  const int64_t full_blocks = gemm_core::padded_blocks(full_panels, tiles_m);
+  ScaleEpilogue epi{a_scale, w_scale, nullptr, nullptr, 0.0f};
+  int64_t tile_m, panel;
+  if (int64_t(blockIdx.x) < full_blocks) {
+    if (!gemm_core::tile_of(blockIdx.x, tiles_m, full_panels, tile_m, panel)) return;
+    frag::run<2>(a, K, w_frag, ntiles, epi, y, M, N, K / 128, tile_m * 256, panel * 256, lds);
+  } else {
+    const int64_t n_full = full_panels * 256;
+    if (!gemm_core::tile_of(blockIdx.x - full_blocks, tiles_m, (N - n_full + 127) / 128, tile_m, panel)) return;
+    frag::run<1>(a, K, w_frag, ntiles, epi, y, M, N, K / 128, tile_m * 256, n_full + panel * 128, lds);
+  }
+}
+
+// Weight re-layout into fragment order, from [K,N] (nk = 0) or [N,K] (nk = 1).  One 16-byte chunk per
+// thread.  (w, w_frag, K, N, nk) ; K % 128 == 0 ; w_frag holds 32 * ceil(N/32) * K bytes.
+extern "C" __global__ void __launch_bounds__(256) mtrt_w8_prepack_frag(const int8_t* __restrict__ w, v4i* __restrict__ w_frag,
+                                                                     int64_t K, int64_t N, int32_t nk) {
+  const int64_t slices = K / 128, ntiles = (N + 31) / 32;
+  const int64_t total = ntiles * slices * 256;
+  for (int64_t id = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; id < total; id += int64_t(gridDim.x) * blockDim.x) {
+    const int lane = int(id & 63), p = int((id >> 6) & 3);
+    const int64_t slice = (id >> 8) % slices, tile = (id >> 8) / slices;
+    const int64_t n = tile * 32 + (lane & 31), k0 = slice * 128 + 32 * p + 16 * (lane >> 5);
+    union { v4i v; int8_t b[16]; } c;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) c.b[i] = n < N ? (nk ? w[n * K + k0 + i] : w[(k0 + i) * N + n]) : int8_t(0);
+    w_frag[id] = c.v;
   }
 }
 

@@ -301,6 +301,64 @@ int32_t mtrt_hip_gemm_w8a8(mtrt_stream_t stream, const void *a, const void *w_nk
   return launch(st, "mtrt_gemm_w8a8_nk_any", blocks_for(M * N, kBlock), kBlock, as_hip(stream), args);
 }
 
+int64_t mtrt_hip_gemm_w8a8_fragments_bytes(int64_t K, int64_t N) {
+  if (K <= 0 || N <= 0 || K % 128 != 0)
+    return 0;
+  return ((N + 31) / 32) * 32 * K;
+}
+
+int32_t mtrt_hip_gemm_w8a8_prepack_fragments(mtrt_stream_t stream, const void *w, int32_t w_is_nk, void *w_frag,
+                                             int64_t K, int64_t N) {
+  clear_error();
+  if (K <= 0 || N <= 0 || K % 128 != 0)
+    return set_error(MTRT_INVALID_ARGUMENT, "fragment order needs positive extents and K %% 128 == 0, got K=%lld N=%lld",
+                     (long long)K, (long long)N);
+  if (!w || !w_frag)
+    return set_error(MTRT_INVALID_ARGUMENT, "null operand");
+  if (!aligned(w_frag, 16))
+    return set_error(MTRT_INVALID_ARGUMENT, "fragment buffer must be 16-byte aligned");
+  DeviceState *st = device_state();
+  if (!st)
+    return MTRT_RUNTIME_ERROR;
+  const int64_t chunks = mtrt_hip_gemm_w8a8_fragments_bytes(K, N) / 16;
+  void *args[] = {&w, &w_frag, &K, &N, &w_is_nk};
+  return launch(st, "mtrt_w8_prepack_frag", blocks_for(chunks, kBlock), kBlock, as_hip(stream), args);
+}
+
+int32_t mtrt_hip_gemm_w8a8_fragments(mtrt_stream_t stream, const void *a, const void *w_frag, const float *a_scale,
+                                     const float *w_scale, void *y, int64_t M, int64_t K, int64_t N) {
+  clear_error();
+  if (M < 0 || K <= 0 || N < 0 || K % 128 != 0)
+    return set_error(MTRT_INVALID_ARGUMENT, "fragment-order GEMM needs K %% 128 == 0 and non-negative extents, got M=%lld K=%lld N=%lld",
+                     (long long)M, (long long)K, (long long)N);
+  if (M == 0 || N == 0)
+    return MTRT_OK;
+  if (!a || !w_frag || !a_scale || !w_scale || !y)
+    return set_error(MTRT_INVALID_ARGUMENT, "null operand");
+  if (!aligned(y, 2) || !aligned(a, 16) || !aligned(w_frag, 16))
+    return set_error(MTRT_INVALID_ARGUMENT, "a and w_frag must be 16-byte aligned, y 2-byte aligned");
+  if (M * K >= (int64_t(1) << 32))
+    return set_error(MTRT_INVALID_ARGUMENT, "activations of %lld bytes exceed the kernel's 32-bit offsets", (long long)(M * K));
+  DeviceState *st = device_state();
+  if (!st)
+    return MTRT_RUNTIME_ERROR;
+  // Tiles and rounds as in mtrt_hip_gemm_w8a8: 256 x 256, one workgroup per compute unit at a time;
+  // a last round that would use at most half of the units is cut into 128-wide half tiles.
+  const int64_t panels = (N + 255) / 256, tiles_m = (M + 255) / 256, units = num_compute_units(st);
+  const int64_t tiles = panels * tiles_m, rest = tiles % units;
+  int64_t full_panels = panels;
+  if (tiles * 2 <= units)
+    full_panels = 0;
+  else if (rest > 0 && rest * 2 <= units)
+    full_panels = panels - (rest + tiles_m - 1) / tiles_m;
+  const int64_t half_panels = (N - full_panels * 256 + 127) / 128;
+  const int64_t grid = 8 * ((full_panels + 7) / 8) * tiles_m + 8 * ((half_panels + 7) / 8) * tiles_m;
+  if (grid > int64_t(kMaxGrid) * 1024)
+    return set_error(MTRT_INVALID_ARGUMENT, "problem [%lld, %lld] needs too many tiles", (long long)M, (long long)N);
+  void *args[] = {&a, &w_frag, &a_scale, &w_scale, &y, &M, &K, &N, &full_panels};
+  return launch(st, "mtrt_gemm_w8a8_frag", uint32_t(grid), 512, as_hip(stream), args);
+}
+
 int64_t mtrt_hip_gemm_w4a16_prepacked_bytes(int64_t K, int64_t N) {
   if (K <= 0 || N <= 0 || K % 64 != 0)
     return 0;

@@ -47,6 +47,29 @@ def test_w8a8_mfma_kernel_small_shapes(pkg, orc, shape):
     assert np.array_equal(bits16(y).reshape(M, N), orc.gemm_w8a8(a, w, a_s, w_s))
 
 
+def _run_w8a8_frag(pkg, a, w, a_s, w_s, from_nk=False):
+    import torch
+    ad, wd = torch.from_numpy(a).cuda(), torch.from_numpy(w).cuda()
+    wf = pkg.gemm_w8a8_prepack_fragments(wd.t().contiguous(), is_nk=True) if from_nk else pkg.gemm_w8a8_prepack_fragments(wd)
+    y = pkg.gemm_w8a8_fragments(ad, wf, torch.from_numpy(a_s).cuda(), torch.from_numpy(w_s).cuda(), w.shape[1])
+    return y, pkg.last_kernel()
+
+
+@pytest.mark.parametrize("shape", [(256, 128, 128), (512, 512, 256), (300, 256, 200), (1, 128, 1), (37, 384, 129),
+                                   (257, 1024, 130), (700, 256, 8200), (2000, 128, 16416)])
+def test_w8a8_weights_in_registers_kernel(pkg, orc, shape):
+    """Full tiles, half-width tiles of a partial last round, ragged M and N, one slice and many."""
+    M, K, N = shape
+    a, w, a_s, w_s = _w8a8_inputs(rng(M + K + N), M, K, N)
+    print("case: w8a8 fragments", shape, flush=True)
+    y, kernel = _run_w8a8_frag(pkg, a, w, a_s, w_s, from_nk=(M % 2 == 1))
+    assert kernel == "mtrt_gemm_w8a8_frag"
+    orc.set_threads(16)
+    ref = orc.gemm_w8a8(a, w, a_s, w_s)
+    orc.set_threads(1)
+    assert np.array_equal(bits16(y).reshape(M, N), ref)
+
+
 @pytest.mark.parametrize("shape", [(5, 7, 3), (33, 100, 65), (2, 130, 4)])
 def test_w8a8_generic_kernel(pkg, orc, shape):
     M, K, N = shape
@@ -89,6 +112,10 @@ def test_c4_w8a8_full_size(pkg, orc):
     acc = (torch.from_numpy(a).cuda().double() @ torch.from_numpy(w).cuda().double())
     expect = ((acc.float() * torch.from_numpy(a_s).cuda()[:, None]) * torch.from_numpy(w_s).cuda()[None, :]).half()
     assert torch.equal(y, expect)
+    # the weights-in-registers kernel gives the same bits
+    y2, kernel2 = _run_w8a8_frag(pkg, a, w, a_s, w_s)
+    assert kernel2 == "mtrt_gemm_w8a8_frag"
+    assert torch.equal(y2, expect)
 
 
 def test_w8a8_argument_checks(pkg):
