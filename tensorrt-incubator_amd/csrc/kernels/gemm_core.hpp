@@ -282,6 +282,31 @@ __device__ __forceinline__ bool tile_of(int64_t id, int64_t tiles_m, int64_t pan
   tile_m = local % tiles_m;
   return panel < panels;
 }
+// The same, with the M tiles walked in groups of `group` rows of tiles: an XCD's 32 units then
+// work on `group` M tiles x 32/group panels at a time instead of on all M tiles of a few panels.
+// What an XCD's L2 has to fetch per K slice is group x (A panel slice) + 32/group x (B panel
+// slice); the group size that minimises it depends on the bytes per row of the two operands
+// (for 4-bit weights under f16 activations a B slice is a quarter of an A slice, so few M tiles and
+// many panels re-read far less).  group >= tiles_m gives tile_of's order.
+__device__ __forceinline__ bool tile_of_grouped(int64_t id, int64_t tiles_m, int64_t panels, int64_t group, int64_t& tile_m,
+                                                int64_t& panel) {
+  const int64_t xcd = id & 7, local = id >> 3;
+  const int64_t slots = (panels + 7) / 8;                // panel slots of one XCD
+  const int64_t full = tiles_m / group;                  // whole groups; a last group holds the remainder
+  const int64_t per_group = slots * group;
+  int64_t g = local / per_group, r, size;
+  if (g < full) {
+    r = local - g * per_group;
+    size = group;
+  } else {
+    g = full;
+    r = local - full * per_group;
+    size = tiles_m - full * group;
+  }
+  panel = (r / size) * 8 + xcd;
+  tile_m = g * group + r % size;
+  return panel < panels;
+}
 __device__ __forceinline__ bool tile_origin(int64_t M, int64_t N, int64_t& m0, int64_t& n0) {
   int64_t tile_m, panel;
   if (!tile_of(blockIdx.x, (M + BM - 1) / BM, (N + BN - 1) / BN, tile_m, panel)) return false;

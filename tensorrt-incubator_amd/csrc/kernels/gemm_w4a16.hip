@@ -306,7 +306,9 @@ __device__ __forceinline__ void weight_regs_kernel(const uint16_t* __restrict__ 
                                                    const uint16_t* __restrict__ scale, uint16_t* __restrict__ y, int64_t M,
                                                    int64_t K, int64_t N, int64_t block, int8_t* lds) {
   int64_t tile_m, panel;
-  if (!gemm_core::tile_of(blockIdx.x, (M + S::kBM - 1) / S::kBM, (N + S::kBN - 1) / S::kBN, tile_m, panel)) return;
+  // A slice of a 4-bit weight panel is a quarter of the bytes of an activation panel slice of the same
+  // width: groups of four M tiles, eight panels at a time per XCD
+  if (!gemm_core::tile_of_grouped(blockIdx.x, (M + S::kBM - 1) / S::kBM, (N + S::kBN - 1) / S::kBN, 4, tile_m, panel)) return;
   const int64_t m0 = tile_m * S::kBM, n0 = panel * S::kBN;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int slot = wave % S::kSlots;
