@@ -140,6 +140,30 @@ def build_workloads(pkg, torch, which):
         out.append(dict(name="mtrt_qdq_uniform_bf16_f8", config="C3", bound="hbm", work=5.0 * n, nslots=ns, make=qdq,
                         keep=(qs, ys)))
 
+    if which == "nvfp4":
+        # Not a BASELINE config (and not part of "all"): the NVFP4 block quantize / dequantize pair on the
+        # tensor of config 3, for its own roofline line.
+        rows, cols = 16384, 8192
+        n = rows * cols
+        ns = 2
+        xs = [gen((rows, cols), torch.float32, 80 + i, float(np.sqrt(2.0))).to(torch.bfloat16) for i in range(ns)]
+        qs = [torch.empty(n // 2, dtype=torch.uint8, device=dev) for _ in range(ns)]
+        ss = [torch.empty(n // 16, dtype=torch.uint8, device=dev) for _ in range(ns)]
+        ys = [torch.empty_like(x) for x in xs]
+        am = [x.float().abs().max().reshape(1).contiguous() for x in xs]
+
+        def nvq(i, xs=xs, qs=qs, ss=ss, am=am, rows=rows, cols=cols):
+            a = (xs[i].data_ptr(), pkg.BF16, qs[i].data_ptr(), ss[i].data_ptr(), am[i].data_ptr(), rows, cols)
+            return lambda: pkg.check(L.mtrt_hip_nvfp4_quantize(stream(), *a))
+
+        def nvdq(i, qs=qs, ss=ss, am=am, ys=ys, rows=rows, cols=cols):
+            a = (qs[i].data_ptr(), ss[i].data_ptr(), am[i].data_ptr(), ys[i].data_ptr(), pkg.BF16, rows, cols)
+            return lambda: pkg.check(L.mtrt_hip_nvfp4_dequantize(stream(), *a))
+        out.append(dict(name="mtrt_nvfp4_q_bf16", config="NVFP4 (C3 tensor)", bound="hbm", work=(2.0 + 0.5 + 1.0 / 16) * n,
+                        nslots=ns, make=nvq, keep=(xs, qs, ss, am)))
+        out.append(dict(name="mtrt_nvfp4_dq_bf16", config="NVFP4 (C3 tensor)", bound="hbm", work=(2.0 + 0.5 + 1.0 / 16) * n,
+                        nslots=ns, make=nvdq, keep=(ys,)))
+
     if which in ("all", "c4"):
         M, K, N = 2048, 4096, 11008
         ns = slots_for(M * K + K * N + 2 * M * N)
@@ -350,7 +374,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="all", choices=["all", "c1", "c2a", "c2b", "c3", "c4", "c5"])
+    ap.add_argument("--workload", default="all", choices=["all", "c1", "c2a", "c2b", "c3", "c4", "c5", "nvfp4"])
     ap.add_argument("--kernel-reps", type=int, default=100, help="launches per kernel for the per-kernel timing")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()

@@ -189,6 +189,21 @@ MTRT_CAPI_EXPORTED int32_t mtrt_hip_quantize_dequantize(mtrt_stream_t stream, co
                                                         int32_t scale_kind, int64_t d0, int64_t d1,
                                                         int64_t nb, int32_t flags);
 
+/* NVFP4 block quantization, the two-level scaling of tensorrt.dynamic_quantize (TensorRTOps.td:3279-3358;
+ * verifier mlir-tensorrt/tensorrt/lib/TensorRT/IR/Verification.cpp:1271-1290) in the program form of
+ * mlir-tensorrt/integrations/PJRT/test/JAX/test_q_dq_nvfp4.py:21-45: blocks of 16 along the LAST axis
+ * of the [d0, d1] view (d1 % 16 == 0), q = f4E2M1FN codes two per byte (element 2i in the low nibble),
+ * scales = one f8E4M3FN byte per block ([d0, d1/16]), tensor_amax = device pointer to the f32 amax of
+ * the whole tensor (mtrt_hip_amax writes it); the second-level scale of the op is tensor_amax / 2688.
+ * x / y: f32, f16 or bf16, 16-byte aligned; q 16-byte aligned.  The op's other axis choice
+ * (second-last) is not built. */
+MTRT_CAPI_EXPORTED int32_t mtrt_hip_nvfp4_quantize(mtrt_stream_t stream, const void *x, int32_t x_dtype,
+                                                   void *q_packed, void *scales, const float *tensor_amax,
+                                                   int64_t d0, int64_t d1);
+MTRT_CAPI_EXPORTED int32_t mtrt_hip_nvfp4_dequantize(mtrt_stream_t stream, const void *q_packed,
+                                                     const void *scales, const float *tensor_amax, void *y,
+                                                     int32_t y_dtype, int64_t d0, int64_t d1);
+
 /* LayerNorm over the last dimension, one launch
  * (RaiseNormalizations.pdll:277-308; TensorRTOps.td:1303-1373); x, gamma, beta, y share dtype. */
 MTRT_CAPI_EXPORTED int32_t mtrt_hip_layernorm(mtrt_stream_t stream, const void *x, const void *gamma,

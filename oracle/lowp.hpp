@@ -187,4 +187,34 @@ inline int8_t int4_sign_extend(uint8_t nibble) {
   return int8_t((nibble & 0x8) ? (nibble | 0xF0) : (nibble & 0xF));
 }
 
+// f4E2M1FN (values 0, 0.5, 1, 1.5, 2, 3, 4, 6 with a sign bit; no inf, no NaN) from f16, restating
+// the executor's expansion of `truncf f16 -> f4E2M1FN`
+// (mlir-tensorrt/executor/lib/Passes/ExpandOps.cpp:471-694): classification by f16 exponent and
+// mantissa thresholds, which is round-to-nearest-even with saturation to +-6; inf -> +-6, NaN -> 0.
+// kRefHost keeps the expansion's treatment of zero: an f16 that is exactly +-0 gives code 0 (the
+// sign is dropped, :687), while a negative f16 subnormal gives code 8 (-0).  kIeee keeps the sign
+// of zero in both cases (what a hardware conversion does).
+inline uint8_t f16_to_f4e2m1fn(uint16_t h, ConvMode mode) {
+  const uint32_t sign = (h >> 15) & 1u, exp = (h >> 10) & 0x1Fu, mant = h & 0x3FFu;
+  if (exp == 31)
+    return mant ? 0 : uint8_t(sign ? 15 : 7);
+  if (mode == kRefHost && exp == 0 && mant == 0)
+    return 0;
+  uint32_t code;
+  if (exp < 13) code = 0;
+  else if (exp == 13) code = mant == 0 ? 0 : 1;            // 0.25 ties to 0
+  else if (exp == 14) code = mant < 512 ? 1 : 2;           // 0.75 ties to 1.0
+  else if (exp == 15) code = mant <= 256 ? 2 : (mant < 768 ? 3 : 4);
+  else if (exp == 16) code = mant <= 256 ? 4 : (mant < 768 ? 5 : 6);
+  else if (exp == 17) code = mant <= 256 ? 6 : 7;          // 5.0 ties to 4.0
+  else code = 7;
+  return uint8_t(code | (sign << 3));
+}
+// exact widening (ExpandOps.cpp:365-461 goes f4 -> f16; every value is representable)
+inline float f4e2m1fn_to_f32(uint8_t code) {
+  static const float kMag[8] = {0.0f, 0.5f, 1.0f, 1.5f, 2.0f, 3.0f, 4.0f, 6.0f};
+  const float v = kMag[code & 7];
+  return (code & 8) ? -v : v;
+}
+
 } // namespace orc

@@ -90,6 +90,25 @@ void orc_quantize(const void *x, int in_dtype, void *q, int out_dtype, const flo
 void orc_dequantize(const void *q, int in_dtype, void *y, int out_dtype, const float *scale,
                     int scale_kind, int64_t d0, int64_t d1, int64_t nscale_or_block, int mode);
 
+/* f4E2M1FN <-> f16/f32 scalar conversions (mlir-tensorrt/executor/lib/Passes/ExpandOps.cpp:365-694) */
+uint8_t orc_f16_to_f4e2m1fn(uint16_t h, int mode);
+float orc_f4e2m1fn_to_f32(uint8_t code);
+
+/* NVFP4 quantize / dequantize over blocks of 16 along the last axis, as the program of
+ * mlir-tensorrt/integrations/PJRT/test/JAX/test_q_dq_nvfp4.py:21-45 (the two-level scaling of
+ * tensorrt.dynamic_quantize, TensorRTOps.td:3279-3358), every op in f32:
+ *   S_dec_x = max|x_block| / 6 ; S_enc = 2688 / tensor_amax ; s8 = f8e4m3fn(S_dec_x * S_enc)
+ *   S_enc_x = S_enc / f32(s8)  ; q = f4e2m1fn(f16(x * S_enc_x))
+ *   y = narrow(f32(q) * (f32(s8) * (tensor_amax / 2688)))
+ * x: [d0, d1] of in_dtype, d1 % 16 == 0; q: two codes per byte, element 2i in the low nibble;
+ * scales: [d0, d1/16] f8e4m3fn bytes.  Conversions to f4 go through f16 (the only f4 truncation the
+ * reference defines).  TensorRT's own IDynamicQuantize arithmetic is closed: "parity unpinned"
+ * against it; pinned here are the conversions and the op order of the JAX program. */
+void orc_nvfp4_quantize(const void *x, int in_dtype, uint8_t *q_packed, uint8_t *scales, float tensor_amax,
+                        int64_t d0, int64_t d1, int mode);
+void orc_nvfp4_dequantize(const uint8_t *q_packed, const uint8_t *scales, float tensor_amax, void *y,
+                          int out_dtype, int64_t d0, int64_t d1, int mode);
+
 /* LayerNorm over the last dim (RaiseNormalizations.pdll:277-308):
  * mu = sum(xf)/D; d = xf-mu; var = sum(d*d)/D; y = narrow(d * (1/sqrt(var+eps)) * gamma + beta) */
 void orc_layernorm(const void *x, const void *gamma, const void *beta, void *y, int dtype,

@@ -1,0 +1,189 @@
+// NVFP4 block quantize / dequantize for gfx950: the two-level scaling of tensorrt.dynamic_quantize
+// (mlir-tensorrt/tensorrt/include/mlir-tensorrt-dialect/TensorRT/IR/TensorRTOps.td:3279-3358) in the
+// program form of mlir-tensorrt/integrations/PJRT/test/JAX/test_q_dq_nvfp4.py:21-45, blocks of 16
+// along the last axis, every op in f32 and in this order:
+//     S_dec_x = max|x_block| / 6        S_enc = 2688 / tensor_amax
+//     s8      = f8e4m3fn(S_dec_x * S_enc)                  (block scale, stored)
+//     S_enc_x = S_enc / f32(s8)         q = f4e2m1fn(f16(x * S_enc_x))
+//     y       = narrow(f32(q) * (f32(s8) * (tensor_amax / 2688)))
+// Conversions to f4 go through f16, the only f4 truncation the reference defines (RNE, saturation
+// to +-6, inf -> +-6, NaN -> 0: mlir-tensorrt/executor/lib/Passes/ExpandOps.cpp:471-694).  An all-zero
+// block has s8 = 0, S_enc_x = inf and x * S_enc_x = NaN, which that conversion maps to code 0; the
+// same chain is evaluated here, nothing is special-cased.
+//
+// Data movement: as in the quantize/dequantize clusters a lane owns one 128-bit vector of the float
+// operand per trip (4 f32 or 8 f16/bf16), so a block of 16 is held by 4 (or 2) neighbouring lanes
+// and its amax is two (one) cross-lane exchanges; every lane of the block then evaluates the
+// block's scalar chain itself.  A wave handles 8 consecutive trips (8 KiB of the float operand);
+// its codes (1 or 2 KiB) and block scales (128 or 256 B) are parked in the wave's own LDS region
+// and written out as whole cache lines, 16 bytes per lane.
+#include "common.hpp"
+
+namespace nvfp4_cluster {
+
+using namespace mtrt_dev;
+using qdq_cluster::FloatGroup;
+
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef float f2 __attribute__((ext_vector_type(2)));
+
+constexpr int kThreads = 256;
+constexpr int kTrips = 8;
+
+// two f32 -> f16 (RNE) -> two f4E2M1FN codes in the low byte.  The hardware conversion is used for
+// ordinary values; NaN (code 0 by the reference's rule) is patched in by the caller per block.
+__device__ __forceinline__ uint32_t f32x2_to_f4(float a, float b) {
+  // f32_to_f16_bits keeps the product's own f32 rounding in front of the f16 rounding (see common.hpp)
+  union { uint32_t u; h2 h; } c;
+  c.u = f32_to_f16_bits(a) | (f32_to_f16_bits(b) << 16);
+  return __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(0u, c.h, 1.0f, 0) & 0xFFu;
+}
+// the reference's table on one f16 bit pattern (exact, slow): used for blocks that contain NaN
+__device__ __forceinline__ uint32_t f16_bits_to_f4_exact(uint32_t h) {
+  const uint32_t a = h & 0x7FFFu, sign = (h >> 12) & 8u;
+  if (a > 0x7C00u) return 0;
+  const uint32_t code = (a > 0x3400u) + (a >= 0x3A00u) + (a > 0x3D00u) + (a >= 0x3F00u) + (a > 0x4100u) + (a >= 0x4300u) +
+                        (a > 0x4500u);
+  return code | sign;
+}
+
+// (x, q_packed, scales, tensor_amax, nvec) ; nvec 128-bit vectors of x, a multiple of the vectors per block
+template <typename X>
+__device__ __forceinline__ void quantize_body(const typename X::storage* __restrict__ x, uint8_t* __restrict__ q,
+                                              uint8_t* __restrict__ scales, const float* __restrict__ tensor_amax,
+                                              int64_t nvec) {
+  constexpr int G = FloatGroup<X>::G;                  // elements per vector: 4 or 8
+  constexpr int LPB = 16 / G;                          // lanes per block: 4 or 2
+  constexpr int kCodeBytes = G / 2;                    // code bytes per lane and trip
+  constexpr int kSpanCodes = kTrips * 64 * kCodeBytes; // 1 or 2 KiB per wave
+  constexpr int kSpanScales = kTrips * 64 / LPB;       // 128 or 256 B per wave
+  __shared__ __attribute__((aligned(16))) uint8_t lds[(kThreads / 64) * (kSpanCodes + kSpanScales)];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  uint8_t* my_codes = lds + wave * (kSpanCodes + kSpanScales);
+  uint8_t* my_scales = my_codes + kSpanCodes;
+  const int64_t span = (int64_t(blockIdx.x) * (kThreads / 64) + wave) * (kTrips * 64);   // first vector of this wave
+  if (span >= nvec) return;                            // whole wave
+  const float s_enc = 2688.0f / *tensor_amax;
+
+  u32x4 t[kTrips];
+#pragma unroll
+  for (int j = 0; j < kTrips; ++j) {
+    int64_t v = span + j * 64 + lane;
+    v = v < nvec ? v : nvec - 1;                       // past the end: a valid vector, its results are not stored
+    t[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(x) + v);
+  }
+#pragma unroll
+  for (int j = 0; j < kTrips; ++j) {
+    float v[G];
+    FloatGroup<X>::unpack(t[j], v);
+    float amax = 0.0f;
+#pragma unroll
+    for (int k = 0; k < G; ++k) amax = fmaxf(amax, fabsf(v[k]));
+#pragma unroll
+    for (int off = 1; off < LPB; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off, kWave));
+    const float s_dec_x = amax / 6.0f;
+    uint32_t s8 = f32x2_to_f8_ieee(s_dec_x * s_enc, 0.0f) & 0xFFu;
+    s8 = (s8 & 0x7Fu) == 0x7Fu ? 0x7Fu : s8;             // NaN (0 * inf when the tensor amax is 0): 0x7F whatever its sign, as the host class
+    const float s_enc_x = s_enc / f8_to_f32<0>(s8);
+    float w[G];
+#pragma unroll
+    for (int k = 0; k < G; ++k) w[k] = v[k] * s_enc_x;
+    uint32_t codes = 0;
+#pragma unroll
+    for (int k = 0; k < G; k += 2) codes |= f32x2_to_f4(w[k], w[k + 1]) << (4 * k);
+    // s8 of 0 (or NaN) makes S_enc_x infinite (or NaN) and the products of zeros NaN: those blocks
+    // are converted again by the reference's table (a wave-uniform branch that is rarely taken)
+    const bool special = s8 == 0u || s8 == 0x7Fu;
+    if (__builtin_amdgcn_ballot_w64(special) != 0) {
+      uint32_t exact = 0;
+#pragma unroll
+      for (int k = 0; k < G; ++k) exact |= f16_bits_to_f4_exact(f32_to_f16_bits(w[k])) << (4 * k);
+      codes = special ? exact : codes;
+    }
+    if (G == 4) *reinterpret_cast<uint16_t*>(my_codes + (j * 64 + lane) * 2) = uint16_t(codes);
+    else *reinterpret_cast<uint32_t*>(my_codes + (j * 64 + lane) * 4) = codes;
+    if ((lane & (LPB - 1)) == 0) my_scales[(j * 64 + lane) / LPB] = uint8_t(s8);
+  }
+  // this wave's own LDS region only: program order suffices, no barrier
+  const int64_t left = nvec - span;                    // vectors of this span that exist (>= 1)
+  const int64_t code_bytes = (left < kTrips * 64 ? left : kTrips * 64) * kCodeBytes;
+  const int64_t scale_bytes = (left < kTrips * 64 ? left : kTrips * 64) / LPB;
+  uint8_t* qo = q + span * kCodeBytes;
+  uint8_t* so = scales + span / LPB;
+#pragma unroll
+  for (int c = 0; c < kSpanCodes / 1024; ++c) {
+    const int o = (c * 64 + lane) * 16;
+    const u32x4 vv = *reinterpret_cast<const u32x4*>(my_codes + o);
+    if (o + 16 <= code_bytes) {
+      *reinterpret_cast<u32x4*>(qo + o) = vv;            // q is 16-byte aligned (checked by the host side)
+    } else {
+      for (int b = 0; b < 16; b += 2)                    // ragged end: code bytes come in pairs at least
+        if (o + b < code_bytes) *reinterpret_cast<uint16_t*>(qo + o + b) = uint16_t(vv[b >> 2] >> (8 * (b & 3)));
+    }
+  }
+  if (lane * 4 < kSpanScales) {
+    const int o = lane * 4;
+    const uint32_t vv = *reinterpret_cast<const uint32_t*>(my_scales + o);
+    if (o + 4 <= scale_bytes && (reinterpret_cast<uintptr_t>(so) & 3) == 0) {
+      *reinterpret_cast<uint32_t*>(so + o) = vv;
+    } else {
+      for (int b = 0; b < 4; ++b)
+        if (o + b < scale_bytes) so[o + b] = uint8_t(vv >> (8 * b));
+    }
+  }
+}
+
+// (q_packed, scales, tensor_amax, y, nvec) ; nvec 128-bit vectors of y
+template <typename Y>
+__device__ __forceinline__ void dequantize_body(const uint8_t* __restrict__ q, const uint8_t* __restrict__ scales,
+                                                const float* __restrict__ tensor_amax, typename Y::storage* __restrict__ y,
+                                                int64_t nvec) {
+  constexpr int G = FloatGroup<Y>::G;
+  constexpr int LPB = 16 / G;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t span = (int64_t(blockIdx.x) * (kThreads / 64) + wave) * (kTrips * 64);
+  if (span >= nvec) return;
+  const float s_dec = *tensor_amax / 2688.0f;
+  uint32_t codes[kTrips], s8[kTrips];
+#pragma unroll
+  for (int j = 0; j < kTrips; ++j) {
+    int64_t v = span + j * 64 + lane;
+    v = v < nvec ? v : nvec - 1;
+    codes[j] = G == 4 ? uint32_t(*reinterpret_cast<const uint16_t*>(q + v * 2)) : *reinterpret_cast<const uint32_t*>(q + v * 4);
+    s8[j] = scales[v / LPB];
+  }
+#pragma unroll
+  for (int j = 0; j < kTrips; ++j) {
+    const int64_t v = span + j * 64 + lane;
+    const float u = f8_to_f32<0>(s8[j]) * s_dec;
+    float out[G];
+#pragma unroll
+    for (int k = 0; k < G; k += 2) {
+      f2 p;
+      if (k == 0) p = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(codes[j], 1.0f, 0);
+      else if (k == 2) p = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(codes[j], 1.0f, 1);
+      else if (k == 4) p = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(codes[j], 1.0f, 2);
+      else p = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(codes[j], 1.0f, 3);
+      out[k] = p[0] * u;
+      out[k + 1] = p[1] * u;
+    }
+    if (v < nvec) FloatGroup<Y>::store(y + v * G, out);
+  }
+}
+
+}  // namespace nvfp4_cluster
+
+// mtrt_nvfp4_q_<t>(x, q_packed, scales, tensor_amax, nvec) ; mtrt_nvfp4_dq_<t>(q_packed, scales, tensor_amax, y, nvec)
+// grid = ceil(nvec / (4 waves * 8 trips * 64)), block = 256; x / y and q_packed 16-byte aligned.
+#define MTRT_NVFP4_KERNELS(XN, XT)                                                                                      \
+  extern "C" __global__ void __launch_bounds__(nvfp4_cluster::kThreads) mtrt_nvfp4_q_##XN(                               \
+      const XT::storage* x, uint8_t* q, uint8_t* scales, const float* tensor_amax, int64_t nvec) {                      \
+    nvfp4_cluster::quantize_body<XT>(x, q, scales, tensor_amax, nvec);                                                  \
+  }                                                                                                                     \
+  extern "C" __global__ void __launch_bounds__(nvfp4_cluster::kThreads) mtrt_nvfp4_dq_##XN(                              \
+      const uint8_t* q, const uint8_t* scales, const float* tensor_amax, XT::storage* y, int64_t nvec) {                \
+    nvfp4_cluster::dequantize_body<XT>(q, scales, tensor_amax, y, nvec);                                                \
+  }
+MTRT_NVFP4_KERNELS(f32, mtrt_dev::F32)
+MTRT_NVFP4_KERNELS(f16, mtrt_dev::F16)
+MTRT_NVFP4_KERNELS(bf16, mtrt_dev::BF16)

@@ -183,6 +183,49 @@ int32_t mtrt_hip_quantize_dequantize(mtrt_stream_t stream, const void *x, int32_
   return qdq_dispatch(2, as_hip(stream), x, x_dtype, q, q_dtype, y, scale, scale_kind, d0, d1, nb, flags);
 }
 
+namespace {
+int32_t nvfp4_dispatch(bool quantize, hipStream_t stream, const void *xy, int32_t dtype, const void *q, const void *scales,
+                       const float *tensor_amax, int64_t d0, int64_t d1) {
+  clear_error();
+  const char *xn = float_name(dtype);
+  if (!xn)
+    return set_error(MTRT_INVALID_ARGUMENT, "float operand dtype %d is not one of f32/f16/bf16", dtype);
+  if (d0 < 0 || d1 < 0)
+    return set_error(MTRT_INVALID_ARGUMENT, "negative extent [%lld, %lld]", (long long)d0, (long long)d1);
+  if (d1 % 16 != 0)
+    return set_error(MTRT_INVALID_ARGUMENT, "shape(input)[axis] must be divisible by 16, got %lld", (long long)d1);
+  if (d0 == 0 || d1 == 0)
+    return MTRT_OK;
+  if (!xy || !q || !scales || !tensor_amax)
+    return set_error(MTRT_INVALID_ARGUMENT, "null operand");
+  if (!aligned(xy, 16) || !aligned(q, 16) || !aligned(tensor_amax, 4))
+    return set_error(MTRT_INVALID_ARGUMENT, "the float operand and the codes must be 16-byte aligned");
+  DeviceState *st = device_state();
+  if (!st)
+    return MTRT_RUNTIME_ERROR;
+  int64_t nvec = d0 * d1 / (dtype == MTRT_F32 ? 4 : 8);
+  const int64_t blocks = (nvec + 4 * 8 * 64 - 1) / (4 * 8 * 64);   // 4 waves x 8 trips x 64 lanes per workgroup
+  if (blocks > int64_t(kMaxGrid) * 1024)
+    return set_error(MTRT_INVALID_ARGUMENT, "tensor of %lld elements is too large", (long long)(d0 * d1));
+  if (quantize) {
+    void *args[] = {&xy, &q, &scales, &tensor_amax, &nvec};
+    return launch(st, std::string("mtrt_nvfp4_q_") + xn, uint32_t(blocks), kBlock, stream, args);
+  }
+  void *args[] = {&q, &scales, &tensor_amax, &xy, &nvec};
+  return launch(st, std::string("mtrt_nvfp4_dq_") + xn, uint32_t(blocks), kBlock, stream, args);
+}
+} // namespace
+
+int32_t mtrt_hip_nvfp4_quantize(mtrt_stream_t stream, const void *x, int32_t x_dtype, void *q_packed, void *scales,
+                                const float *tensor_amax, int64_t d0, int64_t d1) {
+  return nvfp4_dispatch(true, as_hip(stream), x, x_dtype, q_packed, scales, tensor_amax, d0, d1);
+}
+
+int32_t mtrt_hip_nvfp4_dequantize(mtrt_stream_t stream, const void *q_packed, const void *scales,
+                                  const float *tensor_amax, void *y, int32_t y_dtype, int64_t d0, int64_t d1) {
+  return nvfp4_dispatch(false, as_hip(stream), y, y_dtype, q_packed, scales, tensor_amax, d0, d1);
+}
+
 int32_t mtrt_hip_layernorm(mtrt_stream_t stream, const void *x, const void *gamma, const void *beta, void *y,
                            int32_t dtype, int64_t rows, int64_t d, float eps) {
   clear_error();
