@@ -113,9 +113,13 @@ enum mtrt_hip_dtype {
   MTRT_F8E4M3FN = 4,
   MTRT_I4 = 5,        /* one int4 per byte, low nibble: the executor's host/buffer storage
                          (mlir-tensorrt/executor/lib/Runtime/Backend/Common/DataTypes.cpp:494-519) */
-  MTRT_I4_PACKED = 6  /* two per byte, element 2i in the low nibble: what the reference hands to
+  MTRT_I4_PACKED = 6, /* two per byte, element 2i in the low nibble: what the reference hands to
                          TensorRT (mlir-tensorrt/tensorrt/lib/Target/TensorRTEncodingOpInterface/
                          NetworkEncoder.cpp:552-595) */
+  MTRT_F4_PACKED = 8  /* f4E2M1FN (0, 0.5, 1, 1.5, 2, 3, 4, 6 and a sign), two per byte, element 2i in
+                         the low nibble; the block modes of quantize / dequantize allow it
+                         (TensorRTOps.td:3133-3194).  Converted through f16 as the reference does
+                         (mlir-tensorrt/executor/lib/Passes/ExpandOps.cpp:471-694); 7 is unused */
 };
 
 /* how `scale` is addressed; the data tensor is viewed as row-major [d0, d1] */
@@ -170,7 +174,7 @@ MTRT_CAPI_EXPORTED int32_t mtrt_hip_amax(mtrt_stream_t stream, const void *x, in
 
 /* tensorrt.quantize semantics (TensorRTOps.td:3133-3194) in the StableHLO form
  * of StablehloRaiseQDQ.cpp:233-265: q = convert(clamp(lo, rne(f32(x) / scale), hi)).
- * x_dtype in {F32,F16,BF16}; q_dtype in {I8,F8E4M3FN,I4,I4_PACKED}; scale is f32. */
+ * x_dtype in {F32,F16,BF16}; q_dtype in {I8,F8E4M3FN,I4,I4_PACKED,F4_PACKED}; scale is f32. */
 MTRT_CAPI_EXPORTED int32_t mtrt_hip_quantize(mtrt_stream_t stream, const void *x, int32_t x_dtype,
                                              void *q, int32_t q_dtype, const float *scale,
                                              int32_t scale_kind, int64_t d0, int64_t d1, int64_t nb,

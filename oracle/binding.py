@@ -13,7 +13,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "liboracle.so")
 REF_PATH = os.path.join(HERE, "_ref", "libref_datatypes.so")
 
-F32, F16, BF16, I8, F8E4M3FN, I4, I4_PACKED, I32 = range(8)
+F32, F16, BF16, I8, F8E4M3FN, I4, I4_PACKED, I32, F4_PACKED = range(9)
 IEEE, REFHOST = 0, 1
 SCALE_UNIFORM, SCALE_ROW, SCALE_COL = range(3)
 Q_ROUND_TO_INT = 1
@@ -95,7 +95,7 @@ def ref():
 
 
 _NP_OF = {F32: np.float32, F16: np.uint16, BF16: np.uint16, I8: np.int8, F8E4M3FN: np.uint8, I4: np.uint8,
-          I4_PACKED: np.uint8, I32: np.int32}
+          I4_PACKED: np.uint8, I32: np.int32, F4_PACKED: np.uint8}
 
 
 def _p(a):
@@ -109,7 +109,7 @@ def _c_arr(a, dtype):
 
 
 def storage_count(dtype, n):
-    return (n + 1) // 2 if dtype == I4_PACKED else n
+    return (n + 1) // 2 if dtype in (I4_PACKED, F4_PACKED) else n
 
 
 def narrow(x_f32, dst_dtype, mode=IEEE):

@@ -35,7 +35,8 @@ enum {
   ORC_F8E4M3FN = 4,
   ORC_I4 = 5,        /* one int4 per byte, low nibble (host / executor storage) */
   ORC_I4_PACKED = 6, /* two per byte, element 2i in the low nibble (TensorRT storage) */
-  ORC_I32 = 7
+  ORC_I32 = 7,
+  ORC_F4_PACKED = 8  /* f4E2M1FN, two per byte, element 2i in the low nibble */
 };
 
 /* conversion behaviour, see lowp.hpp */
@@ -82,7 +83,7 @@ float orc_scale_from_amax(float amax, float qmax);
 
 /* q = convert(clamp(lo, [rne](f32(x) / scale), hi))
  *   (StablehloRaiseQDQ.cpp:233-265; TensorRTOps.td:3133-3194)
- * lo/hi follow out_dtype: i8 [-128,127], f8 [-448,448], i4 [-8,7]. */
+ * lo/hi follow out_dtype: i8 [-128,127], f8 [-448,448], i4 [-8,7], f4 [-6,6] (converted through f16). */
 void orc_quantize(const void *x, int in_dtype, void *q, int out_dtype, const float *scale,
                   int scale_kind, int64_t d0, int64_t d1, int64_t nscale_or_block, int flags,
                   int mode);

@@ -44,6 +44,10 @@ inline float load_as_f32(const void *p, int dtype, int64_t i) {
   }
   case ORC_I32:
     return float(static_cast<const int32_t *>(p)[i]);
+  case ORC_F4_PACKED: {
+    const uint8_t byte = static_cast<const uint8_t *>(p)[i >> 1];
+    return f4e2m1fn_to_f32((i & 1) ? (byte >> 4) : (byte & 0xF));
+  }
   }
   std::abort();
 }
@@ -152,6 +156,10 @@ void orc_quantize(const void *x, int in_dtype, void *q, int out_dtype, const flo
   case ORC_I4_PACKED:
     lo = -8.0f, hi = 7.0f;
     break;
+  case ORC_F4_PACKED:
+    lo = -6.0f, hi = 6.0f;
+    round_int = (flags & ORC_Q_ROUND_TO_INT) != 0;
+    break;
   default:
     std::abort();
   }
@@ -178,6 +186,12 @@ void orc_quantize(const void *x, int in_dtype, void *q, int out_dtype, const flo
         // Pairs (2j, 2j+1) of the flattened array share a byte; rows have even
         // length or the caller pads, so the pair is owned by one thread.
         const uint8_t nib = uint8_t(int4_saturate(int(std::trunc(v)))) & 0xF;
+        uint8_t *b = static_cast<uint8_t *>(q) + (i >> 1);
+        *b = (i & 1) ? uint8_t((*b & 0x0F) | (nib << 4)) : uint8_t((*b & 0xF0) | nib);
+        break;
+      }
+      case ORC_F4_PACKED: {
+        const uint8_t nib = f16_to_f4e2m1fn(f32_to_f16(v, m), m);
         uint8_t *b = static_cast<uint8_t *>(q) + (i >> 1);
         *b = (i & 1) ? uint8_t((*b & 0x0F) | (nib << 4)) : uint8_t((*b & 0xF0) | nib);
         break;

@@ -19,6 +19,7 @@ FIXTURE_MODULE_PATH = os.path.join(LIB_DIR, "mtrt_test_fixtures.hsaco")
 
 # enum mtrt_hip_dtype
 F32, F16, BF16, I8, F8E4M3FN, I4, I4_PACKED = range(7)
+F4_PACKED = 8
 # enum mtrt_hip_scale_kind
 SCALE_UNIFORM, SCALE_ROW, SCALE_COL = range(3)
 # enum mtrt_hip_flags
@@ -151,7 +152,7 @@ def code_tensor(q_dtype, numel, device):
     torch = _torch()
     if q_dtype == I8:
         return torch.empty(numel, dtype=torch.int8, device=device)
-    if q_dtype == I4_PACKED:
+    if q_dtype in (I4_PACKED, F4_PACKED):
         return torch.empty((numel + 1) // 2, dtype=torch.uint8, device=device)
     return torch.empty(numel, dtype=torch.uint8, device=device)
 

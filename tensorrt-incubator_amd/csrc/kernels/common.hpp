@@ -22,6 +22,7 @@ struct I8 { using storage = int8_t;    static constexpr int kBits = 8; };
 struct F8 { using storage = uint8_t;   static constexpr int kBits = 8; };
 struct I4 { using storage = uint8_t;   static constexpr int kBits = 8; };  // one per byte, low nibble
 struct I4P { using storage = uint8_t;  static constexpr int kBits = 4; };  // two per byte, even index low
+struct F4P { using storage = uint8_t;  static constexpr int kBits = 4; };  // f4E2M1FN, two per byte, even index low
 
 // flag bits passed by value to the quantize kernels
 constexpr int kFlagRoundToInt = 1;   // round_nearest_even before the clamp (f8 target only; ints always round)

@@ -115,6 +115,24 @@ template <> struct Codes<I4P> {
   static __device__ __forceinline__ float dec(uint32_t c) { return float(int(c << 28) >> 28); }
 };
 
+// f4E2M1FN packed two per byte (element 2i in the low nibble).  The value goes through f16 first,
+// the only f4 truncation the reference defines (RNE, saturation:
+// mlir-tensorrt/executor/lib/Passes/ExpandOps.cpp:471-694); callers clamp to [-6, 6], so no NaN or
+// infinity reaches the hardware conversion.
+typedef _Float16 qdq_h2 __attribute__((ext_vector_type(2)));
+typedef float qdq_f2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t f32x2_to_f4x2(float a, float b) {
+  union { uint32_t u; qdq_h2 h; } c;
+  c.u = f32_to_f16_bits(a) | (f32_to_f16_bits(b) << 16);
+  return __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(0u, c.h, 1.0f, 0) & 0xFFu;
+}
+template <> struct Codes<F4P> {
+  static constexpr float kLo = -6.0f, kHi = 6.0f;
+  static constexpr bool kAlwaysRound = false;
+  static __device__ __forceinline__ uint32_t enc(float v, int) { return f32x2_to_f4x2(v, 0.0f) & 0xFu; }
+  static __device__ __forceinline__ float dec(uint32_t c) { return __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(c & 0xFu, 1.0f, 0)[0]; }
+};
+
 // Four byte-wide codes <-> one 32-bit word.  The f8 IEEE path converts pairs in
 // hardware; everything else goes through enc/dec.
 template <typename Q>
@@ -189,6 +207,34 @@ template <int G> struct CodeGroup<I4P, G> {
   static __device__ __forceinline__ void decode(const uint32_t (&w)[2], float (&v)[G]) {
 #pragma unroll
     for (int k = 0; k < G; ++k) v[k] = float(int(w[0] << (28 - 4 * k)) >> 28);
+  }
+};
+
+template <int G> struct CodeGroup<F4P, G> {
+  static __device__ __forceinline__ void store(uint8_t* base, int64_t e, float (&v)[G], int) {
+    uint32_t w = 0;
+#pragma unroll
+    for (int k = 0; k < G; k += 2) w |= f32x2_to_f4x2(v[k], v[k + 1]) << (4 * k);
+    const uint32_t keep[2] = {w, 0};
+    decode(keep, v);
+    if (G == 4) __builtin_nontemporal_store(uint16_t(w), reinterpret_cast<uint16_t*>(base + (e >> 1)));
+    else __builtin_nontemporal_store(w, reinterpret_cast<uint32_t*>(base + (e >> 1)));
+  }
+  static __device__ __forceinline__ void load_raw(const uint8_t* base, int64_t e, uint32_t (&w)[2]) {
+    if (G == 4) w[0] = __builtin_nontemporal_load(reinterpret_cast<const uint16_t*>(base + (e >> 1)));
+    else w[0] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(base + (e >> 1)));
+  }
+  static __device__ __forceinline__ void decode(const uint32_t (&w)[2], float (&v)[G]) {
+    qdq_f2 p = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[0], 1.0f, 0);
+    v[0] = p[0]; v[1] = p[1];
+    p = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[0], 1.0f, 1);
+    v[2] = p[0]; v[3] = p[1];
+    if (G == 8) {
+      p = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[0], 1.0f, 2);
+      v[4 % G] = p[0]; v[5 % G] = p[1];
+      p = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[0], 1.0f, 3);
+      v[6 % G] = p[0]; v[7 % G] = p[1];
+    }
   }
 };
 
@@ -446,7 +492,8 @@ using namespace qdq_cluster;
   MTRT_QDQ_KERNELS(XN, XT, i8, I8)    \
   MTRT_QDQ_KERNELS(XN, XT, f8, F8)    \
   MTRT_QDQ_KERNELS(XN, XT, i4, I4)    \
-  MTRT_QDQ_KERNELS(XN, XT, i4p, I4P)
+  MTRT_QDQ_KERNELS(XN, XT, i4p, I4P)   \
+  MTRT_QDQ_KERNELS(XN, XT, f4p, F4P)
 
 MTRT_QDQ_FOR_FLOAT(f32, F32)
 MTRT_QDQ_FOR_FLOAT(f16, F16)

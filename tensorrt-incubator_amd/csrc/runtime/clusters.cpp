@@ -33,6 +33,7 @@ const char *code_name(int32_t dt) {
   case MTRT_F8E4M3FN: return "f8";
   case MTRT_I4: return "i4";
   case MTRT_I4_PACKED: return "i4p";
+  case MTRT_F4_PACKED: return "f4p";
   }
   return nullptr;
 }
@@ -91,7 +92,8 @@ int32_t qdq_dispatch(int mode, hipStream_t stream, const void *x, int32_t x_dtyp
   // aligned to the G codes a lane moves at once, and - whenever the scale changes
   // along or across rows - rows that are whole groups.
   const int group = x_dtype == MTRT_F32 ? 4 : 8;
-  const uintptr_t q_align = q_dtype == MTRT_I4_PACKED ? group / 2 : group;
+  const bool nibbles = q_dtype == MTRT_I4_PACKED || q_dtype == MTRT_F4_PACKED;
+  const uintptr_t q_align = nibbles ? group / 2 : group;
   bool tiles = aligned(q, q_align) && (mode == 1 || aligned(x, 16)) && (mode == 0 || aligned(y, 16));
   if (kind != MTRT_SCALE_UNIFORM)
     tiles = tiles && (d1 % group == 0);
@@ -119,7 +121,7 @@ int32_t qdq_dispatch(int mode, hipStream_t stream, const void *x, int32_t x_dtyp
   if (!tiles) args[na++] = &kind_arg;
   if (mode != 1) args[na++] = &flags_arg;
 
-  const int64_t units = tiles ? (n + kTile - 1) / kTile : (q_dtype == MTRT_I4_PACKED ? (n + 1) / 2 : n);
+  const int64_t units = tiles ? (n + kTile - 1) / kTile : (nibbles ? (n + 1) / 2 : n);
   return launch(st, name, blocks_for(units, kBlock), kBlock, stream, args);
 }
 

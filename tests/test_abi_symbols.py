@@ -61,7 +61,7 @@ def test_embedded_code_object_is_gfx950_and_has_the_kernels(pkg):
     for mode in ("q", "dq", "qdq"):
         for kind in ("uniform", "row", "col", "any"):
             for x in ("f32", "f16", "bf16"):
-                for q in ("i8", "f8", "i4", "i4p"):
+                for q in ("i8", "f8", "i4", "i4p", "f4p"):
                     names.append("mtrt_%s_%s_%s_%s" % (mode, kind, x, q))
     for x in ("f32", "f16", "bf16"):
         names.append("mtrt_amax_" + x)

@@ -9,12 +9,12 @@ from helpers import bits16, f32_bits, float_storage, rng, to_device_float, torch
 
 pytestmark = pytest.mark.gpu
 
-QMAX = {"i8": 127.0, "f8": 448.0, "i4": 7.0, "i4p": 7.0}
+QMAX = {"i8": 127.0, "f8": 448.0, "i4": 7.0, "i4p": 7.0, "f4p": 6.0}
 
 
 def _q(pkg, orc, name):
     return {"i8": (pkg.I8, orc.I8), "f8": (pkg.F8E4M3FN, orc.F8E4M3FN), "i4": (pkg.I4, orc.I4),
-            "i4p": (pkg.I4_PACKED, orc.I4_PACKED)}[name]
+            "i4p": (pkg.I4_PACKED, orc.I4_PACKED), "f4p": (pkg.F4_PACKED, orc.F4_PACKED)}[name]
 
 
 def _x(pkg, orc, name):
@@ -120,7 +120,7 @@ def test_c3_dynamic_fp8_full_size(pkg, orc):
 
 
 @pytest.mark.parametrize("xname", ["f32", "f16", "bf16"])
-@pytest.mark.parametrize("qname", ["i8", "f8", "i4", "i4p"])
+@pytest.mark.parametrize("qname", ["i8", "f8", "i4", "i4p", "f4p"])
 @pytest.mark.parametrize("shape", [(64, 1024), (37, 515), (1, 1), (1, 15), (3, 16)])
 def test_per_tensor_all_type_pairs(pkg, orc, xname, qname, shape):
     d0, d1 = shape
@@ -133,7 +133,7 @@ def test_per_tensor_all_type_pairs(pkg, orc, xname, qname, shape):
 
 
 @pytest.mark.parametrize("xname", ["f32", "bf16"])
-@pytest.mark.parametrize("qname", ["i8", "f8", "i4p"])
+@pytest.mark.parametrize("qname", ["i8", "f8", "i4p", "f4p"])
 def test_misaligned_pointers_take_the_any_kernels(pkg, orc, xname, qname):
     d0, d1 = 5, 333
     x = rng(7).standard_normal((d0, d1), dtype=np.float32)
@@ -169,7 +169,7 @@ def test_per_channel(pkg, orc, xname, qname):
 
 
 @pytest.mark.parametrize("xname", ["f32", "f16", "bf16"])
-@pytest.mark.parametrize("qname", ["i4", "i4p"])
+@pytest.mark.parametrize("qname", ["i4", "i4p", "f4p"])
 def test_int4_blockwise(pkg, orc, xname, qname):
     g = rng(13)
     # blocks of 128 rows along axis 0 (the weight layout of config 5: scale [K/128, N])
@@ -197,7 +197,7 @@ def test_ties_saturation_and_special_values(pkg, orc):
     x = np.concatenate([(ks + 0.5) * s, ks * s, (ks + 0.25) * s, np.float32([0.0, -0.0, 1e-40, -1e-40, 3e38, -3e38,
                         np.nextafter(np.float32(0.125), np.float32(1)), np.nextafter(np.float32(0.125), np.float32(0))])])
     x = np.resize(x, (1, 1024)).astype(np.float32)
-    for qname in ("i8", "i4", "i4p", "f8"):
+    for qname in ("i8", "i4", "i4p", "f8", "f4p"):
         _check_all(pkg, orc, x, "f32", qname, pkg.SCALE_UNIFORM, 1, 1024, 1, [s])
     # closed form for the int8 codes: numpy's rint is round-half-even too
     import torch
