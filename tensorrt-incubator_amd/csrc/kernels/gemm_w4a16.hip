@@ -123,14 +123,14 @@ struct PlainEpilogue {
 // dequantisation (8 VALU instructions) for the next k-step, every other chunk an A fragment
 // read, and in k-step 0 one direct-to-LDS load.  Raw nibbles and scales of slice s+2 are
 // fetched in the last k-step of slice s into the register set that k-step 2 finished with.
-template <int JT>
+template <int JT, int D>                               // D register sets = slices fetched ahead
 struct WeightRegs {
   const uint32_t* wp;
   const uint16_t* scale;
   int64_t kblocks, N, tile0;                         // tile0: first 32-column tile of this wave
   uint32_t slices_per_block;
-  u4 raw[2][JT];
-  uint32_t sc_bits[2][JT];
+  u4 raw[D][JT];
+  uint32_t sc_bits[D][JT];
   uint32_t mask = nibble_pair_mask();
   template <int SET>
   __device__ __forceinline__ void fetch(int64_t slice) {
@@ -149,6 +149,10 @@ struct WeightRegs {
   }
   template <int SET, int P>
   __device__ __forceinline__ void half(int j, int part, u4& frag) const {
+    // Keeps all four dwords of the set allocated until here.  A wave that splits a slice with another
+    // uses only two of them; the allocator would hand the other two out as scratch registers right
+    // after the load was issued, and every write to such a register has to wait for the load first.
+    __asm__ volatile("" ::"v"(raw[SET][j]));
     H2Bits t;
     t.u = sc_bits[SET][j] * 0x00010001u;
     dequant4(raw[SET][j][P], t.h, part, mask, frag);
@@ -161,13 +165,17 @@ struct WeightRegs {
 // tile without making the tile smaller.  A wave's own VALU, LDS and memory instructions do not
 // overlap its MFMAs (each takes its issue cycles out of the MFMA stream), only another wave's
 // do, so with the dequantisation in the loop two waves per SIMD are the faster shape.
-template <int MW, int NWN, int JT, int KW>
+// DEPTH: slices fetched ahead (weight register sets, and activation stages in flight); STAGES: activation
+// stages in LDS, at least DEPTH + 1.  A tile with little work per slice needs the deeper ring: its loads
+// must be issued a memory latency (about 2000 cycles under load) ahead, however few MFMA cycles a slice is.
+template <int MW, int NWN, int JT, int KW, int DEPTH = 2, int STAGES = 4>
 struct Shape {
-  static constexpr int kMW = MW, kNWN = NWN, kJT = JT, kKW = KW;
+  static constexpr int kMW = MW, kNWN = NWN, kJT = JT, kKW = KW, kDepth = DEPTH, kStages = STAGES;
+  static_assert(STAGES >= DEPTH + 1, "the stage being filled must not be one that is read");
   static constexpr int kSlots = MW * NWN, kWaves = KW * kSlots;
   static constexpr int kBM = 128 * MW, kBN = 32 * JT * NWN;
   static constexpr int kStageBytes = kBM * 128;        // one slice of the activation panel
-  static constexpr int kRingBytes = 4 * kStageBytes;
+  static constexpr int kRingBytes = STAGES * kStageBytes;
   static constexpr int kOutBytes = kSlots * gemm_core::kOutWave + 2048;
   static constexpr int kSumBytes = KW == 2 ? kSlots * 128 * 32 * JT * 4 : 0;
   static constexpr int kLds = kRingBytes > kOutBytes ? (kRingBytes > kSumBytes ? kRingBytes : kSumBytes)
@@ -175,12 +183,18 @@ struct Shape {
 };
 
 template <class S, int KH, class Epilogue>
-__device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, int64_t a_row_bytes, WeightRegs<S::kJT>& wr,
+__device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, int64_t a_row_bytes,
+                                                WeightRegs<S::kJT, S::kDepth>& wr,
                                                 Epilogue& epi, uint16_t* __restrict__ y, int64_t M, int64_t N, int64_t slices,
                                                 int64_t m0, int64_t n0, int8_t* lds, int slot) {
   using namespace gemm_core;
   constexpr int JT = S::kJT, NWN = S::kNWN, KW = S::kKW, G = (16 * S::kMW) / S::kWaves, NK = 4 / KW;
-  static_assert(G >= 4 && G % 4 == 0 && G <= 15, "direct-to-LDS loads per wave and slice");
+  constexpr int D = S::kDepth, NS = S::kStages;
+  // loads that may still be in flight when slice s+1 must have landed: those of the slices fetched
+  // after it (G direct-to-LDS loads and 2 * JT register loads each) and this slice's own G
+  constexpr int kFly = (D - 2) * (G + 2 * JT) + G;
+  static_assert(kFly < 64, "wait counter range");
+  static_assert((G == 2 || (G >= 4 && G % 4 == 0)) && G <= 15, "direct-to-LDS loads per wave and slice");
   const int lane = threadIdx.x & 63;
   const int wm = slot / NWN;
   const int frow = lane & 31, fhalf = lane >> 5;
@@ -201,14 +215,22 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
   auto read_a = [&](FragSet& f, const int8_t* pa, int chunk, int i) {
     f.a[i] = *reinterpret_cast<const v4i*>(pa + lds_off(wm * 128 + i * 32 + frow, chunk));
   };
-  auto stage = [&](int64_t slice) { return lds + int(slice & 3) * S::kStageBytes; };
+  auto stage = [&](int64_t slice) { return lds + int(uint32_t(slice) % uint32_t(NS)) * S::kStageBytes; };
 
+  auto prefetch = [&](auto d) {
+    constexpr int DD = decltype(d)::value;
+    const int64_t sl = DD < last ? DD : last;
 #pragma unroll
-  for (int g = 0; g < G; ++g) al.dma(0, stage(0), g);
-#pragma unroll
-  for (int g = 0; g < G; ++g) al.dma(1 < last ? 1 : last, stage(1), g);
-  wr.template fetch<0>(0);
-  wr.template fetch<1>(1 < last ? 1 : last);
+    for (int g = 0; g < G; ++g) al.dma(sl, stage(DD), g);
+    wr.template fetch<DD>(sl);
+  };
+  prefetch(IntC<0>{});
+  prefetch(IntC<1>{});
+  if constexpr (D > 2) {
+    prefetch(IntC<2>{});
+    prefetch(IntC<3 % D>{});
+  }
+  static_assert(D == 2 || D == 4, "register sets are named at compile time");
   drain_and_barrier();
 #pragma unroll
   for (int i = 0; i < 4; ++i) read_a(f0, stage(0), 2 * KH + fhalf, i);
@@ -226,7 +248,7 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
   auto kstep = [&](auto par, auto step, const FragSet& cur, FragSet& nxt, const int8_t* ra, int64_t s2, int8_t* nd) {
     constexpr int PAR = decltype(par)::value, T = decltype(step)::value;
     constexpr bool kLast = T == NK - 1;
-    constexpr int NSET = kLast ? (PAR ^ 1) : PAR;      // register set and dword the next k-step's weights come from
+    constexpr int NSET = kLast ? (PAR + 1) % D : PAR;  // register set and dword the next k-step's weights come from
     constexpr int NP = kLast ? KH : KH + (T + 1) * KW;
     const int chunk = 2 * NP + fhalf;
 #pragma unroll
@@ -238,8 +260,12 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
       for (int u = 0; u < 2 * JT; ++u)
         if ((u * 4) / (2 * JT) == c) wr.template half<NSET, NP>(u >> 1, u & 1, nxt.b[u >> 1]);
       if (T == 0) {
+        if constexpr (G >= 4) {
 #pragma unroll
-        for (int g = 0; g < G / 4; ++g) al.dma(s2, nd, c * (G / 4) + g);
+          for (int g = 0; g < G / 4; ++g) al.dma(s2, nd, c * (G / 4) + g);
+        } else {
+          if (c < G) al.dma(s2, nd, c);
+        }
       }
       if (kLast && c == 0) wr.template fetch<PAR>(s2);
       __builtin_amdgcn_sched_barrier(0);
@@ -247,8 +273,8 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
   };
   auto slice_body = [&](auto par, int64_t s) {
     const int8_t* pa = stage(s);
-    const int64_t s2 = s + 2 < last ? s + 2 : last;
-    int8_t* nd = stage(s + 2);
+    const int64_t s2 = s + D < last ? s + D : last;    // the slice fetched during this one
+    int8_t* nd = stage(s + D);
     if (NK == 4) {
       kstep(par, IntC<0>{}, f0, f1, pa, s2, nd);
       kstep(par, IntC<1>{}, f1, f0, pa, s2, nd);
@@ -256,18 +282,26 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
     } else {
       kstep(par, IntC<0>{}, f0, f1, pa, s2, nd);
     }
-    // slice s+1 and the registers of slice s+1 have landed; only this slice's G loads may still fly
-    __builtin_amdgcn_s_waitcnt(0x0070 | G);            // vmcnt(G) lgkmcnt(0)
+    // slice s+1 and the registers of slice s+1 have landed; only younger loads may still fly
+    __builtin_amdgcn_s_waitcnt(0x0070 | (kFly & 15) | ((kFly >> 4) << 14));   // vmcnt(kFly) lgkmcnt(0)
     __asm__ volatile("s_barrier" ::: "memory");
     kstep(par, IntC<NK - 1>{}, f1, f0, stage(s + 1), s2, nd);
   };
 
   int64_t s = 0;
-  for (; s + 1 < slices; s += 2) {
+  for (; s + D - 1 < slices; s += D) {
     slice_body(IntC<0>{}, s);
     slice_body(IntC<1>{}, s + 1);
+    if constexpr (D > 2) {
+      slice_body(IntC<2 % D>{}, s + 2);
+      slice_body(IntC<3 % D>{}, s + 3);
+    }
   }
   if (s < slices) slice_body(IntC<0>{}, s);
+  if (s + 1 < slices) slice_body(IntC<1>{}, s + 1);
+  if constexpr (D > 2) {
+    if (s + 2 < slices) slice_body(IntC<2 % D>{}, s + 2);
+  }
   __builtin_amdgcn_s_waitcnt(0x0070);                  // the surplus loads of the last slices have landed
 
   if (KW == 2) {                                       // second set hands its sums to the first through LDS
@@ -312,7 +346,7 @@ __device__ __forceinline__ void weight_regs_kernel(const uint16_t* __restrict__ 
   const int64_t m0 = tile_m * S::kBM, n0 = panel * S::kBN;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int slot = wave % S::kSlots;
-  WeightRegs<S::kJT> wr;
+  WeightRegs<S::kJT, S::kDepth> wr;
   wr.wp = wp; wr.scale = scale; wr.kblocks = K / BKH; wr.N = N; wr.slices_per_block = uint32_t(block / BKH);
   wr.tile0 = n0 / 32 + (slot % S::kNWN) * S::kJT;
   PlainEpilogue epi;
@@ -332,12 +366,24 @@ extern "C" __global__ void __launch_bounds__(512, 1) mtrt_gemm_w4a16_t256x256(
 }
 // Medium M: 128 x 64 tiles so that the grid still fills the chip, two wave sets splitting each slice.
 // Same argument list.  grid = 8 * ceil(ceil(N/64) / 8) * ceil(M/128), block = 256.
-using MidShape = Shape<1, 2, 1, 2>;                    // 128 x 64, 4 waves
+using MidShape = Shape<1, 2, 1, 2, 4, 5>;              // 128 x 64, 4 waves, four slices ahead (two workgroups share a CU's LDS)
 extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w4a16_t128x64(
     const uint16_t* __restrict__ a, const uint32_t* __restrict__ wp, const uint16_t* __restrict__ scale,
     uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t block) {
   __shared__ __attribute__((aligned(16))) int8_t lds[MidShape::kLds];
   weight_regs_kernel<MidShape>(a, wp, scale, y, M, K, N, block, lds);
+}
+
+// Medium M, wider: 128 x 128 tiles.  What a workgroup moves through its CU's L1 is dominated by the
+// activation panel (16 KiB per slice against 2 KiB of weights per 64 columns), and the L1 is what bounds
+// these launches, so the widest tile that still gives every compute unit a workgroup of its own is the
+// fastest.
+using MidWideShape = Shape<1, 4, 1, 2, 4, 5>;          // 128 x 128, 8 waves (two sets of four), four slices ahead
+extern "C" __global__ void __launch_bounds__(512) mtrt_gemm_w4a16_t128x128(
+    const uint16_t* __restrict__ a, const uint32_t* __restrict__ wp, const uint16_t* __restrict__ scale,
+    uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t block) {
+  __shared__ __attribute__((aligned(16))) int8_t lds[MidWideShape::kLds];
+  weight_regs_kernel<MidWideShape>(a, wp, scale, y, M, K, N, block, lds);
 }
 
 // Small M (<= 32): one workgroup per 32 columns, four waves split K.

@@ -171,7 +171,7 @@ def test_w4a16_small_shapes(pkg, orc, shape):
     B = 128
     a, w, wp, s = _w4a16_inputs(orc, rng(M + K + N), M, K, N, B)
     y, kernel = _run_w4a16(pkg, a, wp, s, K, N, B)
-    assert kernel == ("mtrt_gemm_w4a16_skinny16" if M <= 16 else "mtrt_gemm_w4a16_skinny" if M <= 32 else "mtrt_gemm_w4a16_t128x64")
+    assert kernel == ("mtrt_gemm_w4a16_skinny16" if M <= 16 else "mtrt_gemm_w4a16_skinny" if M <= 32 else "mtrt_gemm_w4a16_t128x128")
     _check_w4a16(orc, y, a, w, s, K, N, B, orc.gemm_w4a16(a, wp, s, K, N, B))
 
 
@@ -207,7 +207,7 @@ def test_c5_w4a16_full_size(pkg, orc, M):
     K, N, B = 4096, 11008, 128
     a, w, wp, s = _w4a16_inputs(orc, rng(5), M, K, N, B)
     y, kernel = _run_w4a16(pkg, a, wp, s, K, N, B)
-    assert kernel == {16: "mtrt_gemm_w4a16_skinny16", 256: "mtrt_gemm_w4a16_t128x64", 4096: "mtrt_gemm_w4a16_t256x256"}[M]
+    assert kernel == {16: "mtrt_gemm_w4a16_skinny16", 256: "mtrt_gemm_w4a16_t128x128", 4096: "mtrt_gemm_w4a16_t256x256"}[M]
     rows = sorted(set([0, M - 1] + list(range(0, M, max(1, M // 38)))))[:40]
     orc.set_threads(16)
     import torch
@@ -215,6 +215,20 @@ def test_c5_w4a16_full_size(pkg, orc, M):
     ref = np.concatenate([orc.gemm_w4a16(a, wp, s, K, N, B, m0=r, mcount=1) for r in rows])
     orc.set_threads(1)
     _check_w4a16(orc, got, a[rows], w, s, K, N, B, ref)
+
+
+def test_w4a16_narrow_mid_tile_kernel(pkg, orc):
+    """128 x 64 tiles: more 128-wide tiles than compute units, too few 256-wide ones for the large kernel
+    (M = 600, N = 8480: 5 x 67 = 335 wide tiles; ragged in M and N), K = 320 (five slices: main loop and tail)."""
+    M, K, N, B = 600, 320, 8480, 64
+    a, w, wp, s = _w4a16_inputs(orc, rng(78), M, K, N, B)
+    y, kernel = _run_w4a16(pkg, a, wp, s, K, N, B)
+    assert kernel == "mtrt_gemm_w4a16_t128x64"
+    rows = sorted(set([0, 1, 127, 128, 255, 256, 511, 512, 598, 599] + list(range(3, M, 41))))
+    orc.set_threads(16)
+    ref = np.concatenate([orc.gemm_w4a16(a, wp, s, K, N, B, m0=r, mcount=1) for r in rows])
+    orc.set_threads(1)
+    _check_w4a16(orc, y[rows].contiguous(), a[rows], w, s, K, N, B, ref)
 
 
 def test_w4a16_big_tile_kernel_ragged_edges(pkg, orc):
