@@ -123,7 +123,8 @@ struct PlainEpilogue {
 // dequantisation (8 VALU instructions) for the next k-step, every other chunk an A fragment
 // read, and in k-step 0 one direct-to-LDS load.  Raw nibbles and scales of slice s+2 are
 // fetched in the last k-step of slice s into the register set that k-step 2 finished with.
-template <int JT, int D>                               // D register sets = slices fetched ahead
+// D register sets = slices fetched ahead; KEEP: the waves use only part of each vector (see half)
+template <int JT, int D, bool KEEP>
 struct WeightRegs {
   const uint32_t* wp;
   const uint16_t* scale;
@@ -152,7 +153,7 @@ struct WeightRegs {
     // Keeps all four dwords of the set allocated until here.  A wave that splits a slice with another
     // uses only two of them; the allocator would hand the other two out as scratch registers right
     // after the load was issued, and every write to such a register has to wait for the load first.
-    __asm__ volatile("" ::"v"(raw[SET][j]));
+    if (KEEP) __asm__ volatile("" ::"v"(raw[SET][j]));
     H2Bits t;
     t.u = sc_bits[SET][j] * 0x00010001u;
     dequant4(raw[SET][j][P], t.h, part, mask, frag);
@@ -184,7 +185,7 @@ struct Shape {
 
 template <class S, int KH, class Epilogue>
 __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, int64_t a_row_bytes,
-                                                WeightRegs<S::kJT, S::kDepth>& wr,
+                                                WeightRegs<S::kJT, S::kDepth, (S::kKW > 1)>& wr,
                                                 Epilogue& epi, uint16_t* __restrict__ y, int64_t M, int64_t N, int64_t slices,
                                                 int64_t m0, int64_t n0, int8_t* lds, int slot) {
   using namespace gemm_core;
@@ -346,7 +347,7 @@ __device__ __forceinline__ void weight_regs_kernel(const uint16_t* __restrict__ 
   const int64_t m0 = tile_m * S::kBM, n0 = panel * S::kBN;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int slot = wave % S::kSlots;
-  WeightRegs<S::kJT, S::kDepth> wr;
+  WeightRegs<S::kJT, S::kDepth, (S::kKW > 1)> wr;
   wr.wp = wp; wr.scale = scale; wr.kblocks = K / BKH; wr.N = N; wr.slices_per_block = uint32_t(block / BKH);
   wr.tile0 = n0 / 32 + (slot % S::kNWN) * S::kJT;
   PlainEpilogue epi;
