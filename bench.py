@@ -153,11 +153,11 @@ def build_workloads(pkg, torch, which):
         am = [x.float().abs().max().reshape(1).contiguous() for x in xs]
 
         def nvq(i, xs=xs, qs=qs, ss=ss, am=am, rows=rows, cols=cols):
-            a = (xs[i].data_ptr(), pkg.BF16, qs[i].data_ptr(), ss[i].data_ptr(), am[i].data_ptr(), rows, cols)
+            a = (xs[i].data_ptr(), pkg.BF16, qs[i].data_ptr(), ss[i].data_ptr(), am[i].data_ptr(), rows, cols, 1)
             return lambda: pkg.check(L.mtrt_hip_nvfp4_quantize(stream(), *a))
 
         def nvdq(i, qs=qs, ss=ss, am=am, ys=ys, rows=rows, cols=cols):
-            a = (qs[i].data_ptr(), ss[i].data_ptr(), am[i].data_ptr(), ys[i].data_ptr(), pkg.BF16, rows, cols)
+            a = (qs[i].data_ptr(), ss[i].data_ptr(), am[i].data_ptr(), ys[i].data_ptr(), pkg.BF16, rows, cols, 1)
             return lambda: pkg.check(L.mtrt_hip_nvfp4_dequantize(stream(), *a))
         out.append(dict(name="mtrt_nvfp4_q_bf16", config="NVFP4 (C3 tensor)", bound="hbm", work=(2.0 + 0.5 + 1.0 / 16) * n,
                         nslots=ns, make=nvq, keep=(xs, qs, ss, am)))

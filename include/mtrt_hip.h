@@ -195,18 +195,20 @@ MTRT_CAPI_EXPORTED int32_t mtrt_hip_quantize_dequantize(mtrt_stream_t stream, co
 
 /* NVFP4 block quantization, the two-level scaling of tensorrt.dynamic_quantize (TensorRTOps.td:3279-3358;
  * verifier mlir-tensorrt/tensorrt/lib/TensorRT/IR/Verification.cpp:1271-1290) in the program form of
- * mlir-tensorrt/integrations/PJRT/test/JAX/test_q_dq_nvfp4.py:21-45: blocks of 16 along the LAST axis
- * of the [d0, d1] view (d1 % 16 == 0), q = f4E2M1FN codes two per byte (element 2i in the low nibble),
- * scales = one f8E4M3FN byte per block ([d0, d1/16]), tensor_amax = device pointer to the f32 amax of
- * the whole tensor (mtrt_hip_amax writes it); the second-level scale of the op is tensor_amax / 2688.
- * x / y: f32, f16 or bf16, 16-byte aligned; q 16-byte aligned.  The op's other axis choice
- * (second-last) is not built. */
+ * mlir-tensorrt/integrations/PJRT/test/JAX/test_q_dq_nvfp4.py:21-45, over the [d0, d1] view of the tensor
+ * (leading axes folded into d0).  block_axis = 1: blocks of 16 along the last axis (d1 % 16 == 0), scales
+ * [d0, d1/16]; block_axis = 0: blocks of 16 along the second-to-last axis (its extent % 16 == 0, d1 % 8 == 0
+ * for f16/bf16 or % 4 for f32), scales [d0/16, d1].  q = f4E2M1FN codes two per byte over the flattened array
+ * (element 2i in the low nibble), scales = one f8E4M3FN byte per block, tensor_amax = device pointer to the
+ * f32 amax of the whole tensor (mtrt_hip_amax writes it); the second-level scale of the op is
+ * tensor_amax / 2688.  x / y: f32, f16 or bf16, 16-byte aligned; q 16-byte aligned; scales 8-byte aligned. */
 MTRT_CAPI_EXPORTED int32_t mtrt_hip_nvfp4_quantize(mtrt_stream_t stream, const void *x, int32_t x_dtype,
                                                    void *q_packed, void *scales, const float *tensor_amax,
-                                                   int64_t d0, int64_t d1);
+                                                   int64_t d0, int64_t d1, int32_t block_axis);
 MTRT_CAPI_EXPORTED int32_t mtrt_hip_nvfp4_dequantize(mtrt_stream_t stream, const void *q_packed,
                                                      const void *scales, const float *tensor_amax, void *y,
-                                                     int32_t y_dtype, int64_t d0, int64_t d1);
+                                                     int32_t y_dtype, int64_t d0, int64_t d1,
+                                                     int32_t block_axis);
 
 /* LayerNorm over the last dimension, one launch
  * (RaiseNormalizations.pdll:277-308; TensorRTOps.td:1303-1373); x, gamma, beta, y share dtype. */

@@ -59,9 +59,9 @@ def lib():
         L.orc_f16_to_f4e2m1fn.restype, L.orc_f16_to_f4e2m1fn.argtypes = _c.c_uint8, [_c.c_uint16, _i32]
         L.orc_f4e2m1fn_to_f32.restype, L.orc_f4e2m1fn_to_f32.argtypes = _f32, [_c.c_uint8]
         L.orc_nvfp4_quantize.restype = None
-        L.orc_nvfp4_quantize.argtypes = [_vp, _i32, _vp, _vp, _f32, _i64, _i64, _i32]
+        L.orc_nvfp4_quantize.argtypes = [_vp, _i32, _vp, _vp, _f32, _i64, _i64, _i32, _i32]
         L.orc_nvfp4_dequantize.restype = None
-        L.orc_nvfp4_dequantize.argtypes = [_vp, _vp, _f32, _vp, _i32, _i64, _i64, _i32]
+        L.orc_nvfp4_dequantize.argtypes = [_vp, _vp, _f32, _vp, _i32, _i64, _i64, _i32, _i32]
         _lib = L
     return _lib
 
@@ -212,19 +212,20 @@ def gemm_w4a16(a_f16_bits, w_packed, scale_f16_bits, K, N, block, m0=0, mcount=N
     return y[m0:m0 + mcount]
 
 
-def nvfp4_quantize(x, in_dtype, tensor_amax, d0, d1, mode=IEEE):
-    """Returns (codes packed two per byte [d0*d1/2], block scales as f8e4m3fn bytes [d0*d1/16])."""
+def nvfp4_quantize(x, in_dtype, tensor_amax, d0, d1, mode=IEEE, block_axis=1):
+    """Returns (codes packed two per byte [d0*d1/2], block scales as f8e4m3fn bytes [d0*d1/16]);
+    block_axis 1: blocks of 16 along d1, 0: along d0."""
     x = _c_arr(x, in_dtype)
-    assert d1 % 16 == 0
+    assert (d1 if block_axis else d0) % 16 == 0 and (d0 * d1) % 2 == 0
     q = np.zeros(d0 * d1 // 2, dtype=np.uint8)
     s = np.zeros(d0 * d1 // 16, dtype=np.uint8)
-    lib().orc_nvfp4_quantize(_p(x), in_dtype, _p(q), _p(s), float(tensor_amax), d0, d1, mode)
+    lib().orc_nvfp4_quantize(_p(x), in_dtype, _p(q), _p(s), float(tensor_amax), d0, d1, block_axis, mode)
     return q, s
 
 
-def nvfp4_dequantize(q, scales, tensor_amax, out_dtype, d0, d1, mode=IEEE):
+def nvfp4_dequantize(q, scales, tensor_amax, out_dtype, d0, d1, mode=IEEE, block_axis=1):
     q = np.ascontiguousarray(q, dtype=np.uint8)
     s = np.ascontiguousarray(scales, dtype=np.uint8)
     y = np.empty(d0 * d1, dtype=_NP_OF[out_dtype])
-    lib().orc_nvfp4_dequantize(_p(q), _p(s), float(tensor_amax), _p(y), out_dtype, d0, d1, mode)
+    lib().orc_nvfp4_dequantize(_p(q), _p(s), float(tensor_amax), _p(y), out_dtype, d0, d1, block_axis, mode)
     return y

@@ -101,14 +101,16 @@ float orc_f4e2m1fn_to_f32(uint8_t code);
  *   S_dec_x = max|x_block| / 6 ; S_enc = 2688 / tensor_amax ; s8 = f8e4m3fn(S_dec_x * S_enc)
  *   S_enc_x = S_enc / f32(s8)  ; q = f4e2m1fn(f16(x * S_enc_x))
  *   y = narrow(f32(q) * (f32(s8) * (tensor_amax / 2688)))
- * x: [d0, d1] of in_dtype, d1 % 16 == 0; q: two codes per byte, element 2i in the low nibble;
- * scales: [d0, d1/16] f8e4m3fn bytes.  Conversions to f4 go through f16 (the only f4 truncation the
+ * x: [d0, d1] of in_dtype; block_axis 1: blocks along d1 (d1 % 16 == 0), scales [d0, d1/16];
+ * block_axis 0: blocks along d0 (d0 % 16 == 0), scales [d0/16, d1] (the op's two axis choices,
+ * mlir-tensorrt/tensorrt/lib/TensorRT/IR/Verification.cpp:1279-1283); q: two codes per byte over the
+ * flattened array, element 2i in the low nibble; scales are f8e4m3fn bytes.  Conversions to f4 go through f16 (the only f4 truncation the
  * reference defines).  TensorRT's own IDynamicQuantize arithmetic is closed: "parity unpinned"
  * against it; pinned here are the conversions and the op order of the JAX program. */
 void orc_nvfp4_quantize(const void *x, int in_dtype, uint8_t *q_packed, uint8_t *scales, float tensor_amax,
-                        int64_t d0, int64_t d1, int mode);
+                        int64_t d0, int64_t d1, int block_axis, int mode);
 void orc_nvfp4_dequantize(const uint8_t *q_packed, const uint8_t *scales, float tensor_amax, void *y,
-                          int out_dtype, int64_t d0, int64_t d1, int mode);
+                          int out_dtype, int64_t d0, int64_t d1, int block_axis, int mode);
 
 /* LayerNorm over the last dim (RaiseNormalizations.pdll:277-308):
  * mu = sum(xf)/D; d = xf-mu; var = sum(d*d)/D; y = narrow(d * (1/sqrt(var+eps)) * gamma + beta) */

@@ -216,48 +216,54 @@ void orc_dequantize(const void *q, int in_dtype, void *y, int out_dtype, const f
 uint8_t orc_f16_to_f4e2m1fn(uint16_t h, int mode) { return f16_to_f4e2m1fn(h, ConvMode(mode)); }
 float orc_f4e2m1fn_to_f32(uint8_t code) { return f4e2m1fn_to_f32(code); }
 
+// block_axis 1: blocks of 16 along the last axis (d1); 0: along the second-to-last axis (d0).
+// Scales are laid out like the input with the blocked extent divided by 16.
 void orc_nvfp4_quantize(const void *x, int in_dtype, uint8_t *q_packed, uint8_t *scales, float tensor_amax,
-                        int64_t d0, int64_t d1, int mode) {
+                        int64_t d0, int64_t d1, int block_axis, int mode) {
   const ConvMode m = ConvMode(mode);
-  const int64_t blocks = d1 / 16;
+  const int64_t nb0 = block_axis ? d0 : d0 / 16, nb1 = block_axis ? d1 / 16 : d1;
+  const int64_t step = block_axis ? 1 : d1;              // element stride inside a block
   const float s_enc = 2688.0f / tensor_amax;             // 6 * 448 / amax, one f32 divide
 #pragma omp parallel for schedule(static)
-  for (int64_t r = 0; r < d0; ++r) {
-    for (int64_t b = 0; b < blocks; ++b) {
-      const int64_t base = r * d1 + b * 16;
+  for (int64_t b0 = 0; b0 < nb0; ++b0) {
+    for (int64_t b1 = 0; b1 < nb1; ++b1) {
+      const int64_t base = block_axis ? b0 * d1 + b1 * 16 : b0 * 16 * d1 + b1;
       float amax = 0.0f;
       for (int i = 0; i < 16; ++i)
-        amax = std::fmax(amax, std::fabs(load_as_f32(x, in_dtype, base + i)));
+        amax = std::fmax(amax, std::fabs(load_as_f32(x, in_dtype, base + i * step)));
       const float s_dec_x = amax / 6.0f;
       const uint8_t s8 = f32_to_f8e4m3fn(s_dec_x * s_enc, m);
-      scales[r * blocks + b] = s8;
+      scales[b0 * nb1 + b1] = s8;
       const float s_enc_x = s_enc / f8e4m3fn_to_f32(s8);
-      for (int i = 0; i < 16; i += 2) {
-        uint8_t c[2];
-        for (int e = 0; e < 2; ++e) {
-          const float v = load_as_f32(x, in_dtype, base + i + e) * s_enc_x;
-          c[e] = f16_to_f4e2m1fn(f32_to_f16(v, m), m);
+      for (int i = 0; i < 16; ++i) {
+        const int64_t e = base + i * step;
+        const float v = load_as_f32(x, in_dtype, e) * s_enc_x;
+        const uint8_t c = f16_to_f4e2m1fn(f32_to_f16(v, m), m);
+        uint8_t *byte = q_packed + (e >> 1);             // neighbours along d1 share a byte
+        if (block_axis) {
+          *byte = (e & 1) ? uint8_t((*byte & 0x0F) | (c << 4)) : uint8_t((*byte & 0xF0) | c);
+        } else {
+#pragma omp critical(nvfp4_nibble)
+          *byte = (e & 1) ? uint8_t((*byte & 0x0F) | (c << 4)) : uint8_t((*byte & 0xF0) | c);
         }
-        q_packed[(base + i) / 2] = uint8_t(c[0] | (c[1] << 4));
       }
     }
   }
 }
 
 void orc_nvfp4_dequantize(const uint8_t *q_packed, const uint8_t *scales, float tensor_amax, void *y,
-                          int out_dtype, int64_t d0, int64_t d1, int mode) {
+                          int out_dtype, int64_t d0, int64_t d1, int block_axis, int mode) {
   const ConvMode m = ConvMode(mode);
-  const int64_t blocks = d1 / 16;
+  const int64_t nb1 = block_axis ? d1 / 16 : d1;
   const float s_dec = tensor_amax / 2688.0f;
 #pragma omp parallel for schedule(static)
   for (int64_t r = 0; r < d0; ++r) {
-    for (int64_t b = 0; b < blocks; ++b) {
-      const float u = f8e4m3fn_to_f32(scales[r * blocks + b]) * s_dec;
-      for (int i = 0; i < 16; ++i) {
-        const int64_t e = r * d1 + b * 16 + i;
-        const uint8_t code = (q_packed[e / 2] >> (4 * (e & 1))) & 0xF;
-        store_float(y, out_dtype, e, f4e2m1fn_to_f32(code) * u, m);
-      }
+    for (int64_t c = 0; c < d1; ++c) {
+      const int64_t e = r * d1 + c;
+      const int64_t si = block_axis ? r * nb1 + c / 16 : (r / 16) * nb1 + c;
+      const float u = f8e4m3fn_to_f32(scales[si]) * s_dec;
+      const uint8_t code = (q_packed[e / 2] >> (4 * (e & 1))) & 0xF;
+      store_float(y, out_dtype, e, f4e2m1fn_to_f32(code) * u, m);
     }
   }
 }

@@ -76,8 +76,8 @@ PROTOTYPES = {
     "mtrt_hip_quantize": (_i32, [_vp, _vp, _i32, _vp, _i32, _vp, _i32, _i64, _i64, _i64, _i32]),
     "mtrt_hip_dequantize": (_i32, [_vp, _vp, _i32, _vp, _i32, _vp, _i32, _i64, _i64, _i64]),
     "mtrt_hip_quantize_dequantize": (_i32, [_vp, _vp, _i32, _vp, _i32, _vp, _vp, _i32, _i64, _i64, _i64, _i32]),
-    "mtrt_hip_nvfp4_quantize": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _i64, _i64]),
-    "mtrt_hip_nvfp4_dequantize": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i64, _i64]),
+    "mtrt_hip_nvfp4_quantize": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _i64, _i64, _i32]),
+    "mtrt_hip_nvfp4_dequantize": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i64, _i64, _i32]),
     "mtrt_hip_layernorm": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i64, _i64, _f32]),
     "mtrt_hip_softmax": (_i32, [_vp, _vp, _vp, _i32, _i64, _i64]),
     "mtrt_hip_gemm_w8a8_prepack": (_i32, [_vp, _vp, _vp, _i64, _i64]),
@@ -197,28 +197,33 @@ def quantize_dequantize(x, scale, q_dtype, kind=SCALE_UNIFORM, d0=None, d1=None,
     return q, y
 
 
-def nvfp4_quantize(x, tensor_amax):
-    """NVFP4 codes (uint8, two per byte) and block scales (uint8 f8e4m3fn bytes, shape [..., d1/16]) of `x`,
-    blocks of 16 along the last axis; `tensor_amax` is a 0-d f32 device tensor (what amax() returns)."""
+def nvfp4_quantize(x, tensor_amax, axis=-1):
+    """NVFP4 codes (uint8, two per byte) and block scales (uint8 f8e4m3fn bytes, the shape of `x` with the blocked
+    extent divided by 16) of `x`, blocks of 16 along `axis` (-1 or -2); `tensor_amax` is a 0-d f32 device
+    tensor (what amax() returns)."""
     torch = _torch()
     assert x.is_cuda and x.is_contiguous() and tensor_amax.is_cuda and tensor_amax.dtype == torch.float32
+    assert axis in (-1, -2, x.dim() - 1, x.dim() - 2)
+    last = axis in (-1, x.dim() - 1)
     d1 = x.shape[-1]
     d0 = x.numel() // d1 if d1 else 0
     q = torch.empty(x.numel() // 2, dtype=torch.uint8, device=x.device)
-    s = torch.empty(x.shape[:-1] + (d1 // 16,), dtype=torch.uint8, device=x.device)
+    sshape = x.shape[:-1] + (d1 // 16,) if last else x.shape[:-2] + (x.shape[-2] // 16, d1)
+    s = torch.empty(sshape, dtype=torch.uint8, device=x.device)
     check(lib().mtrt_hip_nvfp4_quantize(_stream(), x.data_ptr(), float_dtype_of(x), q.data_ptr(), s.data_ptr(),
-                                        tensor_amax.data_ptr(), d0, d1))
+                                        tensor_amax.data_ptr(), d0, d1, 1 if last else 0))
     return q, s
 
 
-def nvfp4_dequantize(q, scales, tensor_amax, out_torch_dtype, shape):
+def nvfp4_dequantize(q, scales, tensor_amax, out_torch_dtype, shape, axis=-1):
     torch = _torch()
     assert q.is_cuda and q.dtype == torch.uint8 and scales.dtype == torch.uint8 and tensor_amax.dtype == torch.float32
     y = torch.empty(shape, dtype=out_torch_dtype, device=q.device)
+    last = axis in (-1, y.dim() - 1)
     d1 = y.shape[-1]
     d0 = y.numel() // d1 if d1 else 0
     check(lib().mtrt_hip_nvfp4_dequantize(_stream(), q.data_ptr(), scales.data_ptr(), tensor_amax.data_ptr(),
-                                          y.data_ptr(), float_dtype_of(y), d0, d1))
+                                          y.data_ptr(), float_dtype_of(y), d0, d1, 1 if last else 0))
     return y
 
 

@@ -1,7 +1,7 @@
 // NVFP4 block quantize / dequantize for gfx950: the two-level scaling of tensorrt.dynamic_quantize
 // (mlir-tensorrt/tensorrt/include/mlir-tensorrt-dialect/TensorRT/IR/TensorRTOps.td:3279-3358) in the
 // program form of mlir-tensorrt/integrations/PJRT/test/JAX/test_q_dq_nvfp4.py:21-45, blocks of 16
-// along the last axis, every op in f32 and in this order:
+// along the last axis (or, in the *_cols kernels at the end, the second-to-last), every op in f32 and in this order:
 //     S_dec_x = max|x_block| / 6        S_enc = 2688 / tensor_amax
 //     s8      = f8e4m3fn(S_dec_x * S_enc)                  (block scale, stored)
 //     S_enc_x = S_enc / f32(s8)         q = f4e2m1fn(f16(x * S_enc_x))
@@ -171,6 +171,116 @@ __device__ __forceinline__ void dequantize_body(const uint8_t* __restrict__ q, c
   }
 }
 
+// ---- blocks of 16 along the SECOND-TO-LAST axis ([d0, d1] view, d0 % 16 == 0) ----------------------
+// A lane owns G neighbouring columns of one block row: 16 vectors, one per row, a row's 64 vectors
+// of a wave being 1 KiB of contiguous memory.  The block amax is a maximum down the lane's own
+// registers, one chain per column.  Per row a wave stores 64 x G/2 bytes of codes and per block row
+// 64 x G scale bytes, each contiguous.
+// (x, q_packed, scales, tensor_amax, d0, d1) ; d1 % G == 0 ; one lane per (block row, column group)
+template <typename X>
+__device__ __forceinline__ void quantize_cols_body(const typename X::storage* __restrict__ x, uint8_t* __restrict__ q,
+                                                   uint8_t* __restrict__ scales, const float* __restrict__ tensor_amax,
+                                                   int64_t d0, int64_t d1) {
+  constexpr int G = FloatGroup<X>::G;
+  const int64_t groups = d1 / G, units = (d0 / 16) * groups;
+  const int64_t u = int64_t(blockIdx.x) * kThreads + threadIdx.x;
+  if (u >= units) return;
+  const int64_t rb = u / groups, c0 = (u - rb * groups) * G;
+  const float s_enc = 2688.0f / *tensor_amax;
+  const typename X::storage* xp = x + rb * 16 * d1 + c0;
+  u32x4 t[16];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) t[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xp + r * d1));
+  float amax[G];
+#pragma unroll
+  for (int k = 0; k < G; ++k) amax[k] = 0.0f;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    float v[G];
+    FloatGroup<X>::unpack(t[r], v);
+#pragma unroll
+    for (int k = 0; k < G; ++k) amax[k] = fmaxf(amax[k], fabsf(v[k]));
+  }
+  float s_enc_x[G];
+  uint32_t s8[G];
+  bool special = false;
+#pragma unroll
+  for (int k = 0; k < G; ++k) {
+    const float s_dec_x = amax[k] / 6.0f;
+    uint32_t b = f32x2_to_f8_ieee(s_dec_x * s_enc, 0.0f) & 0xFFu;
+    b = (b & 0x7Fu) == 0x7Fu ? 0x7Fu : b;
+    s8[k] = b;
+    special = special || b == 0u || b == 0x7Fu;
+    s_enc_x[k] = s_enc / f8_to_f32<0>(b);
+  }
+  uint8_t* sp = scales + rb * d1 + c0;
+  if (G == 4) {
+    *reinterpret_cast<uint32_t*>(sp) = s8[0] | (s8[1] << 8) | (s8[2] << 16) | (s8[3] << 24);
+  } else {
+    u32x2 w = {s8[0] | (s8[1] << 8) | (s8[2] << 16) | (s8[3] << 24),
+               s8[4 % G] | (s8[5 % G] << 8) | (s8[6 % G] << 16) | (s8[7 % G] << 24)};
+    *reinterpret_cast<u32x2*>(sp) = w;
+  }
+  const bool any_special = __builtin_amdgcn_ballot_w64(special) != 0;
+  uint8_t* qp = q + (rb * 16 * d1 + c0) / 2;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    float v[G], w[G];
+    FloatGroup<X>::unpack(t[r], v);
+#pragma unroll
+    for (int k = 0; k < G; ++k) w[k] = v[k] * s_enc_x[k];
+    uint32_t codes = 0;
+#pragma unroll
+    for (int k = 0; k < G; k += 2) codes |= f32x2_to_f4(w[k], w[k + 1]) << (4 * k);
+    if (any_special) {                                 // columns whose scale byte is 0 or NaN: the exact table
+      uint32_t exact = 0;
+#pragma unroll
+      for (int k = 0; k < G; ++k) {
+        const bool sk = s8[k] == 0u || s8[k] == 0x7Fu;
+        const uint32_t e = f16_bits_to_f4_exact(f32_to_f16_bits(w[k]));
+        exact |= (sk ? e : ((codes >> (4 * k)) & 0xFu)) << (4 * k);
+      }
+      codes = exact;
+    }
+    if (G == 4) *reinterpret_cast<uint16_t*>(qp + r * (d1 / 2)) = uint16_t(codes);
+    else *reinterpret_cast<uint32_t*>(qp + r * (d1 / 2)) = codes;
+  }
+}
+
+// (q_packed, scales, tensor_amax, y, d0, d1) ; one lane per output vector
+template <typename Y>
+__device__ __forceinline__ void dequantize_cols_body(const uint8_t* __restrict__ q, const uint8_t* __restrict__ scales,
+                                                     const float* __restrict__ tensor_amax,
+                                                     typename Y::storage* __restrict__ y, int64_t d0, int64_t d1) {
+  constexpr int G = FloatGroup<Y>::G;
+  const int64_t groups = d1 / G, nvec = d0 * groups;
+  const float s_dec = *tensor_amax / 2688.0f;
+  const int64_t stride = int64_t(gridDim.x) * kThreads;
+  for (int64_t v = int64_t(blockIdx.x) * kThreads + threadIdx.x; v < nvec; v += stride) {
+    const int64_t r = v / groups, c0 = (v - r * groups) * G;
+    const uint32_t codes = G == 4 ? uint32_t(*reinterpret_cast<const uint16_t*>(q + v * 2)) : *reinterpret_cast<const uint32_t*>(q + v * 4);
+    const uint8_t* sp = scales + (r / 16) * d1 + c0;
+    uint32_t sw[2];
+    sw[0] = *reinterpret_cast<const uint32_t*>(sp);
+    sw[1] = G == 8 ? *reinterpret_cast<const uint32_t*>(sp + 4) : 0u;
+    float out[G];
+#pragma unroll
+    for (int k = 0; k < G; k += 2) {
+      f2 p;
+      if (k == 0) p = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(codes, 1.0f, 0);
+      else if (k == 2) p = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(codes, 1.0f, 1);
+      else if (k == 4) p = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(codes, 1.0f, 2);
+      else p = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(codes, 1.0f, 3);
+      const uint32_t word = sw[k / 4];
+      const float u0 = ((k & 3) == 0 ? f8_to_f32<0>(word) : f8_to_f32<2>(word)) * s_dec;
+      const float u1 = ((k & 3) == 0 ? f8_to_f32<1>(word) : f8_to_f32<3>(word)) * s_dec;
+      out[k] = p[0] * u0;
+      out[k + 1] = p[1] * u1;
+    }
+    FloatGroup<Y>::store(y + v * G, out);
+  }
+}
+
 }  // namespace nvfp4_cluster
 
 // mtrt_nvfp4_q_<t>(x, q_packed, scales, tensor_amax, nvec) ; mtrt_nvfp4_dq_<t>(q_packed, scales, tensor_amax, y, nvec)
@@ -184,6 +294,21 @@ __device__ __forceinline__ void dequantize_body(const uint8_t* __restrict__ q, c
       const uint8_t* q, const uint8_t* scales, const float* tensor_amax, XT::storage* y, int64_t nvec) {                \
     nvfp4_cluster::dequantize_body<XT>(q, scales, tensor_amax, y, nvec);                                                \
   }
+// Blocks along the second-to-last axis: mtrt_nvfp4_qc_<t>(x, q_packed, scales, tensor_amax, d0, d1) with
+// grid = ceil((d0 / 16) * (d1 / G) / 256); mtrt_nvfp4_dqc_<t>(q_packed, scales, tensor_amax, y, d0, d1).
+// d1 % G == 0 (G = 4 for f32, 8 for f16 / bf16), x / y rows 16-byte aligned, scales 4- (G = 4) or 8-byte aligned.
+#define MTRT_NVFP4_COL_KERNELS(XN, XT)                                                                                  \
+  extern "C" __global__ void __launch_bounds__(nvfp4_cluster::kThreads) mtrt_nvfp4_qc_##XN(                              \
+      const XT::storage* x, uint8_t* q, uint8_t* scales, const float* tensor_amax, int64_t d0, int64_t d1) {            \
+    nvfp4_cluster::quantize_cols_body<XT>(x, q, scales, tensor_amax, d0, d1);                                           \
+  }                                                                                                                     \
+  extern "C" __global__ void __launch_bounds__(nvfp4_cluster::kThreads) mtrt_nvfp4_dqc_##XN(                             \
+      const uint8_t* q, const uint8_t* scales, const float* tensor_amax, XT::storage* y, int64_t d0, int64_t d1) {      \
+    nvfp4_cluster::dequantize_cols_body<XT>(q, scales, tensor_amax, y, d0, d1);                                         \
+  }
+MTRT_NVFP4_COL_KERNELS(f32, mtrt_dev::F32)
+MTRT_NVFP4_COL_KERNELS(f16, mtrt_dev::F16)
+MTRT_NVFP4_COL_KERNELS(bf16, mtrt_dev::BF16)
 MTRT_NVFP4_KERNELS(f32, mtrt_dev::F32)
 MTRT_NVFP4_KERNELS(f16, mtrt_dev::F16)
 MTRT_NVFP4_KERNELS(bf16, mtrt_dev::BF16)

@@ -187,25 +187,45 @@ int32_t mtrt_hip_quantize_dequantize(mtrt_stream_t stream, const void *x, int32_
 
 namespace {
 int32_t nvfp4_dispatch(bool quantize, hipStream_t stream, const void *xy, int32_t dtype, const void *q, const void *scales,
-                       const float *tensor_amax, int64_t d0, int64_t d1) {
+                       const float *tensor_amax, int64_t d0, int64_t d1, int32_t block_axis) {
   clear_error();
   const char *xn = float_name(dtype);
   if (!xn)
     return set_error(MTRT_INVALID_ARGUMENT, "float operand dtype %d is not one of f32/f16/bf16", dtype);
   if (d0 < 0 || d1 < 0)
     return set_error(MTRT_INVALID_ARGUMENT, "negative extent [%lld, %lld]", (long long)d0, (long long)d1);
-  if (d1 % 16 != 0)
-    return set_error(MTRT_INVALID_ARGUMENT, "shape(input)[axis] must be divisible by 16, got %lld", (long long)d1);
+  if (block_axis != 0 && block_axis != 1)
+    return set_error(MTRT_INVALID_ARGUMENT, "invalid axis! Axis can be either last (1) or second last (0) dimension of the [d0, d1] view, got %d",
+                     block_axis);
+  const int64_t blocked = block_axis ? d1 : d0;
+  if (blocked % 16 != 0)
+    return set_error(MTRT_INVALID_ARGUMENT, "shape(input)[axis] must be divisible by 16, got %lld", (long long)blocked);
   if (d0 == 0 || d1 == 0)
     return MTRT_OK;
   if (!xy || !q || !scales || !tensor_amax)
     return set_error(MTRT_INVALID_ARGUMENT, "null operand");
-  if (!aligned(xy, 16) || !aligned(q, 16) || !aligned(tensor_amax, 4))
-    return set_error(MTRT_INVALID_ARGUMENT, "the float operand and the codes must be 16-byte aligned");
+  if (!aligned(xy, 16) || !aligned(q, 16) || !aligned(tensor_amax, 4) || !aligned(scales, 8))
+    return set_error(MTRT_INVALID_ARGUMENT, "the float operand and the codes must be 16-byte aligned, the scales 8-byte aligned");
   DeviceState *st = device_state();
   if (!st)
     return MTRT_RUNTIME_ERROR;
-  int64_t nvec = d0 * d1 / (dtype == MTRT_F32 ? 4 : 8);
+  const int group = dtype == MTRT_F32 ? 4 : 8;
+  if (block_axis == 0) {
+    if (d1 % group != 0)
+      return set_error(MTRT_INVALID_ARGUMENT, "blocks along the second-to-last axis need the last extent %% %d == 0, got %lld",
+                       group, (long long)d1);
+    const int64_t units = quantize ? (d0 / 16) * (d1 / group) : d0 * (d1 / group);
+    if ((units + kBlock - 1) / kBlock > int64_t(kMaxGrid) * 1024)
+      return set_error(MTRT_INVALID_ARGUMENT, "tensor of %lld elements is too large", (long long)(d0 * d1));
+    if (quantize) {
+      void *args[] = {&xy, &q, &scales, &tensor_amax, &d0, &d1};
+      return launch(st, std::string("mtrt_nvfp4_qc_") + xn, uint32_t((units + kBlock - 1) / kBlock), kBlock, stream, args);
+    }
+    void *args[] = {&q, &scales, &tensor_amax, &xy, &d0, &d1};
+    const int64_t blocks = std::min<int64_t>((units + kBlock - 1) / kBlock, int64_t(num_compute_units(st)) * 64);
+    return launch(st, std::string("mtrt_nvfp4_dqc_") + xn, uint32_t(blocks), kBlock, stream, args);
+  }
+  int64_t nvec = d0 * d1 / group;
   const int64_t blocks = (nvec + 4 * 8 * 64 - 1) / (4 * 8 * 64);   // 4 waves x 8 trips x 64 lanes per workgroup
   if (blocks > int64_t(kMaxGrid) * 1024)
     return set_error(MTRT_INVALID_ARGUMENT, "tensor of %lld elements is too large", (long long)(d0 * d1));
@@ -219,13 +239,14 @@ int32_t nvfp4_dispatch(bool quantize, hipStream_t stream, const void *xy, int32_
 } // namespace
 
 int32_t mtrt_hip_nvfp4_quantize(mtrt_stream_t stream, const void *x, int32_t x_dtype, void *q_packed, void *scales,
-                                const float *tensor_amax, int64_t d0, int64_t d1) {
-  return nvfp4_dispatch(true, as_hip(stream), x, x_dtype, q_packed, scales, tensor_amax, d0, d1);
+                                const float *tensor_amax, int64_t d0, int64_t d1, int32_t block_axis) {
+  return nvfp4_dispatch(true, as_hip(stream), x, x_dtype, q_packed, scales, tensor_amax, d0, d1, block_axis);
 }
 
 int32_t mtrt_hip_nvfp4_dequantize(mtrt_stream_t stream, const void *q_packed, const void *scales,
-                                  const float *tensor_amax, void *y, int32_t y_dtype, int64_t d0, int64_t d1) {
-  return nvfp4_dispatch(false, as_hip(stream), y, y_dtype, q_packed, scales, tensor_amax, d0, d1);
+                                  const float *tensor_amax, void *y, int32_t y_dtype, int64_t d0, int64_t d1,
+                                  int32_t block_axis) {
+  return nvfp4_dispatch(false, as_hip(stream), y, y_dtype, q_packed, scales, tensor_amax, d0, d1, block_axis);
 }
 
 int32_t mtrt_hip_layernorm(mtrt_stream_t stream, const void *x, const void *gamma, const void *beta, void *y,

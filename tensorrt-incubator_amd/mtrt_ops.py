@@ -167,8 +167,7 @@ def mtrt_dequantize(input, scale, *, mode, axis=None, output_dtype="float32"):
 def mtrt_dynamic_quantize(input, double_quant_scale, *, axis, block_size=16, output_dtype="float4_e2m1fn",
                           scale_dtype="float8_e4m3fn"):
     """`tensorrt.dynamic_quantize` marker (NVFP4): returns (float4 codes, float8 block scales); the block scale
-    is quantized against `double_quant_scale`, the per-tensor second-level scale (tensor amax / 2688).
-    Only the last axis is built."""
+    is quantized against `double_quant_scale`, the per-tensor second-level scale (tensor amax / 2688)."""
     torch = _torch()
     rank = input.dim()
     assert axis is not None, "axis is required for dynamic quantization"
@@ -185,12 +184,9 @@ def mtrt_dynamic_quantize(input, double_quant_scale, *, axis, block_size=16, out
         f"dynamic quantization supports scale_dtype to be one of ['float8_e4m3fn'], got {scale_dtype}")
     assert input.dtype in [torch.float16, torch.bfloat16, torch.float32], (
         f"Unsupported input dtype for dynamic quantization: {input.dtype}")
-    if axis != rank - 1:
-        raise NotImplementedError("dynamic quantization along the second-to-last axis is not built")
     amax = torch.tensor(float(np.float32(dqs) * np.float32(2688.0)), dtype=torch.float32, device=input.device)
-    q, s = nvfp4_quantize(input.contiguous(), amax)
-    return (QuantizedArray(q, "float4_e2m1fn", input.shape),
-            QuantizedArray(s.reshape(-1), "float8_e4m3fn", input.shape[:-1] + (input.shape[-1] // block_size,)))
+    q, s = nvfp4_quantize(input.contiguous(), amax, axis=axis - rank)
+    return QuantizedArray(q, "float4_e2m1fn", input.shape), QuantizedArray(s.reshape(-1), "float8_e4m3fn", s.shape)
 
 
 def custom_call(call_target_name, operands, mode=None, axis=None, **attrs):

@@ -9,7 +9,7 @@ from helpers import bits16, rng
 pytestmark = pytest.mark.gpu
 
 
-def _run(pkg, orc, x_f32, dname, amax=None):
+def _run(pkg, orc, x_f32, dname, amax=None, axis=-1):
     import torch
     o_dt = {"f32": orc.F32, "f16": orc.F16, "bf16": orc.BF16}[dname]
     t_dt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[dname]
@@ -28,12 +28,13 @@ def _run(pkg, orc, x_f32, dname, amax=None):
         assert np.float32(amax) == orc.amax(store, o_dt)
     else:
         a_dev = torch.tensor(amax, dtype=torch.float32, device="cuda")
-    q, s = pkg.nvfp4_quantize(x, a_dev.clone())
-    q_ref, s_ref = orc.nvfp4_quantize(store, o_dt, amax, d0, d1)
+    ba = 1 if axis == -1 else 0
+    q, s = pkg.nvfp4_quantize(x, a_dev.clone(), axis=axis)
+    q_ref, s_ref = orc.nvfp4_quantize(store, o_dt, amax, d0, d1, block_axis=ba)
     assert np.array_equal(s.cpu().numpy().ravel(), s_ref), "block scales (%s)" % pkg.last_kernel()
     assert np.array_equal(q.cpu().numpy(), q_ref), "codes (%s)" % pkg.last_kernel()
-    y = pkg.nvfp4_dequantize(q, s, a_dev.clone(), t_dt, shape)
-    y_ref = orc.nvfp4_dequantize(q_ref, s_ref, amax, o_dt, d0, d1)
+    y = pkg.nvfp4_dequantize(q, s, a_dev.clone(), t_dt, shape, axis=axis)
+    y_ref = orc.nvfp4_dequantize(q_ref, s_ref, amax, o_dt, d0, d1, block_axis=ba)
     got = y.cpu().numpy().ravel().view(np.uint32) if dname == "f32" else bits16(y)
     ref = y_ref.view(got.dtype)
     # a NaN result (tensor amax 0: 0 * NaN) must be NaN on both sides; sign and payload of a NaN are not compared
@@ -53,6 +54,22 @@ def test_reference_shapes(pkg, orc, dname, shape):
     xs = x if dname == "f32" else None
     if xs is not None:   # the reference test's acceptance bound
         assert np.all(np.abs(y.cpu().numpy() - x) <= 0.2 + 0.25 * np.abs(x))
+
+
+@pytest.mark.parametrize("dname", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("shape", [(16, 8), (32, 64), (2, 48, 1000), (4096, 264), (3, 5, 160, 24)])
+def test_blocks_along_the_second_to_last_axis(pkg, orc, dname, shape):
+    """The op's other axis choice: blocks of 16 rows, scales [.., rows/16, cols]; with zero blocks, a block whose
+    scale underflows, negative zeros and an outlier."""
+    x = (rng(41 + len(shape)).standard_normal(shape) * 1.5).astype(np.float32)
+    flat = x.reshape(-1, shape[-2], shape[-1])
+    flat[0, :16, 0] = 0.0
+    flat[0, :16, 1] *= 1e-7
+    flat[0, 3, 1] = 0.0
+    flat[-1, -16:, -1] = -0.0
+    flat[0, 5, 2] = 700.0
+    y = _run(pkg, orc, x, dname, axis=-2)
+    assert y.shape == x.shape
 
 
 def test_every_f16_value_through_the_f4_conversion(pkg, orc):
@@ -100,9 +117,13 @@ def test_argument_checks(pkg):
     L = pkg.lib()
     t = torch.zeros(64, device="cuda")
     p = t.data_ptr()
-    assert L.mtrt_hip_nvfp4_quantize(None, p, pkg.F32, p, p, p, 2, 24) == 1
+    assert L.mtrt_hip_nvfp4_quantize(None, p, pkg.F32, p, p, p, 2, 24, 1) == 1
     assert b"divisible by 16" in L.mtrt_hip_last_error()
-    assert L.mtrt_hip_nvfp4_quantize(None, p, pkg.I8, p, p, p, 2, 16) == 1
-    assert L.mtrt_hip_nvfp4_quantize(None, p + 4, pkg.F32, p, p, p, 2, 16) == 1
-    assert L.mtrt_hip_nvfp4_quantize(None, p, pkg.F32, p, p, None, 2, 16) == 1
-    assert L.mtrt_hip_nvfp4_dequantize(None, p, p, p, p, pkg.F32, 0, 16) == 0
+    assert L.mtrt_hip_nvfp4_quantize(None, p, pkg.F32, p, p, p, 24, 16, 0) == 1     # blocked extent 24
+    assert L.mtrt_hip_nvfp4_quantize(None, p, pkg.F32, p, p, p, 16, 6, 0) == 1      # last extent not whole vectors
+    assert L.mtrt_hip_nvfp4_quantize(None, p, pkg.F32, p, p, p, 16, 16, 2) == 1
+    assert b"invalid axis" in L.mtrt_hip_last_error()
+    assert L.mtrt_hip_nvfp4_quantize(None, p, pkg.I8, p, p, p, 2, 16, 1) == 1
+    assert L.mtrt_hip_nvfp4_quantize(None, p + 4, pkg.F32, p, p, p, 2, 16, 1) == 1
+    assert L.mtrt_hip_nvfp4_quantize(None, p, pkg.F32, p, p, None, 2, 16, 1) == 1
+    assert L.mtrt_hip_nvfp4_dequantize(None, p, p, p, p, pkg.F32, 0, 16, 1) == 0

@@ -123,6 +123,22 @@ def test_dynamic_quantize_known_answer(ops):
 
 
 @pytest.mark.gpu
+def test_dynamic_quantize_along_the_second_to_last_axis(ops, orc):
+    """axis = rank - 2: the same chain as the reference's test on the transposed input gives the transposed result."""
+    import torch
+    g = GOLD["dynamic_quantize_pt"]
+    x = torch.tensor(g["x"], dtype=torch.float32).t().contiguous().cuda()           # [32, 2]: blocks down the rows
+    x4 = torch.cat([x, x, x, x], dim=1).contiguous()                                   # [32, 8]: whole vectors
+    dqs = np.array(1.0)
+    fp4_out, fp8_scale = ops.mtrt_dynamic_quantize(x4, dqs, axis=0)
+    assert fp8_scale.shape == (2, 8)
+    scales = ops.mtrt_dequantize(fp8_scale, dqs, mode="tensorrt.pt_dq", output_dtype=np.float32)
+    out = ops.mtrt_dequantize(fp4_out, scales, mode="tensorrt.block_dq", output_dtype=np.float32)
+    expected = np.array(g["expected"], dtype=np.float32).T
+    np.testing.assert_allclose(out.cpu().numpy(), np.concatenate([expected] * 4, axis=1), rtol=1e-6, atol=0)
+
+
+@pytest.mark.gpu
 def test_block_modes_on_both_axes_against_oracle(ops, orc):
     """block_q / block_dq with int4 and float4 codes, blocks along the last and the second-to-last axis,
     with a leading batch axis; bit-exact against the oracle addressed per element."""

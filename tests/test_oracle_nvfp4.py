@@ -99,3 +99,24 @@ def test_identity_on_the_f4_grid_and_zero_blocks(orc):
     # an all-zero tensor: S_enc is infinite, every scale byte is the e4m3 NaN, every code 0
     q, s = orc.nvfp4_quantize(np.zeros((1, 32), np.float32), orc.F32, 0.0, 1, 32)
     assert not q.any() and list(s) == [0x7F, 0x7F]
+
+
+def test_blocks_along_the_other_axis_are_the_transposed_problem(orc):
+    """Blocks along d0 of x equal blocks along d1 of x^T: pins the block and scale indexing of block_axis = 0
+    against the (numpy-pinned) block_axis = 1 path, codes compared after unpacking."""
+    def unpack(q, n):
+        out = np.empty(n, np.uint8)
+        out[0::2] = q & 0xF
+        out[1::2] = q >> 4
+        return out
+    for d0, d1 in ((16, 3), (48, 10), (32, 64)):
+        x = (rng(d0 + d1).standard_normal((d0, d1)) * 2).astype(np.float32)
+        x[:16, 0] = 0.0
+        amax = np.float32(np.abs(x).max())
+        q0, s0 = orc.nvfp4_quantize(x, orc.F32, amax, d0, d1, block_axis=0)
+        qt, st = orc.nvfp4_quantize(np.ascontiguousarray(x.T), orc.F32, amax, d1, d0, block_axis=1)
+        assert np.array_equal(unpack(q0, d0 * d1).reshape(d0, d1), unpack(qt, d0 * d1).reshape(d1, d0).T)
+        assert np.array_equal(s0.reshape(d0 // 16, d1), st.reshape(d1, d0 // 16).T)
+        y0 = orc.nvfp4_dequantize(q0, s0, amax, orc.F32, d0, d1, block_axis=0)
+        yt = orc.nvfp4_dequantize(qt, st, amax, orc.F32, d1, d0, block_axis=1)
+        assert np.array_equal(y0.reshape(d0, d1), yt.reshape(d1, d0).T)
