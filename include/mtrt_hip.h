@@ -306,6 +306,29 @@ MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_memcpy(uintptr_t stream, uintptr_t src,
  * fill kernel on `stream` (no memset node, so it can be captured into a graph). */
 MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_memset(uintptr_t stream, uintptr_t ptr, uint64_t offset,
                                                 uint64_t nbytes, uint32_t fill, int32_t width);
+/* __cuda_event_create(device) / _release / __cuda_stream_record_event / __cuda_stream_wait_event /
+ * __cuda_event_sync / __cuda_event_elapsed_msec (CUDAModule.cpp:112-155).  As in the reference events come
+ * from a per-device pool (mlir-tensorrt/executor/lib/Runtime/Support/CUDAEventPool.cpp): release returns the
+ * event to the pool, the next create on that device reuses it. */
+MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_event_create(int32_t device, uintptr_t *out_event);
+MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_event_release(uintptr_t event);
+MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_stream_record_event(uintptr_t stream, uintptr_t event);
+MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_stream_wait_event(uintptr_t stream, uintptr_t event);
+MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_event_sync(uintptr_t event);
+MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_event_elapsed_msec(uintptr_t start, uintptr_t end, float *out_ms);
+/* __cuda_alloc_host_pinned(nbytes, alignment) / __cuda_free_host_pinned(stream, ptr) (CUDAModule.cpp:354-376,
+ * 400-411).  Pinned memory is allocated, never registered.  The free is ordered after the work already queued
+ * on `stream` (the reference's PinnedMemoryAllocator::freeAsync): the block is released once the stream has
+ * passed that point, at the latest by a later alloc / free call or at process exit. */
+MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_alloc_host_pinned(uint64_t nbytes, int32_t alignment, uintptr_t *out_ptr);
+MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_free_host_pinned(uintptr_t stream, uintptr_t ptr);
+/* __cuda_memcpy_strided_async_{device2device,device2host,host2device}(stream, rank, elemSize, src, srcOffset,
+ * srcShapeAndStrides, dst, dstOffset, dstShapeAndStrides) (CUDAModule.cpp:210-255): shapes then strides, in
+ * elements, `rank` values each; offsets in bytes.  Issued as one copy per contiguous run. */
+MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_memcpy_strided(uintptr_t stream, int64_t rank, int64_t elemSize,
+                                                        uintptr_t src, uint64_t srcOffset,
+                                                        const int64_t *srcShapeAndStrides, uintptr_t dst,
+                                                        uint64_t dstOffset, const int64_t *dstShapeAndStrides);
 /* __cuda_num_devices (CUDAModule.cpp:86-90) and __cuda_get_program_device(logicalId) (:560-571) */
 MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_num_devices(int32_t *out_count);
 MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_get_program_device(int32_t logicalId, int32_t *out_device);

@@ -64,6 +64,16 @@ PROTOTYPES = {
     "mtrt_lua_cuda_free_device": (_i32, [_sz, _sz]),
     "mtrt_lua_cuda_memcpy": (_i32, [_sz, _sz, _c.c_uint64, _sz, _c.c_uint64, _c.c_uint64]),
     "mtrt_lua_cuda_memset": (_i32, [_sz, _sz, _c.c_uint64, _c.c_uint64, _c.c_uint32, _i32]),
+    "mtrt_lua_cuda_event_create": (_i32, [_i32, _c.POINTER(_sz)]),
+    "mtrt_lua_cuda_event_release": (_i32, [_sz]),
+    "mtrt_lua_cuda_stream_record_event": (_i32, [_sz, _sz]),
+    "mtrt_lua_cuda_stream_wait_event": (_i32, [_sz, _sz]),
+    "mtrt_lua_cuda_event_sync": (_i32, [_sz]),
+    "mtrt_lua_cuda_event_elapsed_msec": (_i32, [_sz, _sz, _c.POINTER(_f32)]),
+    "mtrt_lua_cuda_alloc_host_pinned": (_i32, [_c.c_uint64, _i32, _c.POINTER(_sz)]),
+    "mtrt_lua_cuda_free_host_pinned": (_i32, [_sz, _sz]),
+    "mtrt_lua_cuda_memcpy_strided": (_i32, [_sz, _i64, _i64, _sz, _c.c_uint64, _c.POINTER(_i64), _sz, _c.c_uint64,
+                                            _c.POINTER(_i64)]),
     "mtrt_lua_cuda_num_devices": (_i32, [_c.POINTER(_i32)]),
     "mtrt_lua_cuda_get_program_device": (_i32, [_i32, _c.POINTER(_i32)]),
     "mtrt_lua_cuda_builtins": (_vp, [_c.POINTER(_sz)]),

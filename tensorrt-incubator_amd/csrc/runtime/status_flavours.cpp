@@ -13,6 +13,10 @@
 
 #include <algorithm>
 #include <cstring>
+#include <map>
+#include <mutex>
+#include <utility>
+#include <vector>
 
 using namespace mtrt_rt;
 
@@ -331,6 +335,181 @@ int32_t mtrt_lua_cuda_memset(uintptr_t stream, uintptr_t ptr, uint64_t offset, u
   return launch(st, "mtrt_fill", uint32_t(blocks), 256, reinterpret_cast<hipStream_t>(stream), args);
 }
 
+// ---- events from a per-device pool -------------------------------------------------------------
+namespace {
+struct EventPool {
+  std::mutex mu;
+  std::map<int, std::vector<hipEvent_t>> free_by_device;
+  std::map<hipEvent_t, int> device_of;                   // every event this pool ever created
+};
+EventPool &event_pool() {
+  static EventPool *pool = new EventPool();              // never destroyed: events may outlive static teardown
+  return *pool;
+}
+} // namespace
+
+int32_t mtrt_lua_cuda_event_create(int32_t device, uintptr_t *out_event) {
+  if (!out_event)
+    return set_error(MTRT_INVALID_ARGUMENT, "out_event must not be null");
+  *out_event = 0;
+  EventPool &pool = event_pool();
+  {
+    std::lock_guard<std::mutex> lock(pool.mu);
+    auto &free_list = pool.free_by_device[device];
+    if (!free_list.empty()) {
+      *out_event = reinterpret_cast<uintptr_t>(free_list.back());
+      free_list.pop_back();
+      return MTRT_OK;
+    }
+  }
+  mtrt_event_t e = nullptr;
+  const int32_t st = mtrt::cuda_event_create(device, &e);
+  if (st != MTRT_OK)
+    return st;
+  std::lock_guard<std::mutex> lock(pool.mu);
+  pool.device_of[reinterpret_cast<hipEvent_t>(e)] = device;
+  *out_event = reinterpret_cast<uintptr_t>(e);
+  return MTRT_OK;
+}
+
+int32_t mtrt_lua_cuda_event_release(uintptr_t event) {
+  if (!event)
+    return MTRT_OK;
+  EventPool &pool = event_pool();
+  std::lock_guard<std::mutex> lock(pool.mu);
+  auto it = pool.device_of.find(reinterpret_cast<hipEvent_t>(event));
+  if (it == pool.device_of.end())
+    return set_error(MTRT_INVALID_ARGUMENT, "event was not created by mtrt_lua_cuda_event_create");
+  pool.free_by_device[it->second].push_back(it->first);
+  return MTRT_OK;
+}
+
+int32_t mtrt_lua_cuda_stream_record_event(uintptr_t stream, uintptr_t event) {
+  return mtrt::cuda_stream_record_event(reinterpret_cast<mtrt_stream_t>(stream), reinterpret_cast<mtrt_event_t>(event));
+}
+int32_t mtrt_lua_cuda_stream_wait_event(uintptr_t stream, uintptr_t event) {
+  return mtrt::cuda_stream_wait_event(reinterpret_cast<mtrt_stream_t>(stream), reinterpret_cast<mtrt_event_t>(event));
+}
+int32_t mtrt_lua_cuda_event_sync(uintptr_t event) { return mtrt::cuda_event_sync(reinterpret_cast<mtrt_event_t>(event)); }
+int32_t mtrt_lua_cuda_event_elapsed_msec(uintptr_t start, uintptr_t end, float *out_ms) {
+  return mtrt::cuda_event_elapsed_msec(reinterpret_cast<mtrt_event_t>(start), reinterpret_cast<mtrt_event_t>(end), out_ms);
+}
+
+// ---- pinned host memory with stream-ordered release -------------------------------------------
+namespace {
+struct PinnedFrees {
+  std::mutex mu;
+  std::vector<std::pair<hipEvent_t, void *>> pending;    // block is free once the event has completed
+};
+PinnedFrees &pinned_frees() {
+  static PinnedFrees *p = new PinnedFrees();
+  return *p;
+}
+// releases every block whose stream has passed the point of its free call
+void reap_pinned(bool wait) {
+  PinnedFrees &pf = pinned_frees();
+  std::lock_guard<std::mutex> lock(pf.mu);
+  size_t keep = 0;
+  for (auto &entry : pf.pending) {
+    const hipError_t q = wait ? hipEventSynchronize(entry.first) : hipEventQuery(entry.first);
+    if (q == hipSuccess) {
+      (void)hipEventDestroy(entry.first);
+      (void)hipHostFree(entry.second);
+    } else {
+      if (q != hipErrorNotReady)
+        (void)hipGetLastError();
+      pf.pending[keep++] = entry;
+    }
+  }
+  pf.pending.resize(keep);
+}
+} // namespace
+
+int32_t mtrt_lua_cuda_alloc_host_pinned(uint64_t nbytes, int32_t alignment, uintptr_t *out_ptr) {
+  if (!out_ptr)
+    return set_error(MTRT_INVALID_ARGUMENT, "out_ptr must not be null");
+  *out_ptr = 0;
+  if (alignment <= 0 || (alignment & (alignment - 1)) != 0)
+    return set_error(MTRT_INVALID_ARGUMENT, "alignment must be a positive power of two, got %d", alignment);
+  reap_pinned(false);
+  if (nbytes == 0)
+    return MTRT_OK;
+  void *p = nullptr;
+  RETURN_IF_RT(hipHostMalloc(&p, size_t(nbytes), hipHostMallocDefault));
+  if (reinterpret_cast<uintptr_t>(p) % uint32_t(alignment) != 0) {
+    (void)hipHostFree(p);
+    return set_error(MTRT_INTERNAL_ERROR, "allocated host pinned pointer %p does not have desired alignment %d", p, alignment);
+  }
+  *out_ptr = reinterpret_cast<uintptr_t>(p);
+  return MTRT_OK;
+}
+
+int32_t mtrt_lua_cuda_free_host_pinned(uintptr_t stream, uintptr_t ptr) {
+  if (!ptr)
+    return MTRT_OK;
+  hipEvent_t e = nullptr;
+  RETURN_IF_RT(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+  const hipError_t r = hipEventRecord(e, reinterpret_cast<hipStream_t>(stream));
+  if (r != hipSuccess) {
+    (void)hipEventDestroy(e);
+    return runtime_error(r, "hipEventRecord");
+  }
+  {
+    PinnedFrees &pf = pinned_frees();
+    std::lock_guard<std::mutex> lock(pf.mu);
+    pf.pending.emplace_back(e, reinterpret_cast<void *>(ptr));
+  }
+  reap_pinned(false);
+  return MTRT_OK;
+}
+
+// ---- strided copies --------------------------------------------------------------------------
+int32_t mtrt_lua_cuda_memcpy_strided(uintptr_t stream, int64_t rank, int64_t elemSize, uintptr_t src, uint64_t srcOffset,
+                                     const int64_t *srcShapeAndStrides, uintptr_t dst, uint64_t dstOffset,
+                                     const int64_t *dstShapeAndStrides) {
+  if (rank < 0 || rank > 16 || elemSize <= 0)
+    return set_error(MTRT_INVALID_ARGUMENT, "rank %lld / element size %lld out of range", (long long)rank, (long long)elemSize);
+  if (rank > 0 && (!srcShapeAndStrides || !dstShapeAndStrides))
+    return set_error(MTRT_INVALID_ARGUMENT, "shape/stride arrays must not be null");
+  if (!src || !dst)
+    return set_error(MTRT_INVALID_ARGUMENT, "src/dst must not be null");
+  const int64_t *shape = srcShapeAndStrides, *ss = srcShapeAndStrides + rank, *ds = dstShapeAndStrides + rank;
+  int64_t total = 1;
+  for (int64_t i = 0; i < rank; ++i) {
+    if (shape[i] != dstShapeAndStrides[i])
+      return set_error(MTRT_INVALID_ARGUMENT, "source and destination shapes differ in dimension %lld", (long long)i);
+    if (shape[i] < 0)
+      return set_error(MTRT_INVALID_ARGUMENT, "negative extent in dimension %lld", (long long)i);
+    total *= shape[i];
+  }
+  if (total == 0)
+    return MTRT_OK;
+  // innermost dimensions that are densely packed in BOTH operands form one contiguous run
+  int64_t run = 1, inner = rank;
+  while (inner > 0 && ss[inner - 1] == run && ds[inner - 1] == run) {
+    run *= shape[inner - 1];
+    --inner;
+  }
+  std::vector<int64_t> idx(size_t(inner), 0);
+  const char *sbase = reinterpret_cast<const char *>(src + srcOffset);
+  char *dbase = reinterpret_cast<char *>(dst + dstOffset);
+  for (;;) {
+    int64_t so = 0, dof = 0;
+    for (int64_t i = 0; i < inner; ++i) {
+      so += idx[size_t(i)] * ss[i];
+      dof += idx[size_t(i)] * ds[i];
+    }
+    RETURN_IF_RT(hipMemcpyAsync(dbase + dof * elemSize, sbase + so * elemSize, size_t(run * elemSize), hipMemcpyDefault,
+                                reinterpret_cast<hipStream_t>(stream)));
+    int64_t d = inner - 1;
+    while (d >= 0 && ++idx[size_t(d)] == shape[d])
+      idx[size_t(d--)] = 0;
+    if (d < 0)
+      break;
+  }
+  return MTRT_OK;
+}
+
 int32_t mtrt_lua_cuda_num_devices(int32_t *out_count) {
   if (!out_count)
     return set_error(MTRT_INVALID_ARGUMENT, "out_count must not be null");
@@ -374,6 +553,19 @@ const struct mtrt_lua_builtin *mtrt_lua_cuda_builtins(size_t *count) {
       {"__cuda_memset_8", "mtrt_lua_cuda_memset"},
       {"__cuda_memset_16", "mtrt_lua_cuda_memset"},
       {"__cuda_memset_32", "mtrt_lua_cuda_memset"},
+      {"__cuda_event_create", "mtrt_lua_cuda_event_create"},
+      {"__cuda_event_release", "mtrt_lua_cuda_event_release"},
+      {"__cuda_stream_record_event", "mtrt_lua_cuda_stream_record_event"},
+      {"__cuda_stream_wait_event", "mtrt_lua_cuda_stream_wait_event"},
+      {"__cuda_event_sync", "mtrt_lua_cuda_event_sync"},
+      {"__cuda_event_elapsed_msec", "mtrt_lua_cuda_event_elapsed_msec"},
+      {"__cuda_alloc_host_pinned", "mtrt_lua_cuda_alloc_host_pinned"},
+      {"__cuda_free_host_pinned", "mtrt_lua_cuda_free_host_pinned"},
+      {"__cuda_memcpy_strided_async_device2device", "mtrt_lua_cuda_memcpy_strided"},
+      {"__cuda_memcpy_strided_async_device2host", "mtrt_lua_cuda_memcpy_strided"},
+      {"__cuda_memcpy_strided_async_host2device", "mtrt_lua_cuda_memcpy_strided"},
+      {"__cuda_memcpy_strided_async_host_pinned2device", "mtrt_lua_cuda_memcpy_strided"},
+      {"__cuda_memcpy_strided_async_device2host_pinned", "mtrt_lua_cuda_memcpy_strided"},
       {"__cuda_num_devices", "mtrt_lua_cuda_num_devices"},
       {"__cuda_get_program_device", "mtrt_lua_cuda_get_program_device"},
   };

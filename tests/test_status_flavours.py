@@ -83,6 +83,22 @@ def test_builtin_argument_validation(pkg):
     assert L.mtrt_lua_cuda_get_program_device(3, ctypes.byref(dev)) == 7
     assert b"out of range" in L.mtrt_hip_last_error()
     assert L.mtrt_lua_cuda_stream_destroy(0) == 1
+    assert L.mtrt_lua_cuda_event_create(0, None) == 1
+    assert L.mtrt_lua_cuda_event_release(0) == 0
+    assert L.mtrt_lua_cuda_event_release(4096) == 1                  # not an event of the pool
+    assert L.mtrt_lua_cuda_stream_record_event(0, 0) == 1
+    ms = ctypes.c_float(1.0)
+    assert L.mtrt_lua_cuda_event_elapsed_msec(0, 0, ctypes.byref(ms)) == 1
+    p = ctypes.c_size_t(1)
+    assert L.mtrt_lua_cuda_alloc_host_pinned(64, 3, ctypes.byref(p)) == 1 and p.value == 0
+    assert L.mtrt_lua_cuda_alloc_host_pinned(64, 16, None) == 1
+    assert L.mtrt_lua_cuda_free_host_pinned(0, 0) == 0
+    shp = (ctypes.c_int64 * 4)(2, 3, 3, 1)
+    bad = (ctypes.c_int64 * 4)(2, 4, 4, 1)
+    assert L.mtrt_lua_cuda_memcpy_strided(0, 2, 4, 16, 0, shp, 16, 0, bad) == 1
+    assert b"shapes differ" in L.mtrt_hip_last_error()
+    assert L.mtrt_lua_cuda_memcpy_strided(0, 2, 0, 16, 0, shp, 16, 0, shp) == 1
+    assert L.mtrt_lua_cuda_memcpy_strided(0, 2, 4, 0, 0, shp, 16, 0, shp) == 1
 
 
 @pytest.mark.gpu
@@ -141,5 +157,54 @@ def test_builtin_bodies_known_answers(pkg):
     assert L.mtrt_lua_cuda_launch(fn.value, 1, 1, 1, 4096, 1, 1, 0, stream.value, ctypes.addressof(argv)) == 4
     assert L.mtrt_lua_cuda_free_device(stream.value, a.value) == 0
     assert L.mtrt_lua_cuda_free_device(stream.value, b.value) == 0
+    assert L.mtrt_lua_cuda_stream_sync(stream.value) == 0
+    assert L.mtrt_lua_cuda_stream_destroy(stream.value) == 0
+
+
+@pytest.mark.gpu
+def test_builtin_events_pinned_memory_and_strided_copies(pkg):
+    L = pkg.lib()
+    sz = ctypes.c_size_t
+    dev = L.mtrt_cuda_get_current_device()
+    stream, e0, e1, e2 = sz(0), sz(0), sz(0), sz(0)
+    assert L.mtrt_lua_cuda_stream_create(ctypes.byref(stream)) == 0
+    assert L.mtrt_lua_cuda_event_create(dev, ctypes.byref(e0)) == 0 and e0.value
+    assert L.mtrt_lua_cuda_event_create(dev, ctypes.byref(e1)) == 0 and e1.value != e0.value
+    # pinned staging buffers, 3 x 5 f32 matrix inside a 4 x 8 parent (row stride 8), copied to a dense device matrix
+    hsrc, hdst, dbuf = sz(0), sz(0), sz(0)
+    assert L.mtrt_lua_cuda_alloc_host_pinned(4 * 8 * 4, 64, ctypes.byref(hsrc)) == 0 and hsrc.value % 64 == 0
+    assert L.mtrt_lua_cuda_alloc_host_pinned(6 * 5 * 4, 64, ctypes.byref(hdst)) == 0
+    assert L.mtrt_lua_cuda_alloc_device(stream.value, 3 * 5 * 4, ctypes.byref(dbuf)) == 0
+    src = np.ctypeslib.as_array(ctypes.cast(hsrc.value, ctypes.POINTER(ctypes.c_float)), shape=(4, 8))
+    dst = np.ctypeslib.as_array(ctypes.cast(hdst.value, ctypes.POINTER(ctypes.c_float)), shape=(6, 5))
+    src[:] = np.arange(32, dtype=np.float32).reshape(4, 8)
+    dst[:] = -1.0
+    strided = (ctypes.c_int64 * 4)(3, 5, 8, 1)
+    dense = (ctypes.c_int64 * 4)(3, 5, 5, 1)
+    every_other_row = (ctypes.c_int64 * 4)(3, 5, 10, 1)
+    assert L.mtrt_lua_cuda_stream_record_event(stream.value, e0.value) == 0
+    # host (offset: row 1, column 2) -> device, then device -> every other row of the host destination
+    assert L.mtrt_lua_cuda_memcpy_strided(stream.value, 2, 4, hsrc.value, (1 * 8 + 2) * 4, strided, dbuf.value, 0, dense) == 0
+    assert L.mtrt_lua_cuda_memcpy_strided(stream.value, 2, 4, dbuf.value, 0, dense, hdst.value, 0, every_other_row) == 0
+    assert L.mtrt_lua_cuda_stream_record_event(stream.value, e1.value) == 0
+    assert L.mtrt_lua_cuda_stream_wait_event(stream.value, e1.value) == 0
+    assert L.mtrt_lua_cuda_event_sync(e1.value) == 0
+    ms = ctypes.c_float(-1.0)
+    assert L.mtrt_lua_cuda_event_elapsed_msec(e0.value, e1.value, ctypes.byref(ms)) == 0 and ms.value >= 0.0
+    expect = np.full((6, 5), -1.0, np.float32)
+    expect[0::2] = src[1:4, 2:7]
+    assert np.array_equal(dst, expect)
+    # a released event comes back from the pool
+    assert L.mtrt_lua_cuda_event_release(e1.value) == 0
+    assert L.mtrt_lua_cuda_event_create(dev, ctypes.byref(e2)) == 0 and e2.value == e1.value
+    assert L.mtrt_lua_cuda_event_release(e2.value) == 0 and L.mtrt_lua_cuda_event_release(e0.value) == 0
+    # stream-ordered frees
+    assert L.mtrt_lua_cuda_free_host_pinned(stream.value, hsrc.value) == 0
+    assert L.mtrt_lua_cuda_free_host_pinned(stream.value, hdst.value) == 0
+    assert L.mtrt_lua_cuda_free_device(stream.value, dbuf.value) == 0
+    assert L.mtrt_lua_cuda_stream_sync(stream.value) == 0
+    again = sz(0)
+    assert L.mtrt_lua_cuda_alloc_host_pinned(128, 16, ctypes.byref(again)) == 0      # reaps the finished frees
+    assert L.mtrt_lua_cuda_free_host_pinned(stream.value, again.value) == 0
     assert L.mtrt_lua_cuda_stream_sync(stream.value) == 0
     assert L.mtrt_lua_cuda_stream_destroy(stream.value) == 0
