@@ -14,11 +14,12 @@
 //   k = 64*kb + 8*(2j + h) + [0..7] of column n.  Inside a dword nibble p (p < 4) is
 //   weight 2p and nibble p + 4 is weight 2p + 1, each stored as (value + 8).
 // A wave therefore loads 1 KiB of contiguous memory and every lane gets exactly its
-// B-fragments for four v_mfma_f32_32x32x16_f16 steps; (w >> 4p) & 0x000F000F isolates
-// the pair (2p, 2p+1) in the two halves of a register, OR-ing 0x6400 into each half
-// makes the f16 numbers 1024 + (value + 8), a packed subtract of 1032 gives the exact
-// integer value and a packed f16 multiply by the scale gives wd with the single
-// rounding the program asks for.
+// B-fragments for four v_mfma_f32_32x32x16_f16 steps; w & 0x000F000F isolates the pair
+// (0, 1) in the two halves of a register, OR-ing 0x6400 into each half makes the f16
+// numbers 1024 + (value + 8), a packed subtract of 1032 gives the exact integer value and
+// a packed f16 multiply by the scale gives wd with the single rounding the program asks
+// for; the pair (2, 3) is read where it sits (w & 0x00F000F0 under 0x5400: 64 + (value + 8),
+// minus 72), the pairs (4, 5) and (6, 7) the same way from w >> 8.
 //
 // All kernels take the weight fragments straight from global memory into registers and
 // dequantise them there; only the activations go through LDS (direct-to-LDS loads).
@@ -44,32 +45,28 @@ __device__ __forceinline__ int lds_off(int row, int chunk) { return row * 128 + 
 
 union H2Bits { uint32_t u; h2 h; };
 
-// One prepacked dword -> 8 dequantised f16 weights (k order 0..7), as a 16-byte chunk.
-__device__ __forceinline__ u4 dequant8(uint32_t w, h2 scale2) {
-  u4 out;
-#pragma unroll
-  for (int p = 0; p < 4; ++p) {
-    H2Bits t;
-    t.u = ((w >> (4 * p)) & 0x000F000Fu) | 0x64006400u;   // {1024 + u(2p), 1024 + u(2p+1)}
-    const h2 bias = {(_Float16)1032.0f, (_Float16)1032.0f};
-    t.h = (t.h - bias) * scale2;                            // exact integer, then one f16 rounding
-    out[p] = t.u;
-  }
-  return out;
+// One prepacked dword -> 8 dequantised f16 weights with a single shift: nibbles 0 and 2 are read in
+// place under 0x6400 (1024 + u, minus 1032), nibbles 1 and 3 in place four bits higher under 0x5400
+// (64 + 16 u / 16, minus 72); both differences are the exact integer, the multiply rounds once.
+// The two masks (0x000F000F and 0x00F000F0) are held in vector registers: the and-or then is ONE
+// instruction (it may name a single scalar or literal operand, and the exponent pattern is that one).
+// dequant4 is half of it: dwords 2*part and 2*part + 1 of the chunk.
+__device__ __forceinline__ void dequant4(uint32_t w, h2 scale2, int part, uint32_t mask_lo, uint32_t mask_hi, u4& out) {
+  const h2 bias_lo = {(_Float16)1032.0f, (_Float16)1032.0f}, bias_hi = {(_Float16)72.0f, (_Float16)72.0f};
+  const uint32_t v = part ? w >> 8 : w;
+  H2Bits t0, t1;
+  t0.u = (v & mask_lo) | 0x64006400u;
+  t1.u = (v & mask_hi) | 0x54005400u;
+  t0.h = (t0.h - bias_lo) * scale2;                    // exact integer, then one f16 rounding
+  t1.h = (t1.h - bias_hi) * scale2;
+  out[2 * part] = t0.u;
+  out[2 * part + 1] = t1.u;
 }
-
-// Half of dequant8: dwords 2*part and 2*part + 1 of the chunk.  `mask` is 0x000F000F held in a
-// vector register: the and-or then is ONE instruction (it may name a single scalar or literal
-// operand, and 0x64006400 is that one).
-__device__ __forceinline__ void dequant4(uint32_t w, h2 scale2, int part, uint32_t mask, u4& out) {
-#pragma unroll
-  for (int p = 2 * part; p < 2 * part + 2; ++p) {
-    H2Bits t;
-    t.u = ((w >> (4 * p)) & mask) | 0x64006400u;
-    const h2 bias = {(_Float16)1032.0f, (_Float16)1032.0f};
-    t.h = (t.h - bias) * scale2;
-    out[p] = t.u;
-  }
+__device__ __forceinline__ u4 dequant8_in_place(uint32_t w, h2 scale2, uint32_t mask_lo, uint32_t mask_hi) {
+  u4 out;
+  dequant4(w, scale2, 0, mask_lo, mask_hi, out);
+  dequant4(w, scale2, 1, mask_lo, mask_hi, out);
+  return out;
 }
 __device__ __forceinline__ uint32_t nibble_pair_mask() {
   uint32_t m = 0x000F000Fu;
@@ -132,7 +129,7 @@ struct WeightRegs {
   uint32_t slices_per_block;
   u4 raw[D][JT];
   uint32_t sc_bits[D][JT];
-  uint32_t mask = nibble_pair_mask();
+  uint32_t mask = nibble_pair_mask(), mask_hi = nibble_pair_mask() << 4;
   template <int SET>
   __device__ __forceinline__ void fetch(int64_t slice) {
     const int lane = threadIdx.x & 63;
@@ -156,7 +153,7 @@ struct WeightRegs {
     if (KEEP) __asm__ volatile("" ::"v"(raw[SET][j]));
     H2Bits t;
     t.u = sc_bits[SET][j] * 0x00010001u;
-    dequant4(raw[SET][j][P], t.h, part, mask, frag);
+    dequant4(raw[SET][j][P], t.h, part, mask, mask_hi, frag);
   }
 };
 
@@ -449,7 +446,7 @@ __device__ __forceinline__ void skinny(const uint16_t* __restrict__ a, const uin
   v16f acc;
 #pragma unroll
   for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
-  const uint32_t mask = nibble_pair_mask();
+  const uint32_t mask = nibble_pair_mask(), mask_hi = mask << 4;
   auto multiply = [&](int64_t kb, const Slice& sl) {
     const int8_t* st = ring + int(kb & (kStages - 1)) * kStageBytes;
     H2Bits sp;
@@ -459,8 +456,7 @@ __device__ __forceinline__ void skinny(const uint16_t* __restrict__ a, const uin
       const int arow = frow < 8 * G ? frow : 8 * G - 1;   // rows past the ring: any valid data, never stored
       const v8h fa = *reinterpret_cast<const v8h*>(st + gemm_core::lds_off(arow, 2 * ks + fhalf));
       union { u4 u; v8h h; } fb;
-      dequant4(sl.w[ks], sp.h, 0, mask, fb.u);
-      dequant4(sl.w[ks], sp.h, 1, mask, fb.u);
+      fb.u = dequant8_in_place(sl.w[ks], sp.h, mask, mask_hi);
       acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, fb.h, acc, 0, 0, 0);
     }
   };
