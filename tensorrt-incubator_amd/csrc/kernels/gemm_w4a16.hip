@@ -385,8 +385,9 @@ extern "C" __global__ void __launch_bounds__(512) mtrt_gemm_w4a16_t128x128(
 }
 
 // Small M (<= 32): one workgroup per 32 columns, four waves split K.
-// G: groups of 8 activation rows kept per stage (M <= 8 * G); WAVES: waves that split K.
-template <int G, int WAVES>
+// G: groups of 8 activation rows kept per stage (M <= 8 * G); WAVES: waves that split K;
+// JT: column tiles of the workgroup (blockIdx.x, blockIdx.x + gridDim.x), sharing the activations.
+template <int G, int WAVES, int JT>
 __device__ __forceinline__ void skinny(const uint16_t* __restrict__ a, const uint32_t* __restrict__ wp,
                                        const uint16_t* __restrict__ scale, uint16_t* __restrict__ y, int64_t M, int64_t K,
                                        int64_t N, int64_t block, int8_t* lds) {
@@ -395,18 +396,22 @@ __device__ __forceinline__ void skinny(const uint16_t* __restrict__ a, const uin
   // touch 64 different cache lines per instruction (32 rows 8 KiB apart), the ring is filled
   // with whole 128-byte row segments.  The waves never touch each other's ring: no barriers.
   constexpr int kStages = 4, kStageBytes = 8 * G * 128;
-  constexpr int kLoads = G + 2;                      // memory instructions per slice and wave
+  constexpr int kLoads = G + 2 * JT;                 // memory instructions per slice and wave
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int frow = lane & 31, fhalf = lane >> 5;
-  const int64_t tile = blockIdx.x;
   const int64_t kblocks = K / BKH;
   const int64_t kb0 = kblocks * wave / WAVES, kb1 = kblocks * (wave + 1) / WAVES;
-  const int64_t klast = kb1 - 1;
-  int64_t col = tile * 32 + frow;
-  col = col < N ? col : N - 1;                       // columns past N: the last column's scales, never stored
   const uint32_t slices_per_block = uint32_t(block / BKH);
-  const u4* bp = reinterpret_cast<const u4*>(wp) + (tile * kblocks) * 64 + lane;
+  int64_t tile[JT], col[JT];
+  const u4* bp[JT];
+#pragma unroll
+  for (int j = 0; j < JT; ++j) {
+    tile[j] = blockIdx.x + int64_t(j) * gridDim.x;
+    col[j] = tile[j] * 32 + frow;
+    col[j] = col[j] < N ? col[j] : N - 1;            // columns past N: the last column's scales, never stored
+    bp[j] = reinterpret_cast<const u4*>(wp) + (tile[j] * kblocks) * 64 + lane;
+  }
   int8_t* ring = lds + wave * (kStages * kStageBytes);
 
   // direct-to-LDS load g (of G) of a slice: rows 8g .. 8g+7, lane l <-> (row l >> 3, LDS chunk l & 7)
@@ -419,10 +424,10 @@ __device__ __forceinline__ void skinny(const uint16_t* __restrict__ a, const uin
   }
   const int8_t* abase = reinterpret_cast<const int8_t*>(a);
   struct Slice {
-    u4 w;
-    uint32_t sc;
+    u4 w[JT];
+    uint32_t sc[JT];
   };
-  // everything slice kb needs from memory: G + 2 loads, always, so that the waits can count
+  // everything slice kb needs from memory: G + 2 JT loads, always, so that the waits can count
   auto fetch = [&](int64_t kb, int64_t clamp, Slice& dst) {
     kb = kb < clamp ? kb : clamp;
     int8_t* st = ring + int(kb & (kStages - 1)) * kStageBytes;
@@ -433,31 +438,46 @@ __device__ __forceinline__ void skinny(const uint16_t* __restrict__ a, const uin
     // Register loads issued as opaque instructions: the compiler's own wait-count bookkeeping
     // gives up on loads carried around a loop and drains everything (vmcnt(0)) before their first
     // use, which would leave nothing in flight.  The waits are placed by hand in `landed`.
-    const u4* wsrc = bp + kb * 64;
-    const uint16_t* ssrc = scale + int64_t(uint32_t(kb) / slices_per_block) * N + col;
-    __asm__ volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(dst.w) : "v"(wsrc) : "memory");
-    __asm__ volatile("global_load_ushort %0, %1, off" : "=v"(dst.sc) : "v"(ssrc) : "memory");
+#pragma unroll
+    for (int j = 0; j < JT; ++j) {
+      const u4* wsrc = bp[j] + kb * 64;
+      const uint16_t* ssrc = scale + int64_t(uint32_t(kb) / slices_per_block) * N + col[j];
+      __asm__ volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(dst.w[j]) : "v"(wsrc) : "memory");
+      __asm__ volatile("global_load_ushort %0, %1, off" : "=v"(dst.sc[j]) : "v"(ssrc) : "memory");
+    }
   };
   // ties the registers of a slice to the wait, so that no use can be scheduled in front of it:
   // four slices issued, the loads of three may fly -> those of the oldest slice have landed
-  auto landed = [&](Slice& sl) { __asm__ volatile("s_waitcnt vmcnt(%2)" : "+v"(sl.w), "+v"(sl.sc) : "n"(3 * kLoads) : "memory"); };
-  auto landed_all = [&](Slice& sl) { __asm__ volatile("s_waitcnt vmcnt(0)" : "+v"(sl.w), "+v"(sl.sc)::"memory"); };
-
-  v16f acc;
+  auto landed = [&](Slice& sl) {
 #pragma unroll
-  for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+    for (int j = 0; j < JT; ++j)
+      __asm__ volatile("s_waitcnt vmcnt(%2)" : "+v"(sl.w[j]), "+v"(sl.sc[j]) : "n"(3 * kLoads) : "memory");
+  };
+  auto landed_all = [&](Slice& sl) {
+#pragma unroll
+    for (int j = 0; j < JT; ++j) __asm__ volatile("s_waitcnt vmcnt(0)" : "+v"(sl.w[j]), "+v"(sl.sc[j])::"memory");
+  };
+
+  v16f acc[JT];
+#pragma unroll
+  for (int j = 0; j < JT; ++j)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[j][r] = 0.0f;
   const uint32_t mask = nibble_pair_mask(), mask_hi = mask << 4;
   auto multiply = [&](int64_t kb, const Slice& sl) {
     const int8_t* st = ring + int(kb & (kStages - 1)) * kStageBytes;
-    H2Bits sp;
-    sp.u = sl.sc * 0x00010001u;
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
       const int arow = frow < 8 * G ? frow : 8 * G - 1;   // rows past the ring: any valid data, never stored
       const v8h fa = *reinterpret_cast<const v8h*>(st + gemm_core::lds_off(arow, 2 * ks + fhalf));
-      union { u4 u; v8h h; } fb;
-      fb.u = dequant8_in_place(sl.w[ks], sp.h, mask, mask_hi);
-      acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, fb.h, acc, 0, 0, 0);
+#pragma unroll
+      for (int j = 0; j < JT; ++j) {
+        H2Bits sp;
+        sp.u = sl.sc[j] * 0x00010001u;
+        union { u4 u; v8h h; } fb;
+        fb.u = dequant8_in_place(sl.w[j][ks], sp.h, mask, mask_hi);
+        acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, fb.h, acc[j], 0, 0, 0);
+      }
     }
   };
 
@@ -497,20 +517,38 @@ __device__ __forceinline__ void skinny(const uint16_t* __restrict__ a, const uin
     multiply(kb, sl);
   }
   __builtin_amdgcn_s_waitcnt(0x0070);                  // surplus loads have landed before the ring is reused
-  __syncthreads();
   float (*partial)[16][64] = reinterpret_cast<float (*)[16][64]>(lds);
 #pragma unroll
-  for (int r = 0; r < 16; ++r) partial[wave][r][lane] = acc[r];
-  __syncthreads();
-  for (int e = threadIdx.x; e < 16 * 64; e += 64 * WAVES) {
-    const int r = e >> 6, l = e & 63;
-    float v = partial[0][r][l];
+  for (int j = 0; j < JT; ++j) {
+    __syncthreads();
 #pragma unroll
-    for (int w = 1; w < WAVES; ++w) v = v + partial[w][r][l];
-    const int64_t row = (r >> 2) * 8 + (l >> 5) * 4 + (r & 3);
-    const int64_t c = tile * 32 + (l & 31);
-    if (row < M && c < N) y[row * N + c] = uint16_t(f32_to_f16_bits(v));
+    for (int r = 0; r < 16; ++r) partial[wave][r][lane] = acc[j][r];
+    __syncthreads();
+    for (int e = threadIdx.x; e < 16 * 64; e += 64 * WAVES) {
+      const int r = e >> 6, l = e & 63;
+      float v = partial[0][r][l];
+#pragma unroll
+      for (int w = 1; w < WAVES; ++w) v = v + partial[w][r][l];
+      const int64_t row = (r >> 2) * 8 + (l >> 5) * 4 + (r & 3);
+      const int64_t c = tile[j] * 32 + (l & 31);
+      if (row < M && c < N) y[row * N + c] = uint16_t(f32_to_f16_bits(v));
+    }
   }
+}
+
+// The grid is one workgroup per column tile, or, while that would leave some compute units with two
+// workgroups and the rest with one (tiles between one and two times the compute units), one workgroup
+// per compute unit: workgroup g then also takes tile g + gridDim.x if there is one, and reads the
+// activations once for both.
+template <int G>
+__device__ __forceinline__ void skinny_tiles(const uint16_t* __restrict__ a, const uint32_t* __restrict__ wp,
+                                             const uint16_t* __restrict__ scale, uint16_t* __restrict__ y, int64_t M,
+                                             int64_t K, int64_t N, int64_t block, int8_t* lds) {
+  const int64_t tiles = (N + 31) / 32;
+  if (int64_t(blockIdx.x) + gridDim.x < tiles)
+    skinny<G, 4, 2>(a, wp, scale, y, M, K, N, block, lds);
+  else
+    skinny<G, 4, 1>(a, wp, scale, y, M, K, N, block, lds);
 }
 
 // M <= 16: half the activation rows per stage (8 waves splitting K were no faster than 4).
@@ -518,14 +556,14 @@ extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w4a16_skinny16(
     const uint16_t* __restrict__ a, const uint32_t* __restrict__ wp, const uint16_t* __restrict__ scale,
     uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t block) {
   __shared__ __attribute__((aligned(16))) int8_t lds[4 * 4 * 2 * 1024];
-  skinny<2, 4>(a, wp, scale, y, M, K, N, block, lds);
+  skinny_tiles<2>(a, wp, scale, y, M, K, N, block, lds);
 }
 // M <= 32: 4 waves split K.
 extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w4a16_skinny(
     const uint16_t* __restrict__ a, const uint32_t* __restrict__ wp, const uint16_t* __restrict__ scale,
     uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t block) {
   __shared__ __attribute__((aligned(16))) int8_t lds[4 * 4 * 4 * 1024];
-  skinny<4, 4>(a, wp, scale, y, M, K, N, block, lds);
+  skinny_tiles<4>(a, wp, scale, y, M, K, N, block, lds);
 }
 
 // Any shape: one output per lane, reading the ORIGINAL packed [K,N] nibbles; not a fast path.

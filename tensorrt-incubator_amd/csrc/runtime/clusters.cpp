@@ -469,10 +469,14 @@ int32_t mtrt_hip_gemm_w4a16(mtrt_stream_t stream, const void *a, const void *w_k
   const bool fast = w_prepacked && K > 0 && K % 64 == 0 && block % 64 == 0 && aligned(a, 16) && aligned(w_prepacked, 16);
   if (fast) {
     void *args[] = {&a, &w_prepacked, &scale, &y, &M, &K, &N, &block};
-    if (M <= 16)
-      return launch(st, "mtrt_gemm_w4a16_skinny16", uint32_t((N + 31) / 32), kBlock, as_hip(stream), args);
-    if (M <= 32)
-      return launch(st, "mtrt_gemm_w4a16_skinny", uint32_t((N + 31) / 32), kBlock, as_hip(stream), args);
+    if (M <= 32) {
+      // one workgroup per 32-column tile; between one and two tiles per compute unit, one workgroup per
+      // compute unit instead (the kernel then gives workgroup g the tiles g and g + grid, which share the
+      // activations; measured: 6 % faster at M = 16, 21 % at M = 32, 3 % slower at M = 5)
+      const int64_t tiles = (N + 31) / 32, cus = num_compute_units(st);
+      const uint32_t grid = uint32_t(M > 8 && tiles > cus && tiles <= 2 * cus ? cus : tiles);
+      return launch(st, M <= 16 ? "mtrt_gemm_w4a16_skinny16" : "mtrt_gemm_w4a16_skinny", grid, kBlock, as_hip(stream), args);
+    }
     // 256 x 256 tiles (512 threads) once they cover at least half of the compute units (measured:
     // from M = 1024 on at N = 11008 they beat the small tiles) and the activations stay inside
     // 32-bit byte offsets; 128 x 64 tiles otherwise.

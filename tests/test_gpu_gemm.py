@@ -217,6 +217,22 @@ def test_c5_w4a16_full_size(pkg, orc, M):
     _check_w4a16(orc, got, a[rows], w, s, K, N, B, ref)
 
 
+@pytest.mark.parametrize("shape", [(9, 192, 8209), (20, 320, 12000), (32, 256, 16384), (12, 128, 16400), (3, 256, 9000)])
+def test_w4a16_small_m_workgroups_with_two_column_tiles(pkg, orc, shape):
+    """Between one and two 32-column tiles per compute unit the small-M kernels run one workgroup per
+    compute unit and the first ones take a second tile (M > 8); N = 8209 gives 257 tiles (one workgroup
+    with two, the last tile ragged), 16384 exactly two each, 16400 one tile too many for that form."""
+    M, K, N = shape
+    B = 64
+    a, w, wp, s = _w4a16_inputs(orc, rng(M + K + N), M, K, N, B)
+    y, kernel = _run_w4a16(pkg, a, wp, s, K, N, B)
+    assert kernel == ("mtrt_gemm_w4a16_skinny16" if M <= 16 else "mtrt_gemm_w4a16_skinny")
+    orc.set_threads(16)
+    ref = orc.gemm_w4a16(a, wp, s, K, N, B)
+    orc.set_threads(1)
+    _check_w4a16(orc, y, a, w, s, K, N, B, ref)
+
+
 def test_w4a16_narrow_mid_tile_kernel(pkg, orc):
     """128 x 64 tiles: more 128-wide tiles than compute units, too few 256-wide ones for the large kernel
     (M = 600, N = 8480: 5 x 67 = 335 wide tiles; ragged in M and N), K = 320 (five slices: main loop and tail)."""
