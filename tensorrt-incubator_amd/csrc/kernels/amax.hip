@@ -19,8 +19,8 @@
 // (its pattern is the largest), unlike the host's std::max which would drop it
 // (CoreModule.cpp:540-551); the programs this serves are NaN-free.
 //
-// scratch: (1 + 32) lines of 128 bytes owned by the caller's stream, each holding a
-// (running max, arrival ticket) pair, all zero on entry; whoever arrives last at a
+// scratch: (1 + 32) lines of 128 bytes owned by the caller's stream, each holding an
+// (arrival ticket, running max) pair in its first eight bytes, all zero on entry; whoever arrives last at a
 // pair restores its zeros, so back-to-back launches on one stream need no memset.
 #include "common.hpp"
 
@@ -31,7 +31,7 @@ namespace amax_cluster {
 constexpr int kAmaxThreads = 256;
 constexpr int kAmaxUnroll = 4;     // 128-bit loads in flight per lane per step
 constexpr uint32_t kAmaxFanIn = 32;     // first-level groups of the cross-workgroup arrival tree
-constexpr uint32_t kAmaxLineWords = 32; // one 128-byte line per (max, ticket) pair
+constexpr uint32_t kAmaxLineWords = 32; // one 128-byte line per (ticket, max) pair
 
 template <typename X> struct AbsBits;
 template <> struct AbsBits<F32> {  // returns max over the 4 floats, as f32 bit pattern
@@ -73,23 +73,24 @@ template <> struct AbsBits<F16> {  // 8 f16 per vector; result kept as f16 bit p
   static constexpr int kPerVec = 8;
 };
 
-// One arrival at a (max, ticket) pair.  Device-scope atomics execute at the memory
-// side, the one place all eight XCDs agree on, so no cache write-back or invalidate
-// is needed (an acquire/release pair at device scope would flush and invalidate the
-// XCD's L2 once per workgroup).  Ordering is by completion: the max RETURNS its old
-// value and the empty asm consumes it, so the wave waits for that value before it
-// issues the ticket; every max is therefore performed before the ticket of the same
-// arrival, and all of them before the last ticket.  Returns true for the last of
-// `expected` arrivals, with the combined max in `m`; that caller has also put the
-// pair back to zero.
+// One arrival at a (ticket, max) pair: one 64-bit word, ticket count in the low half, running max in
+// the high half.  Device-scope atomics execute at the memory side, the one place all eight XCDs agree
+// on, so no cache write-back or invalidate is needed (an acquire/release pair at device scope would
+// flush and invalidate the XCD's L2 once per workgroup).  Ordering is by completion: the 32-bit max on
+// the high half RETURNS its old value and the empty asm consumes it, so the wave waits for that value
+// before it issues the 64-bit add that takes the ticket; every max is therefore performed before the
+// ticket of the same arrival, and all of them before the last ticket, whose add returns the whole old
+// word: the last of `expected` arrivals finds the combined max in its high half (two dependent trips
+// to memory per arrival instead of three).  Returns true for that arrival, with the max in `m`; it has
+// also put the word back to zero.
 __device__ __forceinline__ bool arrive(uint32_t* pair, uint32_t expected, uint32_t& m) {
-  const uint32_t before = __hip_atomic_fetch_max(&pair[0], m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const uint32_t before = __hip_atomic_fetch_max(&pair[1], m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __asm__ volatile("" ::"v"(before) : "memory");
-  const uint32_t ticket = __hip_atomic_fetch_add(&pair[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  if (ticket != expected - 1) return false;
-  // read-modify-write, so the value comes from the memory side, not from a cache
-  m = __hip_atomic_exchange(&pair[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __hip_atomic_exchange(&pair[1], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  unsigned long long* word = reinterpret_cast<unsigned long long*>(pair);
+  const unsigned long long old = __hip_atomic_fetch_add(word, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (uint32_t(old) != expected - 1) return false;
+  m = uint32_t(old >> 32);
+  __hip_atomic_exchange(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   return true;
 }
 
