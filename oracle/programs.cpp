@@ -163,7 +163,10 @@ void orc_quantize(const void *x, int in_dtype, void *q, int out_dtype, const flo
   default:
     std::abort();
   }
-#pragma omp parallel for schedule(static)
+  // packed codes: a byte holds elements (2j, 2j+1) of the flattened array, so rows of odd length share
+  // bytes with their neighbours and must not be handed to different threads
+  const bool rows_share_bytes = (out_dtype == ORC_I4_PACKED || out_dtype == ORC_F4_PACKED) && (d1 & 1);
+#pragma omp parallel for schedule(static) if (!rows_share_bytes)
   for (int64_t r = 0; r < d0; ++r) {
     for (int64_t c = 0; c < d1; ++c) {
       const int64_t i = r * d1 + c;
@@ -183,8 +186,6 @@ void orc_quantize(const void *x, int in_dtype, void *q, int out_dtype, const flo
         static_cast<uint8_t *>(q)[i] = uint8_t(int4_saturate(int(std::trunc(v)))) & 0xF;
         break;
       case ORC_I4_PACKED: {
-        // Pairs (2j, 2j+1) of the flattened array share a byte; rows have even
-        // length or the caller pads, so the pair is owned by one thread.
         const uint8_t nib = uint8_t(int4_saturate(int(std::trunc(v)))) & 0xF;
         uint8_t *b = static_cast<uint8_t *>(q) + (i >> 1);
         *b = (i & 1) ? uint8_t((*b & 0x0F) | (nib << 4)) : uint8_t((*b & 0xF0) | nib);

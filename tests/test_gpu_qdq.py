@@ -189,6 +189,33 @@ def test_int4_blockwise(pkg, orc, xname, qname):
     assert "_any_" in k[0]
 
 
+@pytest.mark.parametrize("seed", range(48))
+def test_random_shapes_kinds_and_type_pairs(pkg, orc, seed):
+    """Seeded sweep over scale addressing, extents (aligned and ragged, down to one element), block sizes,
+    type pairs and pointer alignment; a tenth of the values are scaled up so that saturation occurs."""
+    g = rng(9000 + seed)
+    xname = ("f32", "f16", "bf16")[int(g.integers(3))]
+    qname = ("i8", "f8", "i4", "i4p", "f4p")[int(g.integers(5))]
+    kind = (pkg.SCALE_UNIFORM, pkg.SCALE_ROW, pkg.SCALE_COL)[int(g.integers(3))]
+    d0 = int(g.choice([1, 2, 3, 8, 17, 64, 100, 257]))
+    d1 = int(g.choice([1, 2, 7, 8, 16, 24, 64, 120, 128, 255, 512, 1000]))
+    if qname in ("i4p", "f4p") and (d0 * d1) % 2:
+        d1 += 1                                        # packed codes come in pairs
+    if kind == pkg.SCALE_UNIFORM:
+        nb, ns = 1, 1
+    elif kind == pkg.SCALE_ROW:
+        nb = int(g.choice([c for c in (1, 2, 3, 8, d0) if d0 % c == 0]))
+        ns = nb
+    else:
+        nb = int(g.choice([c for c in (1, 2, 8, d0) if d0 % c == 0]))
+        ns = (d0 // nb) * d1
+    x = g.standard_normal((d0, d1), dtype=np.float32)
+    x *= np.where(g.random((d0, d1)) < 0.1, np.float32(40.0), np.float32(1.0))
+    scale = g.uniform(0.01, 0.5, ns).astype(np.float32)
+    misalign = 1 if (kind == pkg.SCALE_UNIFORM and g.random() < 0.3) else 0
+    _check_all(pkg, orc, x, xname, qname, kind, d0, d1, nb, scale, misalign=misalign)
+
+
 def test_ties_saturation_and_special_values(pkg, orc):
     """Inputs that land exactly on k+0.5 after the divide, beyond the clamp, on signed
     zeros and on subnormals; scale chosen so that x/scale is exact."""

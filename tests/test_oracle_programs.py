@@ -68,6 +68,21 @@ def test_quantize_packed_int4_nibble_order(orc):
     assert list(un) == [0, 1, 2, 3, 0xF, 0xE, 0x8, 0x7]      # one per byte, low nibble, upper nibble clear
 
 
+def test_quantize_packed_rows_of_odd_length_with_threads(orc):
+    """Rows of odd length share bytes with their neighbours: the threaded run must equal the nibbles of the
+    one-code-per-byte form (two rows of one element each, the case two threads would split)."""
+    g = rng(61)
+    orc.set_threads(8)
+    try:
+        for _ in range(1500):
+            x = (g.standard_normal((2, 1)) * 3).astype(np.float32)
+            one_per_byte = orc.quantize(x, orc.F32, orc.I4, [np.float32(1)], orc.SCALE_UNIFORM, 2, 1)
+            packed = orc.quantize(x, orc.F32, orc.I4_PACKED, [np.float32(1)], orc.SCALE_UNIFORM, 2, 1)
+            assert packed[0] == (one_per_byte[0] | (one_per_byte[1] << 4))
+    finally:
+        orc.set_threads(1)
+
+
 def test_quantize_fp8_forms(orc):
     import torch
     g = rng(3)
