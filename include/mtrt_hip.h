@@ -100,6 +100,55 @@ MTRT_CAPI_EXPORTED void mtrt_cuda_launch_kernel(mtrt_function_t func, int32_t gr
 MTRT_CAPI_EXPORTED int32_t mtrt_cuda_get_current_device(void);
 MTRT_CAPI_EXPORTED int32_t mtrt_cuda_get_program_device(int32_t logicalId);
 
+/* CUDAModule.h:130-205: the type-erased `<name>_cwrapper` twins that emitted C/C++ calls (every handle
+ * travels as `void *`).  Header-only, as in the reference; each one forwards to the entry point above. */
+#define MTRT_HANDLE(type, p) ((type)(p))
+static inline void *mtrt_cuda_stream_create_cwrapper(void) { return (void *)mtrt_cuda_stream_create(); }
+static inline void mtrt_cuda_stream_destroy_cwrapper(void *stream) {
+  mtrt_cuda_stream_destroy(MTRT_HANDLE(mtrt_stream_t, stream));
+}
+static inline void mtrt_cuda_stream_sync_cwrapper(void *stream) { mtrt_cuda_stream_sync(MTRT_HANDLE(mtrt_stream_t, stream)); }
+static inline void *mtrt_cuda_event_create_cwrapper(int32_t device) { return (void *)mtrt_cuda_event_create(device); }
+static inline void mtrt_cuda_event_release_cwrapper(void *event) { mtrt_cuda_event_release(MTRT_HANDLE(mtrt_event_t, event)); }
+static inline void mtrt_cuda_stream_record_event_cwrapper(void *stream, void *event) {
+  mtrt_cuda_stream_record_event(MTRT_HANDLE(mtrt_stream_t, stream), MTRT_HANDLE(mtrt_event_t, event));
+}
+static inline void mtrt_cuda_stream_wait_event_cwrapper(void *stream, void *event) {
+  mtrt_cuda_stream_wait_event(MTRT_HANDLE(mtrt_stream_t, stream), MTRT_HANDLE(mtrt_event_t, event));
+}
+static inline void mtrt_cuda_event_sync_cwrapper(void *event) { mtrt_cuda_event_sync(MTRT_HANDLE(mtrt_event_t, event)); }
+static inline float mtrt_cuda_event_elapsed_msec_cwrapper(void *start, void *end) {
+  return mtrt_cuda_event_elapsed_msec(MTRT_HANDLE(mtrt_event_t, start), MTRT_HANDLE(mtrt_event_t, end));
+}
+static inline void *mtrt_cuda_alloc_async_cwrapper(void *stream, int64_t size, int32_t alignment, int8_t isHostPinned,
+                                                   int8_t isManaged) {
+  return mtrt_cuda_alloc_async(MTRT_HANDLE(mtrt_stream_t, stream), size, alignment, isHostPinned, isManaged);
+}
+static inline void mtrt_cuda_memcpy_async_cwrapper(void *stream, void *src, void *dest, int64_t size) {
+  mtrt_cuda_memcpy_async(MTRT_HANDLE(mtrt_stream_t, stream), src, dest, size);
+}
+static inline void mtrt_cuda_free_cwrapper(void *stream, void *ptr, int8_t isHostPinned, int8_t isManaged) {
+  mtrt_cuda_free(MTRT_HANDLE(mtrt_stream_t, stream), ptr, isHostPinned, isManaged);
+}
+static inline void *mtrt_cuda_module_load_from_ptx_cwrapper(void *ptxData, size_t ptxLen) {
+  return (void *)mtrt_cuda_module_load_from_ptx((const char *)ptxData, ptxLen);
+}
+static inline void *mtrt_cuda_module_load_from_ptx_file_cwrapper(void *filename, size_t filenameLength) {
+  return (void *)mtrt_cuda_module_load_from_ptx_file((const char *)filename, filenameLength);
+}
+static inline void mtrt_cuda_module_unload_cwrapper(void *module) { mtrt_cuda_module_unload(MTRT_HANDLE(mtrt_module_t, module)); }
+static inline void *mtrt_cuda_module_get_function_cwrapper(void *module, void *name, int64_t length) {
+  return (void *)mtrt_cuda_module_get_function(MTRT_HANDLE(mtrt_module_t, module), (const char *)name, length);
+}
+static inline void mtrt_cuda_launch_kernel_cwrapper(void *func, int32_t gridX, int32_t gridY, int32_t gridZ, int32_t blockX,
+                                                    int32_t blockY, int32_t blockZ, int32_t dynamicSharedMemory,
+                                                    void *stream, void *args) {
+  mtrt_cuda_launch_kernel(MTRT_HANDLE(mtrt_function_t, func), gridX, gridY, gridZ, blockX, blockY, blockZ,
+                          dynamicSharedMemory, MTRT_HANDLE(mtrt_stream_t, stream), (void **)args);
+}
+static inline int32_t mtrt_cuda_get_current_device_cwrapper(void) { return mtrt_cuda_get_current_device(); }
+#undef MTRT_HANDLE
+
 /* ------------------------------------------------------------------------- */
 /* Part 2 — kernel clusters of the quantization hot path                       */
 /* ------------------------------------------------------------------------- */

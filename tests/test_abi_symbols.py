@@ -38,6 +38,21 @@ def test_header_declares_the_reference_names():
         assert name in declared, name
 
 
+def test_header_is_plain_c_and_carries_the_type_erased_twins(tmp_path):
+    """Emitted C calls `<name>_cwrapper(void *...)` (reference CUDAModule.h:130-205): the header must compile
+    as C and define one twin per wrapped entry point."""
+    twins = ["stream_create", "stream_destroy", "stream_sync", "event_create", "event_release", "stream_record_event",
+             "stream_wait_event", "event_sync", "event_elapsed_msec", "alloc_async", "memcpy_async", "free",
+             "module_load_from_ptx", "module_load_from_ptx_file", "module_unload", "module_get_function",
+             "launch_kernel", "get_current_device"]
+    src = tmp_path / "twins.c"
+    body = "".join("  p[%d] = (void *)&mtrt_cuda_%s_cwrapper;\n" % (i, t) for i, t in enumerate(twins))
+    src.write_text('#include "mtrt_hip.h"\nvoid fill(void **p) {\n%s}\n' % body)
+    out = subprocess.run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Wno-pedantic", "-Werror", "-I", os.path.dirname(HEADER),
+                          "-c", str(src), "-o", str(tmp_path / "twins.o")], capture_output=True, text=True)
+    assert out.returncode == 0, out.stderr
+
+
 def test_library_exports_every_declared_symbol(pkg):
     L = pkg.lib()
     for name in _declared():
