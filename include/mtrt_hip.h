@@ -53,6 +53,11 @@ typedef struct mtrt_opaque_event *mtrt_event_t;       /* hipEvent_t    (referenc
 MTRT_CAPI_EXPORTED int32_t mtrt_cuda_get_active_device(void);
 MTRT_CAPI_EXPORTED int32_t mtrt_cuda_set_active_device(int32_t device);
 MTRT_CAPI_EXPORTED int32_t mtrt_cuda_get_device(int32_t device);
+/* Called by the LLVM lowering of cuda.num_devices (CUDAToLLVM.cpp:155-156) but neither declared nor
+ * defined by the reference's C backend; defined here so that such programs link.  The lowering's other
+ * orphan, mtrt_cuda_memcpy_strided_async(stream, rank, descriptor, rank, descriptor) (CUDAToLLVM.cpp:143-150,
+ * 502-513), is NOT provided: the call carries no element size, so the bytes to move are not determined. */
+MTRT_CAPI_EXPORTED int32_t mtrt_cuda_get_device_count(void);
 
 /* CUDAModule.h:61-65.  The reference header declares stream_create without a
  * parameter while its LLVM lowering passes an i32 device

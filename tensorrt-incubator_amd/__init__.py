@@ -34,6 +34,7 @@ PROTOTYPES = {
     "mtrt_cuda_get_active_device": (_i32, []),
     "mtrt_cuda_set_active_device": (_i32, [_i32]),
     "mtrt_cuda_get_device": (_i32, [_i32]),
+    "mtrt_cuda_get_device_count": (_i32, []),
     "mtrt_cuda_stream_create": (_vp, []),
     "mtrt_cuda_stream_destroy": (None, [_vp]),
     "mtrt_cuda_stream_sync": (None, [_vp]),

@@ -62,6 +62,12 @@ int32_t mtrt_cuda_set_active_device(int32_t device) {
 
 int32_t mtrt_cuda_get_device(int32_t device) { return device; }
 
+int32_t mtrt_cuda_get_device_count(void) {
+  int count = 0;
+  MTRT_FATAL_IF_HIP_ERROR(hipGetDeviceCount(&count));
+  return count;
+}
+
 mtrt_stream_t mtrt_cuda_stream_create(void) {
   hipStream_t stream = nullptr;
   MTRT_FATAL_IF_HIP_ERROR(hipStreamCreate(&stream)); // default priority only

@@ -97,6 +97,7 @@ def test_events_and_devices(pkg):
     dev = L.mtrt_cuda_get_current_device()
     assert dev == L.mtrt_cuda_get_active_device() == L.mtrt_cuda_get_program_device(0)
     assert L.mtrt_cuda_get_device(3) == 3
+    assert L.mtrt_cuda_get_device_count() >= 1
     assert L.mtrt_cuda_set_active_device(dev) == dev
     s = L.mtrt_cuda_stream_create()
     e0, e1 = L.mtrt_cuda_event_create(dev), L.mtrt_cuda_event_create(dev)
