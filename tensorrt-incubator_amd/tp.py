@@ -7,6 +7,8 @@ What is mirrored (names, argument meaning, validation order and error text):
   check_qdq_args                             tripy/nvtripy/frontend/ops/utils.py:179-256
   cast (the float8 / int4 routes)            tripy/nvtripy/frontend/ops/cast.py:67-84
   Linear (fake-quant forward)                tripy/nvtripy/frontend/module/linear.py:112-151
+  layernorm / LayerNorm                      tripy/nvtripy/frontend/module/layernorm.py:36-156
+  softmax(input, dim=None)                   tripy/nvtripy/frontend/ops/softmax.py:30-82
   scale from calibration amax                tripy/examples/nanogpt/weight_loader.py:67-68
 
 Tripy builds a trace and hands `tensorrt.quantize` / `tensorrt.dequantize` to TensorRT
@@ -141,6 +143,17 @@ def ones(shape, dtype=float32):
     """An operation result, hence not a constant (tripy/tests/frontend/ops/test_quantize.py:76-84 relies on it).
     Values are made on the host and uploaded on first use by a kernel."""
     return _produced(_torch().ones(tuple(shape), dtype=_torch_dtype(dtype)), dtype)
+
+
+def zeros(shape, dtype=float32):
+    return _produced(_torch().zeros(tuple(shape), dtype=_torch_dtype(dtype)), dtype)
+
+
+def allclose(input, other, rtol=1e-5, atol=1e-8):
+    """|input - other| <= atol + rtol * |other| everywhere (tripy/nvtripy/frontend/ops/allclose.py)."""
+    torch = _torch()
+    a, b = input.device_data().float(), other.device_data().float()
+    return bool(torch.all(torch.abs(a - b) <= atol + rtol * torch.abs(b)))
 
 
 def iota(shape, dim=0, dtype=float32):
@@ -371,3 +384,118 @@ class Linear:
         if self.bias is not None:
             out = out + self.bias.device_data().unsqueeze(0)
         return _produced(out, self.dtype)
+
+
+# ---- fused reduce clusters -----------------------------------------------------------------------
+def _check_float_input(func, input):
+    if input.dtype not in (float32, float16, bfloat16):
+        _invalid_inputs(func, "input.dtype to be one of [float32, float16, bfloat16] (but it was '%s')" % input.dtype)
+
+
+def layernorm(input, weight, bias, eps):
+    """tripy/nvtripy/frontend/module/layernorm.py:36-77: normalises over the last D = weight.rank
+    dimensions, y = (x - mean) * rsqrt(var + eps) * weight + bias, in the input's dtype.  One launch of the
+    LayerNorm cluster over [prod(leading dims), prod(normalized_shape)]."""
+    from . import layernorm as _layernorm_rows
+    for t in (input, weight, bias):
+        if not isinstance(t, Tensor):
+            raise_error("layernorm expects tensors.", ["Got %s" % type(t).__name__])
+    _check_float_input("layernorm", input)
+    if weight.dtype != input.dtype:
+        _invalid_inputs("layernorm", "weight.dtype to be the same as input.dtype (but it was '%s' while input.dtype was '%s')"
+                        % (weight.dtype, input.dtype))
+    if bias.dtype != input.dtype:
+        _invalid_inputs("layernorm", "bias.dtype to be the same as input.dtype (but it was '%s' while input.dtype was '%s')"
+                        % (bias.dtype, input.dtype))
+    normalized_shape = weight.shape
+    D = len(normalized_shape)
+    if input.rank < 2:
+        raise_error(f"Input must have a rank of at least 2, but got input of rank: {input.rank}",
+                    ["Input is expected to have shape (N, *) where N is the batch size, and * represents any number "
+                     "of channel dimension + spatial dimensions"])
+    # what the network builder reports when weight, seen as (1,) * (rank - D) + normalized_shape, does not
+    # broadcast against the input (tripy/tests/frontend/module/test_layernorm.py:24-32)
+    lead = input.rank - D
+    if lead < 0:
+        raise_error("The normalization scale has a higher rank than the input.", [f"scale rank={D}, input rank={input.rank}"])
+    for i, extent in enumerate(normalized_shape):
+        if extent != input.shape[lead + i]:
+            raise_error(f"The normalization scale is not broadcast-compatible with the input at dimension {lead + i}",
+                        [f"input has shape {input.shape}, normalized_shape is {tuple(normalized_shape)}"])
+    if bias.shape != normalized_shape:
+        raise_error("The normalization bias must have the shape of the scale.", [f"bias has shape {bias.shape}"])
+    d = 1
+    for extent in normalized_shape:
+        d *= extent
+    x = input.device_data().contiguous()
+    y = _layernorm_rows(x.reshape(-1, d), weight.device_data().contiguous().reshape(d),
+                        bias.device_data().contiguous().reshape(d), eps)
+    return _produced(y.reshape(input.shape), input.dtype)
+
+
+class DefaultParameter:
+    """A parameter that has to be replaced with real weights before the module runs
+    (tripy/nvtripy/frontend/module/parameter.py:27-34)."""
+
+    def __init__(self, shape, dtype):
+        self.shape, self.dtype = tuple(shape), dtype
+
+
+class LayerNorm:
+    """tripy/nvtripy/frontend/module/layernorm.py:80-156."""
+
+    def __init__(self, normalized_shape, dtype=float32, eps=1e-5):
+        if isinstance(normalized_shape, int):
+            normalized_shape = (normalized_shape,)
+        self.dtype = dtype
+        self.normalized_shape = tuple(normalized_shape)
+        self.weight = DefaultParameter(self.normalized_shape, dtype)
+        self.bias = DefaultParameter(self.normalized_shape, dtype)
+        self.eps = eps
+
+    def initialize_dummy_parameters(self):
+        """Fills parameters that are still placeholders (tripy/nvtripy/frontend/module/module.py, same name)."""
+        if isinstance(self.weight, DefaultParameter):
+            self.weight = ones(self.normalized_shape, self.dtype)
+        if isinstance(self.bias, DefaultParameter):
+            self.bias = zeros(self.normalized_shape, self.dtype)
+
+    def __call__(self, x):
+        return self.forward(x)
+
+    def forward(self, x):
+        for name in ("weight", "bias"):
+            if isinstance(getattr(self, name), DefaultParameter):
+                raise_error(f"Parameter '{name}' of LayerNorm has not been set.",
+                            ["Assign real weights or call initialize_dummy_parameters() first."])
+        if not isinstance(x, Tensor):
+            x = Tensor(x)
+        return layernorm(x, self.weight, self.bias, self.eps)
+
+
+def softmax(input, dim=None):
+    """tripy/nvtripy/frontend/ops/softmax.py:30-82: over `dim`, or over the flattened input when dim is None.
+    The cluster works on rows; another dimension is brought last for the launch and put back."""
+    from . import softmax as _softmax_rows
+    if not isinstance(input, Tensor):
+        input = Tensor(input)
+    _check_float_input("softmax", input)
+    # shapes first (softmax.py:62-76): flatten when dim is None, then at least two dimensions, then process_dim
+    flatten = dim is None
+    seen_shape = (int(np.prod(input.shape, dtype=np.int64)),) if flatten else input.shape
+    if flatten:
+        dim = 0
+    if len(seen_shape) < 2:                            # the softmax layer needs two dimensions
+        seen_shape = tuple(seen_shape) + (1,)
+    rank = len(seen_shape)
+    new_dim = dim + rank if dim < 0 else dim           # tripy/nvtripy/frontend/ops/utils.py:120-138
+    if new_dim < 0 or new_dim >= rank:
+        raise_error("Dimension argument is out of bounds.",
+                    [f"Note: provided dimension was: {dim}, while the tensor has a rank of: {rank}.\n"
+                     f"Dimension should be in the half-open interval: [{-rank}, {rank})."])
+    x = input.device_data().reshape(seen_shape)
+    if new_dim == rank - 1:
+        y = _softmax_rows(x.contiguous())
+    else:
+        y = _softmax_rows(x.movedim(new_dim, -1).contiguous()).movedim(-1, new_dim).contiguous()
+    return _produced(y.reshape(input.shape), input.dtype)

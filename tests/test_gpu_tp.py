@@ -4,6 +4,7 @@ Known answers are those of the reference's integration tests:
   tripy/tests/integration/test_quantize.py:32-43, 58-69, 72-114, 121-145
   tripy/tests/integration/test_dequantize.py:30-79
   tripy/tests/integration/test_linear.py:54-130
+  tripy/tests/integration/test_layernorm.py:24-109, test_softmax.py:18-40
   mlir-tensorrt/integrations/PJRT/test/JAX/CustomPrimitives/test_quantize.py:60-83
 and, on seeded random data, the CPU oracle addressed independently of the mirror (the scale is
 broadcast to the full shape with numpy and the oracle runs per-element on a flat view).
@@ -241,3 +242,61 @@ def test_scale_from_amax(tp, orc):
     a_ref = orc.amax(x, orc.F32)
     assert np.float32(amax.item()).tobytes() == a_ref.tobytes()
     assert np.float32(scale.item()).tobytes() == orc.scale_from_amax(a_ref, 448.0).tobytes()
+
+
+@pytest.mark.parametrize("normalized_shape", [(8, 4, 4), (4, 4)])
+def test_layernorm_module_against_torch(tp, normalized_shape):
+    """tripy/tests/integration/test_layernorm.py:57-109: unit weights give mean 0 / variance 1 over the
+    normalized dimensions; with an affine transformation the result equals torch.nn.LayerNorm to atol 1e-6
+    (f32) / 5e-3 (f16); eps = 0 and inputs U(0, 10) as there."""
+    import torch
+    torch.manual_seed(3)
+    for d, atol in ((tp.float32, 1e-6), (tp.float16, 5e-3)):
+        td = _torch_dtypes(tp)[d]
+        ref = torch.nn.LayerNorm(normalized_shape=normalized_shape, eps=0.0, dtype=td, device="cuda")
+        ln = tp.LayerNorm(normalized_shape=normalized_shape, eps=0.0, dtype=d)
+        x = torch.empty(2, 8, 4, 4, dtype=td, device="cuda").uniform_(0, 10)
+        ln.weight, ln.bias = tp.ones(normalized_shape, dtype=d), tp.zeros(normalized_shape, dtype=d)
+        out = ln(tp.Tensor(x)).torch().float()
+        dims = tuple(range(4 - len(normalized_shape), 4))
+        assert out.mean(dim=dims).abs().mean().item() < 1e-4
+        assert (out.var(dim=dims, unbiased=False) - 1).abs().mean().item() < (1e-4 if d == tp.float32 else 2e-3)
+        torch.nn.init.uniform_(ref.weight, 0.2, 2)
+        torch.nn.init.uniform_(ref.bias, 0.2, 2)
+        ln.weight, ln.bias = tp.Tensor(ref.weight.to("cpu").detach()), tp.Tensor(ref.bias.to("cpu").detach())
+        out = ln(tp.Tensor(x)).torch()
+        with torch.no_grad():
+            expected = ref(x)
+        assert out.shape == expected.shape and out.dtype == expected.dtype
+        assert torch.allclose(out, expected, atol=atol)
+
+
+def test_layernorm_docstring_example(tp):
+    """tripy/nvtripy/frontend/module/layernorm.py:116-133: iota weights and bias on a (2, 3) iota input."""
+    import torch
+    ln = tp.LayerNorm(3)
+    ln.weight, ln.bias = tp.iota(ln.weight.shape), tp.iota(ln.bias.shape)
+    x = tp.iota((2, 3), dim=1)
+    out = ln(x)
+    ref = torch.nn.LayerNorm(3)
+    ref.weight.data, ref.bias.data = ln.weight.torch().cpu(), ln.bias.torch().cpu()
+    assert out.shape == (2, 3)
+    assert np.allclose(out.torch().cpu().numpy(), ref(x.torch().cpu()).detach().numpy())
+
+
+@pytest.mark.parametrize("input_shape, dim", [((2, 2), 0), ((2,), 0), ((2, 2), None), ((2, 2), -1), ((3, 5, 7), 1), ((4,), -1)])
+def test_softmax_against_torch(tp, input_shape, dim):
+    """tripy/tests/integration/test_softmax.py:18-40 (atol 1e-4), plus a middle dimension and the rank-1
+    input with dim = -1, which the reference sees as shape (n, 1): a softmax over one element."""
+    import torch
+    x = tp.iota(input_shape, dtype=tp.float32)
+    out = tp.softmax(x, dim=dim)
+    t = x.torch().cpu()
+    if dim is None:
+        expected = torch.softmax(t.flatten(), 0).reshape(input_shape)
+    elif len(input_shape) == 1 and dim == -1:
+        expected = torch.ones(input_shape)
+    else:
+        expected = torch.softmax(t, dim)
+    assert out.shape == input_shape
+    assert tp.allclose(out, tp.Tensor(expected), atol=1e-4)

@@ -4,6 +4,7 @@ The cases and the expected message fragments are those of the reference's own fr
   tripy/tests/frontend/ops/test_quantize.py:24-85
   tripy/tests/frontend/ops/test_dequantize.py:24-84
   tripy/tests/integration/test_linear.py:88-100 (Linear parameter rejection)
+  tripy/tests/frontend/module/test_layernorm.py:22-45 (LayerNorm shape and rank rejection)
 No kernel is launched: every case fails validation before any device work.
 """
 import importlib
@@ -150,3 +151,38 @@ def test_scale_addressing_modes(tp):
     s0 = tp.Tensor(np.float32(1.0))
     assert from_shape((7, 9), s0, None, "quantize op") == (pkg.SCALE_UNIFORM, 7, 9, 1)
     assert from_shape((), s0, None, "quantize op")[0] == pkg.SCALE_UNIFORM
+
+
+class TestLayerNormAndSoftmax:
+    def test_layernorm_improper_dimensions(self, tp):
+        ln = tp.LayerNorm(normalized_shape=[2, 2])
+        ln.initialize_dummy_parameters()
+        with raises(tp, "The normalization scale is not broadcast-compatible with the input at dimension 1"):
+            ln(tp.ones((5, 5, 5)))
+
+    def test_layernorm_improper_rank(self, tp):
+        ln = tp.LayerNorm(normalized_shape=[2])
+        ln.initialize_dummy_parameters()
+        x = tp.ones((2,))
+        with raises(tp, f"Input must have a rank of at least 2, but got input of rank: {x.rank}"):
+            ln(x)
+
+    def test_layernorm_parameters_and_dtypes(self, tp):
+        ln = tp.LayerNorm(3)
+        assert ln.normalized_shape == (3,) and ln.eps == 1e-5 and ln.dtype == tp.float32
+        assert isinstance(ln.weight, tp.DefaultParameter) and ln.weight.shape == (3,)
+        with raises(tp, "Parameter 'weight' of LayerNorm has not been set."):
+            ln(tp.ones((2, 3)))
+        ln.initialize_dummy_parameters()
+        with raises(tp, "Invalid inputs for function: 'layernorm'."):
+            ln(tp.ones((2, 3), dtype=tp.float16))             # weight dtype differs from the input's
+        with raises(tp, "Invalid inputs for function: 'layernorm'."):
+            tp.layernorm(tp.Tensor([[1, 2, 3]]), ln.weight, ln.bias, 1e-5)   # int32 input
+
+    def test_softmax_rejections(self, tp):
+        with raises(tp, "Invalid inputs for function: 'softmax'."):
+            tp.softmax(tp.Tensor([[1, 2]]), dim=0)
+        with raises(tp, "Dimension argument is out of bounds."):
+            tp.softmax(tp.ones((2, 2)), dim=2)
+        with raises(tp, "Dimension argument is out of bounds."):
+            tp.softmax(tp.ones((2,)), dim=-3)              # a rank-1 input is seen as (2, 1): [-2, 2) is valid
