@@ -115,9 +115,11 @@ struct Frags {
 // writes it out as whole 128-byte row segments, 16 bytes per lane.
 // SLOTS waves own a sub-tile each (slot = wm * NWN + wn, 128 rows x 32*JT columns); `active` is
 // false for waves that only take part in the barriers.
-template <int JT, int NWN, int SLOTS, class Acc, class Epilogue>
-__device__ __forceinline__ void write_tile(Acc (&acc)[4][JT], Epilogue& epi, uint16_t* __restrict__ y, int64_t M, int64_t N,
+// IT (deduced): 32-row tiles per wave; the staging holds 128 rows, taller waves go through it IT / 4 times.
+template <int JT, int NWN, int SLOTS, int IT, class Acc, class Epilogue>
+__device__ __forceinline__ void write_tile(Acc (&acc)[IT][JT], Epilogue& epi, uint16_t* __restrict__ y, int64_t M, int64_t N,
                                            int64_t m0, int64_t n0, int8_t* lds, int slot, bool active) {
+  static_assert(IT % 4 == 0, "waves cover whole groups of 128 rows");
   constexpr int WCOLS = 32 * JT;
   constexpr int HC = JT >= 2 ? 2 : 1;                  // column tiles staged at a time: 64 or 32 columns
   constexpr int CHUNKS = HC * 4;                       // 16-byte chunks per staged row
@@ -131,18 +133,21 @@ __device__ __forceinline__ void write_tile(Acc (&acc)[4][JT], Epilogue& epi, uin
   int8_t* out = lds + slot * kOutWave;
   const bool vec_ok = (N % 8 == 0) && ((reinterpret_cast<uintptr_t>(y) & 15) == 0);
 #pragma unroll
+  for (int ib = 0; ib < IT / 4; ++ib)
+#pragma unroll
   for (int half = 0; half < JT / HC; ++half) {
+    const int wrow = wm * (32 * IT) + ib * 128;         // first row of this pass inside the workgroup's tile
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int lrow = i * 32 + frow;
-      epi.row(wm * 128 + lrow);
+      epi.row(wrow + lrow);
 #pragma unroll
       for (int jj = 0; jj < HC; ++jj)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const int lcol = jj * 32 + q * 8 + fhalf * 4;  // columns lcol .. lcol+3 of this group <-> r = 4q .. 4q+3
           uint32_t bits[4];
-          epi.convert4(acc[i][half * HC + jj], q, wn * WCOLS + half * (32 * HC) + lcol, bits);
+          epi.convert4(acc[ib * 4 + i][half * HC + jj], q, wn * WCOLS + half * (32 * HC) + lcol, bits);
           u32x2 packed;
           packed[0] = bits[0] | (bits[1] << 16);
           packed[1] = bits[2] | (bits[3] << 16);
@@ -153,7 +158,7 @@ __device__ __forceinline__ void write_tile(Acc (&acc)[4][JT], Epilogue& epi, uin
 #pragma unroll
     for (int it = 0; it < 128 * CHUNKS / 64; ++it) {
       const int lrow = it * (64 / CHUNKS) + lane / CHUNKS, ch = lane % CHUNKS;
-      const int64_t row = m0 + wm * 128 + lrow;
+      const int64_t row = m0 + wrow + lrow;
       const int64_t col = n0 + wn * WCOLS + half * (32 * HC) + ch * 8;
       const u32x4 v = *reinterpret_cast<const u32x4*>(out + lrow * kOutRow + ch * 16);
       if (row < M) {

@@ -23,7 +23,7 @@
 //
 // All kernels take the weight fragments straight from global memory into registers and
 // dequantise them there; only the activations go through LDS (direct-to-LDS loads).
-// Large M: 256 x 256 tiles, 8 waves.  Medium M: 128 x 64 tiles so that the grid still fills
+// Large M: 256 x 256 tiles, 4 waves of 256 x 64.  Medium M: 128 x 64 / 128 x 128 tiles so that the grid still fills
 // the chip, 4 waves in two sets that split each K slice.
 // Small M (<= 32): the GEMM is bound by reading the weights once.  One workgroup per
 // 32 columns, its four waves split K, partial tiles are added through LDS at the end.
@@ -110,15 +110,16 @@ struct PlainEpilogue {
 
 // ---- large M, weights straight into registers -------------------------------------------
 // The prepacked stream is already in fragment order, so a wave can load the raw nibbles of
-// its own 128 columns (4 column tiles x 16 B per lane and slice) straight into registers and
+// its own columns (JT column tiles x 16 B per lane and slice) straight into registers and
 // dequantise dword p of each into the B fragment of k-step p: the weights never touch LDS.
-// LDS then carries the activations only (direct-to-LDS loads into a ring of four 32 KiB
-// stages, fetched two slices ahead), which takes the fragment reads, the panel stores and
-// half of the direct-to-LDS traffic of the shared loop off the LDS port; the price is that
-// the two waves of a column half dequantise the same weights.
-// Per k-step a wave issues 16 MFMAs in 8 fenced chunks; each chunk also carries half of one
-// dequantisation (8 VALU instructions) for the next k-step, every other chunk an A fragment
-// read, and in k-step 0 one direct-to-LDS load.  Raw nibbles and scales of slice s+2 are
+// LDS then carries the activations only (direct-to-LDS loads into a ring of 32 KiB
+// stages, fetched two or four slices ahead), which takes the fragment reads, the panel stores and
+// half of the direct-to-LDS traffic of the shared loop off the LDS port; waves that share
+// columns (the row halves of a tile, the two sets that split a slice) dequantise the same weights,
+// which is why the large tile gives each wave all 256 rows of its columns.
+// Per k-step a wave issues IT x JT MFMAs in IT fenced chunks; each chunk also carries an A fragment
+// read for the next k-step, its share of the next weights' dequantisation (13 VALU instructions per
+// fragment) and, in k-step 0, its share of the direct-to-LDS loads.  Raw nibbles and scales of slice s+2 are
 // fetched in the last k-step of slice s into the register set that k-step 2 finished with.
 // D register sets = slices fetched ahead; KEEP: the waves use only part of each vector (see half)
 template <int JT, int D, bool KEEP>
@@ -166,16 +167,17 @@ struct WeightRegs {
 // DEPTH: slices fetched ahead (weight register sets, and activation stages in flight); STAGES: activation
 // stages in LDS, at least DEPTH + 1.  A tile with little work per slice needs the deeper ring: its loads
 // must be issued a memory latency (about 2000 cycles under load) ahead, however few MFMA cycles a slice is.
-template <int MW, int NWN, int JT, int KW, int DEPTH = 2, int STAGES = 4>
+// IT: 32-row tiles per wave (4: 128 rows; 8: 256 rows, one wave per SIMD owning a whole column of the tile).
+template <int MW, int NWN, int JT, int KW, int DEPTH = 2, int STAGES = 4, int IT = 4>
 struct Shape {
-  static constexpr int kMW = MW, kNWN = NWN, kJT = JT, kKW = KW, kDepth = DEPTH, kStages = STAGES;
+  static constexpr int kMW = MW, kNWN = NWN, kJT = JT, kKW = KW, kDepth = DEPTH, kStages = STAGES, kIT = IT;
   static_assert(STAGES >= DEPTH + 1, "the stage being filled must not be one that is read");
   static constexpr int kSlots = MW * NWN, kWaves = KW * kSlots;
-  static constexpr int kBM = 128 * MW, kBN = 32 * JT * NWN;
+  static constexpr int kBM = 32 * IT * MW, kBN = 32 * JT * NWN;
   static constexpr int kStageBytes = kBM * 128;        // one slice of the activation panel
   static constexpr int kRingBytes = STAGES * kStageBytes;
   static constexpr int kOutBytes = kSlots * gemm_core::kOutWave + 2048;
-  static constexpr int kSumBytes = KW == 2 ? kSlots * 128 * 32 * JT * 4 : 0;
+  static constexpr int kSumBytes = KW == 2 ? kSlots * (32 * IT) * 32 * JT * 4 : 0;
   static constexpr int kLds = kRingBytes > kOutBytes ? (kRingBytes > kSumBytes ? kRingBytes : kSumBytes)
                                                      : (kOutBytes > kSumBytes ? kOutBytes : kSumBytes);
 };
@@ -186,20 +188,20 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
                                                 Epilogue& epi, uint16_t* __restrict__ y, int64_t M, int64_t N, int64_t slices,
                                                 int64_t m0, int64_t n0, int8_t* lds, int slot) {
   using namespace gemm_core;
-  constexpr int JT = S::kJT, NWN = S::kNWN, KW = S::kKW, G = (16 * S::kMW) / S::kWaves, NK = 4 / KW;
+  constexpr int JT = S::kJT, NWN = S::kNWN, KW = S::kKW, IT = S::kIT, G = (4 * IT * S::kMW) / S::kWaves, NK = 4 / KW;
   constexpr int D = S::kDepth, NS = S::kStages;
   // loads that may still be in flight when slice s+1 must have landed: those of the slices fetched
   // after it (G direct-to-LDS loads and 2 * JT register loads each) and this slice's own G
   constexpr int kFly = (D - 2) * (G + 2 * JT) + G;
   static_assert(kFly < 64, "wait counter range");
-  static_assert((G == 2 || (G >= 4 && G % 4 == 0)) && G <= 15, "direct-to-LDS loads per wave and slice");
+  static_assert((G < IT || G % IT == 0) && G <= 15, "direct-to-LDS loads per wave and slice, spread over the IT chunks");
   const int lane = threadIdx.x & 63;
   const int wm = slot / NWN;
   const int frow = lane & 31, fhalf = lane >> 5;
 
-  v16f acc[4][JT];
+  v16f acc[IT][JT];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < IT; ++i)
 #pragma unroll
     for (int j = 0; j < JT; ++j) acc[i][j] = F16Traits::zero();
 
@@ -207,11 +209,11 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
   DmaLoaderT<G> al;
   al.init(a, M, a_row_bytes, m0);
   struct FragSet {
-    v4i a[4];
+    v4i a[IT];
     u4 b[JT];
   } f0, f1;
   auto read_a = [&](FragSet& f, const int8_t* pa, int chunk, int i) {
-    f.a[i] = *reinterpret_cast<const v4i*>(pa + lds_off(wm * 128 + i * 32 + frow, chunk));
+    f.a[i] = *reinterpret_cast<const v4i*>(pa + lds_off(wm * (32 * IT) + i * 32 + frow, chunk));
   };
   auto stage = [&](int64_t slice) { return lds + int(uint32_t(slice) % uint32_t(NS)) * S::kStageBytes; };
 
@@ -231,7 +233,7 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
   static_assert(D == 2 || D == 4, "register sets are named at compile time");
   drain_and_barrier();
 #pragma unroll
-  for (int i = 0; i < 4; ++i) read_a(f0, stage(0), 2 * KH + fhalf, i);
+  for (int i = 0; i < IT; ++i) read_a(f0, stage(0), 2 * KH + fhalf, i);
 #pragma unroll
   for (int j = 0; j < JT; ++j) {
     wr.template half<0, KH>(j, 0, f0.b[j]);
@@ -250,17 +252,17 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
     constexpr int NP = kLast ? KH : KH + (T + 1) * KW;
     const int chunk = 2 * NP + fhalf;
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
+    for (int c = 0; c < IT; ++c) {
 #pragma unroll
       for (int j = 0; j < JT; ++j) acc[c][j] = F16Traits::mfma(__builtin_bit_cast(v4i, cur.b[j]), cur.a[c], acc[c][j]);
       read_a(nxt, ra, chunk, c);
 #pragma unroll
       for (int u = 0; u < 2 * JT; ++u)
-        if ((u * 4) / (2 * JT) == c) wr.template half<NSET, NP>(u >> 1, u & 1, nxt.b[u >> 1]);
+        if ((u * IT) / (2 * JT) == c) wr.template half<NSET, NP>(u >> 1, u & 1, nxt.b[u >> 1]);
       if (T == 0) {
-        if constexpr (G >= 4) {
+        if constexpr (G >= IT) {
 #pragma unroll
-          for (int g = 0; g < G / 4; ++g) al.dma(s2, nd, c * (G / 4) + g);
+          for (int g = 0; g < G / IT; ++g) al.dma(s2, nd, c * (G / IT) + g);
         } else {
           if (c < G) al.dma(s2, nd, c);
         }
@@ -304,10 +306,10 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
 
   if (KW == 2) {                                       // second set hands its sums to the first through LDS
     __syncthreads();
-    float* sum = reinterpret_cast<float*>(lds) + slot * (128 * 32 * JT);
+    float* sum = reinterpret_cast<float*>(lds) + slot * ((32 * IT) * 32 * JT);
     if (KH == 1) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < IT; ++i)
 #pragma unroll
         for (int j = 0; j < JT; ++j)
 #pragma unroll
@@ -318,7 +320,7 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
     __syncthreads();
     if (KH == 0) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < IT; ++i)
 #pragma unroll
         for (int j = 0; j < JT; ++j)
 #pragma unroll
@@ -355,8 +357,12 @@ __device__ __forceinline__ void weight_regs_kernel(const uint16_t* __restrict__ 
 
 // (a [M,K] f16, w_prepacked, scale [K/block, N] f16, y [M,N] f16, M, K, N, block) ; K % 64 == 0, block % 64 == 0,
 // a 16-byte aligned and below 4 GiB.  grid = 8 * ceil(ceil(N/256) / 8) * ceil(M/256), block = 256.
-using BigShape = Shape<2, 4, 2, 1>;                    // 256 x 256, 8 waves
-extern "C" __global__ void __launch_bounds__(512, 1) mtrt_gemm_w4a16_t256x256(
+// Four waves, each a whole 256-row column of the tile (256 x 64, one wave per SIMD, 256 accumulator registers):
+// a weight fragment is dequantised once per workgroup and a wave issues 16 MFMAs per k-step.  Against eight
+// waves of 128 x 64 (every weight fragment dequantised by two waves) in one process: 343 -> 330 us at
+// M = 4096, 94.9 -> 92.3 us at M = 1024, same bits.
+using BigShape = Shape<1, 4, 2, 1, 2, 4, 8>;           // 256 x 256, 4 waves
+extern "C" __global__ void __launch_bounds__(256, 1) mtrt_gemm_w4a16_t256x256(
     const uint16_t* __restrict__ a, const uint32_t* __restrict__ wp, const uint16_t* __restrict__ scale,
     uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t block) {
   __shared__ __attribute__((aligned(16))) int8_t lds[BigShape::kLds];

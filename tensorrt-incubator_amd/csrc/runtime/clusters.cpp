@@ -479,12 +479,12 @@ int32_t mtrt_hip_gemm_w4a16(mtrt_stream_t stream, const void *a, const void *w_k
       const uint32_t grid = uint32_t(M > 8 && tiles > cus && tiles <= 2 * cus ? cus : tiles);
       return launch(st, M <= 16 ? "mtrt_gemm_w4a16_skinny16" : "mtrt_gemm_w4a16_skinny", grid, kBlock, as_hip(stream), args);
     }
-    // 256 x 256 tiles (512 threads) once they cover at least half of the compute units (measured:
+    // 256 x 256 tiles (256 threads) once they cover at least half of the compute units (measured:
     // from M = 1024 on at N = 11008 they beat the small tiles) and the activations stay inside
     // 32-bit byte offsets; 128 x 64 tiles otherwise.
     const int64_t panels = (N + 255) / 256, tiles_m = (M + 255) / 256;
     if (panels * tiles_m * 2 >= int64_t(num_compute_units(st)) && M * K * 2 < (int64_t(1) << 32))
-      return launch(st, "mtrt_gemm_w4a16_t256x256", uint32_t(8 * ((panels + 7) / 8) * tiles_m), 512, as_hip(stream),
+      return launch(st, "mtrt_gemm_w4a16_t256x256", uint32_t(8 * ((panels + 7) / 8) * tiles_m), 256, as_hip(stream),
                     args);
     if (M * K * 2 < (int64_t(1) << 32)) {
       // 128-row tiles: 128 columns wide while that leaves every compute unit at most one workgroup, else 64
