@@ -275,9 +275,14 @@ int32_t mtrt_hip_layernorm(mtrt_stream_t stream, const void *x, const void *gamm
   int64_t rows_arg = rows, d_arg = d;
   float eps_arg = eps;
   void *args[] = {&x, &gamma, &beta, &y, &rows_arg, &d_arg, &eps_arg};
-  if (nv)
-    return launch(st, std::string("mtrt_layernorm_") + xn + "_v" + std::to_string(nv),
+  if (nv) {
+    // One wave per row.  The eight-vector kernel runs five waves per SIMD; when that leaves a second, partly
+    // filled round and eight waves per SIMD would hold every row at once, its 64-register form is faster.
+    const int64_t simds = int64_t(num_compute_units(st)) * 4;
+    const bool resident = nv == 8 && rows > 5 * simds && rows <= 8 * simds;
+    return launch(st, std::string("mtrt_layernorm_") + xn + "_v" + std::to_string(nv) + (resident ? "r" : ""),
                   blocks_for(rows, kBlock / 64), kBlock, as_hip(stream), args);
+  }
   return launch(st, std::string("mtrt_layernorm_") + xn + "_any",
                 uint32_t(std::min<int64_t>(rows, int64_t(num_compute_units(st)) * 8)), kBlock, as_hip(stream), args);
 }

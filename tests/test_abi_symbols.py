@@ -82,6 +82,7 @@ def test_embedded_code_object_is_gfx950_and_has_the_kernels(pkg):
         names.append("mtrt_amax_" + x)
         for v in ("v1", "v2", "v4", "v8", "v16", "any"):
             names += ["mtrt_layernorm_%s_%s" % (x, v), "mtrt_softmax_%s_%s" % (x, v)]
+        names.append("mtrt_layernorm_%s_v8r" % x)
     names.append("mtrt_copy_b128")
     for n in names:
         assert n.encode() + b"\x00" in blob, "kernel %s is not in the code object" % n

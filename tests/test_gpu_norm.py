@@ -110,7 +110,7 @@ def _run_softmax(pkg, orc, name, rows, d, seed, expect_kernel=None, frac=2e-2, s
 def test_c2a_layernorm_bf16_full_size(pkg, orc):
     """BASELINE config 2a: bf16 [8192,4096], x~N(0,1), gamma~U(0.5,1.5), beta~N(0,0.1), eps 1e-5, seed 2."""
     orc.set_threads(16)
-    _run_layernorm(pkg, orc, "bf16", 8192, 4096, 2, "mtrt_layernorm_bf16_v8")
+    _run_layernorm(pkg, orc, "bf16", 8192, 4096, 2, "mtrt_layernorm_bf16_v8" + ("r" if _resident(8192) else ""))
     orc.set_threads(1)
 
 
@@ -134,6 +134,47 @@ def test_layernorm_shapes(pkg, orc, name, shape):
 @pytest.mark.parametrize("shape", [(5, 8), (33, 512), (7, 1000), (3, 4104), (2, 8192), (9, 16384), (4, 331), (1, 1), (6, 40000)])
 def test_softmax_shapes(pkg, orc, name, shape):
     _run_softmax(pkg, orc, name, shape[0], shape[1], 40 + shape[1] % 97)
+
+
+def _resident(rows):
+    """The dispatch rule of the eight-vector LayerNorm: the 64-register kernel when eight waves per SIMD hold
+    every row at once and five would not."""
+    import torch
+    simds = 4 * torch.cuda.get_device_properties(0).multi_processor_count
+    return 5 * simds < rows <= 8 * simds
+
+
+def test_layernorm_resident_variant_window_and_bits(pkg, orc):
+    """Both eight-vector kernels run the same arithmetic: rows just inside the window (64-register kernel)
+    give the bits of the same rows launched below it (default kernel); the window's edges pick the kernels."""
+    import torch
+    simds = 4 * torch.cuda.get_device_properties(0).multi_processor_count
+    d = 4096
+    torch.manual_seed(5)
+    g = (torch.rand(d, device="cuda") + 0.5).to(torch.bfloat16)
+    b = (torch.randn(d, device="cuda") * 0.1).to(torch.bfloat16)
+    x = torch.randn(8 * simds + 1, d, device="cuda").to(torch.bfloat16)
+    lo = pkg.layernorm(x[:5 * simds], g, b, 1e-5)
+    assert pkg.last_kernel() == "mtrt_layernorm_bf16_v8"
+    mid = pkg.layernorm(x[:5 * simds + 1], g, b, 1e-5)
+    assert pkg.last_kernel() == "mtrt_layernorm_bf16_v8r"
+    top = pkg.layernorm(x[:8 * simds], g, b, 1e-5)
+    assert pkg.last_kernel() == "mtrt_layernorm_bf16_v8r"
+    over = pkg.layernorm(x, g, b, 1e-5)
+    assert pkg.last_kernel() == "mtrt_layernorm_bf16_v8"
+    assert torch.equal(lo.view(torch.int16), mid[:5 * simds].view(torch.int16))
+    assert torch.equal(top.view(torch.int16), over[:8 * simds].view(torch.int16))
+    assert torch.equal(lo.view(torch.int16), over[:5 * simds].view(torch.int16))
+    # a ragged row length (not all 64 * 8 vectors used) through the 64-register kernel
+    d2 = 4000
+    x2 = torch.randn(5 * simds + 7, d2, device="cuda").to(torch.float16)
+    g2 = (torch.rand(d2, device="cuda") + 0.5).half()
+    b2 = (torch.randn(d2, device="cuda") * 0.1).half()
+    a = pkg.layernorm(x2, g2, b2, 1e-5)
+    assert pkg.last_kernel() == "mtrt_layernorm_f16_v8r"
+    c = pkg.layernorm(x2[:100], g2, b2, 1e-5)
+    assert pkg.last_kernel() == "mtrt_layernorm_f16_v8"
+    assert torch.equal(a[:100].view(torch.int16), c.view(torch.int16))
 
 
 def test_kernel_selection(pkg, orc):
