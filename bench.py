@@ -306,6 +306,56 @@ def time_kernel(pkg, torch, w, reps):
     return us
 
 
+def cache_variants(pkg, torch, wl, which, reps):
+    """The two configurations that fit in the 256 MiB Infinity Cache (C1: 38 MB, C2b: 67 MB), measured two more
+    ways beside the rotating-buffer ("cold") figure of the main table: "warm" (one buffer set launched again and
+    again, so it stays in the cache) and the same kernels on 16 times the rows (too large for the cache)."""
+    L = pkg.lib()
+    dev = torch.device("cuda:0")
+
+    def stream():
+        return torch.cuda.current_stream().cuda_stream
+    out = []
+    for w in wl:
+        if w["config"] in ("C1", "C2b"):
+            us = time_kernel(pkg, torch, dict(w, nslots=1), reps)
+            out.append(dict(kernel=w["name"], config=w["config"] + " warm (one buffer set)", us=round(us, 2),
+                            achieved=round(w["work"] / us / 1e3, 1), unit="GB/s"))
+    if which in ("all", "c1"):
+        rows, cols = 16 * 1024, 4096
+        n = rows * cols
+        x = [torch.randn((rows, cols), device=dev) for _ in range(2)]
+        q = [torch.empty(n, dtype=torch.int8, device=dev) for _ in range(2)]
+        y = [torch.empty_like(t) for t in x]
+        sc = [torch.empty(2, dtype=torch.float32, device=dev) for _ in range(2)]
+
+        def amax(i):
+            a = (x[i].data_ptr(), pkg.F32, n, 127.0, sc[i].data_ptr(), sc[i].data_ptr() + 4)
+            return lambda: pkg.check(L.mtrt_hip_amax(stream(), *a))
+
+        def qdq(i):
+            a = (x[i].data_ptr(), pkg.F32, q[i].data_ptr(), pkg.I8, y[i].data_ptr(), sc[i].data_ptr() + 4, pkg.SCALE_UNIFORM,
+                 rows, cols, 1, 0)
+            return lambda: pkg.check(L.mtrt_hip_quantize_dequantize(stream(), *a))
+        for name, make, work in (("mtrt_amax_f32", amax, 4.0 * n), ("mtrt_qdq_uniform_f32_i8", qdq, 9.0 * n)):
+            us = time_kernel(pkg, torch, dict(make=make, nslots=2), max(10, reps // 4))
+            out.append(dict(kernel=name, config="C1 x16 rows [16384, 4096]", us=round(us, 2), achieved=round(work / us / 1e3, 1),
+                            unit="GB/s"))
+        del x, q, y
+    if which in ("all", "c2b"):
+        rows, d = 16 * 4096, 4096
+        x = [(torch.randn((rows, d), device=dev) * 2.0).half() for _ in range(2)]
+        y = [torch.empty_like(t) for t in x]
+
+        def sm(i):
+            a = (x[i].data_ptr(), y[i].data_ptr(), pkg.F16, rows, d)
+            return lambda: pkg.check(L.mtrt_hip_softmax(stream(), *a))
+        us = time_kernel(pkg, torch, dict(make=sm, nslots=2), max(10, reps // 4))
+        out.append(dict(kernel="mtrt_softmax_f16_v8", config="C2b x16 rows [65536, 4096]", us=round(us, 2),
+                        achieved=round(4.0 * rows * d / us / 1e3, 1), unit="GB/s"))
+    return out
+
+
 def cpu_baseline(which):
     """Times the CPU oracle single-threaded on a bounded sample of each program and
     extrapolates linearly to the full configuration; returns (seconds per step, description)."""
@@ -449,6 +499,9 @@ def main():
                            "not reached on non-zero data (power limit)"},
         "workloads": kernels,
     }
+    variants = cache_variants(pkg, torch, wl, args.workload, args.kernel_reps)
+    if variants:
+        line["cache_variants"] = variants
     if not args.no_cpu_baseline:
         cpu_s, sample = cpu_baseline(args.workload)
         line["cpu_baseline"] = {"value": round(100.0 * (ideal_us / 1e6) / cpu_s, 6),
