@@ -430,6 +430,8 @@ def main():
     ap.add_argument("--workload", default="all", choices=["all", "c1", "c2a", "c2b", "c3", "c4", "c5", "nvfp4"])
     ap.add_argument("--kernel-reps", type=int, default=100, help="launches per kernel for the per-kernel timing")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-cache-variants", action="store_true",
+                    help="skip the warm-cache and 16x-rows launches (they reuse kernel names: keeps a profile's per-kernel averages clean)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: every box of this build has one, and the hot path has no "
@@ -499,7 +501,7 @@ def main():
                            "not reached on non-zero data (power limit)"},
         "workloads": kernels,
     }
-    variants = cache_variants(pkg, torch, wl, args.workload, args.kernel_reps)
+    variants = [] if args.no_cache_variants else cache_variants(pkg, torch, wl, args.workload, args.kernel_reps)
     if variants:
         line["cache_variants"] = variants
     if not args.no_cpu_baseline:

@@ -169,7 +169,8 @@ __device__ __forceinline__ void layernorm_rows(const typename X::storage* __rest
                                                const typename X::storage* __restrict__ gamma,
                                                const typename X::storage* __restrict__ beta,
                                                typename X::storage* __restrict__ y, int64_t rows, int64_t d, float eps) {
-  const int64_t row = int64_t(blockIdx.x) * kRowsPerBlock + threadIdx.x / kWave;
+  // the wave index as a scalar: the row pointers are then wave-uniform and the accesses need one lane offset, not an address pair each
+  const int64_t row = int64_t(blockIdx.x) * kRowsPerBlock + __builtin_amdgcn_readfirstlane(int(threadIdx.x / kWave));
   if (row >= rows) return;                           // whole wave leaves together
   if (d == int64_t(Vec<X>::kElems) * kWave * NV)
     layernorm_row<X, NV, true>(x, gamma, beta, y, row, d, eps);
@@ -216,7 +217,8 @@ __device__ __forceinline__ void softmax_row(const typename X::storage* __restric
 template <typename X, int NV>
 __device__ __forceinline__ void softmax_rows(const typename X::storage* __restrict__ x, typename X::storage* __restrict__ y,
                                              int64_t rows, int64_t d) {
-  const int64_t row = int64_t(blockIdx.x) * kRowsPerBlock + threadIdx.x / kWave;
+  // the wave index as a scalar: the row pointers are then wave-uniform and the accesses need one lane offset, not an address pair each
+  const int64_t row = int64_t(blockIdx.x) * kRowsPerBlock + __builtin_amdgcn_readfirstlane(int(threadIdx.x / kWave));
   if (row >= rows) return;
   if (d == int64_t(Vec<X>::kElems) * kWave * NV)
     softmax_row<X, NV, true>(x, y, row, d);
@@ -288,8 +290,13 @@ using namespace norm_cluster;
 // [4096, 4096] 11.3 -> 12.7 us and [16384, 4096] 47.4 -> 50.4 us, hence only inside that window).
 // Entry points.  mtrt_layernorm_<t>_v<NV>(x, gamma, beta, y, rows, d, eps)
 //                mtrt_softmax_<t>_v<NV>(x, y, rows, d)         NV = vectors per lane
+#define MTRT_LN_OCCUPANCY_1
+#define MTRT_LN_OCCUPANCY_2
+#define MTRT_LN_OCCUPANCY_4
+#define MTRT_LN_OCCUPANCY_8 __attribute__((amdgpu_waves_per_eu(5, 5)))
+#define MTRT_LN_OCCUPANCY_16
 #define MTRT_NORM_KERNELS(XN, XT, NV)                                                                         \
-  extern "C" __global__ void __launch_bounds__(kNormThreads) mtrt_layernorm_##XN##_v##NV(                      \
+  extern "C" __global__ void __launch_bounds__(kNormThreads) MTRT_LN_OCCUPANCY_##NV mtrt_layernorm_##XN##_v##NV(                      \
       const XT::storage* x, const XT::storage* gamma, const XT::storage* beta, XT::storage* y, int64_t rows,  \
       int64_t d, float eps) { layernorm_rows<XT, NV>(x, gamma, beta, y, rows, d, eps); }                      \
   extern "C" __global__ void __launch_bounds__(kNormThreads) mtrt_softmax_##XN##_v##NV(                        \
