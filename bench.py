@@ -184,9 +184,17 @@ def build_workloads(pkg, torch, which):
         def gemm8(i, a4=a4, w4=w4, y4=y4, as4=as4, ws4=ws4, M=M, K=K, N=N):
             a = (a4[i].data_ptr(), w4[i].data_ptr(), as4.data_ptr(), ws4.data_ptr(), y4[i].data_ptr(), M, K, N)
             return lambda: pkg.check(L.mtrt_hip_gemm_w8a8_fragments(stream(), *a))
+        # the same launch on all-zero operands: same instructions and memory traffic, no switching activity in the
+        # matrix cores; the difference to the timed launch is what the board's power limit costs on this data
+        az = torch.zeros((M, K), dtype=torch.int8, device=dev)
+        wz = torch.zeros_like(w4[0])
+
+        def gemm8_zero(i, az=az, wz=wz, y4=y4, as4=as4, ws4=ws4, M=M, K=K, N=N):
+            a = (az.data_ptr(), wz.data_ptr(), as4.data_ptr(), ws4.data_ptr(), y4[i].data_ptr(), M, K, N)
+            return lambda: pkg.check(L.mtrt_hip_gemm_w8a8_fragments(stream(), *a))
         out.append(dict(name="mtrt_gemm_w8a8_frag", config="C4", bound="mfma", work=2.0 * M * K * N, peak=INT8_PEAK,
-                        unit="TOP/s", nslots=ns, make=gemm8, keep=(a4, w4, y4, as4, ws4),
-                        probe=("mtrt_mfma_probe_i8", w4[0], 65536.0)))
+                        unit="TOP/s", nslots=ns, make=gemm8, keep=(a4, w4, y4, as4, ws4, az, wz),
+                        probe=("mtrt_mfma_probe_i8", w4[0], 65536.0), zero_operands=gemm8_zero))
 
     if which in ("all", "c5"):
         K, N, B = 4096, 11008, 128
@@ -208,9 +216,17 @@ def build_workloads(pkg, torch, which):
                 out.append(dict(name=kname, config="C5 M=16", bound="hbm", work=float(nbytes), nslots=ns, make=gemm4,
                                 keep=(a5, w5, s5, y5)))
             else:
+                zero = None
+                if M == 4096:    # the same launch with zero activations and zero weights (nibble 8 is the value 0)
+                    az5 = torch.zeros((M, K), dtype=torch.float16, device=dev)
+                    wz5 = torch.full_like(w5[0], 0x88)
+
+                    def zero(i, az5=az5, wz5=wz5, s5=s5, y5=y5, M=M):
+                        a = (az5.data_ptr(), None, wz5.data_ptr(), s5[i].data_ptr(), y5[i].data_ptr(), M, K, N, B)
+                        return lambda: pkg.check(L.mtrt_hip_gemm_w4a16(stream(), *a))
                 out.append(dict(name=kname, config="C5 M=%d" % M, bound="mfma", work=2.0 * M * K * N, peak=F16_PEAK,
                                 unit="TFLOP/s", nslots=ns, make=gemm4, keep=(a5, w5, s5, y5),
-                                probe=("mtrt_mfma_probe_f16", a5[0], 32768.0) if M == 4096 else None))
+                                probe=("mtrt_mfma_probe_f16", a5[0], 32768.0) if M == 4096 else None, zero_operands=zero))
 
     for w in out:
         w["peak"] = HBM_PEAK if w["bound"] == "hbm" else w["peak"]
@@ -501,6 +517,10 @@ def main():
                            "not reached on non-zero data (power limit)"},
         "workloads": kernels,
     }
+    if not args.no_cache_variants:
+        for w, k in zip(wl, kernels):
+            if w.get("zero_operands"):
+                k["us_on_zero_operands"] = round(time_kernel(pkg, torch, dict(w, make=w["zero_operands"]), args.kernel_reps), 2)
     variants = [] if args.no_cache_variants else cache_variants(pkg, torch, wl, args.workload, args.kernel_reps)
     if variants:
         line["cache_variants"] = variants
