@@ -226,6 +226,19 @@ MTRT_CAPI_EXPORTED const char *mtrt_hip_builtin_code_object(size_t *size);
 MTRT_CAPI_EXPORTED int32_t mtrt_hip_amax(mtrt_stream_t stream, const void *x, int32_t dtype,
                                          int64_t n, float qmax, float *amax_out, float *scale_out);
 
+/* mtrt_hip_amax for callers that cannot allocate device memory (code under stream capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same operands and
+ * results as mtrt_hip_amax; the reduction's scratch block (5 KiB) is a device array inside this library,
+ * one copy per GPU, cleared by a small fill kernel at the start of each call.  The call itself allocates
+ * nothing, but mtrt_hip_init() must have run on the current device before (it loads the kernels and looks
+ * the array's address up); otherwise MTRT_RUNTIME_ERROR.  n above MTRT_HIP_AMAX_NO_ALLOC_MAX_ELEMENTS
+ * is MTRT_INVALID_ARGUMENT.  All calls on one GPU share the block: calls that overlap in time on one GPU
+ * (different streams) race; serialise them. */
+#define MTRT_HIP_AMAX_NO_ALLOC_MAX_ELEMENTS ((int64_t)1 << 36)
+MTRT_CAPI_EXPORTED int32_t mtrt_hip_amax_no_alloc(mtrt_stream_t stream, const void *x, int32_t dtype,
+                                                  int64_t n, float qmax, float *amax_out,
+                                                  float *scale_out);
+
 /* tensorrt.quantize semantics (TensorRTOps.td:3133-3194) in the StableHLO form
  * of StablehloRaiseQDQ.cpp:233-265: q = convert(clamp(lo, rne(f32(x) / scale), hi)).
  * x_dtype in {F32,F16,BF16}; q_dtype in {I8,F8E4M3FN,I4,I4_PACKED,F4_PACKED}; scale is f32. */

@@ -62,6 +62,14 @@ def build_runtime():
     rdir = os.path.join(CSRC, "runtime")
     srcs = sorted(os.path.join(rdir, f) for f in os.listdir(rdir) if f.endswith(".cpp"))
     hsaco = os.path.join(LIB, "mtrt_kernels.hsaco")
+    # Host files that own device-side objects (a device array whose address the host looks up) are
+    # compiled by hipcc as ordinary HIP translation units and linked in as objects.
+    for f in sorted(os.listdir(rdir)):
+        if f.endswith(".hip"):
+            obj = os.path.join(LIB, f[:-4] + ".o")
+            _run([hipcc(), "-c", "-fPIC", "-fvisibility=hidden"] + DEVICE_FLAGS + EXACT_FLAGS +
+                 ["-I" + os.path.join(ROOT, "include"), os.path.join(rdir, f), "-o", obj])
+            srcs.append(obj)
     _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-Wall", "-Wextra",
           "-D__HIP_PLATFORM_AMD__", '-DMTRT_HSACO_PATH="%s"' % hsaco,
           "-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(ROCM, "include")] + srcs +

@@ -134,6 +134,12 @@ DeviceState *device_state() {
     delete st;
     return nullptr;
   }
+  if (no_alloc_setup(st, device) != MTRT_OK) {
+    (void)hipFree(st->slots);
+    (void)hipModuleUnload(st->module);
+    delete st;
+    return nullptr;
+  }
   g_states[device] = st;
   return st;
 }

@@ -36,6 +36,10 @@ hipFunction_t find_kernel(DeviceState *, const std::string &name);   // nullptr 
 uint32_t *reduction_slot(DeviceState *, hipStream_t stream);         // nullptr + set_error
 void forget_stream(hipStream_t stream);
 
+// Set-up half of the allocation-free entry point (no_alloc.hip): looks up, with `device` current, the
+// device address of that file's scratch array and the kernel handles it launches.
+int32_t no_alloc_setup(DeviceState *, int device);
+
 // Launch through the same driver call as mtrt_cuda_launch_kernel, returning a status.
 int32_t launch(DeviceState *, const std::string &kernel, uint32_t grid, uint32_t block,
                hipStream_t stream, void **args);
