@@ -226,6 +226,14 @@ MTRT_CAPI_EXPORTED const char *mtrt_hip_builtin_code_object(size_t *size);
 MTRT_CAPI_EXPORTED int32_t mtrt_hip_amax(mtrt_stream_t stream, const void *x, int32_t dtype,
                                          int64_t n, float qmax, float *amax_out, float *scale_out);
 
+/* Grid reductions (mtrt_hip_amax and the kernels that fold an amax into another pass) meet in a small
+ * block of device memory that the library keeps per stream and that every launch leaves zeroed.  A launch
+ * that did not run to completion (a device fault, a killed process sharing the context) can leave it
+ * non-zero; this call clears the block of `stream` in stream order.  Blocks are also cleared when first
+ * bound to a stream and return to the pool when the stream is destroyed through any of the stream-destroy
+ * entry points of this library. */
+MTRT_CAPI_EXPORTED int32_t mtrt_hip_reset_reductions(mtrt_stream_t stream);
+
 /* mtrt_hip_amax for callers that cannot allocate device memory (code under stream capture, tight
  * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same operands and
  * results as mtrt_hip_amax; the reduction's scratch block (5 KiB) is a device array inside this library,
@@ -391,7 +399,9 @@ MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_alloc_host_pinned(uint64_t nbytes, int3
 MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_free_host_pinned(uintptr_t stream, uintptr_t ptr);
 /* __cuda_memcpy_strided_async_{device2device,device2host,host2device}(stream, rank, elemSize, src, srcOffset,
  * srcShapeAndStrides, dst, dstOffset, dstShapeAndStrides) (CUDAModule.cpp:210-255): shapes then strides, in
- * elements, `rank` values each; offsets in bytes.  Issued as one copy per contiguous run. */
+ * elements, `rank` values each; the offsets are memref offsets, in ELEMENTS as well (the copy starts at
+ * pointer + offset * elemSize, mlir-tensorrt/executor/lib/Support/StridedCopy.cpp:37-38).  Issued as one copy
+ * per contiguous run. */
 MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_memcpy_strided(uintptr_t stream, int64_t rank, int64_t elemSize,
                                                         uintptr_t src, uint64_t srcOffset,
                                                         const int64_t *srcShapeAndStrides, uintptr_t dst,

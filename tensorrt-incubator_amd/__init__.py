@@ -84,6 +84,7 @@ PROTOTYPES = {
     "mtrt_hip_builtin_module": (_vp, []),
     "mtrt_hip_builtin_code_object": (_vp, [_c.POINTER(_sz)]),
     "mtrt_hip_amax": (_i32, [_vp, _vp, _i32, _i64, _f32, _vp, _vp]),
+    "mtrt_hip_reset_reductions": (_i32, [_vp]),
     "mtrt_hip_amax_no_alloc": (_i32, [_vp, _vp, _i32, _i64, _f32, _vp, _vp]),
     "mtrt_hip_quantize": (_i32, [_vp, _vp, _i32, _vp, _i32, _vp, _i32, _i64, _i64, _i64, _i32]),
     "mtrt_hip_dequantize": (_i32, [_vp, _vp, _i32, _vp, _i32, _vp, _i32, _i64, _i64, _i64]),

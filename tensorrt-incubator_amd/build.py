@@ -79,7 +79,8 @@ def build_runtime():
 
 def build_selftest():
     src = os.path.join(CSRC, "selftest", "standalone_selftest.cpp")
-    _run(["g++", "-O1", "-std=c++17", "-Wall", "-Wextra", "-I" + os.path.join(ROOT, "include"), src,
+    # include/standalone holds the reference's header NAMES (MTRTRuntimeCuda.h ...), as generated code includes them
+    _run(["g++", "-O1", "-std=c++17", "-Wall", "-Wextra", "-I" + os.path.join(ROOT, "include", "standalone"), src,
           "-L" + LIB, "-lmtrt_hip", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + os.path.join(ROCM, "lib"),
           "-o", os.path.join(LIB, "mtrt_standalone_selftest")])
 

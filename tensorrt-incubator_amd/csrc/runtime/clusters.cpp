@@ -18,6 +18,10 @@ namespace {
 constexpr int kTile = 16;           // elements per lane per trip in qdq.hip
 constexpr uint32_t kBlock = 256;
 constexpr uint32_t kMaxGrid = 1u << 20;
+// The one-wave-per-row kernels (layernorm / softmax `_v*`) map rows to waves from the workgroup index and do
+// not loop, so their grid must cover every row: ceil(rows / 4) workgroups, which blocks_for() caps at
+// kMaxGrid.  Tensors with more rows take the `_any` kernels, which loop over rows.
+constexpr int64_t kMaxRowsPerWaveKernels = int64_t(kMaxGrid) * (kBlock / 64);
 
 const char *float_name(int32_t dt) {
   switch (dt) {
@@ -95,8 +99,10 @@ int32_t qdq_dispatch(int mode, hipStream_t stream, const void *x, int32_t x_dtyp
   const bool nibbles = q_dtype == MTRT_I4_PACKED || q_dtype == MTRT_F4_PACKED;
   const uintptr_t q_align = nibbles ? group / 2 : group;
   bool tiles = aligned(q, q_align) && (mode == 1 || aligned(x, 16)) && (mode == 0 || aligned(y, 16));
+  // The row- and column-scaled group kernels keep group, row and scale-block indices in 32 bits; a tensor
+  // beyond that (64 GiB of f32 and more) takes the element-wise kernel, which indexes in 64 bits throughout.
   if (kind != MTRT_SCALE_UNIFORM)
-    tiles = tiles && (d1 % group == 0);
+    tiles = tiles && (d1 % group == 0) && n / group < (int64_t(1) << 32) && nb < (int64_t(1) << 32);
   if (kind == MTRT_SCALE_COL)
     tiles = tiles && aligned(scale, 16);
 
@@ -275,7 +281,7 @@ int32_t mtrt_hip_layernorm(mtrt_stream_t stream, const void *x, const void *gamm
   int64_t rows_arg = rows, d_arg = d;
   float eps_arg = eps;
   void *args[] = {&x, &gamma, &beta, &y, &rows_arg, &d_arg, &eps_arg};
-  if (nv) {
+  if (nv && rows <= kMaxRowsPerWaveKernels) {
     // One wave per row.  The eight-vector kernel runs five waves per SIMD; when that leaves a second, partly
     // filled round and eight waves per SIMD would hold every row at once, its 64-register form is faster.
     const int64_t simds = int64_t(num_compute_units(st)) * 4;
@@ -309,7 +315,7 @@ int32_t mtrt_hip_softmax(mtrt_stream_t stream, const void *x, void *y, int32_t d
   const int nv = vec_ok ? pick_nv(d / per_vec) : 0;
   int64_t rows_arg = rows, d_arg = d;
   void *args[] = {&x, &y, &rows_arg, &d_arg};
-  if (nv)
+  if (nv && rows <= kMaxRowsPerWaveKernels)
     return launch(st, std::string("mtrt_softmax_") + xn + "_v" + std::to_string(nv),
                   blocks_for(rows, kBlock / 64), kBlock, as_hip(stream), args);
   return launch(st, std::string("mtrt_softmax_") + xn + "_any",

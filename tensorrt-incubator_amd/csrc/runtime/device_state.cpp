@@ -13,6 +13,7 @@
 #include <map>
 #include <mutex>
 #include <unordered_map>
+#include <vector>
 
 #ifndef MTRT_HSACO_PATH
 #error "MTRT_HSACO_PATH must name the code object to embed"
@@ -83,6 +84,7 @@ struct DeviceState {
   static constexpr int kSlotWords = 40 * 32;
   uint32_t *slots = nullptr;
   std::map<hipStream_t, int> slot_of;
+  std::vector<int> free_slots;   // slots of destroyed streams, handed out again before new ones
   int next_slot = 0;
 };
 
@@ -163,27 +165,92 @@ hipFunction_t find_kernel(DeviceState *st, const std::string &name) {
   return f;
 }
 
+namespace {
+// Stream-ordered clear of one reduction block (a fill kernel, so that it may sit inside a captured graph).
+int32_t clear_slot(DeviceState *st, uint32_t *block, hipStream_t stream) {
+  uint8_t *p = reinterpret_cast<uint8_t *>(block);
+  int64_t count = DeviceState::kSlotWords;
+  uint32_t fill = 0;
+  int32_t width = 4;
+  void *args[] = {&p, &count, &fill, &width};
+  return launch(st, "mtrt_fill", 1, 256, stream, args);
+}
+} // namespace
+
 uint32_t *reduction_slot(DeviceState *st, hipStream_t stream) {
-  std::lock_guard<std::mutex> lock(st->mu);
-  auto it = st->slot_of.find(stream);
   int slot;
-  if (it != st->slot_of.end()) {
-    slot = it->second;
-  } else {
-    if (st->next_slot >= DeviceState::kSlots) {
-      set_error(MTRT_RUNTIME_ERROR, "more than %d live streams use grid reductions", DeviceState::kSlots);
-      return nullptr;
+  bool fresh = false;
+  {
+    std::lock_guard<std::mutex> lock(st->mu);
+    auto it = st->slot_of.find(stream);
+    if (it != st->slot_of.end()) {
+      slot = it->second;
+    } else {
+      if (!st->free_slots.empty()) {
+        slot = st->free_slots.back();
+        st->free_slots.pop_back();
+      } else if (st->next_slot < DeviceState::kSlots) {
+        slot = st->next_slot++;
+      } else {
+        set_error(MTRT_RUNTIME_ERROR, "more than %d live streams use grid reductions", DeviceState::kSlots);
+        return nullptr;
+      }
+      st->slot_of.emplace(stream, slot);
+      fresh = true;
     }
-    slot = st->next_slot++;
-    st->slot_of.emplace(stream, slot);
   }
-  return st->slots + size_t(slot) * DeviceState::kSlotWords;
+  uint32_t *block = st->slots + size_t(slot) * DeviceState::kSlotWords;
+  // A block newly bound to a stream is cleared in stream order before its first use: whatever an earlier
+  // owner (a destroyed stream, or a launch that never finished) left in it cannot reach this stream's results.
+  if (fresh && clear_slot(st, block, stream) != MTRT_OK) {
+    std::lock_guard<std::mutex> lock(st->mu);
+    st->slot_of.erase(stream);
+    st->free_slots.push_back(slot);
+    return nullptr;
+  }
+  return block;
 }
 
-void forget_stream(hipStream_t) {
-  // Slots are never reused for a different stream: a destroyed stream's slot is
-  // zero again once its last kernel has finished, but handing it to another stream
-  // before that would race.  256 slots outlive any realistic stream count.
+int32_t reset_reduction_slot(DeviceState *st, hipStream_t stream) {
+  int slot = -1;
+  {
+    std::lock_guard<std::mutex> lock(st->mu);
+    auto it = st->slot_of.find(stream);
+    if (it != st->slot_of.end())
+      slot = it->second;
+  }
+  if (slot < 0)
+    return MTRT_OK;   // nothing bound: the next reduction on this stream clears its block itself
+  return clear_slot(st, st->slots + size_t(slot) * DeviceState::kSlotWords, stream);
+}
+
+void forget_stream(hipStream_t stream) {
+  // Called by every stream-destroy entry point before the stream goes away.  The stream's block returns
+  // to the free list only after the stream has drained, so a kernel still running on the old stream can
+  // never share the block with its next owner; HIP reusing the handle value for a new stream is harmless
+  // for the same reason (the mapping is gone by then).
+  std::vector<DeviceState *> states;
+  {
+    std::lock_guard<std::mutex> lock(g_mu);
+    for (auto &kv : g_states)
+      states.push_back(kv.second);
+  }
+  for (DeviceState *st : states) {
+    bool bound;
+    {
+      std::lock_guard<std::mutex> lock(st->mu);
+      bound = st->slot_of.count(stream) != 0;
+    }
+    if (!bound)
+      continue;
+    (void)hipStreamSynchronize(stream);
+    std::lock_guard<std::mutex> lock(st->mu);
+    auto it = st->slot_of.find(stream);
+    if (it != st->slot_of.end()) {
+      st->free_slots.push_back(it->second);
+      st->slot_of.erase(it);
+    }
+  }
 }
 
 int32_t launch(DeviceState *st, const std::string &kernel, uint32_t grid, uint32_t block,
@@ -214,6 +281,14 @@ const char *mtrt_hip_last_kernel(void) { return mtrt_rt::last_kernel_name(); }
 int32_t mtrt_hip_init(void) {
   mtrt_rt::clear_error();
   return mtrt_rt::device_state() ? MTRT_OK : MTRT_RUNTIME_ERROR;
+}
+
+int32_t mtrt_hip_reset_reductions(mtrt_stream_t stream) {
+  mtrt_rt::clear_error();
+  mtrt_rt::DeviceState *st = mtrt_rt::device_state();
+  if (!st)
+    return MTRT_RUNTIME_ERROR;
+  return mtrt_rt::reset_reduction_slot(st, mtrt_rt::as_hip(stream));
 }
 
 mtrt_module_t mtrt_hip_builtin_module(void) {

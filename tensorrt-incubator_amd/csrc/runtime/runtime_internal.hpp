@@ -15,6 +15,9 @@ inline hipStream_t as_hip(mtrt_stream_t s) { return reinterpret_cast<hipStream_t
 
 [[noreturn]] void fatal(const char *file, int line, const char *msg);
 bool read_file(const std::string &path, std::vector<char> &out);
+// Reads a program artifact by name: absolute names as they are, relative ones under $MTRT_ARTIFACTS_DIR first and
+// then under the working directory.  MTRT_NOT_FOUND (message lists what was tried) / MTRT_IO_ERROR via set_error.
+int32_t read_artifact(const char *filename, std::vector<char> &out);
 
 // Thread-local error text for the status-returning entry points.
 int32_t set_error(int32_t code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
@@ -34,7 +37,8 @@ hipModule_t builtin_module(DeviceState *);
 int num_compute_units(DeviceState *);
 hipFunction_t find_kernel(DeviceState *, const std::string &name);   // nullptr + set_error
 uint32_t *reduction_slot(DeviceState *, hipStream_t stream);         // nullptr + set_error
-void forget_stream(hipStream_t stream);
+int32_t reset_reduction_slot(DeviceState *, hipStream_t stream);     // stream-ordered clear of the stream's block
+void forget_stream(hipStream_t stream);                              // before a stream is destroyed
 
 // Set-up half of the allocation-free entry point (no_alloc.hip): looks up, with `device` current, the
 // device address of that file's scratch array and the kernel handles it launches.

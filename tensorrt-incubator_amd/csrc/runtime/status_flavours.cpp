@@ -74,8 +74,9 @@ Status cuda_module_create_from_ptx_file(const char *filename, mtrt_module_t *out
   if (!filename || filename[0] == '\0')
     return set_error(MTRT_INVALID_ARGUMENT, "filename must not be empty");
   std::vector<char> bytes;
-  if (!read_file(filename, bytes))
-    return set_error(MTRT_IO_ERROR, "failed to open file: %s", filename);
+  const int32_t rd = read_artifact(filename, bytes);
+  if (rd != MTRT_OK)
+    return rd;
   hipModule_t module = nullptr;
   std::string err;
   const int32_t st = load_code_object(bytes.data(), bytes.size(), &module, &err);
@@ -491,8 +492,9 @@ int32_t mtrt_lua_cuda_memcpy_strided(uintptr_t stream, int64_t rank, int64_t ele
     --inner;
   }
   std::vector<int64_t> idx(size_t(inner), 0);
-  const char *sbase = reinterpret_cast<const char *>(src + srcOffset);
-  char *dbase = reinterpret_cast<char *>(dst + dstOffset);
+  // offsets are memref offsets, in ELEMENTS (mlir-tensorrt/executor/lib/Support/StridedCopy.cpp:37-38)
+  const char *sbase = reinterpret_cast<const char *>(src) + int64_t(srcOffset) * elemSize;
+  char *dbase = reinterpret_cast<char *>(dst) + int64_t(dstOffset) * elemSize;
   for (;;) {
     int64_t so = 0, dof = 0;
     for (int64_t i = 0; i < inner; ++i) {

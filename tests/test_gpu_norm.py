@@ -204,3 +204,36 @@ def test_softmax_extremes_and_empty(pkg, orc):
     out = pkg.layernorm(z, torch.ones(128, device="cuda", dtype=torch.bfloat16),
                         torch.full((128,), 0.5, device="cuda", dtype=torch.bfloat16), 1e-5)
     assert torch.equal(out, torch.full_like(out, 0.5))
+
+
+def test_more_rows_than_the_row_per_wave_grid_covers(pkg, orc):
+    """The one-wave-per-row kernels do not loop over rows and their grid is capped at 2^20 workgroups of four
+    rows; beyond 2^22 rows the looping kernels must take over so that the last rows are still written."""
+    import torch
+    rows, d = (1 << 22) + 7, 8
+    x = torch.randn(rows, d, device="cuda", dtype=torch.float16)
+    y = torch.full_like(x, float("nan"))
+    pkg.softmax(x, out=y)
+    assert pkg.last_kernel() == "mtrt_softmax_f16_any"
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(y).all())
+    tail = slice(rows - 64, rows)
+    xs = bits16_of(x[tail])
+    ref = orc.softmax(xs, orc.F16, 64, d)
+    got = bits16_of(y[tail])
+    assert np.max(np.abs(orc.widen(got, orc.F16) - orc.widen(ref, orc.F16))) <= 2.0 ** -10
+    g = torch.ones(d, device="cuda", dtype=torch.float16)
+    b = torch.zeros(d, device="cuda", dtype=torch.float16)
+    z = torch.full_like(x, float("nan"))
+    pkg.layernorm(x, g, b, 1e-5, out=z)
+    assert pkg.last_kernel() == "mtrt_layernorm_f16_any"
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(z).all())
+    refz = orc.layernorm(xs, bits16_of(g), bits16_of(b), orc.F16, 64, d, 1e-5)
+    gotz = bits16_of(z[tail])
+    assert np.max(np.abs(orc.widen(gotz, orc.F16) - orc.widen(refz, orc.F16))) <= 2.0 ** -8
+
+
+def bits16_of(t):
+    from helpers import bits16
+    return bits16(t)

@@ -26,7 +26,19 @@ REFERENCE_STANDALONE = [
     "cuda_module_create_from_ptx_file", "cuda_module_destroy", "cuda_module_get_func", "cuda_launch_kernel",
     "cuda_event_create", "cuda_event_release", "cuda_stream_record_event", "cuda_stream_wait_event",
     "cuda_event_sync", "cuda_event_elapsed_msec", "get_last_error_message", "clear_last_error_message",
+    # MTRTRuntimeStatus.h:55-58 and MTRTRuntimeCore.h:220-236 (abort_on_error, make_status and the memref
+    # descriptor helpers are header-inline there and here: exercised by the selftest program)
+    "set_last_error_message_v", "host_aligned_alloc", "host_free", "constant_load_from_file", "constant_destroy",
 ]
+
+
+def _constant_env(tmp_path):
+    """A 100-byte constant blob 0, 1, ..., 99 in a fresh artifacts directory, named through the environment."""
+    (tmp_path / "weights.bin").write_bytes(bytes(range(100)))
+    env = dict(os.environ)
+    env["MTRT_ARTIFACTS_DIR"] = str(tmp_path)
+    env["MTRT_SELFTEST_CONSTANT"] = "weights.bin"
+    return env
 
 
 def _selftest(pkg):
@@ -38,15 +50,33 @@ def test_standalone_header_and_exports(pkg):
     declared = re.findall(r"MTRT_CAPI_EXPORTED[^;(]*?\b([a-z_]+)\s*\(", text)
     assert sorted(declared) == sorted(REFERENCE_STANDALONE)
     out = subprocess.run(["nm", "-DC", "--defined-only", pkg.LIB_PATH], capture_output=True, text=True).stdout
-    exported = set(re.findall(r" T mtrt::(\w+)\(", out))
+    exported = set(re.findall(r" T mtrt::(?:detail::)?(\w+)\(", out))
     assert exported == set(REFERENCE_STANDALONE)
+    # the header-inline part of the reference's interface
+    for name in ("abort_on_error", "make_status", "make_memref_descriptor", "make_unranked_descriptor",
+                 "make_ptr_shape_descriptor", "memref_descriptor_get_aligned_ptr", "memref_descriptor_get_stride",
+                 "struct RankedMemRef", "struct UnrankedMemRef", "struct PtrAndShape", "bit_cast"):
+        assert name in text, name
+    # generated code includes the runtime under the reference's header names
+    for shim in ("MTRTRuntimeStatus.h", "MTRTRuntimeCore.h", "MTRTRuntimeCuda.h"):
+        assert os.path.exists(os.path.join(os.path.dirname(STANDALONE_HEADER), "standalone", shim))
 
 
-def test_standalone_argument_validation(pkg):
-    """null out-parameters, empty names, negative sizes, missing files: status + message, no device needed."""
-    res = subprocess.run([_selftest(pkg), "--validate"], capture_output=True, text=True, timeout=60)
+def test_standalone_argument_validation(pkg, tmp_path):
+    """null out-parameters, empty names, negative sizes, missing files, descriptor helpers, host-space constants
+    from $MTRT_ARTIFACTS_DIR: status + message, no device needed."""
+    res = subprocess.run([_selftest(pkg), "--validate"], capture_output=True, text=True, timeout=60,
+                         env=_constant_env(tmp_path))
     assert res.returncode == 0, res.stdout + res.stderr
     assert "standalone selftest ok" in res.stdout
+
+
+def test_abort_on_error_prints_the_message_and_aborts(pkg):
+    """What generated code does after every runtime call (HostToEmitCPatternsCuda.cpp:39-42): a failed status
+    prints the thread's last message to stderr and abort()s (MTRTRuntimeStatus.h:70-81)."""
+    res = subprocess.run([_selftest(pkg), "--abort"], capture_output=True, text=True, timeout=60)
+    assert res.returncode == -6, res.returncode
+    assert "Error opening file 'mtrt_no_such_module.hsaco'" in res.stderr and "Tried:" in res.stderr
 
 
 def test_builtin_name_table(pkg):
@@ -102,9 +132,13 @@ def test_builtin_argument_validation(pkg):
 
 
 @pytest.mark.gpu
-def test_standalone_launch_known_answer(pkg):
+def test_standalone_launch_known_answer(pkg, tmp_path):
+    """The reference's argpack known answer through the status-returning calls, then the same through functions
+    written in the shape the EmitC lowering emits (alloc -> descriptor -> launch -> abort_on_error, copies of
+    offset views), then constants loaded into the pinned, device and unified spaces."""
     print("case: standalone selftest on", pkg.FIXTURE_MODULE_PATH, flush=True)
-    res = subprocess.run([_selftest(pkg), pkg.FIXTURE_MODULE_PATH], capture_output=True, text=True, timeout=100)
+    res = subprocess.run([_selftest(pkg), pkg.FIXTURE_MODULE_PATH], capture_output=True, text=True, timeout=100,
+                         env=_constant_env(tmp_path))
     assert res.returncode == 0, res.stdout + res.stderr
     assert "standalone selftest ok" in res.stdout
 
@@ -184,15 +218,20 @@ def test_builtin_events_pinned_memory_and_strided_copies(pkg):
     every_other_row = (ctypes.c_int64 * 4)(3, 5, 10, 1)
     assert L.mtrt_lua_cuda_stream_record_event(stream.value, e0.value) == 0
     # host (offset: row 1, column 2) -> device, then device -> every other row of the host destination
-    assert L.mtrt_lua_cuda_memcpy_strided(stream.value, 2, 4, hsrc.value, (1 * 8 + 2) * 4, strided, dbuf.value, 0, dense) == 0
-    assert L.mtrt_lua_cuda_memcpy_strided(stream.value, 2, 4, dbuf.value, 0, dense, hdst.value, 0, every_other_row) == 0
+    # offsets are memref offsets in ELEMENTS (reference: executor/lib/Support/StridedCopy.cpp:37-38)
+    assert L.mtrt_lua_cuda_memcpy_strided(stream.value, 2, 4, hsrc.value, 1 * 8 + 2, strided, dbuf.value, 0, dense) == 0
+    # ... and a non-zero destination offset of one row (5 elements): rows 1, 3, 5 of the destination
+    assert L.mtrt_lua_cuda_memcpy_strided(stream.value, 2, 4, dbuf.value, 0, dense, hdst.value, 5, every_other_row) == 0
+    # rank 0: exactly one element, element 3 of the device matrix -> element 2 of the host destination
+    assert L.mtrt_lua_cuda_memcpy_strided(stream.value, 0, 4, dbuf.value, 3, None, hdst.value, 2, None) == 0
     assert L.mtrt_lua_cuda_stream_record_event(stream.value, e1.value) == 0
     assert L.mtrt_lua_cuda_stream_wait_event(stream.value, e1.value) == 0
     assert L.mtrt_lua_cuda_event_sync(e1.value) == 0
     ms = ctypes.c_float(-1.0)
     assert L.mtrt_lua_cuda_event_elapsed_msec(e0.value, e1.value, ctypes.byref(ms)) == 0 and ms.value >= 0.0
     expect = np.full((6, 5), -1.0, np.float32)
-    expect[0::2] = src[1:4, 2:7]
+    expect[1::2] = src[1:4, 2:7]
+    expect[0, 2] = src[1, 2 + 3]
     assert np.array_equal(dst, expect)
     # a released event comes back from the pool
     assert L.mtrt_lua_cuda_event_release(e1.value) == 0
