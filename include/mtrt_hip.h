@@ -188,8 +188,14 @@ enum mtrt_hip_scale_kind {
 enum mtrt_hip_flags {
   MTRT_Q_ROUND_TO_INT = 1, /* f8 target: apply round_nearest_even before the clamp, the form
                               StablehloRaiseQDQ.cpp:233-265 matches; integer targets always round */
-  MTRT_F8_REFHOST = 2      /* f8 target: reproduce the reference HOST class bit for bit
+  MTRT_F8_REFHOST = 2,     /* f8 target: reproduce the reference HOST class bit for bit
                               (DataTypes.cpp:43-122) instead of IEEE RNE + saturate           */
+  MTRT_F8_VIA_F16 = 4      /* f8 target: convert f32 -> f16 -> f8, rounding to nearest even TWICE, which is
+                              what the reference's generated GPU kernels do
+                              (mlir-tensorrt/kernel/lib/Kernel/Transforms/NormalizeQuantizedConversions.cpp:38-118).
+                              Differs from the single rounding of the default where the f16 rounding lands on
+                              an f8 midpoint (about one input in 250 on normally distributed data).  Not
+                              combinable with MTRT_F8_REFHOST.                                 */
 };
 
 /* status codes, MTRTRuntimeStatus.h:31-41 */
@@ -339,6 +345,16 @@ MTRT_CAPI_EXPORTED int32_t mtrt_hip_gemm_w4a16(mtrt_stream_t stream, const void 
                                                const void *w_kn_packed, const void *w_prepacked,
                                                const void *scale, void *y, int64_t M, int64_t K,
                                                int64_t N, int64_t block);
+
+/* Dense Linear in one float type: y[m,n] = narrow(sum_k f32(x[m,k]) * f32(w_nk[n,k]) + f32(bias[n])), f32
+ * accumulation; bias may be NULL.  The float matmul of the fake-quant Linear (linear.py:112-151:
+ * out = x' @ W'^T + b on dequantized operands) for the parameter combinations the two matrix-core clusters
+ * above do not express, and of the unquantized module; w_nk is the module's own [out_features, in_features]
+ * weight.  A tiled FMA kernel, the class of code the reference generates for a matmul
+ * (fallback-schedule-matmul.mlir:24); any shape, no alignment needs. */
+MTRT_CAPI_EXPORTED int32_t mtrt_hip_linear_dense(mtrt_stream_t stream, const void *x, const void *w_nk,
+                                                 const void *bias, void *y, int32_t dtype, int64_t M,
+                                                 int64_t K, int64_t N);
 
 /* ------------------------------------------------------------------------- */
 /* Part 3 — the interpreter's builtin set, status-returning                    */

@@ -15,6 +15,7 @@ REF_PATH = os.path.join(HERE, "_ref", "libref_datatypes.so")
 
 F32, F16, BF16, I8, F8E4M3FN, I4, I4_PACKED, I32, F4_PACKED = range(9)
 IEEE, REFHOST = 0, 1
+F8_VIA_F16 = 4
 SCALE_UNIFORM, SCALE_ROW, SCALE_COL = range(3)
 Q_ROUND_TO_INT = 1
 

@@ -54,8 +54,14 @@ enum {
 
 /* flags */
 enum {
-  ORC_Q_ROUND_TO_INT = 1 /* apply round_nearest_even before the clamp (always on
-                            for integer targets; optional for f8)                */
+  ORC_Q_ROUND_TO_INT = 1, /* apply round_nearest_even before the clamp (always on
+                             for integer targets; optional for f8)                */
+  ORC_F8_VIA_F16 = 4      /* f8 target: f32 -> f16 -> f8, each step RNE (IEEE mode of lowp.hpp): the chain
+                             the reference's GPU code generator emits
+                             (mlir-tensorrt/kernel/lib/Kernel/Transforms/NormalizeQuantizedConversions.cpp:38-118).
+                             Pinned as the composition of two pinned conversions: numpy's float16 cast and the
+                             golden f16 -> f8 table minted from the reference build agree with it on every
+                             witness and random input of tests/test_oracle_programs.py. */
 };
 
 /* scalar conversions */

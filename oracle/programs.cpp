@@ -180,7 +180,9 @@ void orc_quantize(const void *x, int in_dtype, void *q, int out_dtype, const flo
         static_cast<int8_t *>(q)[i] = static_cast<int8_t>(v);
         break;
       case ORC_F8E4M3FN:
-        static_cast<uint8_t *>(q)[i] = f32_to_f8e4m3fn(v, m);
+        if (flags & ORC_F8_VIA_F16)
+          v = f16_to_f32(f32_to_f16(v, kIeee));   // first rounding; the widening back is exact
+        static_cast<uint8_t *>(q)[i] = f32_to_f8e4m3fn(v, (flags & ORC_F8_VIA_F16) ? kIeee : m);
         break;
       case ORC_I4:
         static_cast<uint8_t *>(q)[i] = uint8_t(int4_saturate(int(std::trunc(v)))) & 0xF;

@@ -25,6 +25,7 @@ SCALE_UNIFORM, SCALE_ROW, SCALE_COL = range(3)
 # enum mtrt_hip_flags
 Q_ROUND_TO_INT = 1
 F8_REFHOST = 2
+F8_VIA_F16 = 4
 
 _c = ctypes
 _vp, _i32, _i64, _f32, _sz, _i8 = _c.c_void_p, _c.c_int32, _c.c_int64, _c.c_float, _c.c_size_t, _c.c_int8
@@ -98,6 +99,7 @@ PROTOTYPES = {
     "mtrt_hip_gemm_w8a8_fragments_bytes": (_i64, [_i64, _i64]),
     "mtrt_hip_gemm_w8a8_prepack_fragments": (_i32, [_vp, _vp, _i32, _vp, _i64, _i64]),
     "mtrt_hip_gemm_w8a8_fragments": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64]),
+    "mtrt_hip_linear_dense": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i64, _i64, _i64]),
     "mtrt_hip_gemm_w4a16_prepacked_bytes": (_i64, [_i64, _i64]),
     "mtrt_hip_gemm_w4a16_prepack": (_i32, [_vp, _vp, _vp, _i64, _i64]),
     "mtrt_hip_gemm_w4a16": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64]),
@@ -327,6 +329,19 @@ def gemm_w4a16(a, scale, K, N, block, w_kn_packed=None, w_prepacked=None, out=No
     y = torch.empty((M, N), dtype=torch.float16, device=a.device) if out is None else out
     check(lib().mtrt_hip_gemm_w4a16(_stream(), a.data_ptr(), _ptr(w_kn_packed), _ptr(w_prepacked), scale.data_ptr(),
                                     y.data_ptr(), M, K, N, block))
+    return y
+
+
+def linear_dense(x, w_nk, bias=None, out=None):
+    """y = x @ w_nk^T (+ bias) in the operands' float type, f32 accumulation; x [M,K], w_nk [N,K]."""
+    torch = _torch()
+    assert x.is_cuda and x.is_contiguous() and w_nk.is_contiguous() and w_nk.dtype == x.dtype and x.dim() == 2
+    M, K = x.shape
+    N = w_nk.shape[0]
+    assert w_nk.shape[1] == K and (bias is None or (bias.dtype == x.dtype and bias.numel() == N and bias.is_contiguous()))
+    y = torch.empty((M, N), dtype=x.dtype, device=x.device) if out is None else out
+    check(lib().mtrt_hip_linear_dense(_stream(), x.data_ptr(), w_nk.data_ptr(), _ptr(bias), y.data_ptr(),
+                                      float_dtype_of(x), M, K, N))
     return y
 
 

@@ -6,4 +6,5 @@
 #include "norm.hip"
 #include "gemm_w8a8.hip"
 #include "gemm_w4a16.hip"
+#include "gemm_dense.hip"
 #include "util.hip"

@@ -27,6 +27,7 @@ struct F4P { using storage = uint8_t;  static constexpr int kBits = 4; };  // f4
 // flag bits passed by value to the quantize kernels
 constexpr int kFlagRoundToInt = 1;   // round_nearest_even before the clamp (f8 target only; ints always round)
 constexpr int kFlagF8RefHost = 2;    // reproduce the reference host class instead of IEEE RNE+saturate
+constexpr int kFlagF8ViaF16 = 4;     // f32 -> f16 -> f8, both RNE: the conversion chain of the reference's GPU path
 
 __device__ __forceinline__ float bits_to_f32(uint32_t u) { return __uint_as_float(u); }
 __device__ __forceinline__ uint32_t f32_to_bits(float f) { return __float_as_uint(f); }

@@ -94,7 +94,9 @@ template <> struct Codes<F8> {
   static constexpr float kLo = -448.0f, kHi = 448.0f;
   static constexpr bool kAlwaysRound = false;
   static __device__ __forceinline__ uint32_t enc(float v, int flags) {
-    return (flags & kFlagF8RefHost) ? f32_to_f8_refhost(v) : (f32x2_to_f8_ieee(v, 0.0f) & 0xFFu);
+    if (flags & kFlagF8RefHost) return f32_to_f8_refhost(v);
+    if (flags & kFlagF8ViaF16) v = f16_bits_to_f32(f32_to_f16_bits(v));
+    return f32x2_to_f8_ieee(v, 0.0f) & 0xFFu;
   }
   static __device__ __forceinline__ float dec(uint32_t c) { return f8_to_f32<0>(c); }
 };
@@ -145,8 +147,18 @@ __device__ __forceinline__ uint32_t pack4<F8>(const float* v, int flags) {
   if (flags & kFlagF8RefHost)
     return f32_to_f8_refhost(v[0]) | (f32_to_f8_refhost(v[1]) << 8) | (f32_to_f8_refhost(v[2]) << 16) |
            (f32_to_f8_refhost(v[3]) << 24);
-  int w = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], 0, false);
-  return uint32_t(__builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], w, true));
+  // The reference's generated GPU code never converts f32 to f8 directly: it truncates to f16 first and
+  // converts that (mlir-tensorrt/kernel/lib/Kernel/Transforms/NormalizeQuantizedConversions.cpp:38-118,
+  // cvt.rn.satfinite.e4m3x2.f16x2 in LowerToNVVM.cpp:281-339).  Both steps round to nearest even, so a value
+  // within half an f16 ulp of an f8 midpoint first lands ON the midpoint and then goes to the even code.
+  // Widening f16 to f32 is exact, so the second step can use the f32 conversion instruction.
+  float t[4] = {v[0], v[1], v[2], v[3]};
+  if (flags & kFlagF8ViaF16) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) t[k] = f16_bits_to_f32(f32_to_f16_bits(t[k]));
+  }
+  int w = __builtin_amdgcn_cvt_pk_fp8_f32(t[0], t[1], 0, false);
+  return uint32_t(__builtin_amdgcn_cvt_pk_fp8_f32(t[2], t[3], w, true));
 }
 template <typename Q>
 __device__ __forceinline__ void unpack4(uint32_t w, float* v) {

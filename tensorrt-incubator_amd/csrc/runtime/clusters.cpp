@@ -71,8 +71,10 @@ int32_t qdq_dispatch(int mode, hipStream_t stream, const void *x, int32_t x_dtyp
   if (kind == MTRT_SCALE_COL && d0 % nb != 0)
     return set_error(MTRT_INVALID_ARGUMENT, "block size %lld does not divide the blocked extent %lld",
                      (long long)nb, (long long)d0);
-  if (flags & ~(MTRT_Q_ROUND_TO_INT | MTRT_F8_REFHOST))
+  if (flags & ~(MTRT_Q_ROUND_TO_INT | MTRT_F8_REFHOST | MTRT_F8_VIA_F16))
     return set_error(MTRT_INVALID_ARGUMENT, "unknown flag bits 0x%x", flags);
+  if ((flags & MTRT_F8_REFHOST) && (flags & MTRT_F8_VIA_F16))
+    return set_error(MTRT_INVALID_ARGUMENT, "MTRT_F8_REFHOST and MTRT_F8_VIA_F16 name two different conversions; pass one");
   const int64_t n = d0 * d1;
   if (n == 0)
     return MTRT_OK;
@@ -436,6 +438,32 @@ int32_t mtrt_hip_gemm_w8a8_fragments(mtrt_stream_t stream, const void *a, const 
     return set_error(MTRT_INVALID_ARGUMENT, "problem [%lld, %lld] needs too many tiles", (long long)M, (long long)N);
   void *args[] = {&a, &w_frag, &a_scale, &w_scale, &y, &M, &K, &N, &full_panels};
   return launch(st, "mtrt_gemm_w8a8_frag", uint32_t(grid), 512, as_hip(stream), args);
+}
+
+int32_t mtrt_hip_linear_dense(mtrt_stream_t stream, const void *x, const void *w_nk, const void *bias, void *y,
+                              int32_t dtype, int64_t M, int64_t K, int64_t N) {
+  clear_error();
+  const char *xn = float_name(dtype);
+  if (!xn)
+    return set_error(MTRT_INVALID_ARGUMENT, "dense linear dtype %d is not one of f32/f16/bf16", dtype);
+  if (M < 0 || K < 0 || N < 0)
+    return set_error(MTRT_INVALID_ARGUMENT, "negative extent M=%lld K=%lld N=%lld", (long long)M, (long long)K,
+                     (long long)N);
+  if (M == 0 || N == 0)
+    return MTRT_OK;
+  if (!y || (K > 0 && (!x || !w_nk)))
+    return set_error(MTRT_INVALID_ARGUMENT, "null operand");
+  const int eb = float_bytes(dtype);
+  if (!aligned(x, eb) || !aligned(w_nk, eb) || !aligned(y, eb) || !aligned(bias, eb))
+    return set_error(MTRT_INVALID_ARGUMENT, "operand is not aligned to its element size");
+  DeviceState *st = device_state();
+  if (!st)
+    return MTRT_RUNTIME_ERROR;
+  const int64_t tiles = ((M + 63) / 64) * ((N + 63) / 64);
+  if (tiles > int64_t(kMaxGrid) * 1024)
+    return set_error(MTRT_INVALID_ARGUMENT, "problem [%lld, %lld] needs too many tiles", (long long)M, (long long)N);
+  void *args[] = {&x, &w_nk, &bias, &y, &M, &K, &N};
+  return launch(st, std::string("mtrt_gemm_dense_") + xn, uint32_t(tiles), kBlock, as_hip(stream), args);
 }
 
 int64_t mtrt_hip_gemm_w4a16_prepacked_bytes(int64_t K, int64_t N) {

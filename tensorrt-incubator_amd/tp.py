@@ -324,15 +324,24 @@ def scale_from_amax(input, dtype):
 
 class Linear:
     """tp.Linear (linear.py:30-151): out = x @ W^T + b, with the fake-quant pair on the input and on the
-    weight when `quant_dtype` is set.  weight: [out_features, in_features].
+    weight when `quant_dtype` is set.  weight: [out_features, in_features]; x: [*, in_features].
 
-    With int8, an input scale and a per-output-channel (dim 0) or per-tensor weight scale the product of
-    the two dequantized operands equals (q_x . q_W^T) * s_x * s_w[n] exactly in real arithmetic; `fused=True`
-    runs that form on the integer matrix cores (W8A8 cluster, int32 accumulation, f16 result) instead of
-    a float matmul of the dequantized operands."""
+    Every product runs on a hand-written kernel of this library; which one follows from the parameters:
 
-    def __init__(self, in_features, out_features, bias=True, dtype=float32, quant_dtype=None, weight_quant_dim=None,
-                 fused=False):
+      * int8, an input scale, weight scale per tensor or per output channel (dim 0): the product of the two
+        dequantized operands equals (q_x . q_W^T) * s_x * s_w[n] exactly in real arithmetic, so it runs on the
+        integer matrix cores (W8A8 cluster: int32 accumulation, f16 result widened to the module's dtype).
+      * int4 weight-only in a float16 module, weight scale per tensor or per output channel, in_features a
+        multiple of 64: the W4A16 cluster dequantizes the packed codes on the way into the matrix cores.
+        (The rank-2 scale of this API groups OUTPUT features, [out/B, in] as weight_loader.py:102-115 builds it;
+        the W4A16 cluster's blocks run along the reduction axis, so that form takes the next route.)
+      * everything else (float8 codes, scales along the input features, int4 blocks, other dtypes, no
+        quantization): the literal fake-quant form, DQ(Q(x)) @ DQ(Q(W))^T on the dense Linear kernel.
+
+    Weights are program constants: they are quantized, re-laid out and (for the last route) dequantized ONCE,
+    when first needed after `weight` / `weight_scale` were assigned; the forward pass only touches x."""
+
+    def __init__(self, in_features, out_features, bias=True, dtype=float32, quant_dtype=None, weight_quant_dim=None):
         torch = _torch()
         self.dtype = dtype
         self.weight = _produced(torch.zeros((out_features, in_features), dtype=_torch_dtype(dtype)), dtype)
@@ -341,49 +350,99 @@ class Linear:
         self.weight_quant_dim = weight_quant_dim
         self.weight_scale = None
         self.input_scale = None
-        self.fused = fused
+        self._plan_key = None
+        self._plan = None
 
     def __call__(self, x):
         return self.forward(x)
 
+    def load_state_dict(self, state_dict):
+        """Assigns `weight`, `bias`, `weight_scale`, `input_scale` from a name -> Tensor mapping and prepares the
+        weight side (quantize, re-layout) right away, as a loader does once per model."""
+        for name in ("weight", "bias", "weight_scale", "input_scale"):
+            if name in state_dict:
+                v = state_dict[name]
+                setattr(self, name, v if isinstance(v, Tensor) else Tensor(v))
+        self._prepared()
+
+    def route(self):
+        """'w8a8', 'w4a16' or 'dense': the kernel family the next forward pass uses."""
+        return self._prepared()["route"]
+
+    # -- weight side, once ---------------------------------------------------------------------------
+    def _prepared(self):
+        torch = _torch()
+        def ident(t):      # a new Tensor object or an in-place update of its storage makes a new key
+            return (id(t), t._t._version) if isinstance(t, Tensor) else t
+        key = (ident(self.weight), ident(self.weight_scale), ident(self.input_scale), self.quant_dtype, self.weight_quant_dim)
+        if self._plan is not None and self._plan_key == key:
+            return self._plan
+        from . import gemm_w4a16_prepack, gemm_w8a8_prepack_fragments
+        N, K = self.weight.shape
+        plan = {"route": "dense"}
+        if self.quant_dtype is None:
+            plan["weight"] = self.weight.device_data().contiguous()
+        else:
+            has_x_scale = isinstance(self.input_scale, Tensor)
+            if has_x_scale and self.weight_quant_dim == 1:
+                raise_error("Unsupported quantization parameters for Linear module.",
+                            ["weight_quant_dim cannot be 1 when input_scale is provided. ",
+                             f"input_scale={self.input_scale}, weight_quant_dim={self.weight_quant_dim}"])
+            q_weight = quantize(self.weight, self.weight_scale, self.quant_dtype, self.weight_quant_dim)
+            w_scale = _convert_scale(self.weight_scale, self.dtype)
+            per_out = w_scale.rank == 0 or (w_scale.rank == 1 and self.weight_quant_dim == 0)
+            if self.quant_dtype == int8 and has_x_scale and per_out:
+                plan["route"] = "w8a8"
+                codes = q_weight.device_data().contiguous()          # [N, K], K contiguous
+                plan["s_w"] = _scale_on_device(w_scale).reshape(-1).expand(N).contiguous()
+                if K % 128 == 0:
+                    plan["w_frag"] = gemm_w8a8_prepack_fragments(codes, is_nk=True)
+                else:
+                    plan["w_nk"] = codes
+            elif (self.quant_dtype == int4 and not has_x_scale and per_out and self.dtype == float16 and K % 64 == 0):
+                plan["route"] = "w4a16"
+                # the cluster takes [K, N] codes packed two per byte and f16 scales [K / block, N]: one block = all of K
+                kn = q_weight.device_data().to(torch.uint8).bitwise_and(0xF).transpose(0, 1).contiguous().reshape(-1)
+                packed = (kn[0::2] | (kn[1::2] << 4)).contiguous()
+                plan["w_prepacked"] = gemm_w4a16_prepack(packed, K, N)
+                plan["scale_kn"] = _scale_on_device(w_scale).reshape(-1).expand(N).to(torch.float16).reshape(1, N).contiguous()
+            else:
+                plan["weight"] = dequantize(q_weight, self.weight_scale, self.dtype, self.weight_quant_dim).device_data().contiguous()
+        self._plan_key, self._plan = key, plan
+        return plan
+
+    # -- forward ---------------------------------------------------------------------------------------
     def forward(self, x):
+        from . import gemm_w4a16, gemm_w8a8, gemm_w8a8_fragments, linear_dense
         torch = _torch()
         if not isinstance(x, Tensor):
             x = Tensor(x)
-        if self.quant_dtype is not None:
-            q_x = None
-            if isinstance(self.input_scale, Tensor):
-                if self.weight_quant_dim == 1:
-                    raise_error("Unsupported quantization parameters for Linear module.",
-                                ["weight_quant_dim cannot be 1 when input_scale is provided. ",
-                                 f"input_scale={self.input_scale}, weight_quant_dim={self.weight_quant_dim}"])
-                q_x = quantize(x, self.input_scale, self.quant_dtype)
-            q_weight = quantize(self.weight, self.weight_scale, self.quant_dtype, self.weight_quant_dim)
-            if self.fused and q_x is not None and self.quant_dtype == int8 and x.rank == 2 and self.weight_scale.rank < 2:
-                return self._forward_w8a8(q_x, q_weight)
-            if q_x is not None:
-                x = dequantize(q_x, self.input_scale, self.dtype)
-            weight = dequantize(q_weight, self.weight_scale, self.dtype, self.weight_quant_dim)
+        plan = self._prepared()
+        N, K = self.weight.shape
+        lead = x.shape[:-1]
+        bias = None if self.bias is None else self.bias.device_data().contiguous()
+        if plan["route"] == "w8a8":
+            q_x = quantize(x, self.input_scale, int8).device_data().reshape(-1, K)
+            M = q_x.shape[0]
+            s_x = _scale_on_device(_convert_scale(self.input_scale, self.dtype)).reshape(-1).expand(M).contiguous()
+            if "w_frag" in plan:
+                y = gemm_w8a8_fragments(q_x, plan["w_frag"], s_x, plan["s_w"], N)
+            else:
+                y = gemm_w8a8(q_x, plan["w_nk"], s_x, plan["s_w"])
+            out = y.to(_torch_dtype(self.dtype))
+            if bias is not None:
+                out = out + bias.unsqueeze(0)
+        elif plan["route"] == "w4a16":
+            a = x.device_data().reshape(-1, K).contiguous()
+            out = gemm_w4a16(a, plan["scale_kn"], K, N, K, w_prepacked=plan["w_prepacked"])
+            if bias is not None:
+                out = out + bias.unsqueeze(0)
         else:
-            weight = self.weight
-        out = x.device_data() @ weight.device_data().transpose(1, 0)
-        if self.bias is not None:
-            out = out + self.bias.device_data().unsqueeze(0)
-        return _produced(out, self.dtype)
-
-    def _forward_w8a8(self, q_x, q_weight):
-        from . import gemm_w8a8
-        torch = _torch()
-        M = q_x.shape[0]
-        N = q_weight.shape[0]
-        s_x = _scale_on_device(self.input_scale).expand(M).contiguous()
-        s_w = _scale_on_device(self.weight_scale).expand(N).contiguous()
-        # Tripy's weight is [out, in] = [N, K] with K contiguous: already the layout the int8 cluster reads.
-        y = gemm_w8a8(q_x.device_data(), q_weight.device_data().contiguous(), s_x, s_w)
-        out = y.to(_torch_dtype(self.dtype))
-        if self.bias is not None:
-            out = out + self.bias.device_data().unsqueeze(0)
-        return _produced(out, self.dtype)
+            if self.quant_dtype is not None and isinstance(self.input_scale, Tensor):
+                x = dequantize(quantize(x, self.input_scale, self.quant_dtype), self.input_scale, self.dtype)
+            a = x.device_data().reshape(-1, K).contiguous()
+            out = linear_dense(a, plan["weight"], bias)
+        return _produced(out.reshape(lead + (N,)), self.dtype)
 
 
 # ---- fused reduce clusters -----------------------------------------------------------------------

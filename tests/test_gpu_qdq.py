@@ -108,11 +108,22 @@ def test_c3_dynamic_fp8_full_size(pkg, orc):
     scale_ref = orc.scale_from_amax(amax_ref, 448.0)
     assert f32_bits(amax.cpu().numpy())[0] == f32_bits(amax_ref)[0]
     assert f32_bits(scale.cpu().numpy())[0] == f32_bits(scale_ref)[0]
-    for flags, mode in ((0, orc.IEEE), (pkg.F8_REFHOST, orc.REFHOST)):
+    # three f8 conversions: IEEE single rounding (default), the reference host class, the reference GPU chain via f16
+    direct = None
+    for flags, oflags, mode in ((0, 0, orc.IEEE), (pkg.F8_REFHOST, 0, orc.REFHOST), (pkg.F8_VIA_F16, orc.F8_VIA_F16, orc.IEEE)):
         q, y = pkg.quantize_dequantize(xd, scale.reshape(1), pkg.F8E4M3FN, flags=flags)
         assert pkg.last_kernel() == "mtrt_qdq_uniform_bf16_f8"
-        q_ref = orc.quantize(xs, orc.BF16, orc.F8E4M3FN, [scale_ref], orc.SCALE_UNIFORM, rows, cols, 1, 0, mode)
-        assert np.array_equal(_codes_np(q), q_ref), "fp8 codes, mode %d" % mode
+        q_ref = orc.quantize(xs, orc.BF16, orc.F8E4M3FN, [scale_ref], orc.SCALE_UNIFORM, rows, cols, 1, oflags, mode)
+        assert np.array_equal(_codes_np(q), q_ref), "fp8 codes, flags %d" % flags
+        if flags == 0:
+            direct = q_ref
+        elif flags == pkg.F8_VIA_F16:
+            # bf16 inputs divided by ONE scale take only 128 distinct quotient mantissas per binade, so whether any
+            # of them sits in a double-rounding window is a property of the scale; on f32 inputs about 0.4 % of the
+            # codes differ (test_fp8_via_f16_witnesses_and_rejections, tests/test_oracle_programs.py)
+            frac = np.count_nonzero(q_ref != direct) / q_ref.size
+            print("C3: codes that differ between the direct and the via-f16 conversion: %g" % frac, flush=True)
+            assert frac < 2e-2
         y_ref = orc.dequantize(q_ref, orc.F8E4M3FN, orc.BF16, [scale_ref], orc.SCALE_UNIFORM, rows, cols, 1, mode)
         assert np.array_equal(bits16(y), y_ref), "bf16 dequantized values, mode %d" % mode
         del q, y, q_ref, y_ref
@@ -332,3 +343,31 @@ def test_invalid_arguments_are_reported(pkg):
     assert st == 1 and b"flag" in L.mtrt_hip_last_error()
     st = L.mtrt_hip_amax(None, x.data_ptr(), pkg.I8, 64, 1.0, None, None)
     assert st == 1
+
+
+def test_fp8_via_f16_witnesses_and_rejections(pkg, orc):
+    """MTRT_F8_VIA_F16 = the conversion chain of the reference's generated GPU kernels (f32 -> f16 -> f8, RNE
+    twice): hand-derived double-rounding witnesses, every type pair against the oracle, and the flag checks."""
+    import torch
+    one = torch.ones(1, device="cuda")
+    w = np.float32([1.0625 + 2.0 ** -20, -(1.0625 + 2.0 ** -20), 1.1875 - 2.0 ** -20, 1.0625, 1.0625 + 2.0 ** -10] * 8)
+    x = torch.from_numpy(w).cuda()
+    assert _codes_np(pkg.quantize(x, one, pkg.F8E4M3FN))[:5].tolist() == [0x39, 0xB9, 0x39, 0x38, 0x39]
+    assert _codes_np(pkg.quantize(x, one, pkg.F8E4M3FN, flags=pkg.F8_VIA_F16))[:5].tolist() == [0x38, 0xB8, 0x3A, 0x38, 0x39]
+    g = rng(41)
+    for d0, d1 in ((64, 1024), (7, 13)):           # vector kernels and the element-wise kernel
+        v = (g.standard_normal((d0, d1)) * 40).astype(np.float32)
+        xd = torch.from_numpy(v).cuda()
+        sc = np.float32(0.37)
+        for fl, ofl in ((pkg.F8_VIA_F16, orc.F8_VIA_F16), (pkg.F8_VIA_F16 | pkg.Q_ROUND_TO_INT, orc.F8_VIA_F16 | orc.Q_ROUND_TO_INT)):
+            q = pkg.quantize(xd, torch.full((1,), float(sc), device="cuda"), pkg.F8E4M3FN, flags=fl)
+            ref = orc.quantize(v, orc.F32, orc.F8E4M3FN, [sc], orc.SCALE_UNIFORM, d0, d1, 1, ofl)
+            assert np.array_equal(_codes_np(q), ref), (d0, d1, fl)
+    L = pkg.lib()
+    s = torch.cuda.current_stream().cuda_stream
+    q = torch.empty(40, dtype=torch.uint8, device="cuda")
+    assert L.mtrt_hip_quantize(s, x.data_ptr(), pkg.F32, q.data_ptr(), pkg.F8E4M3FN, one.data_ptr(), pkg.SCALE_UNIFORM, 1, 40,
+                               1, pkg.F8_VIA_F16 | pkg.F8_REFHOST) == 1
+    assert b"two different conversions" in L.mtrt_hip_last_error()
+    assert L.mtrt_hip_quantize(s, x.data_ptr(), pkg.F32, q.data_ptr(), pkg.F8E4M3FN, one.data_ptr(), pkg.SCALE_UNIFORM, 1, 40,
+                               1, 8) == 1

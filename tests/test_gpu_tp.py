@@ -207,32 +207,105 @@ def test_quant_linear_reference_cases(tp):
         assert np.array_equal(out.torch().cpu().numpy(), np.full((4, 8), 5.0, dtype=np.float32))
 
 
-def test_quant_linear_fused_w8a8_matches_fake_quant(tp, orc):
-    """int8 Linear with an input scale and per-output-channel weight scales: the fused integer form
-    against a float64 product of the oracle's dequantized operands, 1e-3 relative (f16 result)."""
-    import torch
+def test_quant_linear_int8_runs_on_the_w8a8_cluster(tp, orc, pkg):
+    """int8 Linear with an input scale and per-output-channel weight scales lands on the integer matrix cores
+    (fragment-order weights prepared once): against a float64 product of the oracle's dequantized operands,
+    1e-3 relative (f16 result)."""
     r = rng(77)
-    M, K, N = 96, 256, 160
-    x = r.standard_normal((M, K)).astype(np.float32)
-    w = (r.standard_normal((N, K)) * 0.05).astype(np.float32)
-    s_x = np.float32(np.abs(x).max() / 127.0)
-    s_w = (np.abs(w).max(axis=1) / 127.0).astype(np.float32)
-    lin = tp.Linear(K, N, bias=False, quant_dtype=tp.int8, weight_quant_dim=0, fused=True)
-    lin.weight = tp.Tensor(w)
-    lin.weight_scale = tp.Tensor(s_w)
-    lin.input_scale = tp.Tensor(s_x)
-    out = lin(tp.Tensor(x)).torch().cpu().numpy().astype(np.float64)
+    for M, K, N, kernel in ((96, 256, 160, "mtrt_gemm_w8a8_frag"), (5, 72, 33, "mtrt_gemm_w8a8_nk_any")):
+        x = r.standard_normal((M, K)).astype(np.float32)
+        w = (r.standard_normal((N, K)) * 0.05).astype(np.float32)
+        b = r.standard_normal(N).astype(np.float32)
+        s_x = np.float32(np.abs(x).max() / 127.0)
+        s_w = (np.abs(w).max(axis=1) / 127.0).astype(np.float32)
+        lin = tp.Linear(K, N, quant_dtype=tp.int8, weight_quant_dim=0)
+        lin.load_state_dict({"weight": tp.Tensor(w), "bias": tp.Tensor(b), "weight_scale": tp.Tensor(s_w),
+                             "input_scale": tp.Tensor(s_x)})
+        assert lin.route() == "w8a8"
+        plan = lin._prepared()
+        out = lin(tp.Tensor(x)).torch().cpu().numpy().astype(np.float64)
+        assert lin._prepared() is plan, "the weight side must be prepared once, not per forward pass"
+        assert pkg.last_kernel() == kernel
 
-    qx = orc.quantize(x.ravel(), orc.F32, orc.I8, np.array([s_x]), orc.SCALE_UNIFORM, M, K)
-    qw = orc.quantize(w.ravel(), orc.F32, orc.I8, s_w, orc.SCALE_ROW, N, K, N)
-    xd = qx.astype(np.float64).reshape(M, K) * np.float64(s_x)
-    wd = qw.astype(np.float64).reshape(N, K) * s_w.astype(np.float64)[:, None]
-    ref = xd @ wd.T
-    tol = 1e-3 * np.abs(ref) + 2.0 ** -10 * np.abs(ref) + 1e-6     # 1e-3 relative + one f16 rounding
-    assert np.all(np.abs(out - ref) <= tol), float(np.max(np.abs(out - ref) / (np.abs(ref) + 1e-9)))
-    lin.fused = False
-    out2 = lin(tp.Tensor(x)).torch().cpu().numpy().astype(np.float64)
-    assert np.all(np.abs(out2 - ref) <= 1e-3 * np.abs(ref) + 1e-4)
+        qx = orc.quantize(x.ravel(), orc.F32, orc.I8, np.array([s_x]), orc.SCALE_UNIFORM, M, K)
+        qw = orc.quantize(w.ravel(), orc.F32, orc.I8, s_w, orc.SCALE_ROW, N, K, N)
+        xd = qx.astype(np.float64).reshape(M, K) * np.float64(s_x)
+        wd = qw.astype(np.float64).reshape(N, K) * s_w.astype(np.float64)[:, None]
+        core = xd @ wd.T
+        ref = core + b
+        tol = (1e-3 + 2.0 ** -10) * np.abs(core) + 1e-6 * (1 + np.abs(b))     # 1e-3 relative + one f16 rounding of the product
+        assert np.all(np.abs(out - ref) <= tol), float(np.max(np.abs(out - ref) / (np.abs(ref) + 1e-9)))
+        # a new weight tensor is picked up (the plan is keyed on the parameter objects)
+        lin.weight = tp.Tensor(2 * w)
+        lin.weight_scale = tp.Tensor(2 * s_w)
+        out2 = lin(tp.Tensor(x)).torch().cpu().numpy().astype(np.float64)
+        assert np.all(np.abs(out2 - (2 * core + b)) <= 2 * tol)
+        # the literal fake-quant form on the dense kernel agrees (weight scales along dim 0, no integer GEMM when
+        # the input scale is absent)
+        lin.input_scale = None
+        assert lin.route() == "dense"
+
+
+def test_quant_linear_int4_weight_only_runs_on_the_w4a16_cluster(tp, orc, pkg):
+    """float16 module, int4 weight-only, per-output-channel scales: W4A16 cluster on a prepack made once; checked
+    against the oracle's W4A16 program (same dequantize-then-accumulate order) and a float64 product."""
+    import torch
+    r = rng(78)
+    M, K, N = 48, 256, 96
+    x = r.standard_normal((M, K)).astype(np.float16)
+    w = (r.standard_normal((N, K)) * 0.1).astype(np.float16)
+    s_w = (np.abs(w.astype(np.float32)).max(axis=1) / 7.0).astype(np.float16)
+    lin = tp.Linear(K, N, bias=False, dtype=tp.float16, quant_dtype=tp.int4, weight_quant_dim=0)
+    lin.load_state_dict({"weight": tp.Tensor(w), "weight_scale": tp.Tensor(s_w)})
+    assert lin.route() == "w4a16"
+    out = lin(tp.Tensor(x)).torch()
+    assert pkg.last_kernel().startswith("mtrt_gemm_w4a16_") and not pkg.last_kernel().endswith("_any")
+    # oracle: codes [N,K] -> [K,N] packed, scales [1,N] with block = K
+    codes = orc.quantize(w.view(np.uint16).ravel(), orc.F16, orc.I4, s_w.astype(np.float32), orc.SCALE_ROW, N, K, N)
+    kn = np.ascontiguousarray(codes.reshape(N, K).T).ravel()
+    packed = (kn[0::2] | (kn[1::2] << 4)).astype(np.uint8)
+    ref = orc.gemm_w4a16(x.view(np.uint16), packed, s_w.view(np.uint16), K, N, K).ravel()
+    got = out.view(torch.int16).cpu().numpy().view(np.uint16).ravel()
+    gf, rf = orc.widen(got, orc.F16).astype(np.float64), orc.widen(ref, orc.F16).astype(np.float64)
+    sgn = np.where(codes >= 8, codes.astype(np.int32) - 16, codes.astype(np.int32))
+    wd = (sgn.reshape(N, K).astype(np.float32) * s_w.astype(np.float32)[:, None]).astype(np.float16).astype(np.float64)
+    exact = x.astype(np.float64) @ wd.T
+    mag = np.abs(x.astype(np.float64)) @ np.abs(wd.T)
+    tol = 1e-3 * np.abs(exact) + 2.0 ** -10 * np.abs(exact) + 3e-6 * mag + 1e-7
+    assert np.all(np.abs(gf - exact.ravel()) <= tol.ravel())
+    assert np.all(np.abs(gf - rf) <= 2 * tol.ravel())
+    # float32 module or a block-wise scale: dense route, same API
+    lin32 = tp.Linear(K, N, bias=False, quant_dtype=tp.int4, weight_quant_dim=0)
+    lin32.load_state_dict({"weight": tp.Tensor(w.astype(np.float32)), "weight_scale": tp.Tensor(s_w.astype(np.float32))})
+    assert lin32.route() == "dense"
+    o32 = lin32(tp.Tensor(x.astype(np.float32))).torch().cpu().numpy().astype(np.float64)
+    assert pkg.last_kernel() == "mtrt_gemm_dense_f32"
+    wd32 = (sgn.reshape(N, K).astype(np.float32) * s_w.astype(np.float32)[:, None]).astype(np.float64)
+    ex32 = x.astype(np.float64) @ wd32.T
+    assert np.all(np.abs(o32 - ex32) <= 1e-5 * (np.abs(x.astype(np.float64)) @ np.abs(wd32.T)) + 1e-6)
+
+
+@pytest.mark.parametrize("dname", ["float32", "float16", "bfloat16"])
+def test_dense_linear_against_float64(tp, pkg, dname):
+    """The unquantized module and ragged shapes on the dense kernel: f32 accumulation, result within the output
+    type's rounding of the float64 product; leading batch dimensions are folded."""
+    import torch
+    d = getattr(tp, dname)
+    td = {"float32": torch.float32, "float16": torch.float16, "bfloat16": torch.bfloat16}[dname]
+    torch.manual_seed(5)
+    for lead, K, N in (((3, 7), 50, 33), ((130,), 64, 129), ((1,), 1, 1)):
+        x = torch.randn(*lead, K, dtype=torch.float32).to(td)
+        w = (torch.randn(N, K, dtype=torch.float32) * 0.2).to(td)
+        b = torch.randn(N, dtype=torch.float32).to(td)
+        lin = tp.Linear(K, N, dtype=d)
+        lin.weight, lin.bias = tp.Tensor(w, dtype=d), tp.Tensor(b, dtype=d)
+        out = lin(tp.Tensor(x, dtype=d)).torch()
+        assert pkg.last_kernel() == "mtrt_gemm_dense_" + {"float32": "f32", "float16": "f16", "bfloat16": "bf16"}[dname]
+        assert tuple(out.shape) == lead + (N,)
+        ref = x.double() @ w.double().T + b.double()
+        mag = x.double().abs() @ w.double().abs().T + b.double().abs()
+        ulp = {"float32": 2.0 ** -23, "float16": 2.0 ** -10, "bfloat16": 2.0 ** -7}[dname]
+        assert bool(torch.all((out.cpu().double() - ref).abs() <= ulp * ref.abs() + 1e-5 * mag + 1e-30))
 
 
 def test_scale_from_amax(tp, orc):

@@ -106,6 +106,38 @@ def test_quantize_fp8_forms(orc):
     assert list(orc.widen(q, orc.F8E4M3FN)) == [448.0, 448.0, 448.0, -448.0]
 
 
+def test_quantize_fp8_via_f16_double_rounding(orc):
+    """The reference's GPU code generator converts f32 -> f16 -> f8 (NormalizeQuantizedConversions.cpp:38-118), two
+    roundings to nearest even.  Pinned as a composition of two independently pinned steps: numpy's float16 cast,
+    then the f16 -> f8 table minted from the reference's compiled DataTypes.cpp (IEEE-agreeing entries only:
+    |v| < 248 and outside the subnormal-carry window, where the host class is correct RNE)."""
+    import os
+    one = [np.float32(1)]
+    # hand-derived witnesses: 1.0625 is the midpoint of the f8 neighbours 1.0 (0x38, even) and 1.125 (0x39).
+    # 1.0625 + 2^-20 lies above it (direct: 0x39) but rounds to 1.0625 in f16 (ulp 2^-10), a tie -> even -> 0x38.
+    # 1.1875 is the midpoint of 1.125 (0x39, odd) and 1.25 (0x3A): from below, direct gives 0x39, via f16 0x3A.
+    w = np.float32([1.0625 + 2.0 ** -20, -(1.0625 + 2.0 ** -20), 1.1875 - 2.0 ** -20, 1.0625, 1.0625 + 2.0 ** -10])
+    direct = orc.quantize(w, orc.F32, orc.F8E4M3FN, one, orc.SCALE_UNIFORM, 1, w.size)
+    via = orc.quantize(w, orc.F32, orc.F8E4M3FN, one, orc.SCALE_UNIFORM, 1, w.size, 1, orc.F8_VIA_F16)
+    assert list(direct) == [0x39, 0xB9, 0x39, 0x38, 0x39]
+    assert list(via) == [0x38, 0xB8, 0x3A, 0x38, 0x39]
+    # composition against numpy + the golden table, on normally distributed quotients
+    tab = np.load(os.path.join(os.path.dirname(__file__), "golden", "lowp_from_f16_grid.npz"))
+    f16_to_f8_ref = tab["f8"]                      # reference host class applied to every f16 value (index = f16 bits)
+    x = (rng(31).standard_normal(1 << 18) * 60).astype(np.float32)
+    x = x[(np.abs(x) < 240) & (np.abs(x) > 0.02)]  # where the host class equals IEEE (quirks Q1-Q3 excluded)
+    via = orc.quantize(x, orc.F32, orc.F8E4M3FN, one, orc.SCALE_UNIFORM, 1, x.size, 1, orc.F8_VIA_F16)
+    h = x.astype(np.float16)                       # numpy: IEEE RNE
+    assert np.array_equal(via, f16_to_f8_ref[h.view(np.uint16)])
+    direct = orc.quantize(x, orc.F32, orc.F8E4M3FN, one, orc.SCALE_UNIFORM, 1, x.size)
+    frac = np.count_nonzero(via != direct) / x.size
+    assert 1e-4 < frac < 2e-2, frac                # the two policies do differ, on a small fraction
+    # f16-representable inputs: one rounding either way
+    hx = h.astype(np.float32)
+    assert np.array_equal(orc.quantize(hx, orc.F32, orc.F8E4M3FN, one, orc.SCALE_UNIFORM, 1, hx.size, 1, orc.F8_VIA_F16),
+                          orc.quantize(hx, orc.F32, orc.F8E4M3FN, one, orc.SCALE_UNIFORM, 1, hx.size))
+
+
 def test_dequantize_closed_form(orc):
     g = rng(4)
     d0, d1 = 16, 24
