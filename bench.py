@@ -234,6 +234,18 @@ def build_workloads(pkg, torch, which):
     return out
 
 
+_YARDSTICKS = []
+
+
+def yardstick_module(pkg):
+    """The code object with the measurement yardsticks (plain copy, matrix-core-only loop); they are not part of
+    the library's built-in module."""
+    if not _YARDSTICKS:
+        path = pkg.FIXTURE_MODULE_PATH.encode()
+        _YARDSTICKS.append(pkg.lib().mtrt_cuda_module_load_from_ptx_file(path, len(path)))
+    return _YARDSTICKS[0]
+
+
 def calibration_copy(pkg, torch):
     """One launch of the plain copy kernel over 128 MiB (reads 128 MiB, writes 128 MiB): the
     yardstick that hardware byte counters of a profiled run are scaled by."""
@@ -244,7 +256,7 @@ def calibration_copy(pkg, torch):
     dst = torch.empty_like(src)
     src.fill_(1)
     name = b"mtrt_copy_b128"
-    fn = L.mtrt_cuda_module_get_function(L.mtrt_hip_builtin_module(), name, len(name))
+    fn = L.mtrt_cuda_module_get_function(yardstick_module(pkg), name, len(name))
     vals = (ctypes.c_void_p(src.data_ptr()), ctypes.c_void_p(dst.data_ptr()), ctypes.c_int64(nbytes // 16))
     args = (ctypes.c_void_p * 3)(*[ctypes.cast(ctypes.pointer(v), ctypes.c_void_p) for v in vals])
     nvec = nbytes // 16
@@ -263,7 +275,7 @@ def mfma_sustained(pkg, torch, kernel, operand, ops_per_mfma):
     out = torch.empty(units * 256, dtype=torch.int32, device="cuda")
     assert operand.numel() * operand.element_size() >= (1 << 24)
     name = kernel.encode()
-    fn = L.mtrt_cuda_module_get_function(L.mtrt_hip_builtin_module(), name, len(name))
+    fn = L.mtrt_cuda_module_get_function(yardstick_module(pkg), name, len(name))
     vals = (ctypes.c_void_p(operand.data_ptr()), ctypes.c_void_p(out.data_ptr()), ctypes.c_int32(ksteps))
     args = (ctypes.c_void_p * 3)(*[ctypes.cast(ctypes.pointer(v), ctypes.c_void_p) for v in vals])
     s = torch.cuda.current_stream().cuda_stream

@@ -83,9 +83,13 @@ def test_embedded_code_object_is_gfx950_and_has_the_kernels(pkg):
         for v in ("v1", "v2", "v4", "v8", "v16", "any"):
             names += ["mtrt_layernorm_%s_%s" % (x, v), "mtrt_softmax_%s_%s" % (x, v)]
         names.append("mtrt_layernorm_%s_v8r" % x)
-    names.append("mtrt_copy_b128")
+    names += ["mtrt_fill", "mtrt_gemm_dense_f32", "mtrt_gemm_dense_f16", "mtrt_gemm_dense_bf16"]
     for n in names:
         assert n.encode() + b"\x00" in blob, "kernel %s is not in the code object" % n
+    # measurement yardsticks and launch-ABI fixtures live in their own module, not in the product code object
+    fixtures = open(pkg.FIXTURE_MODULE_PATH, "rb").read()
+    for n in ("mtrt_copy_b128", "mtrt_mfma_probe_f16", "mtrt_mfma_probe_i8", "add_kernel", "binary_shift_right"):
+        assert n.encode() + b"\x00" in fixtures and n.encode() + b"\x00" not in blob, n
 
 
 def test_status_calls_fail_loudly_without_a_gpu(pkg):

@@ -215,6 +215,28 @@ def test_c5_w4a16_full_size(pkg, orc, M):
     ref = np.concatenate([orc.gemm_w4a16(a, wp, s, K, N, B, m0=r, mcount=1) for r in rows])
     orc.set_threads(1)
     _check_w4a16(orc, got, a[rows], w, s, K, N, B, ref)
+    if M < 256:
+        return
+    # Every element of the launch against an independent evaluation: weights dequantised with torch (one f16
+    # rounding of the exact product), product in float64 on the GPU, the bound of _check_w4a16.
+    dev = y.device
+    af = torch.from_numpy(a.view(np.float16).astype(np.float32)).to(dev).double()
+    wd = (torch.from_numpy(w.astype(np.float16)).to(dev) *
+          torch.from_numpy(s.view(np.float16).copy()).to(dev).repeat_interleave(B, dim=0)).double()
+    exact = af @ wd
+    noise = 1e-3 * np.sqrt(K) * (af ** 2).mean(dim=1).sqrt()[:, None] * (wd ** 2).mean(dim=0).sqrt()[None, :]
+    ulp = torch.exp2(torch.floor(torch.log2(exact.abs().clamp_min(2.0 ** -14)))) * 2.0 ** -10
+    err = (y.double() - exact).abs()
+    excess = err - (1e-3 * exact.abs() + ulp + noise)
+    assert float(excess.max()) <= 0.0, "whole matrix vs float64: worst excess %g at flat index %d" % (
+        float(excess.max()), int(excess.argmax()))
+    del af, wd, exact, noise, ulp, err, excess
+    # ... and every row of one full band of 256-row tiles (all 43 column panels) against the oracle
+    band = list(range(256, 512)) if M >= 512 else list(range(0, 256))
+    orc.set_threads(16)
+    ref = orc.gemm_w4a16(a, wp, s, K, N, B, m0=band[0], mcount=len(band))
+    orc.set_threads(1)
+    _check_w4a16(orc, y[band].contiguous(), a[band], w, s, K, N, B, ref)
 
 
 @pytest.mark.parametrize("shape", [(9, 192, 8209), (20, 320, 12000), (32, 256, 16384), (12, 128, 16400), (3, 256, 9000)])

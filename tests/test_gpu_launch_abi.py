@@ -111,21 +111,46 @@ def test_events_and_devices(pkg):
     L.mtrt_cuda_stream_destroy(s)
 
 
-def test_builtin_module_launch_through_part1(pkg):
-    """A cluster kernel launched by hand through get_function + launch_kernel, with the
-    argument array the reference ABI prescribes (pointer, pointer, i64 size)."""
+def test_builtin_module_launch_through_part1(pkg, orc):
+    """A cluster kernel launched by hand through module_load / get_function / launch_kernel with the argument
+    array the reference's device ABI prescribes (ExpandMemRefArgs.cpp:65-120: bare pointers, i64 sizes, scalars by
+    value): mtrt_q_uniform_f32_i8(x, q, scale, n, d1, nb, flags), seven operands of three widths, checked against
+    the oracle; then the fused quantize+dequantize kernel the same way."""
+    import numpy as np
     import torch
     L = pkg.lib()
-    assert L.mtrt_hip_init() == 0, L.mtrt_hip_last_error()
-    mod = L.mtrt_hip_builtin_module()
-    fn = L.mtrt_cuda_module_get_function(mod, b"mtrt_copy_b128", 14)
-    src = torch.arange(4096, dtype=torch.int32, device="cuda")
-    dst = torch.zeros_like(src)
-    args, keep = _args(ctypes.c_void_p(src.data_ptr()), ctypes.c_void_p(dst.data_ptr()), ctypes.c_int64(1024))
-    stream = torch.cuda.current_stream().cuda_stream
-    L.mtrt_cuda_launch_kernel(fn, 4, 1, 1, 256, 1, 1, 0, stream, args)
-    torch.cuda.synchronize()
-    assert torch.equal(src, dst)
     size = ctypes.c_size_t(0)
     blob = L.mtrt_hip_builtin_code_object(ctypes.byref(size))
     assert blob and size.value > 1000
+    mod = L.mtrt_cuda_module_load_from_ptx(ctypes.string_at(blob, size.value), size.value)   # code object, not PTX
+    assert mod
+    rows, cols = 96, 4096
+    x_np = np.random.Generator(np.random.PCG64(12)).standard_normal((rows, cols), dtype=np.float32)
+    scale_np = np.float32(np.abs(x_np).max() / 127.0)
+    x = torch.from_numpy(x_np).cuda()
+    scale = torch.full((1,), float(scale_np), device="cuda")
+    q = torch.zeros(rows * cols, dtype=torch.int8, device="cuda")
+    n = rows * cols
+    stream = torch.cuda.current_stream().cuda_stream
+    name = b"mtrt_q_uniform_f32_i8"
+    fn = L.mtrt_cuda_module_get_function(mod, name, len(name))
+    args, keep = _args(ctypes.c_void_p(x.data_ptr()), ctypes.c_void_p(q.data_ptr()), ctypes.c_void_p(scale.data_ptr()),
+                       ctypes.c_int64(n), ctypes.c_int64(cols), ctypes.c_int64(1), ctypes.c_int32(0))
+    L.mtrt_cuda_launch_kernel(fn, (n + 4095) // 4096, 1, 1, 256, 1, 1, 0, stream, args)   # 256 lanes x 16 elements each
+    torch.cuda.synchronize()
+    q_ref = orc.quantize(x_np, orc.F32, orc.I8, [scale_np], orc.SCALE_UNIFORM, rows, cols)
+    assert np.array_equal(q.cpu().numpy(), q_ref)
+    # fused form: (x, q, y, scale, n, d1, nb, flags)
+    y = torch.zeros_like(x)
+    q.zero_()
+    name = b"mtrt_qdq_uniform_f32_i8"
+    fn2 = L.mtrt_cuda_module_get_function(mod, name, len(name))
+    args2, keep2 = _args(ctypes.c_void_p(x.data_ptr()), ctypes.c_void_p(q.data_ptr()), ctypes.c_void_p(y.data_ptr()),
+                         ctypes.c_void_p(scale.data_ptr()), ctypes.c_int64(n), ctypes.c_int64(cols), ctypes.c_int64(1),
+                         ctypes.c_int32(0))
+    L.mtrt_cuda_launch_kernel(fn2, (n + 4095) // 4096, 1, 1, 256, 1, 1, 0, stream, args2)
+    torch.cuda.synchronize()
+    assert np.array_equal(q.cpu().numpy(), q_ref)
+    y_ref = orc.dequantize(q_ref, orc.I8, orc.F32, [scale_np], orc.SCALE_UNIFORM, rows, cols)
+    assert np.array_equal(y.cpu().numpy().ravel().view(np.uint32), y_ref.view(np.uint32))
+    L.mtrt_cuda_module_unload(mod)
