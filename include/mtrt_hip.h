@@ -274,6 +274,25 @@ MTRT_CAPI_EXPORTED int32_t mtrt_hip_quantize_dequantize(mtrt_stream_t stream, co
                                                         int32_t scale_kind, int64_t d0, int64_t d1,
                                                         int64_t nb, int32_t flags);
 
+/* Dynamic per-tensor quantization, the whole chain of a dynamic-scale Q/DQ in one call:
+ *   amax = max |f32(x)| ; scale = amax / qmax ; q = convert(clamp(rne?(f32(x) / scale))) ; y = narrow(f32(q) * scale)
+ * (clusters of KernelSegmentation.cpp:53-113 in the program form of StablehloRaiseQDQ.cpp:233-265, 407-418; scale rule
+ * tripy/examples/nanogpt/weight_loader.py:67-68).  q_dtype: MTRT_I8 or MTRT_F8E4M3FN; y may be NULL (codes only);
+ * amax_out may be NULL; scale_out must be given.  Results are bit-identical to mtrt_hip_amax followed by
+ * mtrt_hip_quantize_dequantize.  A tensor that fits in the registers of one grid (n / 4 (f32) or n / 8 (f16, bf16)
+ * at most 16384 per compute unit, n a multiple of that vector length, x and y 16-byte aligned) runs as ONE
+ * launch that reads x once; its workgroups wait for each other's maximum with a bounded number of polls and a
+ * workgroup that gives up reduces the tensor by itself, so the launch finishes whatever else occupies the device.
+ * Larger or unaligned tensors run as the two launches above. */
+MTRT_CAPI_EXPORTED int32_t mtrt_hip_dynamic_quantize_dequantize(mtrt_stream_t stream, const void *x,
+                                                                int32_t x_dtype, void *q, int32_t q_dtype,
+                                                                void *y, int64_t n, float qmax,
+                                                                float *amax_out, float *scale_out,
+                                                                int32_t flags);
+/* Number of polls a workgroup of the one-launch form spends waiting for the grid's maximum before it computes
+ * the maximum by itself (default 65536; 0: never wait).  Returns the previous value.  Process-wide. */
+MTRT_CAPI_EXPORTED int32_t mtrt_hip_set_wait_limit(int32_t polls);
+
 /* NVFP4 block quantization, the two-level scaling of tensorrt.dynamic_quantize (TensorRTOps.td:3279-3358;
  * verifier mlir-tensorrt/tensorrt/lib/TensorRT/IR/Verification.cpp:1271-1290) in the program form of
  * mlir-tensorrt/integrations/PJRT/test/JAX/test_q_dq_nvfp4.py:21-45, over the [d0, d1] view of the tensor

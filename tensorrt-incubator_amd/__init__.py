@@ -90,6 +90,8 @@ PROTOTYPES = {
     "mtrt_hip_quantize": (_i32, [_vp, _vp, _i32, _vp, _i32, _vp, _i32, _i64, _i64, _i64, _i32]),
     "mtrt_hip_dequantize": (_i32, [_vp, _vp, _i32, _vp, _i32, _vp, _i32, _i64, _i64, _i64]),
     "mtrt_hip_quantize_dequantize": (_i32, [_vp, _vp, _i32, _vp, _i32, _vp, _vp, _i32, _i64, _i64, _i64, _i32]),
+    "mtrt_hip_dynamic_quantize_dequantize": (_i32, [_vp, _vp, _i32, _vp, _i32, _vp, _i64, _f32, _vp, _vp, _i32]),
+    "mtrt_hip_set_wait_limit": (_i32, [_i32]),
     "mtrt_hip_nvfp4_quantize": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _i64, _i64, _i32]),
     "mtrt_hip_nvfp4_dequantize": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i64, _i64, _i32]),
     "mtrt_hip_layernorm": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i64, _i64, _f32]),
@@ -210,6 +212,19 @@ def quantize_dequantize(x, scale, q_dtype, kind=SCALE_UNIFORM, d0=None, d1=None,
     check(lib().mtrt_hip_quantize_dequantize(_stream(), x.data_ptr(), float_dtype_of(x), q.data_ptr(), q_dtype,
                                              y.data_ptr(), scale.data_ptr(), kind, d0, d1, nb, flags))
     return q, y
+
+
+def dynamic_quantize_dequantize(x, q_dtype, qmax, flags=0, dequantize=True):
+    """amax -> scale -> quantize (-> dequantize) of the whole tensor in one call; returns (q, y or None, amax, scale)."""
+    torch = _torch()
+    assert x.is_cuda and x.is_contiguous()
+    out = torch.empty(2, dtype=torch.float32, device=x.device)
+    q = code_tensor(q_dtype, x.numel(), x.device)
+    y = torch.empty_like(x) if dequantize else None
+    check(lib().mtrt_hip_dynamic_quantize_dequantize(_stream(), x.data_ptr(), float_dtype_of(x), q.data_ptr(), q_dtype,
+                                                     _ptr(y), x.numel(), float(qmax), out.data_ptr(), out.data_ptr() + 4,
+                                                     flags))
+    return q, y, out[0], out[1]
 
 
 def nvfp4_quantize(x, tensor_amax, axis=-1):

@@ -2,6 +2,7 @@
 // the host side loads one module and resolves kernels by name.
 #include "amax.hip"
 #include "qdq.hip"
+#include "dynq.hip"
 #include "nvfp4.hip"
 #include "norm.hip"
 #include "gemm_w8a8.hip"

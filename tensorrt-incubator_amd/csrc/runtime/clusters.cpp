@@ -9,6 +9,7 @@
 #include "runtime_internal.hpp"
 
 #include <algorithm>
+#include <atomic>
 #include <cstdlib>
 
 using namespace mtrt_rt;
@@ -193,6 +194,58 @@ int32_t mtrt_hip_quantize_dequantize(mtrt_stream_t stream, const void *x, int32_
                                      int32_t q_dtype, void *y, const float *scale, int32_t scale_kind,
                                      int64_t d0, int64_t d1, int64_t nb, int32_t flags) {
   return qdq_dispatch(2, as_hip(stream), x, x_dtype, q, q_dtype, y, scale, scale_kind, d0, d1, nb, flags);
+}
+
+namespace {
+std::atomic<int32_t> g_wait_limit{1 << 16};
+} // namespace
+
+int32_t mtrt_hip_set_wait_limit(int32_t polls) {
+  return g_wait_limit.exchange(polls < 0 ? 0 : polls);
+}
+
+int32_t mtrt_hip_dynamic_quantize_dequantize(mtrt_stream_t stream, const void *x, int32_t x_dtype, void *q, int32_t q_dtype,
+                                             void *y, int64_t n, float qmax, float *amax_out, float *scale_out,
+                                             int32_t flags) {
+  clear_error();
+  const char *xn = float_name(x_dtype);
+  if (!xn)
+    return set_error(MTRT_INVALID_ARGUMENT, "float operand dtype %d is not one of f32/f16/bf16", x_dtype);
+  if (q_dtype != MTRT_I8 && q_dtype != MTRT_F8E4M3FN)
+    return set_error(MTRT_INVALID_ARGUMENT, "dynamic per-tensor quantization targets i8 or f8E4M3FN, got dtype %d", q_dtype);
+  if (n < 0)
+    return set_error(MTRT_INVALID_ARGUMENT, "negative element count %lld", (long long)n);
+  if (n > 0 && (!x || !q))
+    return set_error(MTRT_INVALID_ARGUMENT, "null operand");
+  if (!scale_out)
+    return set_error(MTRT_INVALID_ARGUMENT, "scale_out must point at device memory for one f32 (the quantize step reads the scale there)");
+  if (flags & ~(MTRT_Q_ROUND_TO_INT | MTRT_F8_REFHOST | MTRT_F8_VIA_F16))
+    return set_error(MTRT_INVALID_ARGUMENT, "unknown flag bits 0x%x", flags);
+  DeviceState *st = device_state();
+  if (!st)
+    return MTRT_RUNTIME_ERROR;
+  const int group = x_dtype == MTRT_F32 ? 4 : 8;
+  const int64_t nvec = n / group, units = num_compute_units(st);   // one workgroup per compute unit at most
+  const bool one_launch = n > 0 && n % group == 0 && aligned(x, 16) && aligned(q, group) && (!y || aligned(y, 16)) &&
+                          nvec <= units * 1024 * 16 && !((flags & MTRT_F8_REFHOST) && (flags & MTRT_F8_VIA_F16));
+  if (one_launch) {
+    uint32_t *slot = reduction_slot(st, as_hip(stream));
+    if (!slot)
+      return MTRT_RUNTIME_ERROR;
+    const int nv = nvec <= units * 1024 * 4 ? 4 : 16;
+    const uint32_t grid = uint32_t((nvec + int64_t(1024) * nv - 1) / (int64_t(1024) * nv));
+    int32_t limit = g_wait_limit.load();
+    void *args[] = {&x, &q, &y, &n, &qmax, &amax_out, &scale_out, &slot, &flags, &limit};
+    return launch(st, std::string("mtrt_dynqdq_") + xn + "_" + code_name(q_dtype) + "_v" + std::to_string(nv), grid, 1024,
+                  as_hip(stream), args);
+  }
+  // Does not fit in the registers of one grid (or is not vector-aligned): the reduction, then the element-wise pass.
+  const int32_t st1 = mtrt_hip_amax(stream, x, x_dtype, n, qmax, amax_out, scale_out);
+  if (st1 != MTRT_OK)
+    return st1;
+  if (y)
+    return qdq_dispatch(2, as_hip(stream), x, x_dtype, q, q_dtype, y, scale_out, MTRT_SCALE_UNIFORM, 1, n, 1, flags);
+  return qdq_dispatch(0, as_hip(stream), x, x_dtype, q, q_dtype, nullptr, scale_out, MTRT_SCALE_UNIFORM, 1, n, 1, flags);
 }
 
 namespace {

@@ -78,10 +78,10 @@ struct DeviceState {
   std::mutex mu;
   std::unordered_map<std::string, hipFunction_t> funcs;
   // One zeroed block per stream for single-launch grid reductions: 33 lines of
-  // 128 bytes (root + 32 first-level groups, see amax.hip), rounded up to 40.
-  // Kernels return their block to zero.
+  // 128 bytes for the arrival tree (root + 32 first-level groups, see amax.hip) and
+  // 17 for the broadcast of dynq.hip, rounded up to 64.  Kernels return their block to zero.
   static constexpr int kSlots = 256;
-  static constexpr int kSlotWords = 40 * 32;
+  static constexpr int kSlotWords = 64 * 32;
   uint32_t *slots = nullptr;
   std::map<hipStream_t, int> slot_of;
   std::vector<int> free_slots;   // slots of destroyed streams, handed out again before new ones

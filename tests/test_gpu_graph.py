@@ -65,3 +65,46 @@ def test_captured_pipeline_replays_like_eager(pkg):
         x2 = torch.randn(64, 256, device="cuda").to(torch.bfloat16)
         a2, _ = pkg.amax(x2, 448.0)
         assert float(a2) == float(x2.float().abs().max())
+
+
+def test_captured_one_launch_dynamic_quantization_replays_like_eager(pkg):
+    """The one-launch amax + quantize + dequantize kernel (workgroups that wait for each other, a scratch block that
+    restores itself) recorded into a graph: every replay gives the eager bits, also after eager launches in between."""
+    import torch
+    L = pkg.lib()
+    torch.manual_seed(12)
+    x = torch.randn(1024, 4096, device="cuda")
+    n = x.numel()
+    out = torch.zeros(2, device="cuda")
+    q = torch.zeros(n, dtype=torch.int8, device="cuda")
+    y = torch.zeros_like(x)
+    vp = ctypes.c_void_p
+
+    def run(stream):
+        pkg.check(L.mtrt_hip_dynamic_quantize_dequantize(vp(stream), vp(x.data_ptr()), pkg.F32, vp(q.data_ptr()), pkg.I8,
+                                                         vp(y.data_ptr()), n, ctypes.c_float(127.0), vp(out.data_ptr()),
+                                                         vp(out.data_ptr() + 4), 0))
+
+    run(torch.cuda.current_stream().cuda_stream)
+    assert pkg.last_kernel() == "mtrt_dynqdq_f32_i8_v4"
+    torch.cuda.synchronize()
+    want = (out.clone(), q.clone(), y.clone())
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        run(side.cuda_stream)
+        torch.cuda.synchronize()
+        graph.capture_begin()
+        run(side.cuda_stream)
+        graph.capture_end()
+    for replay in range(4):
+        for t in (out, q, y):
+            t.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for g, w, name in zip((out, q, y), want, ("amax/scale", "codes", "dequantized")):
+            assert torch.equal(g.view(torch.uint8), w.view(torch.uint8)), "replay %d: %s differ from the eager run" % (replay, name)
+        x2 = torch.randn(300, 1024, device="cuda")
+        q2, y2, a2, s2 = pkg.dynamic_quantize_dequantize(x2, pkg.I8, 127.0)
+        assert float(a2) == float(x2.abs().max())

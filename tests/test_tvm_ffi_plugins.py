@@ -88,8 +88,13 @@ def test_symbols_and_rejections_without_a_device(pkg):
 
 
 @pytest.mark.gpu
-def test_plugins_equal_the_cluster_entry_points(pkg):
+def test_plugins_against_the_oracle_and_the_cluster_entry_points(pkg, orc):
+    """Each plugin is called through its exported symbol with the argument array the reference's compiler emits and
+    its output is compared with the CPU oracle (bit for bit for amax, scales, codes, dequantized values and the int8
+    GEMM) and, for the two tolerance-checked reductions, with the cluster entry point it forwards to."""
+    import numpy as np
     import torch
+    from helpers import bits16
     L = pkg.lib()
     torch.manual_seed(21)
     res = Any()
@@ -106,24 +111,35 @@ def test_plugins_equal_the_cluster_entry_points(pkg):
     call("mtrt_amax", x, both, 448.0)
     amax, scale = pkg.amax(x, 448.0)
     assert torch.equal(both, torch.stack([amax.reshape(()), scale.reshape(())]))
+    xs = bits16(x)
+    amax_ref = orc.amax(xs, orc.BF16)
+    scale_ref = orc.scale_from_amax(amax_ref, 448.0)
+    assert both.cpu().numpy().tobytes() == np.array([amax_ref, scale_ref], dtype=np.float32).tobytes()
     q = torch.zeros(x.shape, dtype=torch.float8_e4m3fn, device="cuda")
     call("mtrt_quantize", x, both[1:], q)
     want_q = pkg.quantize(x, both[1:], pkg.F8E4M3FN)
     assert torch.equal(q.view(torch.uint8).ravel(), want_q.view(torch.uint8).ravel())
+    q_ref = orc.quantize(xs, orc.BF16, orc.F8E4M3FN, [scale_ref], orc.SCALE_UNIFORM, 240, 128)
+    assert np.array_equal(q.view(torch.uint8).cpu().numpy().ravel(), q_ref)
     y = torch.zeros_like(x)
     call("mtrt_dequantize", q, both[1:], y, None)
     want_y = pkg.dequantize(want_q, both[1:], pkg.F8E4M3FN, torch.bfloat16, x.shape)
     assert torch.equal(y.view(torch.int16), want_y.view(torch.int16).reshape(y.shape))
+    assert np.array_equal(bits16(y), orc.dequantize(q_ref, orc.F8E4M3FN, orc.BF16, [scale_ref], orc.SCALE_UNIFORM, 240, 128))
     # per-channel int8 on the middle axis (scale[row % 40] over [240, 128]) and on the last axis
     s_mid = (torch.rand(40, device="cuda") * 0.05 + 0.01)
     q8 = torch.zeros(x.shape, dtype=torch.int8, device="cuda")
     call("mtrt_quantize", x, s_mid, q8, 1)
     want = pkg.quantize(x, s_mid, pkg.I8, pkg.SCALE_ROW, 240, 128, 40)
     assert torch.equal(q8.ravel(), want.ravel())
+    assert np.array_equal(q8.cpu().numpy().ravel(),
+                          orc.quantize(xs, orc.BF16, orc.I8, s_mid.cpu().numpy(), orc.SCALE_ROW, 240, 128, 40))
     s_last = (torch.rand(128, device="cuda") * 0.05 + 0.01)
     call("mtrt_quantize", x, s_last, q8, 2)
     want = pkg.quantize(x, s_last, pkg.I8, pkg.SCALE_COL, 240, 128, 240)
     assert torch.equal(q8.ravel(), want.ravel())
+    assert np.array_equal(q8.cpu().numpy().ravel(),
+                          orc.quantize(xs, orc.BF16, orc.I8, s_last.cpu().numpy(), orc.SCALE_COL, 240, 128, 240))
     # block scale along the second-to-last axis: [6, 40, 128] with scale [6, 5, 128] (blocks of 8 rows)
     s_blk = (torch.rand(6, 5, 128, device="cuda") * 0.05 + 0.01)
     xb = x[0].contiguous()                                  # [40, 128] with scale [5, 128]
@@ -131,14 +147,20 @@ def test_plugins_equal_the_cluster_entry_points(pkg):
     call("mtrt_quantize", xb, s_blk[0].contiguous(), qb)
     want = pkg.quantize(xb, s_blk[0].contiguous(), pkg.I8, pkg.SCALE_COL, 40, 128, 8)
     assert torch.equal(qb.ravel(), want.ravel())
+    assert np.array_equal(qb.cpu().numpy().ravel(),
+                          orc.quantize(bits16(xb), orc.BF16, orc.I8, s_blk[0].cpu().numpy().ravel(), orc.SCALE_COL, 40, 128, 8))
     # fused reduce clusters
     g = (torch.rand(128, device="cuda") + 0.5).to(torch.bfloat16)
     b = (torch.randn(128, device="cuda") * 0.1).to(torch.bfloat16)
     out = torch.zeros_like(x)
     call("mtrt_layernorm", x, g, b, out, 1e-5)
     assert torch.equal(out.view(torch.int16), pkg.layernorm(x, g, b, 1e-5).view(torch.int16))
+    ln_ref = orc.widen(orc.layernorm(xs, bits16(g), bits16(b), orc.BF16, 240, 128, 1e-5), orc.BF16)
+    assert np.max(np.abs(orc.widen(bits16(out), orc.BF16) - ln_ref) / (np.abs(ln_ref) + 0.1)) <= 2.0 ** -7   # one bf16 ulp
     call("mtrt_softmax", x, out)
     assert torch.equal(out.view(torch.int16), pkg.softmax(x).view(torch.int16))
+    sm_ref = orc.widen(orc.softmax(xs, orc.BF16, 240, 128), orc.BF16)
+    assert np.max(np.abs(orc.widen(bits16(out), orc.BF16) - sm_ref) / (sm_ref + 1e-6)) <= 2.0 ** -7
     # int8 GEMM
     M, K, N = 96, 256, 160
     a = torch.randint(-128, 128, (M, K), dtype=torch.int8, device="cuda")
@@ -147,6 +169,8 @@ def test_plugins_equal_the_cluster_entry_points(pkg):
     yg = torch.zeros(M, N, dtype=torch.float16, device="cuda")
     call("mtrt_gemm_w8a8", a, w, a_s, w_s, yg)
     assert torch.equal(yg.view(torch.int16), pkg.gemm_w8a8(a, w, a_s, w_s).view(torch.int16))
+    y_ref = orc.gemm_w8a8(a.cpu().numpy(), np.ascontiguousarray(w.cpu().numpy().T), a_s.cpu().numpy(), w_s.cpu().numpy())
+    assert np.array_equal(bits16(yg).reshape(M, N), y_ref)
     # a failing cluster call surfaces as -1 with the cluster's message
     arr, keep = _args(x, torch.zeros(3, device="cuda"), q)       # 3 scale elements fit no mode
     assert _fn(L, "mtrt_quantize")(None, arr, 3, ctypes.byref(res)) == -1
