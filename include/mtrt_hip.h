@@ -232,6 +232,17 @@ MTRT_CAPI_EXPORTED const char *mtrt_hip_builtin_code_object(size_t *size);
 MTRT_CAPI_EXPORTED int32_t mtrt_hip_amax(mtrt_stream_t stream, const void *x, int32_t dtype,
                                          int64_t n, float qmax, float *amax_out, float *scale_out);
 
+/* amax and scale for every scale element of a per-channel or block-wise quantization: the tensor is viewed as
+ * [d0, d1] and `scale_kind` / `nb` address the scales exactly as in mtrt_hip_quantize below; each scale element
+ * gets amax = max |f32(x)| over the elements that address it and scale = amax / qmax
+ * (tripy/examples/nanogpt/weight_loader.py:67-68, 102-115).  MTRT_SCALE_ROW with nb = d0 gives one scale per row
+ * (per-token activation scales, per-output-channel weight scales); MTRT_SCALE_COL with nb = 128 the [d0 / 128, d1]
+ * scales of int4 block quantization along axis 0; MTRT_SCALE_UNIFORM forwards to mtrt_hip_amax.  Outputs hold nb
+ * (row kind) or (d0 / nb) * d1 (col kind) f32 values; either may be NULL. */
+MTRT_CAPI_EXPORTED int32_t mtrt_hip_amax_scales(mtrt_stream_t stream, const void *x, int32_t dtype,
+                                                int32_t scale_kind, int64_t d0, int64_t d1, int64_t nb,
+                                                float qmax, float *amax_out, float *scale_out);
+
 /* Grid reductions (mtrt_hip_amax and the kernels that fold an amax into another pass) meet in a small
  * block of device memory that the library keeps per stream and that every launch leaves zeroed.  A launch
  * that did not run to completion (a device fault, a killed process sharing the context) can leave it

@@ -45,6 +45,8 @@ def lib():
         L.orc_unpack_int4.restype, L.orc_unpack_int4.argtypes = None, [_vp, _vp, _i64]
         L.orc_amax.restype, L.orc_amax.argtypes = _f32, [_vp, _i32, _i64]
         L.orc_scale_from_amax.restype, L.orc_scale_from_amax.argtypes = _f32, [_f32, _f32]
+        L.orc_amax_scales.restype = None
+        L.orc_amax_scales.argtypes = [_vp, _i32, _i32, _i64, _i64, _i64, _f32, _vp, _vp]
         L.orc_quantize.restype = None
         L.orc_quantize.argtypes = [_vp, _i32, _vp, _i32, _vp, _i32, _i64, _i64, _i64, _i32, _i32]
         L.orc_dequantize.restype = None
@@ -149,6 +151,16 @@ def amax(x, dtype):
 
 def scale_from_amax(amax_value, qmax):
     return np.float32(lib().orc_scale_from_amax(float(amax_value), float(qmax)))
+
+
+def amax_scales(x, dtype, kind, d0, d1, nb, qmax):
+    """(amax, scale) arrays, one element per scale element of the addressing (kind, nb)."""
+    x = _c_arr(x, dtype)
+    count = 1 if kind == SCALE_UNIFORM else (nb if kind == SCALE_ROW else (d0 // nb) * d1)
+    amax = np.zeros(count, dtype=np.float32)
+    scale = np.zeros(count, dtype=np.float32)
+    lib().orc_amax_scales(_p(x), dtype, kind, d0, d1, nb, float(qmax), _p(amax), _p(scale))
+    return amax, scale
 
 
 def quantize(x, in_dtype, out_dtype, scale, kind, d0, d1, nb=1, flags=0, mode=IEEE):

@@ -87,6 +87,13 @@ float orc_amax(const void *x, int dtype, int64_t n);
 /* scale = amax / qmax, one f32 divide */
 float orc_scale_from_amax(float amax, float qmax);
 
+/* amax and scale = amax / qmax for EVERY scale element of the addressing (scale_kind, nscale_or_block) over the
+ * [d0, d1] view: the per-channel / block-wise form of the calibration rule
+ * (tripy/examples/nanogpt/weight_loader.py:67-68, 102-115).  Outputs: nscale (row kind) or (d0 / block) * d1
+ * (col kind) values, 1 for uniform; either may be NULL.  Scale elements no input addresses get amax 0. */
+void orc_amax_scales(const void *x, int dtype, int scale_kind, int64_t d0, int64_t d1, int64_t nscale_or_block,
+                     float qmax, float *amax_out, float *scale_out);
+
 /* q = convert(clamp(lo, [rne](f32(x) / scale), hi))
  *   (StablehloRaiseQDQ.cpp:233-265; TensorRTOps.td:3133-3194)
  * lo/hi follow out_dtype: i8 [-128,127], f8 [-448,448], i4 [-8,7], f4 [-6,6] (converted through f16). */

@@ -139,6 +139,24 @@ float orc_amax(const void *x, int dtype, int64_t n) {
 
 float orc_scale_from_amax(float amax, float qmax) { return amax / qmax; }
 
+void orc_amax_scales(const void *x, int dtype, int scale_kind, int64_t d0, int64_t d1, int64_t nb, float qmax,
+                     float *amax_out, float *scale_out) {
+  const int64_t count = scale_kind == ORC_SCALE_UNIFORM ? 1 : (scale_kind == ORC_SCALE_ROW ? nb : (d0 / nb) * d1);
+  std::vector<float> amax(size_t(count), 0.0f);       // reduce init for max(abs(.)) is 0
+  for (int64_t r = 0; r < d0; ++r)
+    for (int64_t c = 0; c < d1; ++c) {
+      const float a = std::fabs(load_as_f32(x, dtype, r * d1 + c));
+      float &m = amax[size_t(scale_index(scale_kind, r, c, d1, nb))];
+      m = a > m ? a : m;
+    }
+  for (int64_t i = 0; i < count; ++i) {
+    if (amax_out)
+      amax_out[i] = amax[size_t(i)];
+    if (scale_out)
+      scale_out[i] = amax[size_t(i)] / qmax;
+  }
+}
+
 void orc_quantize(const void *x, int in_dtype, void *q, int out_dtype, const float *scale,
                   int scale_kind, int64_t d0, int64_t d1, int64_t nb, int flags, int mode) {
   const ConvMode m = ConvMode(mode);

@@ -85,6 +85,7 @@ PROTOTYPES = {
     "mtrt_hip_builtin_module": (_vp, []),
     "mtrt_hip_builtin_code_object": (_vp, [_c.POINTER(_sz)]),
     "mtrt_hip_amax": (_i32, [_vp, _vp, _i32, _i64, _f32, _vp, _vp]),
+    "mtrt_hip_amax_scales": (_i32, [_vp, _vp, _i32, _i32, _i64, _i64, _i64, _f32, _vp, _vp]),
     "mtrt_hip_reset_reductions": (_i32, [_vp]),
     "mtrt_hip_amax_no_alloc": (_i32, [_vp, _vp, _i32, _i64, _f32, _vp, _vp]),
     "mtrt_hip_quantize": (_i32, [_vp, _vp, _i32, _vp, _i32, _vp, _i32, _i64, _i64, _i64, _i32]),
@@ -181,6 +182,19 @@ def amax(x, qmax):
     out = torch.empty(2, dtype=torch.float32, device=x.device)
     check(lib().mtrt_hip_amax(_stream(), x.data_ptr(), float_dtype_of(x), x.numel(), float(qmax),
                               out.data_ptr(), out.data_ptr() + 4))
+    return out[0], out[1]
+
+
+def amax_scales(x, qmax, kind, d0=None, d1=None, nb=1):
+    """(amax, scale) f32 device tensors with one element per scale element of the addressing (kind, nb) over the
+    [d0, d1] view of x: nb elements for SCALE_ROW, (d0 / nb) * d1 for SCALE_COL, one for SCALE_UNIFORM."""
+    torch = _torch()
+    assert x.is_cuda and x.is_contiguous()
+    d0, d1 = _view2d(x, d0, d1)
+    count = 1 if kind == SCALE_UNIFORM else (nb if kind == SCALE_ROW else (d0 // nb) * d1)
+    out = torch.empty((2, max(count, 0)), dtype=torch.float32, device=x.device)
+    check(lib().mtrt_hip_amax_scales(_stream(), x.data_ptr(), float_dtype_of(x), kind, d0, d1, nb, float(qmax),
+                                     out[0].data_ptr(), out[1].data_ptr()))
     return out[0], out[1]
 
 

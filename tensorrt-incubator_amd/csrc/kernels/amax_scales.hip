@@ -1,0 +1,164 @@
+// amax per scale element: the reduction that produces the scales of the per-channel and block-wise modes of
+// tensorrt.quantize (TensorRTOps.td:3133-3194), as the calibration flow computes them
+//   scale = amax.float() / maxbound        tripy/examples/nanogpt/weight_loader.py:67-68
+//   int4 blocks: amax reshaped per block   weight_loader.py:102-115
+// The tensor is viewed as row-major [d0, d1] and the scale addressing is the one of qdq.hip:
+//   row : scale[row % nb]            one scale per row (nb = d0: per-token / per-output-channel, blocks along the last
+//                                    axis) or per channel of a middle axis (rows r, r + nb, ... share a scale)
+//   col : scale[(row / nb) * d1 + c] blocks of nb rows per column (nb = d0: per-channel on the last axis)
+// For every scale element: amax = max |f32(x)| over the elements that address it (exact in any order, so the result
+// is bit-identical to a sequential host reduction), scale = amax / qmax (one IEEE divide).  The reference's generated
+// reduction walks each row serially per thread (mlir-tensorrt/kernel/lib/Utils/TilingUtils.cpp:669-677); here a wave
+// owns a scale (row kinds) or a workgroup a 64-vector-wide strip of one block (col kind), 128-bit loads throughout.
+#include "common.hpp"
+
+namespace amax_scales_cluster {
+
+using namespace mtrt_dev;
+using namespace amax_cluster;
+
+// max |.| of each of the G elements of a vector, as orderable bit patterns (see AbsBits)
+template <typename X> struct AbsEach;
+template <> struct AbsEach<F32> {
+  static constexpr int G = 4;
+  static __device__ __forceinline__ void acc(u32x4 t, uint32_t (&m)[4]) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) { const uint32_t a = t[k] & 0x7FFFFFFFu; m[k] = m[k] > a ? m[k] : a; }
+  }
+};
+template <> struct AbsEach<BF16> {
+  static constexpr int G = 8;
+  static __device__ __forceinline__ void acc(u32x4 t, uint32_t (&m)[8]) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t lo = (t[k] << 16) & 0x7FFF0000u, hi = t[k] & 0x7FFF0000u;
+      m[2 * k] = m[2 * k] > lo ? m[2 * k] : lo;
+      m[2 * k + 1] = m[2 * k + 1] > hi ? m[2 * k + 1] : hi;
+    }
+  }
+};
+template <> struct AbsEach<F16> {
+  static constexpr int G = 8;
+  static __device__ __forceinline__ void acc(u32x4 t, uint32_t (&m)[8]) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t lo = t[k] & 0x7FFFu, hi = (t[k] >> 16) & 0x7FFFu;
+      m[2 * k] = m[2 * k] > lo ? m[2 * k] : lo;
+      m[2 * k + 1] = m[2 * k + 1] > hi ? m[2 * k + 1] : hi;
+    }
+  }
+};
+
+__device__ __forceinline__ void emit(float amax, float qmax, float* amax_out, float* scale_out, int64_t idx) {
+  if (amax_out) amax_out[idx] = amax;
+  if (scale_out) scale_out[idx] = amax / qmax;
+}
+
+// row kind: wave `s` (of nb) reduces rows s, s + nb, ... ; VEC: d1 % G == 0 and x 16-byte aligned
+template <typename X, bool VEC>
+__device__ __forceinline__ void rows_body(const typename X::storage* __restrict__ x, int64_t d0, int64_t d1, int64_t nb,
+                                          float qmax, float* __restrict__ amax_out, float* __restrict__ scale_out) {
+  using A = AbsBits<X>;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t s = (int64_t(blockIdx.x) * blockDim.x + threadIdx.x) / kWave;
+  if (s >= nb) return;                               // whole waves leave together
+  uint32_t m = 0;
+  for (int64_t row = s; row < d0; row += nb) {
+    const typename X::storage* p = x + row * d1;
+    if (VEC) {
+      const u32x4* pv = reinterpret_cast<const u32x4*>(p);
+      const int64_t nvec = d1 / A::kPerVec;
+      int64_t v = lane;
+      for (; v + 3 * kWave < nvec; v += 4 * kWave) {   // four independent loads in flight
+        u32x4 t[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) t[u] = __builtin_nontemporal_load(pv + v + u * kWave);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) { const uint32_t a = A::of(t[u]); m = m > a ? m : a; }
+      }
+      for (; v < nvec; v += kWave) { const uint32_t a = A::of(__builtin_nontemporal_load(pv + v)); m = m > a ? m : a; }
+    } else {
+      for (int64_t c = lane; c < d1; c += kWave) { const uint32_t a = A::one(p + c); m = m > a ? m : a; }
+    }
+  }
+  m = wave_reduce(m, MaxU32());
+  if (lane == 0) emit(A::finish(m), qmax, amax_out, scale_out, s);
+}
+
+// col kind, vector form: workgroup = (block b, strip of 64 vectors of columns); wave w takes rows w, w + 4, ... of
+// the block, lane l the vector column strip * 64 + l; the four waves' partial maxima meet in LDS.
+template <typename X>
+__device__ __forceinline__ void cols_body(const typename X::storage* __restrict__ x, int64_t d0, int64_t d1, int64_t nb,
+                                          float qmax, float* __restrict__ amax_out, float* __restrict__ scale_out) {
+  using E = AbsEach<X>;
+  constexpr int G = E::G;
+  __shared__ uint32_t part[4][kWave][G + 1];
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int64_t nvec = d1 / G, strips = (nvec + kWave - 1) / kWave;
+  const int64_t b = blockIdx.x / strips, strip = blockIdx.x % strips;
+  const int64_t vcol = strip * kWave + lane;
+  uint32_t m[G];
+#pragma unroll
+  for (int k = 0; k < G; ++k) m[k] = 0;
+  if (vcol < nvec) {
+    const u32x4* pv = reinterpret_cast<const u32x4*>(x + (b * nb) * d1) + vcol;
+    int64_t r = wave;
+    for (; r + 12 < nb; r += 16) {                     // four independent loads in flight
+      u32x4 t[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) t[u] = __builtin_nontemporal_load(pv + (r + 4 * u) * nvec);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) E::acc(t[u], m);
+    }
+    for (; r < nb; r += 4) E::acc(__builtin_nontemporal_load(pv + r * nvec), m);
+  }
+#pragma unroll
+  for (int k = 0; k < G; ++k) part[wave][lane][k] = m[k];
+  __syncthreads();
+  if (wave == 0 && vcol < nvec) {
+#pragma unroll
+    for (int k = 0; k < G; ++k) {
+      uint32_t r = part[0][lane][k];
+#pragma unroll
+      for (int w = 1; w < 4; ++w) r = r > part[w][lane][k] ? r : part[w][lane][k];
+      emit(AbsBits<X>::finish(r), qmax, amax_out, scale_out, b * d1 + vcol * G + k);
+    }
+  }
+}
+
+// col kind, any shape: one lane per (block, column)
+template <typename X>
+__device__ __forceinline__ void cols_any_body(const typename X::storage* __restrict__ x, int64_t d0, int64_t d1, int64_t nb,
+                                              float qmax, float* __restrict__ amax_out, float* __restrict__ scale_out) {
+  using A = AbsBits<X>;
+  const int64_t total = (d0 / nb) * d1;
+  for (int64_t e = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; e < total; e += int64_t(gridDim.x) * blockDim.x) {
+    const int64_t b = e / d1, c = e - b * d1;
+    uint32_t m = 0;
+    for (int64_t r = 0; r < nb; ++r) { const uint32_t a = A::one(x + (b * nb + r) * d1 + c); m = m > a ? m : a; }
+    emit(A::finish(m), qmax, amax_out, scale_out, e);
+  }
+}
+
+}  // namespace amax_scales_cluster
+
+// (x, d0, d1, nb, qmax, amax_out or null, scale_out or null)
+//   rows / rows_any : grid = ceil(nb / 4), block = 256 (one wave per scale)
+//   cols            : grid = (d0 / nb) * ceil(d1 / G / 64), block = 256 ; d1 % G == 0, x 16-byte aligned
+//   cols_any        : grid-stride, block = 256
+#define MTRT_AMAX_SCALES_KERNELS(XN, XT)                                                                              \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_amax_rows_##XN(                                               \
+      const XT::storage* x, int64_t d0, int64_t d1, int64_t nb, float qmax, float* amax_out, float* scale_out) {       \
+    amax_scales_cluster::rows_body<XT, true>(x, d0, d1, nb, qmax, amax_out, scale_out); }                              \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_amax_rows_any_##XN(                                           \
+      const XT::storage* x, int64_t d0, int64_t d1, int64_t nb, float qmax, float* amax_out, float* scale_out) {       \
+    amax_scales_cluster::rows_body<XT, false>(x, d0, d1, nb, qmax, amax_out, scale_out); }                             \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_amax_cols_##XN(                                               \
+      const XT::storage* x, int64_t d0, int64_t d1, int64_t nb, float qmax, float* amax_out, float* scale_out) {       \
+    amax_scales_cluster::cols_body<XT>(x, d0, d1, nb, qmax, amax_out, scale_out); }                                    \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_amax_cols_any_##XN(                                           \
+      const XT::storage* x, int64_t d0, int64_t d1, int64_t nb, float qmax, float* amax_out, float* scale_out) {       \
+    amax_scales_cluster::cols_any_body<XT>(x, d0, d1, nb, qmax, amax_out, scale_out); }
+MTRT_AMAX_SCALES_KERNELS(f32, F32)
+MTRT_AMAX_SCALES_KERNELS(f16, F16)
+MTRT_AMAX_SCALES_KERNELS(bf16, BF16)

@@ -1,6 +1,7 @@
 // The built-in kernel module: every cluster kernel in one gfx950 code object, so
 // the host side loads one module and resolves kernels by name.
 #include "amax.hip"
+#include "amax_scales.hip"
 #include "qdq.hip"
 #include "dynq.hip"
 #include "nvfp4.hip"

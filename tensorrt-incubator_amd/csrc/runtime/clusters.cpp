@@ -178,6 +178,53 @@ int32_t mtrt_hip_amax(mtrt_stream_t stream, const void *x, int32_t dtype, int64_
   return launch(st, std::string("mtrt_amax_") + xn, grid, kBlock, as_hip(stream), args);
 }
 
+int32_t mtrt_hip_amax_scales(mtrt_stream_t stream, const void *x, int32_t dtype, int32_t scale_kind, int64_t d0, int64_t d1,
+                             int64_t nb, float qmax, float *amax_out, float *scale_out) {
+  clear_error();
+  const char *xn = float_name(dtype);
+  if (!xn)
+    return set_error(MTRT_INVALID_ARGUMENT, "amax input dtype %d is not one of f32/f16/bf16", dtype);
+  if (d0 < 0 || d1 < 0)
+    return set_error(MTRT_INVALID_ARGUMENT, "negative extent [%lld, %lld]", (long long)d0, (long long)d1);
+  if (scale_kind < MTRT_SCALE_UNIFORM || scale_kind > MTRT_SCALE_COL)
+    return set_error(MTRT_INVALID_ARGUMENT, "unknown scale kind %d", scale_kind);
+  if (scale_kind == MTRT_SCALE_UNIFORM)
+    return mtrt_hip_amax(stream, x, dtype, d0 * d1, qmax, amax_out, scale_out);
+  if (nb <= 0)
+    return set_error(MTRT_INVALID_ARGUMENT, "scale kind %d needs a positive scale count / block size, got %lld", scale_kind,
+                     (long long)nb);
+  if (scale_kind == MTRT_SCALE_ROW && nb > d0 && d0 > 0)
+    return set_error(MTRT_INVALID_ARGUMENT, "%lld scales for %lld rows", (long long)nb, (long long)d0);
+  if (scale_kind == MTRT_SCALE_COL && d0 % nb != 0)
+    return set_error(MTRT_INVALID_ARGUMENT, "block size %lld does not divide the blocked extent %lld", (long long)nb,
+                     (long long)d0);
+  if (d0 == 0 || d1 == 0)
+    return MTRT_OK;                                    // no scale element has an input
+  if (!x || (!amax_out && !scale_out))
+    return set_error(MTRT_INVALID_ARGUMENT, "null operand");
+  if (!aligned(x, float_bytes(dtype)))
+    return set_error(MTRT_INVALID_ARGUMENT, "input is not aligned to its element size");
+  DeviceState *st = device_state();
+  if (!st)
+    return MTRT_RUNTIME_ERROR;
+  const int group = dtype == MTRT_F32 ? 4 : 8;
+  const bool vec = d1 % group == 0 && aligned(x, 16);
+  void *args[] = {&x, &d0, &d1, &nb, &qmax, &amax_out, &scale_out};
+  if (scale_kind == MTRT_SCALE_ROW) {
+    const int64_t blocks = (nb + 3) / 4;
+    if (blocks > int64_t(kMaxGrid) * 1024)
+      return set_error(MTRT_INVALID_ARGUMENT, "%lld scales are too many for one launch", (long long)nb);
+    return launch(st, std::string(vec ? "mtrt_amax_rows_" : "mtrt_amax_rows_any_") + xn, uint32_t(blocks), kBlock,
+                  as_hip(stream), args);
+  }
+  if (vec) {
+    const int64_t blocks = (d0 / nb) * ((d1 / group + 63) / 64);
+    if (blocks <= int64_t(kMaxGrid) * 1024)
+      return launch(st, std::string("mtrt_amax_cols_") + xn, uint32_t(blocks), kBlock, as_hip(stream), args);
+  }
+  return launch(st, std::string("mtrt_amax_cols_any_") + xn, blocks_for((d0 / nb) * d1, kBlock), kBlock, as_hip(stream), args);
+}
+
 int32_t mtrt_hip_quantize(mtrt_stream_t stream, const void *x, int32_t x_dtype, void *q, int32_t q_dtype,
                           const float *scale, int32_t scale_kind, int64_t d0, int64_t d1, int64_t nb,
                           int32_t flags) {

@@ -22,6 +22,34 @@ def test_amax_and_scale(orc):
     assert orc.amax(np.zeros(0, dtype=np.float32), orc.F32) == 0.0
 
 
+def test_amax_per_scale_element_closed_form(orc):
+    """Per-channel and block-wise amax against numpy's reductions over the reshaped tensor; the scale is one f32
+    divide per element.  The index invariants tell the addressings apart: per-row vs per-channel-of-a-middle-axis
+    (rows r and r + C share), blocks of rows per column vs per-column over all rows."""
+    g = rng(11)
+    x = (g.standard_normal((24, 40)) * 5).astype(np.float32)
+    ax = np.abs(x)
+    a, s = orc.amax_scales(x, orc.F32, orc.SCALE_ROW, 24, 40, 24, 127.0)           # one scale per row
+    assert np.array_equal(a, ax.max(axis=1)) and np.array_equal(s, (ax.max(axis=1) / np.float32(127.0)).astype(np.float32))
+    a, _ = orc.amax_scales(x, orc.F32, orc.SCALE_ROW, 24, 40, 6, 127.0)            # [4, 6, 40], channel axis 1
+    assert np.array_equal(a, ax.reshape(4, 6, 40).max(axis=(0, 2)))
+    a, s = orc.amax_scales(x, orc.F32, orc.SCALE_COL, 24, 40, 8, 7.0)              # blocks of 8 rows per column
+    assert np.array_equal(a, ax.reshape(3, 8, 40).max(axis=1).ravel())
+    assert np.array_equal(s, (ax.reshape(3, 8, 40).max(axis=1).ravel() / np.float32(7.0)).astype(np.float32))
+    a, _ = orc.amax_scales(x, orc.F32, orc.SCALE_COL, 24, 40, 24, 448.0)           # per channel on the last axis
+    assert np.array_equal(a, ax.max(axis=0))
+    a, s = orc.amax_scales(x, orc.F32, orc.SCALE_UNIFORM, 24, 40, 1, 448.0)
+    assert a[0] == ax.max() and s[0] == np.float32(ax.max()) / np.float32(448.0)
+    xb = orc.narrow(x, orc.BF16)
+    a, _ = orc.amax_scales(xb, orc.BF16, orc.SCALE_COL, 24, 40, 8, 7.0)
+    assert np.array_equal(a, np.abs(orc.widen(xb, orc.BF16)).reshape(3, 8, 40).max(axis=1).ravel())
+    # quantizing with those scales uses the whole code range and never saturates past it
+    a, s = orc.amax_scales(x, orc.F32, orc.SCALE_COL, 24, 40, 8, 7.0)
+    q = orc.quantize(x, orc.F32, orc.I4, s, orc.SCALE_COL, 24, 40, 8)
+    codes = np.where(q >= 8, q.astype(np.int32) - 16, q.astype(np.int32)).reshape(3, 8, 40)
+    assert np.array_equal(np.abs(codes).max(axis=1).ravel(), np.full(120, 7))
+
+
 @pytest.mark.parametrize("qd,lo,hi", [("I8", -128, 127), ("I4", -8, 7)])
 def test_quantize_int_closed_form(orc, qd, lo, hi):
     g = rng(2)
