@@ -304,6 +304,27 @@ MTRT_CAPI_EXPORTED int32_t mtrt_hip_dynamic_quantize_dequantize(mtrt_stream_t st
  * the maximum by itself (default 65536; 0: never wait).  Returns the previous value.  Process-wide. */
 MTRT_CAPI_EXPORTED int32_t mtrt_hip_set_wait_limit(int32_t polls);
 
+/* quantize / dequantize on rank-2 VIEWS (slices, transposes, offset sub-tensors): each tensor operand is a base
+ * pointer plus (offset, stride0, stride1) in elements, element (r, c) of the [d0, d1] view at
+ * base[offset + r * stride0 + c * stride1], which is how the reference hands a dynamic strided memref to a
+ * generated kernel (ExpandMemRefArgs.cpp:65-120: base, offset, sizes, strides; order pinned by
+ * compiler/test/Passes/1_Core/KernelToCUDA/kernel-to-cuda.mlir:3-48).  Codes are one per byte (MTRT_I8,
+ * MTRT_F8E4M3FN, MTRT_I4); the scale is contiguous and addressed by the logical (r, c) as above.  A view may not
+ * reach below its base pointer; that it stays inside the allocation is the caller's responsibility, as it is for
+ * generated kernels.  Results equal those of the contiguous entry points on a packed copy of the view. */
+typedef struct mtrt_hip_view2d {
+  int64_t offset, stride0, stride1;
+} mtrt_hip_view2d;
+MTRT_CAPI_EXPORTED int32_t mtrt_hip_quantize_view(mtrt_stream_t stream, const void *x, int32_t x_dtype,
+                                                  const mtrt_hip_view2d *x_view, void *q, int32_t q_dtype,
+                                                  const mtrt_hip_view2d *q_view, const float *scale,
+                                                  int32_t scale_kind, int64_t d0, int64_t d1, int64_t nb,
+                                                  int32_t flags);
+MTRT_CAPI_EXPORTED int32_t mtrt_hip_dequantize_view(mtrt_stream_t stream, const void *q, int32_t q_dtype,
+                                                    const mtrt_hip_view2d *q_view, void *y, int32_t y_dtype,
+                                                    const mtrt_hip_view2d *y_view, const float *scale,
+                                                    int32_t scale_kind, int64_t d0, int64_t d1, int64_t nb);
+
 /* NVFP4 block quantization, the two-level scaling of tensorrt.dynamic_quantize (TensorRTOps.td:3279-3358;
  * verifier mlir-tensorrt/tensorrt/lib/TensorRT/IR/Verification.cpp:1271-1290) in the program form of
  * mlir-tensorrt/integrations/PJRT/test/JAX/test_q_dq_nvfp4.py:21-45, over the [d0, d1] view of the tensor

@@ -93,6 +93,8 @@ PROTOTYPES = {
     "mtrt_hip_quantize_dequantize": (_i32, [_vp, _vp, _i32, _vp, _i32, _vp, _vp, _i32, _i64, _i64, _i64, _i32]),
     "mtrt_hip_dynamic_quantize_dequantize": (_i32, [_vp, _vp, _i32, _vp, _i32, _vp, _i64, _f32, _vp, _vp, _i32]),
     "mtrt_hip_set_wait_limit": (_i32, [_i32]),
+    "mtrt_hip_quantize_view": (_i32, [_vp, _vp, _i32, _vp, _vp, _i32, _vp, _vp, _i32, _i64, _i64, _i64, _i32]),
+    "mtrt_hip_dequantize_view": (_i32, [_vp, _vp, _i32, _vp, _vp, _i32, _vp, _vp, _i32, _i64, _i64, _i64]),
     "mtrt_hip_nvfp4_quantize": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _i64, _i64, _i32]),
     "mtrt_hip_nvfp4_dequantize": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i64, _i64, _i32]),
     "mtrt_hip_layernorm": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i64, _i64, _f32]),
@@ -239,6 +241,37 @@ def dynamic_quantize_dequantize(x, q_dtype, qmax, flags=0, dequantize=True):
                                                      _ptr(y), x.numel(), float(qmax), out.data_ptr(), out.data_ptr() + 4,
                                                      flags))
     return q, y, out[0], out[1]
+
+
+class View2d(ctypes.Structure):
+    """struct mtrt_hip_view2d"""
+    _fields_ = [("offset", _i64), ("stride0", _i64), ("stride1", _i64)]
+
+
+def _view_of(t):
+    """(base pointer of the storage, View2d) of a rank-2 torch view."""
+    assert t.dim() == 2
+    base = t.data_ptr() - t.storage_offset() * t.element_size()
+    return base, View2d(t.storage_offset(), t.stride(0), t.stride(1))
+
+
+def quantize_view(x, scale, q_dtype, q_out, kind=SCALE_UNIFORM, nb=1, flags=0):
+    """Quantize the rank-2 view `x` (any strides) into the rank-2 view `q_out` (int8 / uint8 storage, any strides)."""
+    assert x.is_cuda and q_out.is_cuda and tuple(x.shape) == tuple(q_out.shape) and scale.dtype == _torch().float32
+    xb, xv = _view_of(x)
+    qb, qv = _view_of(q_out)
+    check(lib().mtrt_hip_quantize_view(_stream(), xb, float_dtype_of(x), ctypes.byref(xv), qb, q_dtype, ctypes.byref(qv),
+                                       scale.data_ptr(), kind, x.shape[0], x.shape[1], nb, flags))
+    return q_out
+
+
+def dequantize_view(q, scale, q_dtype, y_out, kind=SCALE_UNIFORM, nb=1):
+    assert q.is_cuda and y_out.is_cuda and tuple(q.shape) == tuple(y_out.shape) and scale.dtype == _torch().float32
+    qb, qv = _view_of(q)
+    yb, yv = _view_of(y_out)
+    check(lib().mtrt_hip_dequantize_view(_stream(), qb, q_dtype, ctypes.byref(qv), yb, float_dtype_of(y_out), ctypes.byref(yv),
+                                         scale.data_ptr(), kind, q.shape[0], q.shape[1], nb))
+    return y_out
 
 
 def nvfp4_quantize(x, tensor_amax, axis=-1):

@@ -510,3 +510,53 @@ using namespace qdq_cluster;
 MTRT_QDQ_FOR_FLOAT(f32, F32)
 MTRT_QDQ_FOR_FLOAT(f16, F16)
 MTRT_QDQ_FOR_FLOAT(bf16, BF16)
+
+// ---- strided views ------------------------------------------------------------------
+// The same element-wise programs on rank-2 VIEWS: each tensor operand arrives as the reference expands a fully
+// dynamic memref<?x?xT, strided<[?, ?], offset: ?>> argument (mlir-tensorrt/kernel/lib/Kernel/Transforms/
+// ExpandMemRefArgs.cpp:65-120; operand order pinned by mlir-tensorrt/compiler/test/Passes/1_Core/KernelToCUDA/
+// kernel-to-cuda.mlir:3-48): aligned base pointer, offset, size 0, size 1, stride 0, stride 1, all in elements as
+// 64-bit integers; element (r, c) lives at base[offset + r * stride0 + c * stride1].  The scale is a contiguous
+// constant addressed by the LOGICAL (r, c) of the view: uniform scale[0], row scale[r % nb], col
+// scale[(r / nb) * size1 + c].  One element per lane; codes one per byte (i8, f8E4M3FN, int4 in the low nibble).
+namespace qdq_cluster {
+
+template <typename X, typename Q, int MODE>   // MODE 0: quantize x -> q ; 1: dequantize q -> x
+__device__ __forceinline__ void qdq_view(typename X::storage* __restrict__ xb, int64_t xo, int64_t xs0, int64_t xs1,
+                                         typename Q::storage* __restrict__ qb, int64_t qo, int64_t qs0, int64_t qs1,
+                                         const float* __restrict__ scale, int64_t d0, int64_t d1, int64_t nb, int kind, int flags) {
+  const int64_t n = d0 * d1;
+  const int64_t stride = int64_t(gridDim.x) * blockDim.x;
+  for (int64_t e = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; e < n; e += stride) {
+    const int64_t r = e / d1, c = e - r * d1;
+    const float s = kind == kUniform ? scale[0] : (kind == kRow ? scale[r % nb] : scale[(r / nb) * d1 + c]);
+    typename X::storage* xp = xb + xo + r * xs0 + c * xs1;
+    typename Q::storage* qp = qb + qo + r * qs0 + c * qs1;
+    if (MODE == 0) {
+      const float v = quant_value<Q>(Tile<X>::load1(xp), s, flags);
+      *qp = typename Q::storage(Codes<Q>::enc(v, flags));
+    } else {
+      Tile<X>::store1(xp, Codes<Q>::dec(uint32_t(uint8_t(*qp))) * s);
+    }
+  }
+}
+
+}  // namespace qdq_cluster
+
+//   q_view  (x: base, offset, size0, size1, stride0, stride1 ; q: the same six ; scale, nb, kind, flags)
+//   dq_view (q: six ; y: six ; scale, nb, kind)
+// The two operands of a call have equal sizes; the kernel reads them from the first one.
+#define MTRT_QDQ_VIEW_KERNELS(XN, XT, QN, QT)                                                                        \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_q_view_##XN##_##QN(                                         \
+      const XT::storage* x, int64_t xo, int64_t d0, int64_t d1, int64_t xs0, int64_t xs1, QT::storage* q, int64_t qo, \
+      int64_t, int64_t, int64_t qs0, int64_t qs1, const float* scale, int64_t nb, int32_t kind, int32_t flags) {     \
+    qdq_view<XT, QT, 0>(const_cast<XT::storage*>(x), xo, xs0, xs1, q, qo, qs0, qs1, scale, d0, d1, nb, kind, flags); } \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_dq_view_##XN##_##QN(                                        \
+      const QT::storage* q, int64_t qo, int64_t d0, int64_t d1, int64_t qs0, int64_t qs1, XT::storage* y, int64_t yo, \
+      int64_t, int64_t, int64_t ys0, int64_t ys1, const float* scale, int64_t nb, int32_t kind) {                    \
+    qdq_view<XT, QT, 1>(y, yo, ys0, ys1, const_cast<QT::storage*>(q), qo, qs0, qs1, scale, d0, d1, nb, kind, 0); }
+#define MTRT_QDQ_VIEW_FOR_X(XN, XT)  \
+  MTRT_QDQ_VIEW_KERNELS(XN, XT, i8, I8) MTRT_QDQ_VIEW_KERNELS(XN, XT, f8, F8) MTRT_QDQ_VIEW_KERNELS(XN, XT, i4, I4)
+MTRT_QDQ_VIEW_FOR_X(f32, F32)
+MTRT_QDQ_VIEW_FOR_X(f16, F16)
+MTRT_QDQ_VIEW_FOR_X(bf16, BF16)

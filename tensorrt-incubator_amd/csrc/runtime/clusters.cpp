@@ -245,7 +245,80 @@ int32_t mtrt_hip_quantize_dequantize(mtrt_stream_t stream, const void *x, int32_
 
 namespace {
 std::atomic<int32_t> g_wait_limit{1 << 16};
+
+// Highest and lowest element offset a [d0, d1] view with these strides touches, relative to its base.
+bool view_extent(int64_t offset, int64_t d0, int64_t d1, int64_t s0, int64_t s1, int64_t *lo, int64_t *hi) {
+  const __int128 a = __int128(d0 - 1) * s0, b = __int128(d1 - 1) * s1;
+  const __int128 l = offset + (a < 0 ? a : 0) + (b < 0 ? b : 0), h = offset + (a > 0 ? a : 0) + (b > 0 ? b : 0);
+  if (l < -(__int128(1) << 62) || h > (__int128(1) << 62))
+    return false;
+  *lo = int64_t(l);
+  *hi = int64_t(h);
+  return true;
+}
+
+int32_t view_dispatch(bool quantize, hipStream_t stream, const void *f, int32_t f_dtype, const mtrt_hip_view2d *fv, const void *q,
+                      int32_t q_dtype, const mtrt_hip_view2d *qv, const float *scale, int32_t kind, int64_t d0, int64_t d1,
+                      int64_t nb, int32_t flags) {
+  clear_error();
+  const char *xn = float_name(f_dtype);
+  if (!xn)
+    return set_error(MTRT_INVALID_ARGUMENT, "float operand dtype %d is not one of f32/f16/bf16", f_dtype);
+  if (q_dtype != MTRT_I8 && q_dtype != MTRT_F8E4M3FN && q_dtype != MTRT_I4)
+    return set_error(MTRT_INVALID_ARGUMENT, "views carry one code per byte (i8, f8E4M3FN, i4); dtype %d is packed or unknown", q_dtype);
+  if (!fv || !qv)
+    return set_error(MTRT_INVALID_ARGUMENT, "null view descriptor");
+  if (d0 < 0 || d1 < 0)
+    return set_error(MTRT_INVALID_ARGUMENT, "negative extent [%lld, %lld]", (long long)d0, (long long)d1);
+  if (kind < MTRT_SCALE_UNIFORM || kind > MTRT_SCALE_COL)
+    return set_error(MTRT_INVALID_ARGUMENT, "unknown scale kind %d", kind);
+  if (kind != MTRT_SCALE_UNIFORM && nb <= 0)
+    return set_error(MTRT_INVALID_ARGUMENT, "scale kind %d needs a positive scale count / block size, got %lld", kind, (long long)nb);
+  if (kind == MTRT_SCALE_COL && d0 % nb != 0)
+    return set_error(MTRT_INVALID_ARGUMENT, "block size %lld does not divide the blocked extent %lld", (long long)nb, (long long)d0);
+  if (flags & ~(MTRT_Q_ROUND_TO_INT | MTRT_F8_REFHOST | MTRT_F8_VIA_F16) || ((flags & MTRT_F8_REFHOST) && (flags & MTRT_F8_VIA_F16)))
+    return set_error(MTRT_INVALID_ARGUMENT, "bad flag bits 0x%x", flags);
+  if (d0 == 0 || d1 == 0)
+    return MTRT_OK;
+  if (d0 * d1 >= (int64_t(1) << 40))
+    return set_error(MTRT_INVALID_ARGUMENT, "view of %lld elements is too large", (long long)(d0 * d1));
+  if (!f || !q || !scale)
+    return set_error(MTRT_INVALID_ARGUMENT, "null operand");
+  if (!aligned(f, float_bytes(f_dtype)))
+    return set_error(MTRT_INVALID_ARGUMENT, "float operand is not aligned to its element size");
+  // a view must stay at or above its base pointer (the allocation starts there); its upper end is the caller's word
+  int64_t lo, hi;
+  if (!view_extent(fv->offset, d0, d1, fv->stride0, fv->stride1, &lo, &hi) || lo < 0 ||
+      !view_extent(qv->offset, d0, d1, qv->stride0, qv->stride1, &lo, &hi) || lo < 0)
+    return set_error(MTRT_INVALID_ARGUMENT, "view reaches below its base pointer or overflows 62-bit offsets");
+  DeviceState *st = device_state();
+  if (!st)
+    return MTRT_RUNTIME_ERROR;
+  if (kind == MTRT_SCALE_UNIFORM)
+    nb = 1;
+  int64_t fo = fv->offset, fs0 = fv->stride0, fs1 = fv->stride1, qo = qv->offset, qs0 = qv->stride0, qs1 = qv->stride1;
+  const std::string name = std::string(quantize ? "mtrt_q_view_" : "mtrt_dq_view_") + xn + "_" + code_name(q_dtype);
+  const uint32_t grid = blocks_for(d0 * d1, kBlock);
+  if (quantize) {
+    void *args[] = {&f, &fo, &d0, &d1, &fs0, &fs1, &q, &qo, &d0, &d1, &qs0, &qs1, &scale, &nb, &kind, &flags};
+    return launch(st, name, grid, kBlock, stream, args);
+  }
+  void *args[] = {&q, &qo, &d0, &d1, &qs0, &qs1, &f, &fo, &d0, &d1, &fs0, &fs1, &scale, &nb, &kind};
+  return launch(st, name, grid, kBlock, stream, args);
+}
 } // namespace
+
+int32_t mtrt_hip_quantize_view(mtrt_stream_t stream, const void *x, int32_t x_dtype, const mtrt_hip_view2d *x_view, void *q,
+                               int32_t q_dtype, const mtrt_hip_view2d *q_view, const float *scale, int32_t scale_kind,
+                               int64_t d0, int64_t d1, int64_t nb, int32_t flags) {
+  return view_dispatch(true, as_hip(stream), x, x_dtype, x_view, q, q_dtype, q_view, scale, scale_kind, d0, d1, nb, flags);
+}
+
+int32_t mtrt_hip_dequantize_view(mtrt_stream_t stream, const void *q, int32_t q_dtype, const mtrt_hip_view2d *q_view, void *y,
+                                 int32_t y_dtype, const mtrt_hip_view2d *y_view, const float *scale, int32_t scale_kind,
+                                 int64_t d0, int64_t d1, int64_t nb) {
+  return view_dispatch(false, as_hip(stream), y, y_dtype, y_view, q, q_dtype, q_view, scale, scale_kind, d0, d1, nb, 0);
+}
 
 int32_t mtrt_hip_set_wait_limit(int32_t polls) {
   return g_wait_limit.exchange(polls < 0 ? 0 : polls);
