@@ -200,7 +200,7 @@ def build_workloads(pkg, torch, which):
         K, N, B = 4096, 11008, 128
         g = torch.Generator(device=dev)
         g.manual_seed(5)
-        for M, kname in ((16, "mtrt_gemm_w4a16_skinny16"), (256, "mtrt_gemm_w4a16_t128x128"), (4096, "mtrt_gemm_w4a16_t256x256")):
+        for M, kname in ((16, "mtrt_gemm_w4a16_strips16"), (256, "mtrt_gemm_w4a16_t128x128"), (4096, "mtrt_gemm_w4a16_t256x256")):
             nbytes = K * N // 2 + (K // B) * N * 2 + M * K * 2 + M * N * 2
             ns = min(slots_for(nbytes), 24)
             a5 = [torch.randn((M, K), generator=g, device=dev).half() for _ in range(ns)]

@@ -385,7 +385,9 @@ MTRT_CAPI_EXPORTED int32_t mtrt_hip_gemm_w8a8_fragments(mtrt_stream_t stream, co
  * a: f16 [M,K]; w_kn_packed: int4 [K,N] two per byte over the flattened array, element 2i in the
  * low nibble (NetworkEncoder.cpp:552-595); scale: f16 [K/block, N]; y: f16 [M,N].
  * The matrix-core kernels read the weights from a one-time re-layout (`w_prepacked`, made by the
- * prepack call, mtrt_hip_gemm_w4a16_prepacked_bytes(K, N) bytes, needs K % 64 == 0); they are
+ * prepack call, mtrt_hip_gemm_w4a16_prepacked_bytes(K, N) bytes, needs K % 64 == 0; it holds the weights in
+ * the fragment order of the 32-column kernels and, when K % 128 == 0, once more in the strip order of the
+ * M <= 16 kernel, so it is about K * N bytes); they are
  * used when w_prepacked is given and K % 64 == 0, block % 64 == 0, K % block == 0.  Otherwise the
  * generic kernel reads w_kn_packed directly (any shape, slow).  Either weight pointer may be NULL
  * if the other path applies. */

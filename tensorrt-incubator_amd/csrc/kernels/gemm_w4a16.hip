@@ -572,6 +572,211 @@ extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w4a16_skinny(
   skinny_tiles<4>(a, wp, scale, y, M, K, N, block, lds);
 }
 
+// ---- M <= 16: one strip of columns per compute unit --------------------------------------------------
+// At this size the launch is bound by what each compute unit's L1 takes in: its share of the weights plus ALL of
+// the activations (16 rows x K).  One workgroup per 32-column tile leaves 344 workgroups on 256 compute units at
+// N = 11008, and the 88 units that hold two set the time.  Here the grid is one workgroup per compute unit, each
+// owning a contiguous strip of 16-column tiles (688 tiles -> 2 or 3 per workgroup, at most 48 of the ideal 43
+// columns) over ALL of K: no second round, no partial sums across workgroups.
+// 16-column tiles need v_mfma_f32_16x16x32_f16 (lane l: column l % 16, k group l / 16, 8 consecutive k), so this
+// kernel reads the weights from a second re-layout made by mtrt_w4_prepack_strips:
+//   for each tile of 16 columns and each block of 128 k, 64 lanes x 4 dwords; dword j of lane l holds the 8 weights
+//   k = 128*kb + 32*j + 8*(l / 16) + [0..7] of column 16*tile + l % 16, nibbles ordered as in the 32-column layout.
+// The four waves of a workgroup split K; each keeps its own four-stage ring of activation slices (16 rows x 128 k,
+// whole 256-byte row segments by direct-to-LDS loads, 16-byte chunks XOR-swizzled by the row so that the fragment
+// reads are conflict-free) and never touches another wave's ring: no barriers until the partial tiles are added
+// through LDS at the end.
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+template <int WAVES, int JT>
+__device__ __forceinline__ void strips_chunk(const uint16_t* __restrict__ a, const uint32_t* __restrict__ ws,
+                                             const uint16_t* __restrict__ scale, uint16_t* __restrict__ y, int64_t M,
+                                             int64_t K, int64_t N, int64_t block, int64_t tile0, int8_t* lds) {
+  constexpr int kStages = 4, kStageBytes = 16 * 256;   // 16 rows x 128 k of f16
+  constexpr int kLoads = 4 + 2 * JT;                   // memory instructions per slice and wave
+  static_assert(3 * kLoads < 64, "wait counter range");
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int fcol = lane & 15, fgrp = lane >> 4;
+  const int64_t kblocks = K / 128;
+  const int64_t kb0 = kblocks * wave / WAVES, kb1 = kblocks * (wave + 1) / WAVES;
+  const uint32_t blocks_per_scale = uint32_t(block / 128);
+  int64_t col[JT];
+  const u4* bp[JT];
+#pragma unroll
+  for (int j = 0; j < JT; ++j) {
+    col[j] = (tile0 + j) * 16 + fcol;
+    col[j] = col[j] < N ? col[j] : N - 1;              // columns past N: the last column's scales, never stored
+    bp[j] = reinterpret_cast<const u4*>(ws) + ((tile0 + j) * kblocks) * 64 + lane;
+  }
+  int8_t* ring = lds + wave * (kStages * kStageBytes);
+
+  // direct-to-LDS load g (of 4) of a slice: rows 4g .. 4g+3; lane l <-> (row 4g + l / 16, LDS chunk position l % 16),
+  // which holds chunk (l % 16) ^ row of that row's 256 bytes
+  uint32_t aoff[4];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const int lrow = 4 * g + (lane >> 4);
+    const int64_t row = lrow < M ? lrow : M - 1;       // rows past M repeat the last row; never stored
+    aoff[g] = uint32_t(row * K * 2 + (((lane & 15) ^ lrow) << 4));
+  }
+  const int8_t* abase = reinterpret_cast<const int8_t*>(a);
+  struct Slice {
+    u4 w[JT];
+    uint32_t sc[JT];
+  };
+  auto fetch = [&](int64_t kb, int64_t clamp, Slice& dst) {
+    kb = kb < clamp ? kb : clamp;
+    int8_t* st = ring + int(kb & (kStages - 1)) * kStageBytes;
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+      __builtin_amdgcn_global_load_lds((gemm_core::global_void_t*)(abase + kb * 256 + aoff[g]),
+                                       (gemm_core::lds_void_t*)(st + g * 1024), 16, 0, 0);
+    // opaque register loads, waits placed by hand (see `skinny`)
+#pragma unroll
+    for (int j = 0; j < JT; ++j) {
+      const u4* wsrc = bp[j] + kb * 64;
+      const uint16_t* ssrc = scale + int64_t(uint32_t(kb) / blocks_per_scale) * N + col[j];
+      __asm__ volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(dst.w[j]) : "v"(wsrc) : "memory");
+      __asm__ volatile("global_load_ushort %0, %1, off" : "=v"(dst.sc[j]) : "v"(ssrc) : "memory");
+    }
+  };
+  auto landed = [&](Slice& sl) {
+#pragma unroll
+    for (int j = 0; j < JT; ++j)
+      __asm__ volatile("s_waitcnt vmcnt(%2)" : "+v"(sl.w[j]), "+v"(sl.sc[j]) : "n"(3 * kLoads) : "memory");
+  };
+  auto landed_all = [&](Slice& sl) {
+#pragma unroll
+    for (int j = 0; j < JT; ++j) __asm__ volatile("s_waitcnt vmcnt(0)" : "+v"(sl.w[j]), "+v"(sl.sc[j])::"memory");
+  };
+
+  v4f acc[JT];
+#pragma unroll
+  for (int j = 0; j < JT; ++j) acc[j] = (v4f){0.0f, 0.0f, 0.0f, 0.0f};
+  const uint32_t mask = nibble_pair_mask(), mask_hi = mask << 4;
+  auto multiply = [&](int64_t kb, const Slice& sl) {
+    const int8_t* st = ring + int(kb & (kStages - 1)) * kStageBytes;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const v8h fa = *reinterpret_cast<const v8h*>(st + fcol * 256 + (((4 * ks + fgrp) ^ fcol) << 4));
+#pragma unroll
+      for (int j = 0; j < JT; ++j) {
+        H2Bits sp;
+        sp.u = sl.sc[j] * 0x00010001u;
+        union { u4 u; v8h h; } fb;
+        fb.u = dequant8_in_place(sl.w[j][ks], sp.h, mask, mask_hi);
+        acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa, fb.h, acc[j], 0, 0, 0);
+      }
+    }
+  };
+
+  const int64_t kmain = kb0 + ((kb1 - kb0) & ~int64_t(3));
+  if (kb0 < kmain) {
+    const int64_t clamp = kmain - 1;                   // past the end: the last slice again, into a stage nobody reads
+    Slice s0, s1, s2, s3;
+    fetch(kb0, clamp, s0);
+    fetch(kb0 + 1, clamp, s1);
+    fetch(kb0 + 2, clamp, s2);
+    for (int64_t kb = kb0; kb < kmain; kb += 4) {
+      fetch(kb + 3, clamp, s3);
+      landed(s0);
+      multiply(kb, s0);
+      fetch(kb + 4, clamp, s0);
+      landed(s1);
+      multiply(kb + 1, s1);
+      fetch(kb + 5, clamp, s1);
+      landed(s2);
+      multiply(kb + 2, s2);
+      fetch(kb + 6, clamp, s2);
+      landed(s3);
+      multiply(kb + 3, s3);
+    }
+    landed_all(s0);
+    landed_all(s1);
+    landed_all(s2);
+  }
+  for (int64_t kb = kmain; kb < kb1; ++kb) {           // at most three slices, one at a time
+    Slice sl;
+    __builtin_amdgcn_s_waitcnt(0x0070);
+    fetch(kb, kb, sl);
+    landed_all(sl);
+    multiply(kb, sl);
+  }
+  __builtin_amdgcn_s_waitcnt(0x0070);                  // surplus loads have landed before the ring is reused
+  // partial tiles of the waves meet in LDS: [wave][tile][register][lane]
+  float* partial = reinterpret_cast<float*>(lds);
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < JT; ++j)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) partial[((wave * JT + j) * 4 + r) * 64 + lane] = acc[j][r];
+  __syncthreads();
+  for (int e = threadIdx.x; e < JT * 4 * 64; e += 64 * WAVES) {
+    const int l = e & 63, r = (e >> 6) & 3, j = e >> 8;
+    float v = partial[((0 * JT + j) * 4 + r) * 64 + l];
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) v = v + partial[((w * JT + j) * 4 + r) * 64 + l];
+    const int64_t row = 4 * (l >> 4) + r;
+    const int64_t c = (tile0 + j) * 16 + (l & 15);
+    if (row < M && c < N) y[row * N + c] = uint16_t(f32_to_f16_bits(v));
+  }
+  __syncthreads();                                     // the next chunk of this workgroup reuses the LDS
+}
+
+// (a [M,K] f16, strip-order weights, scale [K/block, N] f16, y [M,N] f16, M <= 16, K % 128 == 0, N, block % 128 == 0)
+// grid = min(compute units, ceil(N / 16)), block = 256: workgroup g owns the 16-column tiles
+// [g * tiles / grid, (g + 1) * tiles / grid), three at a time.
+// Four waves, one per SIMD.  Measured on M = 16, N = 11008, K = 4096 (rocprofv3 kernel durations): 2 / 4 / 8 waves take
+// 12.7 / 9.6 / 10.7 us; more than one workgroup per compute unit (grids of 344, 512, 688) 11.5-12.6 us.  In-kernel
+// timestamps of the four-wave form: 1.3 us until the loads are issued, first slice landed at 3.9 us, K loop done at
+// 10.4 us (1600 cycles per slice against some 800 of issue for 175 dequantisation instructions and 12 MFMAs), so what
+// is left is the dequantisation on one wave per SIMD and the 4 us before the first data; with eight waves the loop
+// shortens to 4.9 us but the first data arrives later by as much.
+constexpr int kStripWaves = 4;
+extern "C" __global__ void __launch_bounds__(64 * kStripWaves) mtrt_gemm_w4a16_strips16(
+    const uint16_t* __restrict__ a, const uint32_t* __restrict__ ws, const uint16_t* __restrict__ scale,
+    uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t block) {
+  __shared__ __attribute__((aligned(16))) int8_t lds[kStripWaves * 4 * 4096];
+  const int64_t tiles = (N + 15) / 16;
+  const int64_t t0 = tiles * blockIdx.x / gridDim.x, t1 = tiles * (int64_t(blockIdx.x) + 1) / gridDim.x;
+  for (int64_t t = t0; t < t1; t += 3) {
+    const int64_t left = t1 - t;
+    if (left >= 3) strips_chunk<kStripWaves, 3>(a, ws, scale, y, M, K, N, block, t, lds);
+    else if (left == 2) strips_chunk<kStripWaves, 2>(a, ws, scale, y, M, K, N, block, t, lds);
+    else strips_chunk<kStripWaves, 1>(a, ws, scale, y, M, K, N, block, t, lds);
+  }
+}
+
+// Re-layout for mtrt_gemm_w4a16_strips16: packed [K,N] nibbles -> strip order (above).  One thread per output dword.
+// (w_kn_packed, ws, K, N) ; K % 128 == 0.
+extern "C" __global__ void __launch_bounds__(256) mtrt_w4_prepack_strips(const uint8_t* __restrict__ w_kn_packed,
+                                                                       uint32_t* __restrict__ ws, int64_t K, int64_t N) {
+  const int64_t kblocks = K / 128;
+  const int64_t ntiles = (N + 15) / 16;
+  const int64_t total = ntiles * kblocks * 256;
+  for (int64_t d = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; d < total; d += int64_t(gridDim.x) * blockDim.x) {
+    const int j = int(d & 3), lane = int((d >> 2) & 63);
+    const int64_t kb = (d >> 8) % kblocks, tile = (d >> 8) / kblocks;
+    const int64_t n = tile * 16 + (lane & 15);
+    const int64_t k0 = kb * 128 + 32 * j + 8 * (lane >> 4);
+    uint32_t w = 0;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      uint32_t nib = 0;                                 // columns past N: value 0
+      if (n < N) {
+        const int64_t i = (k0 + q) * N + n;
+        const uint32_t byte = w_kn_packed[i >> 1];
+        nib = (i & 1) ? (byte >> 4) : (byte & 0xFu);
+      }
+      const uint32_t u = (nib ^ 8u) & 0xFu;             // value + 8
+      const int pos = (q & 1) ? (q >> 1) + 4 : (q >> 1);
+      w |= u << (4 * pos);
+    }
+    ws[d] = w;
+  }
+}
+
 // Any shape: one output per lane, reading the ORIGINAL packed [K,N] nibbles; not a fast path.
 extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w4a16_any(
     const uint16_t* __restrict__ a, const uint8_t* __restrict__ w_kn_packed, const uint16_t* __restrict__ scale,

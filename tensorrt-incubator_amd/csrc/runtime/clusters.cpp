@@ -639,10 +639,18 @@ int32_t mtrt_hip_linear_dense(mtrt_stream_t stream, const void *x, const void *w
   return launch(st, std::string("mtrt_gemm_dense_") + xn, uint32_t(tiles), kBlock, as_hip(stream), args);
 }
 
+namespace {
+// The re-laid weights hold two layouts back to back: fragment order for the 32 x 32 matrix-core tiles (per 32
+// columns and 64 k: 64 lanes x 16 bytes) and, when K is a multiple of 128, strip order for the M <= 16 kernel
+// (per 16 columns and 128 k: 64 lanes x 16 bytes).
+int64_t w4_fragment_bytes(int64_t K, int64_t N) { return ((N + 31) / 32) * (K / 64) * 1024; }
+int64_t w4_strip_bytes(int64_t K, int64_t N) { return K % 128 == 0 ? ((N + 15) / 16) * (K / 128) * 1024 : 0; }
+} // namespace
+
 int64_t mtrt_hip_gemm_w4a16_prepacked_bytes(int64_t K, int64_t N) {
   if (K <= 0 || N <= 0 || K % 64 != 0)
     return 0;
-  return ((N + 31) / 32) * (K / 64) * 1024;   // per 32 columns and 64 k: 64 lanes x 16 bytes
+  return w4_fragment_bytes(K, N) + w4_strip_bytes(K, N);
 }
 
 int32_t mtrt_hip_gemm_w4a16_prepack(mtrt_stream_t stream, const void *w_kn_packed, void *w_prepacked, int64_t K,
@@ -658,9 +666,14 @@ int32_t mtrt_hip_gemm_w4a16_prepack(mtrt_stream_t stream, const void *w_kn_packe
   DeviceState *st = device_state();
   if (!st)
     return MTRT_RUNTIME_ERROR;
-  const int64_t dwords = mtrt_hip_gemm_w4a16_prepacked_bytes(K, N) / 4;
+  const int64_t dwords = w4_fragment_bytes(K, N) / 4;
   void *args[] = {&w_kn_packed, &w_prepacked, &K, &N};
-  return launch(st, "mtrt_w4_prepack", blocks_for(dwords, kBlock), kBlock, as_hip(stream), args);
+  const int32_t rc = launch(st, "mtrt_w4_prepack", blocks_for(dwords, kBlock), kBlock, as_hip(stream), args);
+  if (rc != MTRT_OK || w4_strip_bytes(K, N) == 0)
+    return rc;
+  void *strips = static_cast<char *>(w_prepacked) + w4_fragment_bytes(K, N);
+  void *args2[] = {&w_kn_packed, &strips, &K, &N};
+  return launch(st, "mtrt_w4_prepack_strips", blocks_for(w4_strip_bytes(K, N) / 4, kBlock), kBlock, as_hip(stream), args2);
 }
 
 int32_t mtrt_hip_gemm_w4a16(mtrt_stream_t stream, const void *a, const void *w_kn_packed, const void *w_prepacked,
@@ -683,6 +696,14 @@ int32_t mtrt_hip_gemm_w4a16(mtrt_stream_t stream, const void *a, const void *w_k
   const bool fast = w_prepacked && K > 0 && K % 64 == 0 && block % 64 == 0 && aligned(a, 16) && aligned(w_prepacked, 16);
   if (fast) {
     void *args[] = {&a, &w_prepacked, &scale, &y, &M, &K, &N, &block};
+    if (M <= 16 && K % 128 == 0 && block % 128 == 0) {
+      // one workgroup per compute unit, each a strip of 16-column tiles over all of K (weights in strip order)
+      const void *strips = static_cast<const char *>(w_prepacked) + w4_fragment_bytes(K, N);
+      void *sargs[] = {&a, &strips, &scale, &y, &M, &K, &N, &block};
+      const int64_t tiles = (N + 15) / 16;
+      return launch(st, "mtrt_gemm_w4a16_strips16", uint32_t(std::min<int64_t>(tiles, num_compute_units(st))), kBlock,
+                    as_hip(stream), sargs);
+    }
     if (M <= 32) {
       // one workgroup per 32-column tile; between one and two tiles per compute unit, one workgroup per
       // compute unit instead (the kernel then gives workgroup g the tiles g and g + grid, which share the

@@ -171,7 +171,7 @@ def test_w4a16_small_shapes(pkg, orc, shape):
     B = 128
     a, w, wp, s = _w4a16_inputs(orc, rng(M + K + N), M, K, N, B)
     y, kernel = _run_w4a16(pkg, a, wp, s, K, N, B)
-    assert kernel == ("mtrt_gemm_w4a16_skinny16" if M <= 16 else "mtrt_gemm_w4a16_skinny" if M <= 32 else "mtrt_gemm_w4a16_t128x128")
+    assert kernel == ("mtrt_gemm_w4a16_strips16" if M <= 16 else "mtrt_gemm_w4a16_skinny" if M <= 32 else "mtrt_gemm_w4a16_t128x128")
     _check_w4a16(orc, y, a, w, s, K, N, B, orc.gemm_w4a16(a, wp, s, K, N, B))
 
 
@@ -207,7 +207,7 @@ def test_c5_w4a16_full_size(pkg, orc, M):
     K, N, B = 4096, 11008, 128
     a, w, wp, s = _w4a16_inputs(orc, rng(5), M, K, N, B)
     y, kernel = _run_w4a16(pkg, a, wp, s, K, N, B)
-    assert kernel == {16: "mtrt_gemm_w4a16_skinny16", 256: "mtrt_gemm_w4a16_t128x128", 4096: "mtrt_gemm_w4a16_t256x256"}[M]
+    assert kernel == {16: "mtrt_gemm_w4a16_strips16", 256: "mtrt_gemm_w4a16_t128x128", 4096: "mtrt_gemm_w4a16_t256x256"}[M]
     rows = sorted(set([0, M - 1] + list(range(0, M, max(1, M // 38)))))[:40]
     orc.set_threads(16)
     import torch
@@ -249,6 +249,24 @@ def test_w4a16_small_m_workgroups_with_two_column_tiles(pkg, orc, shape):
     a, w, wp, s = _w4a16_inputs(orc, rng(M + K + N), M, K, N, B)
     y, kernel = _run_w4a16(pkg, a, wp, s, K, N, B)
     assert kernel == ("mtrt_gemm_w4a16_skinny16" if M <= 16 else "mtrt_gemm_w4a16_skinny")
+    orc.set_threads(16)
+    ref = orc.gemm_w4a16(a, wp, s, K, N, B)
+    orc.set_threads(1)
+    _check_w4a16(orc, y, a, w, s, K, N, B, ref)
+
+
+@pytest.mark.parametrize("shape", [(16, 4096, 11008), (16, 384, 16400), (1, 128, 16), (9, 1280, 4099), (13, 640, 8192 + 48),
+                                   (16, 256, 40)])
+def test_w4a16_strip_kernel(pkg, orc, shape):
+    """M <= 16 with K % 128 == 0 and block % 128 == 0: one workgroup per compute unit owning a strip of 16-column
+    tiles over all of K (strip-order weights).  N = 11008 gives 688 tiles = 2 or 3 per workgroup, 16400 gives 1025
+    (4 or 5: chunks of 3 + 1 and 3 + 2), 4099 a ragged last tile; K = 384 leaves one wave without a K block,
+    K = 1280 gives the waves 2 or 3 blocks (no full group of four: the one-at-a-time tail only)."""
+    M, K, N = shape
+    B = 128
+    a, w, wp, s = _w4a16_inputs(orc, rng(M + K + N), M, K, N, B)
+    y, kernel = _run_w4a16(pkg, a, wp, s, K, N, B)
+    assert kernel == "mtrt_gemm_w4a16_strips16"
     orc.set_threads(16)
     ref = orc.gemm_w4a16(a, wp, s, K, N, B)
     orc.set_threads(1)
