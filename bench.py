@@ -6,7 +6,7 @@
 A STEP is one pass of the hot path over one batch of seeded synthetic input: the
 programs of BASELINE.json's configs run back to back through the C ABI
 (libmtrt_hip.so) on tensors already resident in HBM:
-    C1  amax + fused quantize->dequantize   f32 [1024,4096] -> i8          (per-tensor, amax/127)
+    C1  amax + quantize->dequantize, ONE launch   f32 [1024,4096] -> i8    (per-tensor, amax/127)
     C2a LayerNorm                           bf16 [8192,4096]
     C2b softmax                             f16 [4096,4096]
     C3  amax + fused quantize->dequantize   bf16 [16384,8192] -> f8E4M3FN  (amax/448)
@@ -19,14 +19,16 @@ would take at its roofline peak, on its ALGORITHMIC bytes or ops) / (measured ti
 of the step).  Peaks: HBM 8 TB/s, int8 MFMA 5 POP/s, f16 MFMA 2.5 PFLOP/s.
 Every kernel also gets its own line under "workloads" (achieved, peak, fraction),
 timed with HIP events on the launch stream over rotating buffers whose combined
-footprint exceeds the 256 MiB Infinity Cache, so cache hits do not count as HBM.
+footprint exceeds the 256 MiB Infinity Cache, so cache hits do not count as HBM; the
+figure is the MEDIAN over ten batches of launches.
 "roofline" repeats the entry of the kernel with the largest share of the step.
 "mfma_sustained" is the matrix-core rate a loop of nothing but MFMAs reaches on the bench's
 own operand data (the published dense peaks hold for idle data only: the clock drops under
 the board's power limit); GEMM entries carry "frac_of_sustained" beside "frac".
 "cpu_baseline" times the CPU oracle (a C++ restatement of the reference's host
 lowering, NOT the reference binary) on a bounded sample, single-threaded like the
-reference interpreter, and extrapolates linearly to the step.
+reference interpreter, and extrapolates linearly to the step; "cpu_baseline_all_cores"
+is the same sample with the oracle's OpenMP loops on every host core.
 """
 import argparse
 import json
@@ -73,26 +75,23 @@ def build_workloads(pkg, torch, which):
         y1 = [torch.empty_like(x) for x in x1]
         s1 = [torch.empty(2, dtype=torch.float32, device=dev) for _ in range(ns)]
 
-        def amax(i, xs=x1, sc=s1, n=n):
-            a = (xs[i].data_ptr(), pkg.F32, n, 127.0, sc[i].data_ptr(), sc[i].data_ptr() + 4)
-            return lambda: pkg.check(L.mtrt_hip_amax(stream(), *a))
-
-        def qdq(i, xs=x1, qs=q1, ys=y1, sc=s1):
-            a = (xs[i].data_ptr(), pkg.F32, qs[i].data_ptr(), pkg.I8, ys[i].data_ptr(), sc[i].data_ptr() + 4,
-                 pkg.SCALE_UNIFORM, 1024, 4096, 1, 0)
-            return lambda: pkg.check(L.mtrt_hip_quantize_dequantize(stream(), *a))
-        xs, qs, ys, sc = x1, q1, y1, s1
-        out.append(dict(name="mtrt_amax_f32", config="C1", bound="hbm", work=4.0 * n, nslots=ns, make=amax, keep=(xs, sc)))
-        out.append(dict(name="mtrt_qdq_uniform_f32_i8", config="C1", bound="hbm", work=9.0 * n, nslots=ns, make=qdq,
-                        keep=(qs, ys)))
+        def dynq(i, xs=x1, qs=q1, ys=y1, sc=s1, n=n):
+            a = (xs[i].data_ptr(), pkg.F32, qs[i].data_ptr(), pkg.I8, ys[i].data_ptr(), n, 127.0, sc[i].data_ptr(),
+                 sc[i].data_ptr() + 4, 0)
+            return lambda: pkg.check(L.mtrt_hip_dynamic_quantize_dequantize(stream(), *a))
+        # one launch: x read once (kept in registers across the reduction), q and y written: 9 bytes per element
+        out.append(dict(name="mtrt_dynqdq_f32_i8_v4", config="C1", bound="hbm", work=9.0 * n, nslots=ns, make=dynq,
+                        keep=(x1, q1, y1, s1)))
 
     if which in ("all", "c2a"):
         rows, d = 8192, 4096
         ns = slots_for(rows * d * 4)
         xs = [gen((rows, d), torch.bfloat16, 20 + i) for i in range(ns)]
         ys = [torch.empty_like(x) for x in xs]
-        gamma = (torch.rand(d, device=dev) + 0.5).to(torch.bfloat16)
-        beta = (torch.randn(d, device=dev) * 0.1).to(torch.bfloat16)
+        gg = torch.Generator(device=dev)
+        gg.manual_seed(19)
+        gamma = (torch.rand(d, generator=gg, device=dev) + 0.5).to(torch.bfloat16)
+        beta = (torch.randn(d, generator=gg, device=dev) * 0.1).to(torch.bfloat16)
 
         def ln(i, xs=xs, ys=ys, rows=rows, d=d, gamma=gamma, beta=beta):
             a = (xs[i].data_ptr(), gamma.data_ptr(), beta.data_ptr(), ys[i].data_ptr(), pkg.BF16, rows, d, 1e-5)
@@ -314,24 +313,30 @@ def traffic_from_profile(kernel):
 
 
 def time_kernel(pkg, torch, w, reps):
-    """Average launch duration in microseconds, HIP events on the launch stream."""
+    """Launch duration in microseconds: HIP events on the launch stream around batches of back-to-back launches
+    (`reps` launches in ten batches), the MEDIAN of the batch averages."""
     L = pkg.lib()
     dev = L.mtrt_cuda_get_current_device()
     calls = [w["make"](i) for i in range(w["nslots"])]
     s = torch.cuda.current_stream().cuda_stream
     for c in calls:
         c()
-    e0, e1 = L.mtrt_cuda_event_create(dev), L.mtrt_cuda_event_create(dev)
+    batches = 10 if reps >= 20 else 1
+    per = max(1, reps // batches)
+    events = [L.mtrt_cuda_event_create(dev) for _ in range(batches + 1)]
     L.mtrt_cuda_stream_sync(s)
-    L.mtrt_cuda_stream_record_event(s, e0)
-    for r in range(reps):
-        calls[r % len(calls)]()
-    L.mtrt_cuda_stream_record_event(s, e1)
-    L.mtrt_cuda_event_sync(e1)
-    us = L.mtrt_cuda_event_elapsed_msec(e0, e1) * 1e3 / reps
-    L.mtrt_cuda_event_release(e0)
-    L.mtrt_cuda_event_release(e1)
-    return us
+    L.mtrt_cuda_stream_record_event(s, events[0])
+    r = 0
+    for b in range(batches):
+        for _ in range(per):
+            calls[r % len(calls)]()
+            r += 1
+        L.mtrt_cuda_stream_record_event(s, events[b + 1])
+    L.mtrt_cuda_event_sync(events[-1])
+    us = sorted(L.mtrt_cuda_event_elapsed_msec(events[b], events[b + 1]) * 1e3 / per for b in range(batches))
+    for e in events:
+        L.mtrt_cuda_event_release(e)
+    return us[len(us) // 2] if batches % 2 else 0.5 * (us[batches // 2 - 1] + us[batches // 2])
 
 
 def cache_variants(pkg, torch, wl, which, reps):
@@ -352,7 +357,10 @@ def cache_variants(pkg, torch, wl, which, reps):
     if which in ("all", "c1"):
         rows, cols = 16 * 1024, 4096
         n = rows * cols
-        x = [torch.randn((rows, cols), device=dev) for _ in range(2)]
+        gens = [torch.Generator(device=dev) for _ in range(2)]
+        for i, gi in enumerate(gens):
+            gi.manual_seed(900 + i)
+        x = [torch.randn((rows, cols), generator=gi, device=dev) for gi in gens]
         q = [torch.empty(n, dtype=torch.int8, device=dev) for _ in range(2)]
         y = [torch.empty_like(t) for t in x]
         sc = [torch.empty(2, dtype=torch.float32, device=dev) for _ in range(2)]
@@ -372,7 +380,10 @@ def cache_variants(pkg, torch, wl, which, reps):
         del x, q, y
     if which in ("all", "c2b"):
         rows, d = 16 * 4096, 4096
-        x = [(torch.randn((rows, d), device=dev) * 2.0).half() for _ in range(2)]
+        gens = [torch.Generator(device=dev) for _ in range(2)]
+        for i, gi in enumerate(gens):
+            gi.manual_seed(940 + i)
+        x = [(torch.randn((rows, d), generator=gi, device=dev) * 2.0).half() for gi in gens]
         y = [torch.empty_like(t) for t in x]
 
         def sm(i):
@@ -384,11 +395,12 @@ def cache_variants(pkg, torch, wl, which, reps):
     return out
 
 
-def cpu_baseline(which):
-    """Times the CPU oracle single-threaded on a bounded sample of each program and
-    extrapolates linearly to the full configuration; returns (seconds per step, description)."""
+def cpu_baseline(which, threads=1):
+    """Times the CPU oracle on a bounded sample of each program, with `threads` OpenMP threads (1 = like the
+    reference's single-threaded interpreter), and extrapolates linearly to the full configuration; returns
+    (seconds per step, description)."""
     orc = entry.load_oracle()
-    orc.set_threads(1)
+    orc.set_threads(threads)
     g = np.random.Generator(np.random.PCG64(1))
     total = 0.0
     parts = []
@@ -503,11 +515,13 @@ def main():
                             achieved=round(achieved, 1), peak=w["peak"], unit=w["unit"], frac=round(achieved / w["peak"], 4),
                             work=w["work"]))
     # what the matrix cores sustain on this very data with nothing else going on (power-limited)
-    sustained = {}
+    sustained, sustained_zero = {}, {}
     for w in wl:
         if w.get("probe"):
             kname, operand, ops = w["probe"]
             sustained[w["unit"]] = round(mfma_sustained(pkg, torch, kname, operand, ops), 1)
+            # the yardstick's own ceiling: the same loop on all-zero operands (no toggling, full clock)
+            sustained_zero[w["unit"]] = round(mfma_sustained(pkg, torch, kname, torch.zeros_like(operand), ops), 1)
     for k in kernels:
         if k["bound"] == "mfma" and k["unit"] in sustained:
             k["frac_of_sustained"] = round(k["achieved"] / sustained[k["unit"]], 4)
@@ -523,8 +537,10 @@ def main():
         "config": {"workload": {"all": "C1+C2a+C2b+C3+C4+C5 programs of BASELINE.json, one pass each per step"}.get(
             args.workload, args.workload.upper()), "kernels_per_step": len(wl)},
         "roofline": {"kernel": dom["kernel"], "bound": dom["bound"], "achieved": dom["achieved"], "peak": dom["peak"],
-                     "unit": dom["unit"], "frac": dom["frac"], "traffic": traffic_from_profile(dom["kernel"])},
-        "mfma_sustained": {"rates": sustained, "method": "mtrt_mfma_probe_*: 16 independent MFMAs per round and wave, one wave "
+                     "unit": dom["unit"], "frac": dom["frac"], "traffic": traffic_from_profile(dom["kernel"]),
+                     "traffic_source": "profiles/hbm_traffic_bench_suite.md (rocprofv3 --pmc run of this command; "
+                                       "not measured in this run)"},
+        "mfma_sustained": {"rates": sustained, "rates_on_zero_operands": sustained_zero, "method": "mtrt_mfma_probe_*: 16 independent MFMAs per round and wave, one wave "
                            "per SIMD, operands = this bench's own data, no memory traffic; published dense peaks are "
                            "not reached on non-zero data (power limit)"},
         "workloads": kernels,
@@ -541,6 +557,15 @@ def main():
         line["cpu_baseline"] = {"value": round(100.0 * (ideal_us / 1e6) / cpu_s, 6),
                                 "unit": "% of MI355X peak (same definition)", "cores": 1, "kind": "port",
                                 "sample": sample + "; extrapolated linearly", "seconds_per_step": round(cpu_s, 3)}
+        # the same sample with the oracle's OpenMP loops on every core this process may use (16 on the one-GPU box)
+        cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+        cores = max(1, min(cores, int(os.environ.get("OMP_NUM_THREADS", cores))))
+        cpu_all, _ = cpu_baseline(args.workload, cores)
+        entry.load_oracle().set_threads(1)
+        line["cpu_baseline_all_cores"] = {"value": round(100.0 * (ideal_us / 1e6) / cpu_all, 6),
+                                          "unit": "% of MI355X peak (same definition)", "cores": cores, "kind": "port",
+                                          "sample": "same sample, OpenMP over rows / tiles",
+                                          "seconds_per_step": round(cpu_all, 3)}
     print(json.dumps(line))
 
 

@@ -182,6 +182,14 @@ struct Shape {
                                                      : (kOutBytes > kSumBytes ? kOutBytes : kSumBytes);
 };
 
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(gemm_core::IntC<I>{});
+    static_for<I + 1, N>(f);
+  }
+}
+
 template <class S, int KH, class Epilogue>
 __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, int64_t a_row_bytes,
                                                 WeightRegs<S::kJT, S::kDepth, (S::kKW > 1)>& wr,
@@ -224,13 +232,7 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
     for (int g = 0; g < G; ++g) al.dma(sl, stage(DD), g);
     wr.template fetch<DD>(sl);
   };
-  prefetch(IntC<0>{});
-  prefetch(IntC<1>{});
-  if constexpr (D > 2) {
-    prefetch(IntC<2>{});
-    prefetch(IntC<3 % D>{});
-  }
-  static_assert(D == 2 || D == 4, "register sets are named at compile time");
+  static_for<0, D>(prefetch);                          // register sets are named at compile time
   drain_and_barrier();
 #pragma unroll
   for (int i = 0; i < IT; ++i) read_a(f0, stage(0), 2 * KH + fhalf, i);
@@ -289,19 +291,11 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
   };
 
   int64_t s = 0;
-  for (; s + D - 1 < slices; s += D) {
-    slice_body(IntC<0>{}, s);
-    slice_body(IntC<1>{}, s + 1);
-    if constexpr (D > 2) {
-      slice_body(IntC<2 % D>{}, s + 2);
-      slice_body(IntC<3 % D>{}, s + 3);
-    }
-  }
-  if (s < slices) slice_body(IntC<0>{}, s);
-  if (s + 1 < slices) slice_body(IntC<1>{}, s + 1);
-  if constexpr (D > 2) {
-    if (s + 2 < slices) slice_body(IntC<2 % D>{}, s + 2);
-  }
+  for (; s + D - 1 < slices; s += D)                   // D slices per trip: one per register set, no branch inside
+    static_for<0, D>([&](auto p) { slice_body(p, s + decltype(p)::value); });
+  static_for<0, D - 1>([&](auto p) {
+    if (s + decltype(p)::value < slices) slice_body(p, s + decltype(p)::value);
+  });
   __builtin_amdgcn_s_waitcnt(0x0070);                  // the surplus loads of the last slices have landed
 
   if (KW == 2) {                                       // second set hands its sums to the first through LDS

@@ -111,7 +111,8 @@ int32_t qdq_dispatch(int mode, hipStream_t stream, const void *x, int32_t x_dtyp
 
   static const char *kModeName[] = {"q", "dq", "qdq"};
   static const char *kKindName[] = {"uniform", "row", "col"};
-  std::string name = std::string("mtrt_") + kModeName[mode] + "_" + (tiles ? kKindName[kind] : "any") + "_" + xn + "_" + qn;
+  KernelName name("mtrt_");
+  name + kModeName[mode] + "_" + (tiles ? kKindName[kind] : "any") + "_" + xn + "_" + qn;
 
   int64_t n_arg = n, d1_arg = d1, nb_arg = nb;
   int32_t kind_arg = kind, flags_arg = flags;
@@ -175,7 +176,7 @@ int32_t mtrt_hip_amax(mtrt_stream_t stream, const void *x, int32_t dtype, int64_
   int64_t n_arg = n;
   float qmax_arg = qmax;
   void *args[] = {&x_arg, &n_arg, &qmax_arg, &amax_out, &scale_out, &slot};
-  return launch(st, std::string("mtrt_amax_") + xn, grid, kBlock, as_hip(stream), args);
+  return launch(st, KernelName("mtrt_amax_") + xn, grid, kBlock, as_hip(stream), args);
 }
 
 int32_t mtrt_hip_amax_scales(mtrt_stream_t stream, const void *x, int32_t dtype, int32_t scale_kind, int64_t d0, int64_t d1,
@@ -214,15 +215,15 @@ int32_t mtrt_hip_amax_scales(mtrt_stream_t stream, const void *x, int32_t dtype,
     const int64_t blocks = (nb + 3) / 4;
     if (blocks > int64_t(kMaxGrid) * 1024)
       return set_error(MTRT_INVALID_ARGUMENT, "%lld scales are too many for one launch", (long long)nb);
-    return launch(st, std::string(vec ? "mtrt_amax_rows_" : "mtrt_amax_rows_any_") + xn, uint32_t(blocks), kBlock,
+    return launch(st, KernelName(vec ? "mtrt_amax_rows_" : "mtrt_amax_rows_any_") + xn, uint32_t(blocks), kBlock,
                   as_hip(stream), args);
   }
   if (vec) {
     const int64_t blocks = (d0 / nb) * ((d1 / group + 63) / 64);
     if (blocks <= int64_t(kMaxGrid) * 1024)
-      return launch(st, std::string("mtrt_amax_cols_") + xn, uint32_t(blocks), kBlock, as_hip(stream), args);
+      return launch(st, KernelName("mtrt_amax_cols_") + xn, uint32_t(blocks), kBlock, as_hip(stream), args);
   }
-  return launch(st, std::string("mtrt_amax_cols_any_") + xn, blocks_for((d0 / nb) * d1, kBlock), kBlock, as_hip(stream), args);
+  return launch(st, KernelName("mtrt_amax_cols_any_") + xn, blocks_for((d0 / nb) * d1, kBlock), kBlock, as_hip(stream), args);
 }
 
 int32_t mtrt_hip_quantize(mtrt_stream_t stream, const void *x, int32_t x_dtype, void *q, int32_t q_dtype,
@@ -297,7 +298,8 @@ int32_t view_dispatch(bool quantize, hipStream_t stream, const void *f, int32_t 
   if (kind == MTRT_SCALE_UNIFORM)
     nb = 1;
   int64_t fo = fv->offset, fs0 = fv->stride0, fs1 = fv->stride1, qo = qv->offset, qs0 = qv->stride0, qs1 = qv->stride1;
-  const std::string name = std::string(quantize ? "mtrt_q_view_" : "mtrt_dq_view_") + xn + "_" + code_name(q_dtype);
+  KernelName name(quantize ? "mtrt_q_view_" : "mtrt_dq_view_");
+  name + xn + "_" + code_name(q_dtype);
   const uint32_t grid = blocks_for(d0 * d1, kBlock);
   if (quantize) {
     void *args[] = {&f, &fo, &d0, &d1, &fs0, &fs1, &q, &qo, &d0, &d1, &qs0, &qs1, &scale, &nb, &kind, &flags};
@@ -356,7 +358,7 @@ int32_t mtrt_hip_dynamic_quantize_dequantize(mtrt_stream_t stream, const void *x
     const uint32_t grid = uint32_t((nvec + int64_t(1024) * nv - 1) / (int64_t(1024) * nv));
     int32_t limit = g_wait_limit.load();
     void *args[] = {&x, &q, &y, &n, &qmax, &amax_out, &scale_out, &slot, &flags, &limit};
-    return launch(st, std::string("mtrt_dynqdq_") + xn + "_" + code_name(q_dtype) + "_v" + std::to_string(nv), grid, 1024,
+    return launch(st, KernelName("mtrt_dynqdq_") + xn + "_" + code_name(q_dtype) + "_v" + nv, grid, 1024,
                   as_hip(stream), args);
   }
   // Does not fit in the registers of one grid (or is not vector-aligned): the reduction, then the element-wise pass.
@@ -402,11 +404,11 @@ int32_t nvfp4_dispatch(bool quantize, hipStream_t stream, const void *xy, int32_
       return set_error(MTRT_INVALID_ARGUMENT, "tensor of %lld elements is too large", (long long)(d0 * d1));
     if (quantize) {
       void *args[] = {&xy, &q, &scales, &tensor_amax, &d0, &d1};
-      return launch(st, std::string("mtrt_nvfp4_qc_") + xn, uint32_t((units + kBlock - 1) / kBlock), kBlock, stream, args);
+      return launch(st, KernelName("mtrt_nvfp4_qc_") + xn, uint32_t((units + kBlock - 1) / kBlock), kBlock, stream, args);
     }
     void *args[] = {&q, &scales, &tensor_amax, &xy, &d0, &d1};
     const int64_t blocks = std::min<int64_t>((units + kBlock - 1) / kBlock, int64_t(num_compute_units(st)) * 64);
-    return launch(st, std::string("mtrt_nvfp4_dqc_") + xn, uint32_t(blocks), kBlock, stream, args);
+    return launch(st, KernelName("mtrt_nvfp4_dqc_") + xn, uint32_t(blocks), kBlock, stream, args);
   }
   int64_t nvec = d0 * d1 / group;
   const int64_t blocks = (nvec + 4 * 8 * 64 - 1) / (4 * 8 * 64);   // 4 waves x 8 trips x 64 lanes per workgroup
@@ -414,10 +416,10 @@ int32_t nvfp4_dispatch(bool quantize, hipStream_t stream, const void *xy, int32_
     return set_error(MTRT_INVALID_ARGUMENT, "tensor of %lld elements is too large", (long long)(d0 * d1));
   if (quantize) {
     void *args[] = {&xy, &q, &scales, &tensor_amax, &nvec};
-    return launch(st, std::string("mtrt_nvfp4_q_") + xn, uint32_t(blocks), kBlock, stream, args);
+    return launch(st, KernelName("mtrt_nvfp4_q_") + xn, uint32_t(blocks), kBlock, stream, args);
   }
   void *args[] = {&q, &scales, &tensor_amax, &xy, &nvec};
-  return launch(st, std::string("mtrt_nvfp4_dq_") + xn, uint32_t(blocks), kBlock, stream, args);
+  return launch(st, KernelName("mtrt_nvfp4_dq_") + xn, uint32_t(blocks), kBlock, stream, args);
 }
 } // namespace
 
@@ -461,10 +463,10 @@ int32_t mtrt_hip_layernorm(mtrt_stream_t stream, const void *x, const void *gamm
     // filled round and eight waves per SIMD would hold every row at once, its 64-register form is faster.
     const int64_t simds = int64_t(num_compute_units(st)) * 4;
     const bool resident = nv == 8 && rows > 5 * simds && rows <= 8 * simds;
-    return launch(st, std::string("mtrt_layernorm_") + xn + "_v" + std::to_string(nv) + (resident ? "r" : ""),
+    return launch(st, KernelName("mtrt_layernorm_") + xn + "_v" + nv + (resident ? "r" : ""),
                   blocks_for(rows, kBlock / 64), kBlock, as_hip(stream), args);
   }
-  return launch(st, std::string("mtrt_layernorm_") + xn + "_any",
+  return launch(st, KernelName("mtrt_layernorm_") + xn + "_any",
                 uint32_t(std::min<int64_t>(rows, int64_t(num_compute_units(st)) * 8)), kBlock, as_hip(stream), args);
 }
 
@@ -491,9 +493,9 @@ int32_t mtrt_hip_softmax(mtrt_stream_t stream, const void *x, void *y, int32_t d
   int64_t rows_arg = rows, d_arg = d;
   void *args[] = {&x, &y, &rows_arg, &d_arg};
   if (nv && rows <= kMaxRowsPerWaveKernels)
-    return launch(st, std::string("mtrt_softmax_") + xn + "_v" + std::to_string(nv),
+    return launch(st, KernelName("mtrt_softmax_") + xn + "_v" + nv,
                   blocks_for(rows, kBlock / 64), kBlock, as_hip(stream), args);
-  return launch(st, std::string("mtrt_softmax_") + xn + "_any",
+  return launch(st, KernelName("mtrt_softmax_") + xn + "_any",
                 uint32_t(std::min<int64_t>(rows, int64_t(num_compute_units(st)) * 8)), kBlock, as_hip(stream), args);
 }
 
@@ -512,7 +514,7 @@ int32_t mtrt_hip_gemm_w8a8_prepack(mtrt_stream_t stream, const void *w_kn, void 
   if (tiles > int64_t(kMaxGrid) * 1024)
     return set_error(MTRT_INVALID_ARGUMENT, "weight matrix [%lld, %lld] is too large", (long long)K, (long long)N);
   void *args[] = {&w_kn, &w_nk, &K, &N};
-  return launch(st, "mtrt_w8_prepack_kn_to_nk", uint32_t(tiles), kBlock, as_hip(stream), args);
+  return launch(st, KernelName("mtrt_w8_prepack_kn_to_nk"), uint32_t(tiles), kBlock, as_hip(stream), args);
 }
 
 int32_t mtrt_hip_gemm_w8a8(mtrt_stream_t stream, const void *a, const void *w_nk, const float *a_scale,
@@ -549,10 +551,10 @@ int32_t mtrt_hip_gemm_w8a8(mtrt_stream_t stream, const void *a, const void *w_nk
     const int64_t grid = 8 * ((full_panels + 7) / 8) * tiles_m + 8 * ((half_panels + 7) / 8) * tiles_m;
     if (grid <= int64_t(kMaxGrid) * 1024) {
       void *fast_args[] = {&a, &w_nk, &a_scale, &w_scale, &y, &M, &K, &N, &full_panels};
-      return launch(st, "mtrt_gemm_w8a8_nk", uint32_t(grid), kBlock, as_hip(stream), fast_args);
+      return launch(st, KernelName("mtrt_gemm_w8a8_nk"), uint32_t(grid), kBlock, as_hip(stream), fast_args);
     }
   }
-  return launch(st, "mtrt_gemm_w8a8_nk_any", blocks_for(M * N, kBlock), kBlock, as_hip(stream), args);
+  return launch(st, KernelName("mtrt_gemm_w8a8_nk_any"), blocks_for(M * N, kBlock), kBlock, as_hip(stream), args);
 }
 
 int64_t mtrt_hip_gemm_w8a8_fragments_bytes(int64_t K, int64_t N) {
@@ -576,7 +578,7 @@ int32_t mtrt_hip_gemm_w8a8_prepack_fragments(mtrt_stream_t stream, const void *w
     return MTRT_RUNTIME_ERROR;
   const int64_t chunks = mtrt_hip_gemm_w8a8_fragments_bytes(K, N) / 16;
   void *args[] = {&w, &w_frag, &K, &N, &w_is_nk};
-  return launch(st, "mtrt_w8_prepack_frag", blocks_for(chunks, kBlock), kBlock, as_hip(stream), args);
+  return launch(st, KernelName("mtrt_w8_prepack_frag"), blocks_for(chunks, kBlock), kBlock, as_hip(stream), args);
 }
 
 int32_t mtrt_hip_gemm_w8a8_fragments(mtrt_stream_t stream, const void *a, const void *w_frag, const float *a_scale,
@@ -610,7 +612,7 @@ int32_t mtrt_hip_gemm_w8a8_fragments(mtrt_stream_t stream, const void *a, const 
   if (grid > int64_t(kMaxGrid) * 1024)
     return set_error(MTRT_INVALID_ARGUMENT, "problem [%lld, %lld] needs too many tiles", (long long)M, (long long)N);
   void *args[] = {&a, &w_frag, &a_scale, &w_scale, &y, &M, &K, &N, &full_panels};
-  return launch(st, "mtrt_gemm_w8a8_frag", uint32_t(grid), 512, as_hip(stream), args);
+  return launch(st, KernelName("mtrt_gemm_w8a8_frag"), uint32_t(grid), 512, as_hip(stream), args);
 }
 
 int32_t mtrt_hip_linear_dense(mtrt_stream_t stream, const void *x, const void *w_nk, const void *bias, void *y,
@@ -636,7 +638,7 @@ int32_t mtrt_hip_linear_dense(mtrt_stream_t stream, const void *x, const void *w
   if (tiles > int64_t(kMaxGrid) * 1024)
     return set_error(MTRT_INVALID_ARGUMENT, "problem [%lld, %lld] needs too many tiles", (long long)M, (long long)N);
   void *args[] = {&x, &w_nk, &bias, &y, &M, &K, &N};
-  return launch(st, std::string("mtrt_gemm_dense_") + xn, uint32_t(tiles), kBlock, as_hip(stream), args);
+  return launch(st, KernelName("mtrt_gemm_dense_") + xn, uint32_t(tiles), kBlock, as_hip(stream), args);
 }
 
 namespace {
@@ -668,12 +670,12 @@ int32_t mtrt_hip_gemm_w4a16_prepack(mtrt_stream_t stream, const void *w_kn_packe
     return MTRT_RUNTIME_ERROR;
   const int64_t dwords = w4_fragment_bytes(K, N) / 4;
   void *args[] = {&w_kn_packed, &w_prepacked, &K, &N};
-  const int32_t rc = launch(st, "mtrt_w4_prepack", blocks_for(dwords, kBlock), kBlock, as_hip(stream), args);
+  const int32_t rc = launch(st, KernelName("mtrt_w4_prepack"), blocks_for(dwords, kBlock), kBlock, as_hip(stream), args);
   if (rc != MTRT_OK || w4_strip_bytes(K, N) == 0)
     return rc;
   void *strips = static_cast<char *>(w_prepacked) + w4_fragment_bytes(K, N);
   void *args2[] = {&w_kn_packed, &strips, &K, &N};
-  return launch(st, "mtrt_w4_prepack_strips", blocks_for(w4_strip_bytes(K, N) / 4, kBlock), kBlock, as_hip(stream), args2);
+  return launch(st, KernelName("mtrt_w4_prepack_strips"), blocks_for(w4_strip_bytes(K, N) / 4, kBlock), kBlock, as_hip(stream), args2);
 }
 
 int32_t mtrt_hip_gemm_w4a16(mtrt_stream_t stream, const void *a, const void *w_kn_packed, const void *w_prepacked,
@@ -701,7 +703,7 @@ int32_t mtrt_hip_gemm_w4a16(mtrt_stream_t stream, const void *a, const void *w_k
       const void *strips = static_cast<const char *>(w_prepacked) + w4_fragment_bytes(K, N);
       void *sargs[] = {&a, &strips, &scale, &y, &M, &K, &N, &block};
       const int64_t tiles = (N + 15) / 16;
-      return launch(st, "mtrt_gemm_w4a16_strips16", uint32_t(std::min<int64_t>(tiles, num_compute_units(st))), kBlock,
+      return launch(st, KernelName("mtrt_gemm_w4a16_strips16"), uint32_t(std::min<int64_t>(tiles, num_compute_units(st))), kBlock,
                     as_hip(stream), sargs);
     }
     if (M <= 32) {
@@ -710,31 +712,31 @@ int32_t mtrt_hip_gemm_w4a16(mtrt_stream_t stream, const void *a, const void *w_k
       // activations; measured: 6 % faster at M = 16, 21 % at M = 32, 3 % slower at M = 5)
       const int64_t tiles = (N + 31) / 32, cus = num_compute_units(st);
       const uint32_t grid = uint32_t(M > 8 && tiles > cus && tiles <= 2 * cus ? cus : tiles);
-      return launch(st, M <= 16 ? "mtrt_gemm_w4a16_skinny16" : "mtrt_gemm_w4a16_skinny", grid, kBlock, as_hip(stream), args);
+      return launch(st, KernelName(M <= 16 ? "mtrt_gemm_w4a16_skinny16" : "mtrt_gemm_w4a16_skinny"), grid, kBlock, as_hip(stream), args);
     }
     // 256 x 256 tiles (256 threads) once they cover at least half of the compute units (measured:
     // from M = 1024 on at N = 11008 they beat the small tiles) and the activations stay inside
     // 32-bit byte offsets; 128 x 64 tiles otherwise.
     const int64_t panels = (N + 255) / 256, tiles_m = (M + 255) / 256;
     if (panels * tiles_m * 2 >= int64_t(num_compute_units(st)) && M * K * 2 < (int64_t(1) << 32))
-      return launch(st, "mtrt_gemm_w4a16_t256x256", uint32_t(8 * ((panels + 7) / 8) * tiles_m), 256, as_hip(stream),
+      return launch(st, KernelName("mtrt_gemm_w4a16_t256x256"), uint32_t(8 * ((panels + 7) / 8) * tiles_m), 256, as_hip(stream),
                     args);
     if (M * K * 2 < (int64_t(1) << 32)) {
       // 128-row tiles: 128 columns wide while that leaves every compute unit at most one workgroup, else 64
       const int64_t wide_tiles = ((N + 127) / 128) * ((M + 127) / 128);
       if (wide_tiles <= int64_t(num_compute_units(st))) {
         const int64_t wide = 8 * ((((N + 127) / 128) + 7) / 8) * ((M + 127) / 128);
-        return launch(st, "mtrt_gemm_w4a16_t128x128", uint32_t(wide), 512, as_hip(stream), args);
+        return launch(st, KernelName("mtrt_gemm_w4a16_t128x128"), uint32_t(wide), 512, as_hip(stream), args);
       }
       const int64_t small = 8 * ((((N + 63) / 64) + 7) / 8) * ((M + 127) / 128);
-      return launch(st, "mtrt_gemm_w4a16_t128x64", uint32_t(small), kBlock, as_hip(stream), args);
+      return launch(st, KernelName("mtrt_gemm_w4a16_t128x64"), uint32_t(small), kBlock, as_hip(stream), args);
     }
   }
   if (!w_kn_packed)
     return set_error(MTRT_INVALID_ARGUMENT, "this shape needs the original packed weights (K=%lld block=%lld)",
                      (long long)K, (long long)block);
   void *args[] = {&a, &w_kn_packed, &scale, &y, &M, &K, &N, &block};
-  return launch(st, "mtrt_gemm_w4a16_any", blocks_for(M * N, kBlock), kBlock, as_hip(stream), args);
+  return launch(st, KernelName("mtrt_gemm_w4a16_any"), blocks_for(M * N, kBlock), kBlock, as_hip(stream), args);
 }
 
 } // extern "C"

@@ -173,7 +173,7 @@ int32_t clear_slot(DeviceState *st, uint32_t *block, hipStream_t stream) {
   uint32_t fill = 0;
   int32_t width = 4;
   void *args[] = {&p, &count, &fill, &width};
-  return launch(st, "mtrt_fill", 1, 256, stream, args);
+  return launch(st, KernelName("mtrt_fill"), 1, 256, stream, args);
 }
 } // namespace
 
@@ -253,23 +253,68 @@ void forget_stream(hipStream_t stream) {
   }
 }
 
-int32_t launch(DeviceState *st, const std::string &kernel, uint32_t grid, uint32_t block,
-               hipStream_t stream, void **args) {
-  hipFunction_t f = find_kernel(st, kernel);
+namespace {
+// Per-thread cache of resolved kernels: open addressing on the name's hash, entries never removed (the set of
+// kernel names is fixed).  A hit costs one hash of a short string and one compare.
+struct CachedKernel {
+  DeviceState *st = nullptr;
+  hipFunction_t fn = nullptr;
+  uint64_t hash = 0;
+  char name[72] = {0};
+};
+constexpr uint32_t kCacheSlots = 512;                // a thread uses a few dozen kernels; a full table falls back to the locked look-up
+thread_local CachedKernel tl_cache[kCacheSlots];
+thread_local const char *tl_kernel_ptr = "";
+
+uint64_t name_hash(const KernelName &k, DeviceState *st) {
+  uint64_t h = 1469598103934665603ull ^ reinterpret_cast<uintptr_t>(st);
+  for (uint32_t i = 0; i < k.len; ++i)
+    h = (h ^ uint8_t(k.text[i])) * 1099511628211ull;
+  return h | 1;                                      // 0 marks an empty slot
+}
+} // namespace
+
+int32_t launch(DeviceState *st, const KernelName &kernel, uint32_t grid, uint32_t block, hipStream_t stream, void **args) {
+  const uint64_t h = name_hash(kernel, st);
+  CachedKernel *hit = nullptr;
+  for (uint32_t probe = 0; probe < kCacheSlots; ++probe) {
+    CachedKernel &c = tl_cache[(h + probe) & (kCacheSlots - 1)];
+    if (c.hash == h && c.st == st && std::strcmp(c.name, kernel.text) == 0) {
+      hit = &c;
+      break;
+    }
+    if (c.hash == 0) {
+      hipFunction_t f = find_kernel(st, kernel.text);
+      if (!f)
+        return MTRT_NOT_FOUND;
+      c.st = st;
+      c.fn = f;
+      std::memcpy(c.name, kernel.text, kernel.len + 1);
+      c.hash = h;
+      hit = &c;
+      break;
+    }
+  }
+  hipFunction_t f = hit ? hit->fn : find_kernel(st, kernel.text);   // table full: the locked look-up
   if (!f)
     return MTRT_NOT_FOUND;
   const hipError_t e =
       hipModuleLaunchKernel(f, grid, 1, 1, block, 1, 1, /*sharedMemBytes=*/0, stream, args, nullptr);
   if (e != hipSuccess) {
     (void)hipGetLastError(); // reported through the status; do not leave it for the caller's next HIP call
-    return set_error(MTRT_DRIVER_ERROR, "launching '%s' grid %u block %u: %s", kernel.c_str(), grid,
-                     block, hipGetErrorString(e));
+    return set_error(MTRT_DRIVER_ERROR, "launching '%s' grid %u block %u: %s", kernel.text, grid, block,
+                     hipGetErrorString(e));
   }
-  std::snprintf(tl_kernel, sizeof(tl_kernel), "%s", kernel.c_str());
+  if (hit) {
+    tl_kernel_ptr = hit->name;
+  } else {
+    std::snprintf(tl_kernel, sizeof(tl_kernel), "%s", kernel.text);
+    tl_kernel_ptr = tl_kernel;
+  }
   return MTRT_OK;
 }
 
-const char *last_kernel_name() { return tl_kernel; }
+const char *last_kernel_name() { return tl_kernel_ptr; }
 
 } // namespace mtrt_rt
 

@@ -44,8 +44,35 @@ void forget_stream(hipStream_t stream);                              // before a
 // device address of that file's scratch array and the kernel handles it launches.
 int32_t no_alloc_setup(DeviceState *, int device);
 
-// Launch through the same driver call as mtrt_cuda_launch_kernel, returning a status.
-int32_t launch(DeviceState *, const std::string &kernel, uint32_t grid, uint32_t block,
+// A kernel name put together on the stack (no heap, no locale): KernelName("mtrt_q_") + kind + "_" + x.
+struct KernelName {
+  char text[72];
+  uint32_t len = 0;
+  KernelName(const char *s) { text[0] = '\0'; *this + s; }
+  KernelName &operator+(const char *s) {
+    while (*s && len + 1 < sizeof(text))
+      text[len++] = *s++;
+    text[len] = '\0';
+    return *this;
+  }
+  KernelName &operator+(int v) {                       // small non-negative numbers (vector counts)
+    char digits[12];
+    int n = 0;
+    do {
+      digits[n++] = char('0' + v % 10);
+      v /= 10;
+    } while (v > 0 && n < 11);
+    while (n > 0 && len + 1 < sizeof(text))
+      text[len++] = digits[--n];
+    text[len] = '\0';
+    return *this;
+  }
+};
+
+// Launch through the same driver call as mtrt_cuda_launch_kernel, returning a status.  The name is resolved
+// through a per-thread table first (no lock, no allocation); only the first use of a kernel on a thread goes to
+// the device state's table under its mutex.
+int32_t launch(DeviceState *, const KernelName &kernel, uint32_t grid, uint32_t block,
                hipStream_t stream, void **args);
 
 } // namespace mtrt_rt
