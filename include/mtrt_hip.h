@@ -475,6 +475,12 @@ MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_memcpy_strided(uintptr_t stream, int64_
                                                         uintptr_t src, uint64_t srcOffset,
                                                         const int64_t *srcShapeAndStrides, uintptr_t dst,
                                                         uint64_t dstOffset, const int64_t *dstShapeAndStrides);
+/* __cuda_get_active_device / __cuda_set_active_device (CUDAModule.cpp:99-107) and __cuda_get_device(deviceNumber):
+ * the reference registers that last name twice and the later lambda (CUDAModule.cpp:261-267) returns the current
+ * device whatever the argument; so does this one. */
+MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_get_active_device(int32_t *out_device);
+MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_set_active_device(int32_t deviceNumber);
+MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_get_device(int32_t deviceNumber, int32_t *out_device);
 /* __cuda_num_devices (CUDAModule.cpp:86-90) and __cuda_get_program_device(logicalId) (:560-571) */
 MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_num_devices(int32_t *out_count);
 MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_get_program_device(int32_t logicalId, int32_t *out_device);

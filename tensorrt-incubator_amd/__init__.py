@@ -76,6 +76,9 @@ PROTOTYPES = {
     "mtrt_lua_cuda_free_host_pinned": (_i32, [_sz, _sz]),
     "mtrt_lua_cuda_memcpy_strided": (_i32, [_sz, _i64, _i64, _sz, _c.c_uint64, _c.POINTER(_i64), _sz, _c.c_uint64,
                                             _c.POINTER(_i64)]),
+    "mtrt_lua_cuda_get_active_device": (_i32, [_c.POINTER(_i32)]),
+    "mtrt_lua_cuda_set_active_device": (_i32, [_i32]),
+    "mtrt_lua_cuda_get_device": (_i32, [_i32, _c.POINTER(_i32)]),
     "mtrt_lua_cuda_num_devices": (_i32, [_c.POINTER(_i32)]),
     "mtrt_lua_cuda_get_program_device": (_i32, [_i32, _c.POINTER(_i32)]),
     "mtrt_lua_cuda_builtins": (_vp, [_c.POINTER(_sz)]),

@@ -512,6 +512,28 @@ int32_t mtrt_lua_cuda_memcpy_strided(uintptr_t stream, int64_t rank, int64_t ele
   return MTRT_OK;
 }
 
+int32_t mtrt_lua_cuda_get_active_device(int32_t *out_device) {
+  if (!out_device)
+    return set_error(MTRT_INVALID_ARGUMENT, "out_device must not be null");
+  int device = 0;
+  *out_device = 0;
+  RETURN_IF_RT(hipGetDevice(&device));
+  *out_device = device;
+  return MTRT_OK;
+}
+
+int32_t mtrt_lua_cuda_set_active_device(int32_t deviceNumber) {
+  RETURN_IF_RT(hipSetDevice(deviceNumber));
+  return MTRT_OK;
+}
+
+int32_t mtrt_lua_cuda_get_device(int32_t deviceNumber, int32_t *out_device) {
+  // The reference registers this name twice; the later lambda wins and returns the CURRENT device whatever the
+  // argument (CUDAModule.cpp:261-267 over :92-97).  Kept as it behaves.
+  (void)deviceNumber;
+  return mtrt_lua_cuda_get_active_device(out_device);
+}
+
 int32_t mtrt_lua_cuda_num_devices(int32_t *out_count) {
   if (!out_count)
     return set_error(MTRT_INVALID_ARGUMENT, "out_count must not be null");
@@ -569,6 +591,9 @@ const struct mtrt_lua_builtin *mtrt_lua_cuda_builtins(size_t *count) {
       {"__cuda_memcpy_strided_async_host_pinned2device", "mtrt_lua_cuda_memcpy_strided"},
       {"__cuda_memcpy_strided_async_device2host_pinned", "mtrt_lua_cuda_memcpy_strided"},
       {"__cuda_num_devices", "mtrt_lua_cuda_num_devices"},
+      {"__cuda_get_active_device", "mtrt_lua_cuda_get_active_device"},
+      {"__cuda_set_active_device", "mtrt_lua_cuda_set_active_device"},
+      {"__cuda_get_device", "mtrt_lua_cuda_get_device"},
       {"__cuda_get_program_device", "mtrt_lua_cuda_get_program_device"},
   };
   if (count)

@@ -91,6 +91,18 @@ def test_builtin_name_table(pkg):
         assert lua_name in names
     for sym in names.values():
         assert hasattr(L, sym), sym
+    # every `__cuda_*` builtin the reference's CUDA module registers
+    # (mlir-tensorrt/executor/lib/Runtime/Backend/Lua/Modules/CUDA/CUDAModule.cpp:86-571) has a body here
+    reference_names = """__cuda_alloc_device __cuda_alloc_host_pinned __cuda_event_create __cuda_event_elapsed_msec
+        __cuda_event_release __cuda_event_sync __cuda_free_device __cuda_free_host_pinned __cuda_get_active_device
+        __cuda_get_device __cuda_get_function __cuda_get_program_device __cuda_launch __cuda_load_module
+        __cuda_memcpy_device2device __cuda_memcpy_device2host __cuda_memcpy_device2host_pinned __cuda_memcpy_host2device
+        __cuda_memcpy_host_pinned2device __cuda_memcpy_strided_async_device2device __cuda_memcpy_strided_async_device2host
+        __cuda_memcpy_strided_async_device2host_pinned __cuda_memcpy_strided_async_host2device
+        __cuda_memcpy_strided_async_host_pinned2device __cuda_memset_16 __cuda_memset_32 __cuda_memset_8 __cuda_num_devices
+        __cuda_set_active_device __cuda_stream_create __cuda_stream_destroy __cuda_stream_record_event __cuda_stream_sync
+        __cuda_stream_wait_event""".split()
+    assert len(reference_names) == 34 and set(reference_names) == set(names)
 
 
 def test_builtin_argument_validation(pkg):
@@ -200,6 +212,11 @@ def test_builtin_events_pinned_memory_and_strided_copies(pkg):
     L = pkg.lib()
     sz = ctypes.c_size_t
     dev = L.mtrt_cuda_get_current_device()
+    d = ctypes.c_int32(-1)
+    assert L.mtrt_lua_cuda_get_active_device(ctypes.byref(d)) == 0 and d.value == dev
+    assert L.mtrt_lua_cuda_set_active_device(dev) == 0
+    assert L.mtrt_lua_cuda_get_device(0, ctypes.byref(d)) == 0 and d.value == dev
+    assert L.mtrt_lua_cuda_set_active_device(4096) != 0 and L.mtrt_hip_last_error()
     stream, e0, e1, e2 = sz(0), sz(0), sz(0), sz(0)
     assert L.mtrt_lua_cuda_stream_create(ctypes.byref(stream)) == 0
     assert L.mtrt_lua_cuda_event_create(dev, ctypes.byref(e0)) == 0 and e0.value
