@@ -10,21 +10,25 @@
 // tensor fits in the registers of one grid: x is read once (the two-launch form reads it twice) and the time of
 // a second launch is saved, which is most of the cost of a tensor of a few MB.
 //
-// Shape: gridDim.x workgroups of 1024 lanes, one per compute unit at most; each lane keeps NV 128-bit vectors of
-// x in registers.  The workgroups meet in the arrival tree of amax.hip; whoever arrives last at the root
-// publishes the maximum (tag in the high half of a 64-bit word), in kCopies copies on cache lines of their own so
-// that the polls of the waiting workgroups spread over as many memory-side queues (every device-scope atomic on
-// one line is served one after the other; a flat exchange where all workgroups add to and poll one counter was
-// measured 5 us slower on 256 workgroups).  Every workgroup needs that word before it can quantize.
+// Shape: gridDim.x workgroups of 1024 lanes, one per compute unit at most (and at most 256); each lane keeps NV
+// 128-bit vectors of x in registers.  Every workgroup needs the maximum of all before it can quantize, and the
+// exchange is what a launch of a few MB spends most of its time on, so it is built from the cheapest operations
+// the memory system has: every workgroup STORES its maximum, tagged with the launch's number, into a slot of its
+// own (one device-scope store, nobody waits for it) and then reads all slots (64 lanes x 4 slots, one round trip)
+// until every slot carries the tag.  No read-modify-write is on the path: device-scope atomics on one line are
+// served one after the other (an arrival tree cost five dependent trips to memory, about 0.9 us each; a single
+// counter that all 256 workgroups add to and poll was slower still), plain stores and loads are not.
+// The tag is a counter in the scratch block which the workgroups advance when they are done with the slots (a
+// maximum that nobody waits for), so the slots never have to be cleared: what an earlier launch left carries an
+// older tag.
 // Nothing guarantees that all workgroups of a launch are resident at once (another stream may hold compute
-// units), so the wait is BOUNDED: lane 0 polls `spin_limit` times; a workgroup that gives up computes the maximum
+// units), so the wait is BOUNDED: `spin_limit` rounds of reads; a workgroup that gives up computes the maximum
 // of the whole tensor by itself (slow, same bits) and goes on, which frees its compute unit for the workgroups
 // still queued.  No workgroup ever depends on another one making progress.
-// The scratch block restores itself: after reading (or giving up on) the result every workgroup arrives at a
-// second counter, and the last of them clears the result words and the counter.
 //
-// scratch (the stream's reduction block, zero on entry and on exit): lines 0..32 arrival tree, lines 33..48 the
-// copies of the result word {tag, max bits}, line 49 the second counter.
+// scratch (the stream's reduction block, zero when the stream first uses it): lines 0..32 belong to the arrival
+// tree of amax.hip and are not touched here; lines 33..48 hold the 256 slots {tag, max bits}, line 49 the tag
+// counter.  Tags repeat after 2^32 launches.
 #include "common.hpp"
 
 namespace dynq_cluster {
@@ -34,7 +38,7 @@ using namespace qdq_cluster;
 using namespace amax_cluster;
 
 constexpr int kDynThreads = 1024;
-constexpr uint32_t kResultLine = 33, kCopies = 16, kDoneLine = kResultLine + kCopies;
+constexpr uint32_t kSlotLine = 33, kSlots = 256, kTagLine = 49;
 
 __device__ __forceinline__ uint32_t block_max(uint32_t m, uint32_t* wave_max) {
   m = wave_reduce(m, MaxU32());
@@ -61,6 +65,11 @@ __device__ __forceinline__ void dynqdq_body(const typename X::storage* __restric
   const int64_t nvec = n / G;                        // host: n % G == 0, x / y 16-byte aligned
   const int64_t base = int64_t(blockIdx.x) * (kDynThreads * NV) + threadIdx.x;
 
+  unsigned long long* slots = reinterpret_cast<unsigned long long*>(scratch + kAmaxLineWords * kSlotLine);
+  uint32_t* tag_word = scratch + kAmaxLineWords * kTagLine;
+  // asked for before the data, needed after it
+  const uint32_t tag = __hip_atomic_load(tag_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+
   u32x4 xin[NV];
   uint32_t m = 0;
 #pragma unroll
@@ -75,35 +84,34 @@ __device__ __forceinline__ void dynqdq_body(const typename X::storage* __restric
   }
   m = block_max(m, wave_max);
 
-  unsigned long long* result = reinterpret_cast<unsigned long long*>(scratch + kAmaxLineWords * kResultLine);
-  unsigned long long* done = reinterpret_cast<unsigned long long*>(scratch + kAmaxLineWords * kDoneLine);
-  constexpr int kLineQwords = kAmaxLineWords / 2;
-  if (threadIdx.x == 0) {
-    const uint32_t groups = gridDim.x < kAmaxFanIn ? gridDim.x : kAmaxFanIn;
-    const uint32_t g = blockIdx.x % groups;
-    const uint32_t members = (gridDim.x - g + groups - 1) / groups;
-    uint32_t total = m;
-    bool have = false;
-    if (arrive(scratch + kAmaxLineWords * (1 + g), members, total) && arrive(scratch, groups, total)) {
-      // last arrival of the whole grid: publish for the others (tag 1 in the high half)
+  if (threadIdx.x < kWave) {                         // wave 0: publish, then watch the other slots
+    const uint32_t lane = threadIdx.x;
+    if (lane == 0)
+      __hip_atomic_store(slots + blockIdx.x, ((unsigned long long)tag << 32) | m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    uint32_t total = m, have = 0;
+    for (int spin = 0; spin < spin_limit; ++spin) {
+      uint32_t mx = m;
+      bool ok = true;
 #pragma unroll
-      for (uint32_t c = 0; c < kCopies; ++c)
-        __hip_atomic_exchange(result + c * kLineQwords, (1ull << 32) | total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      have = true;
-    } else {
-      const unsigned long long* mine = result + (blockIdx.x % kCopies) * kLineQwords;
-      for (int spin = 0; spin < spin_limit; ++spin) {
-        const unsigned long long w = __hip_atomic_load(mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (w >> 32) {
-          total = uint32_t(w);
-          have = true;
-          break;
+      for (uint32_t c = 0; c < kSlots / kWave; ++c) {
+        const uint32_t idx = lane + kWave * c;
+        if (idx < gridDim.x && idx != blockIdx.x) {  // the own slot is known without reading it back
+          const unsigned long long w = __hip_atomic_load(slots + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          ok = ok && uint32_t(w >> 32) == tag;
+          mx = mx > uint32_t(w) ? mx : uint32_t(w);
         }
-        __builtin_amdgcn_s_sleep(1);
       }
+      if (__ballot(ok) == __ballot(true)) {
+        total = wave_reduce(mx, MaxU32());
+        have = 1;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(1);
     }
-    bcast[0] = have ? 1u : 0u;
-    bcast[1] = total;
+    if (lane == 0) {
+      bcast[0] = have;
+      bcast[1] = total;
+    }
   }
   __syncthreads();
   uint32_t total = bcast[1];
@@ -116,16 +124,14 @@ __device__ __forceinline__ void dynqdq_body(const typename X::storage* __restric
     }
     total = block_max(mm, wave_max);
   }
-  if (threadIdx.x == 0) {
-    // second arrival: once every workgroup has the maximum (or has given up) the block returns to zero
-    const unsigned long long old = __hip_atomic_fetch_add(done, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (uint32_t(old) == gridDim.x - 1) {
-#pragma unroll
-      for (uint32_t c = 0; c < kCopies; ++c)
-        __hip_atomic_exchange(result + c * kLineQwords, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_exchange(done, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-  }
+  // Done with the slots: advance the tag counter for the next launch on this stream.  Every workgroup does it
+  // (a maximum, so it is idempotent) and none waits for an answer: 256 workgroups updating one line within a
+  // microsecond take the memory side up to 3 us to serve, and a lane that waited for its turn would hold its
+  // whole wave back.  The counter cannot move while a workgroup of this launch has yet to read it: nobody gets
+  // here before every slot carries the tag, and a workgroup publishes after it has read the counter.  (Unless
+  // somebody gave up waiting: a workgroup that starts after that reads the advanced counter, finds no slot with
+  // its tag, gives up in turn and computes the maximum itself; right, only slow, like every give-up.)
+  if (threadIdx.x == 0) __hip_atomic_fetch_max(tag_word, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
   const float amax = A::finish(total);
   const float scale = amax / qmax;                   // one IEEE divide, as the host does it; identical in every workgroup
@@ -156,7 +162,7 @@ __device__ __forceinline__ void dynqdq_body(const typename X::storage* __restric
 
 // (x, q, y or null, n, qmax, amax_out or null, scale_out or null, scratch, flags, spin_limit)
 //   n % G == 0 (G = 4 for f32, 8 for f16 / bf16), x and y 16-byte aligned, q aligned to G codes,
-//   gridDim.x = ceil(n / G / (1024 * NV)) <= number of compute units, block = 1024.
+//   gridDim.x = ceil(n / G / (1024 * NV)) <= min(number of compute units, 256), block = 1024.
 #define MTRT_DYNQ_KERNEL(XN, XT, QN, QT, NV)                                                                          \
   extern "C" __global__ void __launch_bounds__(1024) mtrt_dynqdq_##XN##_##QN##_v##NV(                                  \
       const XT::storage* x, QT::storage* q, XT::storage* y, int64_t n, float qmax, float* amax_out, float* scale_out,  \

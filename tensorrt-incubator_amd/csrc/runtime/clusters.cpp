@@ -347,7 +347,8 @@ int32_t mtrt_hip_dynamic_quantize_dequantize(mtrt_stream_t stream, const void *x
   if (!st)
     return MTRT_RUNTIME_ERROR;
   const int group = x_dtype == MTRT_F32 ? 4 : 8;
-  const int64_t nvec = n / group, units = num_compute_units(st);   // one workgroup per compute unit at most
+  // one workgroup per compute unit at most, and one slot of the exchange per workgroup (256 of them)
+  const int64_t nvec = n / group, units = std::min(num_compute_units(st), 256);
   const bool one_launch = n > 0 && n % group == 0 && aligned(x, 16) && aligned(q, group) && (!y || aligned(y, 16)) &&
                           nvec <= units * 1024 * 16 && !((flags & MTRT_F8_REFHOST) && (flags & MTRT_F8_VIA_F16));
   if (one_launch) {

@@ -77,9 +77,9 @@ struct DeviceState {
   hipModule_t module = nullptr;
   std::mutex mu;
   std::unordered_map<std::string, hipFunction_t> funcs;
-  // One zeroed block per stream for single-launch grid reductions: 33 lines of
-  // 128 bytes for the arrival tree (root + 32 first-level groups, see amax.hip) and
-  // 17 for the broadcast of dynq.hip, rounded up to 64.  Kernels return their block to zero.
+  // One block per stream for single-launch grid reductions, zero when a stream first uses it: 33 lines of
+  // 128 bytes for the arrival tree (root + 32 first-level groups, see amax.hip), which the kernels return to
+  // zero, and 18 for the tagged slots and counters of dynq.hip, which never need clearing; rounded up to 64.
   static constexpr int kSlots = 256;
   static constexpr int kSlotWords = 64 * 32;
   uint32_t *slots = nullptr;
