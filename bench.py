@@ -296,20 +296,41 @@ def mfma_sustained(pkg, torch, kernel, operand, ops_per_mfma):
     return ksteps * 16.0 * units * 4 * ops_per_mfma / us / 1e6
 
 
+def kernel_sources_digest():
+    """sha256 over the device sources (csrc/kernels/*, in name order): what a counter profile must have been taken
+    with for its per-kernel figures to describe the kernels that run now."""
+    import hashlib
+    kdir = os.path.join(ROOT, "tensorrt-incubator_amd", "csrc", "kernels")
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(kdir)):
+        if name.endswith((".hip", ".hpp")):
+            h.update(name.encode() + b"\0")
+            h.update(open(os.path.join(kdir, name), "rb").read())
+    return h.hexdigest()
+
+
 def traffic_from_profile(kernel):
-    """HBM bytes per launch of `kernel` as measured by the committed counter profile
-    (profiles/hbm_traffic_bench_suite.md, table rows `| kernel | fetch | write | total |`), or None."""
+    """(HBM bytes per launch of `kernel`, where the figure comes from).  The figure is the one measured by the
+    committed counter profile (profiles/hbm_traffic_bench_suite.md, table rows `| kernel | fetch | write | total |`);
+    it is None when the profile names other kernel sources than the ones in the tree (line `kernel sources sha256:
+    ...`), i.e. when it was taken before a kernel changed."""
     path = os.path.join(ROOT, "profiles", "hbm_traffic_bench_suite.md")
+    where = "profiles/hbm_traffic_bench_suite.md (rocprofv3 --pmc run of this command; not measured in this run)"
     if not os.path.exists(path):
-        return None
+        return None, "no counter profile in the tree"
+    value, digest = None, None
     for line in open(path):
+        if line.startswith("kernel sources sha256:"):
+            digest = line.split(":", 1)[1].strip()
         cells = [c.strip() for c in line.strip().strip("|").split("|")]
         if len(cells) >= 4 and cells[0] == kernel:
             try:
-                return float(cells[3])
+                value = float(cells[3])
             except ValueError:
-                return None
-    return None
+                value = None
+    if digest != kernel_sources_digest():
+        return None, "profiles/hbm_traffic_bench_suite.md was taken with other kernel sources than the tree's: not used"
+    return value, where
 
 
 def time_kernel(pkg, torch, w, reps):
@@ -527,6 +548,7 @@ def main():
             k["frac_of_sustained"] = round(k["achieved"] / sustained[k["unit"]], 4)
     value = 100.0 * (ideal_us / 1e3) / ms_per_step
     dom = max(kernels, key=lambda k: k["us"])
+    traffic = traffic_from_profile(dom["kernel"])
     line = {
         "metric": "Q/DQ+reduce HBM GB/s and W8A8/W4A16 GEMM TOPS, as % of MI355X peak, 1 GPU",
         "value": round(value, 2),
@@ -537,9 +559,7 @@ def main():
         "config": {"workload": {"all": "C1+C2a+C2b+C3+C4+C5 programs of BASELINE.json, one pass each per step"}.get(
             args.workload, args.workload.upper()), "kernels_per_step": len(wl)},
         "roofline": {"kernel": dom["kernel"], "bound": dom["bound"], "achieved": dom["achieved"], "peak": dom["peak"],
-                     "unit": dom["unit"], "frac": dom["frac"], "traffic": traffic_from_profile(dom["kernel"]),
-                     "traffic_source": "profiles/hbm_traffic_bench_suite.md (rocprofv3 --pmc run of this command; "
-                                       "not measured in this run)"},
+                     "unit": dom["unit"], "frac": dom["frac"], "traffic": traffic[0], "traffic_source": traffic[1]},
         "mfma_sustained": {"rates": sustained, "rates_on_zero_operands": sustained_zero, "method": "mtrt_mfma_probe_*: 16 independent MFMAs per round and wave, one wave "
                            "per SIMD, operands = this bench's own data, no memory traffic; published dense peaks are "
                            "not reached on non-zero data (power limit)"},
