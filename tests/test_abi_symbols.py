@@ -116,3 +116,54 @@ def test_argument_validation_needs_no_device(pkg):
     # zero-sized work is a no-op that needs no device either
     assert L.mtrt_hip_quantize(None, 16, pkg.F32, 16, pkg.I8, 16, 0, 0, 4, 1, 0) == 0
     assert L.mtrt_hip_softmax(None, 16, 16, pkg.F32, 0, 4) == 0
+
+
+def test_argument_validation_of_the_newer_entry_points_needs_no_device(pkg):
+    """Every rejection below happens before the device is looked up, so it reads the same on a machine
+    without a GPU; 16 stands for a non-null pointer that is never dereferenced."""
+    import ctypes
+    L = pkg.lib()
+    err = lambda: L.mtrt_hip_last_error().decode()
+    # amax per scale element
+    assert L.mtrt_hip_amax_scales(None, 16, 9, pkg.SCALE_ROW, 4, 4, 4, 127.0, 16, 16) == 1 and "f32/f16/bf16" in err()
+    assert L.mtrt_hip_amax_scales(None, 16, pkg.F32, 7, 4, 4, 4, 127.0, 16, 16) == 1 and "scale kind" in err()
+    assert L.mtrt_hip_amax_scales(None, 16, pkg.F32, pkg.SCALE_ROW, 4, 4, 0, 127.0, 16, 16) == 1 and "positive" in err()
+    assert L.mtrt_hip_amax_scales(None, 16, pkg.F32, pkg.SCALE_ROW, 4, 4, 5, 127.0, 16, 16) == 1 and "5 scales for 4 rows" in err()
+    assert L.mtrt_hip_amax_scales(None, 16, pkg.F32, pkg.SCALE_COL, 6, 4, 4, 127.0, 16, 16) == 1 and "does not divide" in err()
+    assert L.mtrt_hip_amax_scales(None, 16, pkg.F32, pkg.SCALE_COL, 8, 4, 4, 127.0, None, None) == 1 and "null operand" in err()
+    assert L.mtrt_hip_amax_scales(None, 18, pkg.F32, pkg.SCALE_COL, 8, 4, 4, 127.0, 16, 16) == 1 and "aligned" in err()
+    assert L.mtrt_hip_amax_scales(None, 16, pkg.F32, pkg.SCALE_COL, 0, 4, 4, 127.0, 16, 16) == 0      # nothing to reduce
+    # dynamic quantization in one call
+    dq = L.mtrt_hip_dynamic_quantize_dequantize
+    assert dq(None, 16, pkg.F32, 16, pkg.I4, 16, 64, 127.0, 16, 16, 0) == 1 and "i8 or f8E4M3FN" in err()
+    assert dq(None, 16, pkg.F32, 16, pkg.I8, 16, -1, 127.0, 16, 16, 0) == 1 and "negative" in err()
+    assert dq(None, None, pkg.F32, 16, pkg.I8, 16, 64, 127.0, 16, 16, 0) == 1 and "null operand" in err()
+    assert dq(None, 16, pkg.F32, 16, pkg.I8, 16, 64, 127.0, 16, None, 0) == 1 and "scale_out" in err()
+    assert dq(None, 16, pkg.F32, 16, pkg.I8, 16, 64, 127.0, 16, 16, 64) == 1 and "flag" in err()
+    # quantize on views
+    ok_view = pkg.View2d(0, 8, 1)
+    below = pkg.View2d(2, -8, 1)                               # row 1 would start 6 elements below the base pointer
+    qv = L.mtrt_hip_quantize_view
+    ref = ctypes.byref
+    assert qv(None, 16, pkg.F32, ref(ok_view), 16, pkg.I4_PACKED, ref(ok_view), 16, pkg.SCALE_UNIFORM, 4, 8, 1, 0) == 1 and "one code per byte" in err()
+    assert qv(None, 16, pkg.F32, None, 16, pkg.I8, ref(ok_view), 16, pkg.SCALE_UNIFORM, 4, 8, 1, 0) == 1 and "descriptor" in err()
+    assert qv(None, 16, pkg.F32, ref(ok_view), 16, pkg.I8, ref(ok_view), 16, pkg.SCALE_COL, 6, 8, 4, 0) == 1 and "does not divide" in err()
+    assert qv(None, 16, pkg.F32, ref(ok_view), 16, pkg.I8, ref(ok_view), 16, pkg.SCALE_UNIFORM, 4, 8, 1, pkg.F8_REFHOST | pkg.F8_VIA_F16) == 1 and "flag" in err()
+    assert qv(None, 16, pkg.F32, ref(below), 16, pkg.I8, ref(ok_view), 16, pkg.SCALE_UNIFORM, 4, 8, 1, 0) == 1 and "below its base" in err()
+    assert qv(None, 16, pkg.F32, ref(ok_view), 16, pkg.I8, ref(ok_view), 16, pkg.SCALE_UNIFORM, 1 << 20, 1 << 20, 1, 0) == 1 and "too large" in err()
+    assert qv(None, 16, pkg.F32, ref(ok_view), 16, pkg.I8, ref(ok_view), 16, pkg.SCALE_UNIFORM, 0, 8, 1, 0) == 0
+    # dense Linear
+    ld = L.mtrt_hip_linear_dense
+    assert ld(None, 16, 16, None, 16, 9, 4, 4, 4) == 1 and "f32/f16/bf16" in err()
+    assert ld(None, 16, 16, None, 16, pkg.F16, 4, -4, 4) == 1 and "negative" in err()
+    assert ld(None, 16, None, None, 16, pkg.F16, 4, 4, 4) == 1 and "null operand" in err()
+    assert ld(None, 16, 16, 17, 16, pkg.F16, 4, 4, 4) == 1 and "aligned" in err()
+    assert ld(None, 16, 16, None, 16, pkg.F16, 0, 4, 4) == 0
+    # the block-wise GEMM and the size of its re-laid weights
+    assert L.mtrt_hip_gemm_w4a16(None, 16, 16, 16, 16, 16, 4, 256, 64, 96) == 1 and "does not divide" in err()
+    assert L.mtrt_hip_gemm_w4a16(None, 16, None, None, 16, 16, 4, 256, 64, 128) == 1 and "null operand" in err()
+    assert L.mtrt_hip_gemm_w4a16_prepacked_bytes(4096, 11008) == 4096 * 11008            # two layouts of K*N/2 bytes each
+    assert L.mtrt_hip_gemm_w4a16_prepacked_bytes(192, 64) == 192 * 64 // 2               # K % 128 != 0: fragment order only
+    assert L.mtrt_hip_gemm_w4a16_prepacked_bytes(100, 64) == 0
+    # the allocation-free reduction: its own limit, and it needs the library initialised on the device first
+    assert L.mtrt_hip_amax_no_alloc(None, 16, pkg.F32, (1 << 36) + 1, 127.0, 16, 16) == 1 and "allocation-free amax accepts" in err()
