@@ -46,6 +46,12 @@ int float_bytes(int32_t dt) { return dt == MTRT_F32 ? 4 : 2; }
 
 bool aligned(const void *p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
+// Element count of a [d0, d1] operand without signed overflow: false when the product does not fit in 63 bits.
+bool element_count(int64_t d0, int64_t d1, int64_t *n) { return !__builtin_mul_overflow(d0, d1, n); }
+// Matrix extents of the GEMM entry points: below 2^31 each, so that every product of two of them (and twice that)
+// fits in 63 bits.
+constexpr int64_t kMaxMatrixExtent = (int64_t(1) << 31) - 1;
+
 uint32_t blocks_for(int64_t units, uint32_t per_block) {
   const int64_t b = (units + per_block - 1) / per_block;
   return uint32_t(std::max<int64_t>(1, std::min<int64_t>(b, kMaxGrid)));
@@ -76,11 +82,11 @@ int32_t qdq_dispatch(int mode, hipStream_t stream, const void *x, int32_t x_dtyp
     return set_error(MTRT_INVALID_ARGUMENT, "unknown flag bits 0x%x", flags);
   if ((flags & MTRT_F8_REFHOST) && (flags & MTRT_F8_VIA_F16))
     return set_error(MTRT_INVALID_ARGUMENT, "MTRT_F8_REFHOST and MTRT_F8_VIA_F16 name two different conversions; pass one");
-  const int64_t n = d0 * d1;
+  int64_t n;
+  if (!element_count(d0, d1, &n) || n >= (int64_t(1) << 35))
+    return set_error(MTRT_INVALID_ARGUMENT, "[%lld, %lld] elements exceed the supported 2^35", (long long)d0, (long long)d1);
   if (n == 0)
     return MTRT_OK;
-  if (n >= (int64_t(1) << 35))
-    return set_error(MTRT_INVALID_ARGUMENT, "%lld elements exceed the supported 2^35", (long long)n);
   if (!scale || !q || (mode != 1 && !x) || (mode != 0 && !y))
     return set_error(MTRT_INVALID_ARGUMENT, "null operand");
   if (!aligned(mode == 1 ? y : x, float_bytes(x_dtype)) || (mode == 2 && !aligned(y, float_bytes(x_dtype))))
@@ -189,8 +195,11 @@ int32_t mtrt_hip_amax_scales(mtrt_stream_t stream, const void *x, int32_t dtype,
     return set_error(MTRT_INVALID_ARGUMENT, "negative extent [%lld, %lld]", (long long)d0, (long long)d1);
   if (scale_kind < MTRT_SCALE_UNIFORM || scale_kind > MTRT_SCALE_COL)
     return set_error(MTRT_INVALID_ARGUMENT, "unknown scale kind %d", scale_kind);
+  int64_t n;
+  if (!element_count(d0, d1, &n))
+    return set_error(MTRT_INVALID_ARGUMENT, "[%lld, %lld] elements do not fit a 64-bit count", (long long)d0, (long long)d1);
   if (scale_kind == MTRT_SCALE_UNIFORM)
-    return mtrt_hip_amax(stream, x, dtype, d0 * d1, qmax, amax_out, scale_out);
+    return mtrt_hip_amax(stream, x, dtype, n, qmax, amax_out, scale_out);
   if (nb <= 0)
     return set_error(MTRT_INVALID_ARGUMENT, "scale kind %d needs a positive scale count / block size, got %lld", scale_kind,
                      (long long)nb);
@@ -281,8 +290,9 @@ int32_t view_dispatch(bool quantize, hipStream_t stream, const void *f, int32_t 
     return set_error(MTRT_INVALID_ARGUMENT, "bad flag bits 0x%x", flags);
   if (d0 == 0 || d1 == 0)
     return MTRT_OK;
-  if (d0 * d1 >= (int64_t(1) << 40))
-    return set_error(MTRT_INVALID_ARGUMENT, "view of %lld elements is too large", (long long)(d0 * d1));
+  int64_t n;
+  if (!element_count(d0, d1, &n) || n >= (int64_t(1) << 40))
+    return set_error(MTRT_INVALID_ARGUMENT, "view of [%lld, %lld] elements is too large", (long long)d0, (long long)d1);
   if (!f || !q || !scale)
     return set_error(MTRT_INVALID_ARGUMENT, "null operand");
   if (!aligned(f, float_bytes(f_dtype)))
@@ -300,7 +310,7 @@ int32_t view_dispatch(bool quantize, hipStream_t stream, const void *f, int32_t 
   int64_t fo = fv->offset, fs0 = fv->stride0, fs1 = fv->stride1, qo = qv->offset, qs0 = qv->stride0, qs1 = qv->stride1;
   KernelName name(quantize ? "mtrt_q_view_" : "mtrt_dq_view_");
   name + xn + "_" + code_name(q_dtype);
-  const uint32_t grid = blocks_for(d0 * d1, kBlock);
+  const uint32_t grid = blocks_for(n, kBlock);
   if (quantize) {
     void *args[] = {&f, &fo, &d0, &d1, &fs0, &fs1, &q, &qo, &d0, &d1, &qs0, &qs1, &scale, &nb, &kind, &flags};
     return launch(st, name, grid, kBlock, stream, args);
@@ -383,6 +393,9 @@ int32_t nvfp4_dispatch(bool quantize, hipStream_t stream, const void *xy, int32_
   if (block_axis != 0 && block_axis != 1)
     return set_error(MTRT_INVALID_ARGUMENT, "invalid axis! Axis can be either last (1) or second last (0) dimension of the [d0, d1] view, got %d",
                      block_axis);
+  int64_t n;
+  if (!element_count(d0, d1, &n) || n >= (int64_t(1) << 40))
+    return set_error(MTRT_INVALID_ARGUMENT, "tensor of [%lld, %lld] elements is too large", (long long)d0, (long long)d1);
   const int64_t blocked = block_axis ? d1 : d0;
   if (blocked % 16 != 0)
     return set_error(MTRT_INVALID_ARGUMENT, "shape(input)[axis] must be divisible by 16, got %lld", (long long)blocked);
@@ -402,7 +415,7 @@ int32_t nvfp4_dispatch(bool quantize, hipStream_t stream, const void *xy, int32_
                        group, (long long)d1);
     const int64_t units = quantize ? (d0 / 16) * (d1 / group) : d0 * (d1 / group);
     if ((units + kBlock - 1) / kBlock > int64_t(kMaxGrid) * 1024)
-      return set_error(MTRT_INVALID_ARGUMENT, "tensor of %lld elements is too large", (long long)(d0 * d1));
+      return set_error(MTRT_INVALID_ARGUMENT, "tensor of %lld elements is too large", (long long)n);
     if (quantize) {
       void *args[] = {&xy, &q, &scales, &tensor_amax, &d0, &d1};
       return launch(st, KernelName("mtrt_nvfp4_qc_") + xn, uint32_t((units + kBlock - 1) / kBlock), kBlock, stream, args);
@@ -411,10 +424,10 @@ int32_t nvfp4_dispatch(bool quantize, hipStream_t stream, const void *xy, int32_
     const int64_t blocks = std::min<int64_t>((units + kBlock - 1) / kBlock, int64_t(num_compute_units(st)) * 64);
     return launch(st, KernelName("mtrt_nvfp4_dqc_") + xn, uint32_t(blocks), kBlock, stream, args);
   }
-  int64_t nvec = d0 * d1 / group;
+  int64_t nvec = n / group;
   const int64_t blocks = (nvec + 4 * 8 * 64 - 1) / (4 * 8 * 64);   // 4 waves x 8 trips x 64 lanes per workgroup
   if (blocks > int64_t(kMaxGrid) * 1024)
-    return set_error(MTRT_INVALID_ARGUMENT, "tensor of %lld elements is too large", (long long)(d0 * d1));
+    return set_error(MTRT_INVALID_ARGUMENT, "tensor of %lld elements is too large", (long long)n);
   if (quantize) {
     void *args[] = {&xy, &q, &scales, &tensor_amax, &nvec};
     return launch(st, KernelName("mtrt_nvfp4_q_") + xn, uint32_t(blocks), kBlock, stream, args);
@@ -443,6 +456,9 @@ int32_t mtrt_hip_layernorm(mtrt_stream_t stream, const void *x, const void *gamm
     return set_error(MTRT_INVALID_ARGUMENT, "layernorm dtype %d is not one of f32/f16/bf16", dtype);
   if (rows < 0 || d < 0)
     return set_error(MTRT_INVALID_ARGUMENT, "negative extent [%lld, %lld]", (long long)rows, (long long)d);
+  int64_t n;
+  if (!element_count(rows, d, &n) || n >= (int64_t(1) << 40))
+    return set_error(MTRT_INVALID_ARGUMENT, "[%lld, %lld] elements exceed the supported 2^40", (long long)rows, (long long)d);
   if (rows == 0 || d == 0)
     return MTRT_OK;
   if (!x || !gamma || !beta || !y)
@@ -478,6 +494,9 @@ int32_t mtrt_hip_softmax(mtrt_stream_t stream, const void *x, void *y, int32_t d
     return set_error(MTRT_INVALID_ARGUMENT, "softmax dtype %d is not one of f32/f16/bf16", dtype);
   if (rows < 0 || d < 0)
     return set_error(MTRT_INVALID_ARGUMENT, "negative extent [%lld, %lld]", (long long)rows, (long long)d);
+  int64_t n;
+  if (!element_count(rows, d, &n) || n >= (int64_t(1) << 40))
+    return set_error(MTRT_INVALID_ARGUMENT, "[%lld, %lld] elements exceed the supported 2^40", (long long)rows, (long long)d);
   if (rows == 0 || d == 0)
     return MTRT_OK;
   if (!x || !y)
@@ -502,8 +521,8 @@ int32_t mtrt_hip_softmax(mtrt_stream_t stream, const void *x, void *y, int32_t d
 
 int32_t mtrt_hip_gemm_w8a8_prepack(mtrt_stream_t stream, const void *w_kn, void *w_nk, int64_t K, int64_t N) {
   clear_error();
-  if (K < 0 || N < 0)
-    return set_error(MTRT_INVALID_ARGUMENT, "negative extent [%lld, %lld]", (long long)K, (long long)N);
+  if (K < 0 || N < 0 || K > kMaxMatrixExtent || N > kMaxMatrixExtent)
+    return set_error(MTRT_INVALID_ARGUMENT, "extents [%lld, %lld] are negative or beyond 2^31 - 1", (long long)K, (long long)N);
   if (K == 0 || N == 0)
     return MTRT_OK;
   if (!w_kn || !w_nk)
@@ -524,6 +543,9 @@ int32_t mtrt_hip_gemm_w8a8(mtrt_stream_t stream, const void *a, const void *w_nk
   if (M < 0 || K < 0 || N < 0)
     return set_error(MTRT_INVALID_ARGUMENT, "negative extent M=%lld K=%lld N=%lld", (long long)M, (long long)K,
                      (long long)N);
+  if (M > kMaxMatrixExtent || K > kMaxMatrixExtent || N > kMaxMatrixExtent)
+    return set_error(MTRT_INVALID_ARGUMENT, "matrix extents are limited to 2^31 - 1, got M=%lld K=%lld N=%lld", (long long)M,
+                     (long long)K, (long long)N);
   if (M == 0 || N == 0)
     return MTRT_OK;
   if (!a_scale || !w_scale || !y || (K > 0 && (!a || !w_nk)))
@@ -559,7 +581,7 @@ int32_t mtrt_hip_gemm_w8a8(mtrt_stream_t stream, const void *a, const void *w_nk
 }
 
 int64_t mtrt_hip_gemm_w8a8_fragments_bytes(int64_t K, int64_t N) {
-  if (K <= 0 || N <= 0 || K % 128 != 0)
+  if (K <= 0 || N <= 0 || K % 128 != 0 || K > kMaxMatrixExtent || N > kMaxMatrixExtent)
     return 0;
   return ((N + 31) / 32) * 32 * K;
 }
@@ -567,8 +589,8 @@ int64_t mtrt_hip_gemm_w8a8_fragments_bytes(int64_t K, int64_t N) {
 int32_t mtrt_hip_gemm_w8a8_prepack_fragments(mtrt_stream_t stream, const void *w, int32_t w_is_nk, void *w_frag,
                                              int64_t K, int64_t N) {
   clear_error();
-  if (K <= 0 || N <= 0 || K % 128 != 0)
-    return set_error(MTRT_INVALID_ARGUMENT, "fragment order needs positive extents and K %% 128 == 0, got K=%lld N=%lld",
+  if (K <= 0 || N <= 0 || K % 128 != 0 || K > kMaxMatrixExtent || N > kMaxMatrixExtent)
+    return set_error(MTRT_INVALID_ARGUMENT, "fragment order needs positive extents below 2^31 and K %% 128 == 0, got K=%lld N=%lld",
                      (long long)K, (long long)N);
   if (!w || !w_frag)
     return set_error(MTRT_INVALID_ARGUMENT, "null operand");
@@ -588,6 +610,9 @@ int32_t mtrt_hip_gemm_w8a8_fragments(mtrt_stream_t stream, const void *a, const 
   if (M < 0 || K <= 0 || N < 0 || K % 128 != 0)
     return set_error(MTRT_INVALID_ARGUMENT, "fragment-order GEMM needs K %% 128 == 0 and non-negative extents, got M=%lld K=%lld N=%lld",
                      (long long)M, (long long)K, (long long)N);
+  if (M > kMaxMatrixExtent || K > kMaxMatrixExtent || N > kMaxMatrixExtent)
+    return set_error(MTRT_INVALID_ARGUMENT, "matrix extents are limited to 2^31 - 1, got M=%lld K=%lld N=%lld", (long long)M,
+                     (long long)K, (long long)N);
   if (M == 0 || N == 0)
     return MTRT_OK;
   if (!a || !w_frag || !a_scale || !w_scale || !y)
@@ -625,6 +650,9 @@ int32_t mtrt_hip_linear_dense(mtrt_stream_t stream, const void *x, const void *w
   if (M < 0 || K < 0 || N < 0)
     return set_error(MTRT_INVALID_ARGUMENT, "negative extent M=%lld K=%lld N=%lld", (long long)M, (long long)K,
                      (long long)N);
+  if (M > kMaxMatrixExtent || K > kMaxMatrixExtent || N > kMaxMatrixExtent)
+    return set_error(MTRT_INVALID_ARGUMENT, "matrix extents are limited to 2^31 - 1, got M=%lld K=%lld N=%lld", (long long)M,
+                     (long long)K, (long long)N);
   if (M == 0 || N == 0)
     return MTRT_OK;
   if (!y || (K > 0 && (!x || !w_nk)))
@@ -651,7 +679,7 @@ int64_t w4_strip_bytes(int64_t K, int64_t N) { return K % 128 == 0 ? ((N + 15) /
 } // namespace
 
 int64_t mtrt_hip_gemm_w4a16_prepacked_bytes(int64_t K, int64_t N) {
-  if (K <= 0 || N <= 0 || K % 64 != 0)
+  if (K <= 0 || N <= 0 || K % 64 != 0 || K > kMaxMatrixExtent || N > kMaxMatrixExtent)
     return 0;
   return w4_fragment_bytes(K, N) + w4_strip_bytes(K, N);
 }
@@ -659,8 +687,8 @@ int64_t mtrt_hip_gemm_w4a16_prepacked_bytes(int64_t K, int64_t N) {
 int32_t mtrt_hip_gemm_w4a16_prepack(mtrt_stream_t stream, const void *w_kn_packed, void *w_prepacked, int64_t K,
                                     int64_t N) {
   clear_error();
-  if (K <= 0 || N <= 0 || K % 64 != 0)
-    return set_error(MTRT_INVALID_ARGUMENT, "prepack needs positive extents and K %% 64 == 0, got K=%lld N=%lld",
+  if (K <= 0 || N <= 0 || K % 64 != 0 || K > kMaxMatrixExtent || N > kMaxMatrixExtent)
+    return set_error(MTRT_INVALID_ARGUMENT, "prepack needs positive extents below 2^31 and K %% 64 == 0, got K=%lld N=%lld",
                      (long long)K, (long long)N);
   if (!w_kn_packed || !w_prepacked)
     return set_error(MTRT_INVALID_ARGUMENT, "null operand");
@@ -685,6 +713,9 @@ int32_t mtrt_hip_gemm_w4a16(mtrt_stream_t stream, const void *a, const void *w_k
   if (M < 0 || K < 0 || N < 0)
     return set_error(MTRT_INVALID_ARGUMENT, "negative extent M=%lld K=%lld N=%lld", (long long)M, (long long)K,
                      (long long)N);
+  if (M > kMaxMatrixExtent || K > kMaxMatrixExtent || N > kMaxMatrixExtent)
+    return set_error(MTRT_INVALID_ARGUMENT, "matrix extents are limited to 2^31 - 1, got M=%lld K=%lld N=%lld", (long long)M,
+                     (long long)K, (long long)N);
   if (M == 0 || N == 0)
     return MTRT_OK;
   if (block <= 0 || (K > 0 && K % block != 0))

@@ -167,3 +167,19 @@ def test_argument_validation_of_the_newer_entry_points_needs_no_device(pkg):
     assert L.mtrt_hip_gemm_w4a16_prepacked_bytes(100, 64) == 0
     # the allocation-free reduction: its own limit, and it needs the library initialised on the device first
     assert L.mtrt_hip_amax_no_alloc(None, 16, pkg.F32, (1 << 36) + 1, 127.0, 16, 16) == 1 and "allocation-free amax accepts" in err()
+
+
+def test_extents_whose_products_overflow_are_rejected(pkg):
+    """Sizes are formed as products of 64-bit extents; extents that would overflow them are turned away first."""
+    L = pkg.lib()
+    big = 1 << 40
+    assert L.mtrt_hip_quantize(None, 16, pkg.F32, 16, pkg.I8, 16, 0, big, big, 1, 0) == 1 and b"2^35" in L.mtrt_hip_last_error()
+    assert L.mtrt_hip_amax_scales(None, 16, pkg.F32, pkg.SCALE_ROW, big, big, 4, 127.0, 16, 16) == 1
+    assert L.mtrt_hip_softmax(None, 16, 16, pkg.F32, big, big) == 1
+    assert L.mtrt_hip_layernorm(None, 16, 16, 16, 16, pkg.F32, big, big, 1e-5) == 1
+    assert L.mtrt_hip_nvfp4_quantize(None, 16, pkg.F32, 16, 16, 16, big, big, 1) == 1
+    assert L.mtrt_hip_gemm_w8a8(None, 16, 16, 16, 16, 16, 4, 1 << 31, 4) == 1 and b"2^31" in L.mtrt_hip_last_error()
+    assert L.mtrt_hip_gemm_w4a16(None, 16, 16, 16, 16, 16, 1 << 31, 128, 4, 128) == 1
+    assert L.mtrt_hip_linear_dense(None, 16, 16, None, 16, pkg.F16, 4, 4, 1 << 31) == 1
+    assert L.mtrt_hip_gemm_w4a16_prepacked_bytes(1 << 32, 64) == 0
+    assert L.mtrt_hip_gemm_w8a8_fragments_bytes(128, 1 << 31) == 0
