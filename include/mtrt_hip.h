@@ -469,8 +469,10 @@ MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_free_host_pinned(uintptr_t stream, uint
 /* __cuda_memcpy_strided_async_{device2device,device2host,host2device}(stream, rank, elemSize, src, srcOffset,
  * srcShapeAndStrides, dst, dstOffset, dstShapeAndStrides) (CUDAModule.cpp:210-255): shapes then strides, in
  * elements, `rank` values each; the offsets are memref offsets, in ELEMENTS as well (the copy starts at
- * pointer + offset * elemSize, mlir-tensorrt/executor/lib/Support/StridedCopy.cpp:37-38).  Issued as one copy
- * per contiguous run. */
+ * pointer + offset * elemSize, mlir-tensorrt/executor/lib/Support/StridedCopy.cpp:37-38).  When the device can
+ * address both views (device memory, pinned or managed host memory; up to 7 dimensions that are not dense on both
+ * sides) one kernel walks the index space, moving units of up to 16 bytes; otherwise (ordinary host memory on one
+ * side) the copy is issued run by contiguous run.  The reference issues one copy per element (StridedCopy.cpp:57-75). */
 MTRT_CAPI_EXPORTED int32_t mtrt_lua_cuda_memcpy_strided(uintptr_t stream, int64_t rank, int64_t elemSize,
                                                         uintptr_t src, uint64_t srcOffset,
                                                         const int64_t *srcShapeAndStrides, uintptr_t dst,

@@ -476,33 +476,85 @@ int32_t mtrt_lua_cuda_memcpy_strided(uintptr_t stream, int64_t rank, int64_t ele
     return set_error(MTRT_INVALID_ARGUMENT, "src/dst must not be null");
   const int64_t *shape = srcShapeAndStrides, *ss = srcShapeAndStrides + rank, *ds = dstShapeAndStrides + rank;
   int64_t total = 1;
+  bool empty = false;
   for (int64_t i = 0; i < rank; ++i) {
     if (shape[i] != dstShapeAndStrides[i])
       return set_error(MTRT_INVALID_ARGUMENT, "source and destination shapes differ in dimension %lld", (long long)i);
     if (shape[i] < 0)
       return set_error(MTRT_INVALID_ARGUMENT, "negative extent in dimension %lld", (long long)i);
-    total *= shape[i];
+    empty = empty || shape[i] == 0;
+    if (!empty && (__builtin_mul_overflow(total, shape[i], &total) || total >= (int64_t(1) << 48)))
+      return set_error(MTRT_INVALID_ARGUMENT, "shape is too large for one copy");
   }
-  if (total == 0)
+  if (empty)
     return MTRT_OK;
+  if (elemSize > (int64_t(1) << 14))
+    return set_error(MTRT_INVALID_ARGUMENT, "element size %lld out of range", (long long)elemSize);
   // innermost dimensions that are densely packed in BOTH operands form one contiguous run
   int64_t run = 1, inner = rank;
   while (inner > 0 && ss[inner - 1] == run && ds[inner - 1] == run) {
     run *= shape[inner - 1];
     --inner;
   }
-  std::vector<int64_t> idx(size_t(inner), 0);
   // offsets are memref offsets, in ELEMENTS (mlir-tensorrt/executor/lib/Support/StridedCopy.cpp:37-38)
   const char *sbase = reinterpret_cast<const char *>(src) + int64_t(srcOffset) * elemSize;
   char *dbase = reinterpret_cast<char *>(dst) + int64_t(dstOffset) * elemSize;
+  hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+  if (inner == 0) {                                    // dense on both sides: one copy
+    RETURN_IF_RT(hipMemcpyAsync(dbase, sbase, size_t(run * elemSize), hipMemcpyDefault, hs));
+    return MTRT_OK;
+  }
+
+  // Both views in memory the device can address (device memory, pinned or managed host memory): one kernel walks
+  // the index space.  The unit it moves is the largest power of two up to 16 bytes that divides the run, every
+  // outer stride and both base addresses; the units of a run become the innermost dimension.
+  auto device_can_address = [](const void *p) {
+    hipPointerAttribute_t attr;
+    if (hipPointerGetAttributes(&attr, p) != hipSuccess) {
+      (void)hipGetLastError();                           // ordinary host memory: not an error of this call
+      return false;
+    }
+    return attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeHost || attr.type == hipMemoryTypeManaged ||
+           attr.type == hipMemoryTypeUnified;
+  };
+  if (inner <= 7 && device_can_address(sbase) && device_can_address(dbase)) {
+    const int64_t run_bytes = run * elemSize;
+    uint64_t bits = uint64_t(run_bytes) | reinterpret_cast<uintptr_t>(sbase) | reinterpret_cast<uintptr_t>(dbase) | 16u;
+    for (int64_t i = 0; i < inner; ++i)
+      if (shape[i] > 1)
+        bits |= uint64_t(ss[i] * elemSize) | uint64_t(ds[i] * elemSize);
+    const int64_t unit = int64_t(bits & (~bits + 1));     // lowest set bit: 1, 2, 4, 8 or 16
+    struct {
+      int64_t extent[8], src_stride[8], dst_stride[8];
+    } sh = {};
+    int32_t krank = int32_t(inner) + 1;
+    for (int64_t i = 0; i < inner; ++i) {
+      sh.extent[i] = shape[i];
+      sh.src_stride[i] = ss[i] * elemSize;
+      sh.dst_stride[i] = ds[i] * elemSize;
+    }
+    sh.extent[inner] = run_bytes / unit;
+    sh.src_stride[inner] = sh.dst_stride[inner] = unit;
+    int64_t units = total / run * sh.extent[inner];
+    DeviceState *st = device_state();
+    if (!st)
+      return MTRT_RUNTIME_ERROR;
+    const int64_t blocks = std::min<int64_t>((units + 255) / 256, int64_t(num_compute_units(st)) * 32);
+    KernelName name("mtrt_copy_strided_b");
+    name + int(unit);
+    void *args[] = {&sbase, &dbase, &units, &krank, &sh};
+    return launch(st, name, uint32_t(blocks), 256, hs, args);
+  }
+
+  // Ordinary host memory on one side (or more dimensions than the kernel takes): one copy per contiguous run.
+  std::vector<int64_t> idx(size_t(inner), 0);
   for (;;) {
     int64_t so = 0, dof = 0;
     for (int64_t i = 0; i < inner; ++i) {
       so += idx[size_t(i)] * ss[i];
       dof += idx[size_t(i)] * ds[i];
     }
-    RETURN_IF_RT(hipMemcpyAsync(dbase + dof * elemSize, sbase + so * elemSize, size_t(run * elemSize), hipMemcpyDefault,
-                                reinterpret_cast<hipStream_t>(stream)));
+    RETURN_IF_RT(hipMemcpyAsync(dbase + dof * elemSize, sbase + so * elemSize, size_t(run * elemSize), hipMemcpyDefault, hs));
     int64_t d = inner - 1;
     while (d >= 0 && ++idx[size_t(d)] == shape[d])
       idx[size_t(d--)] = 0;

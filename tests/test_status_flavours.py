@@ -264,3 +264,57 @@ def test_builtin_events_pinned_memory_and_strided_copies(pkg):
     assert L.mtrt_lua_cuda_free_host_pinned(stream.value, again.value) == 0
     assert L.mtrt_lua_cuda_stream_sync(stream.value) == 0
     assert L.mtrt_lua_cuda_stream_destroy(stream.value) == 0
+
+
+@pytest.mark.gpu
+def test_strided_copies_between_device_addressable_views(pkg):
+    """Views that the device can address on both sides are copied by one kernel (the reference issues a copy per
+    element from the host, StridedCopy.cpp:57-75); results are those of indexing with the same shapes and strides."""
+    import torch
+    L = pkg.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def copy(src, dst, shape, sstr, dstr, soff=0, doff=0, esize=None):
+        rank = len(shape)
+        s = (ctypes.c_int64 * (2 * rank))(*shape, *sstr)
+        d = (ctypes.c_int64 * (2 * rank))(*shape, *dstr)
+        pkg.check(L.mtrt_lua_cuda_memcpy_strided(stream, rank, esize or src.element_size(), src.data_ptr(), soff, s,
+                                                 dst.data_ptr(), doff, d))
+
+    g = torch.Generator(device="cuda").manual_seed(3)
+    # transpose of a 300 x 500 f32 matrix: no two consecutive elements are contiguous on both sides
+    a = torch.randn(300, 500, device="cuda", generator=g)
+    t = torch.zeros(500, 300, device="cuda")
+    copy(a, t, (500, 300), (1, 500), (300, 1))
+    assert pkg.last_kernel() == "mtrt_copy_strided_b4"
+    assert torch.equal(t, a.t())
+    # rank 3, 2-byte elements, permuted source, destination a window (offset 7 elements) inside a larger buffer
+    b = torch.randn(6, 10, 16, device="cuda", generator=g).to(torch.bfloat16)
+    big = torch.zeros(4096, device="cuda", dtype=torch.bfloat16)
+    copy(b, big, (10, 6, 16), (16, 160, 1), (6 * 20, 20, 1), doff=7)
+    want = torch.zeros_like(big)
+    want[7:7 + 10 * 120].view(10, 6, 20)[:, :, :16] = b.permute(1, 0, 2)
+    assert torch.equal(big.view(torch.int16), want.view(torch.int16))
+    # rows that are contiguous and 16-byte aligned move as 16-byte units; a negative row stride reverses the rows
+    c = torch.arange(64 * 256, device="cuda", dtype=torch.float32).view(64, 256)
+    r = torch.zeros(64, 128, device="cuda")
+    copy(c, r, (64, 128), (-256, 1), (128, 1), soff=63 * 256 + 128)
+    assert pkg.last_kernel() == "mtrt_copy_strided_b16"
+    assert torch.equal(r, c.flip(0)[:, 128:])
+    # 3-byte elements (units of one byte), pinned host source -> device destination with a gap between rows
+    h = torch.arange(5 * 7 * 3, dtype=torch.uint8).pin_memory()
+    d = torch.zeros(5 * 30, dtype=torch.uint8, device="cuda")
+    copy(h, d, (5, 7), (7, 1), (10, 1), esize=3)
+    assert pkg.last_kernel() == "mtrt_copy_strided_b1"
+    torch.cuda.synchronize()
+    want = torch.zeros(5, 30, dtype=torch.uint8)
+    want[:, :21] = h.view(5, 21)
+    assert torch.equal(d.cpu().view(5, 30), want)
+    # ordinary (pageable) host memory on one side still goes run by run through the copy engine
+    ph = np.arange(12, dtype=np.float32).reshape(3, 4)
+    pd = torch.zeros(3, 2, device="cuda")
+    s = (ctypes.c_int64 * 4)(3, 2, 4, 1)
+    dd = (ctypes.c_int64 * 4)(3, 2, 2, 1)
+    pkg.check(L.mtrt_lua_cuda_memcpy_strided(stream, 2, 4, ph.ctypes.data, 1, s, pd.data_ptr(), 0, dd))
+    torch.cuda.synchronize()
+    assert np.array_equal(pd.cpu().numpy(), ph[:, 1:3])
