@@ -220,10 +220,25 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
     v4i a[IT];
     u4 b[JT];
   } f0, f1;
-  auto read_a = [&](FragSet& f, const int8_t* pa, int chunk, int i) {
-    f.a[i] = *reinterpret_cast<const v4i*>(pa + lds_off(wm * (32 * IT) + i * 32 + frow, chunk));
+  // Fragment reads are issued as opaque instructions and waited for by count.  Left to the compiler every
+  // k-step got one s_waitcnt lgkmcnt(0) placed right behind a read that had just been issued (its bookkeeping
+  // of the in-order LDS counter gives up across the loop edge), so each k-step exposed one LDS round trip with
+  // nothing else to issue.  The reads form one stream (chunk c of k-step t reads row tile c of k-step t+1); when
+  // chunk c of k-step t+1 needs its fragment exactly IT - 1 younger reads are outstanding, whatever c is.
+  // Row tile i of a wave sits i * 4096 bytes further; the swizzle depends on the lane and the k chunk only.
+  const uint32_t lds_base = uint32_t(uintptr_t((lds_void_t*)lds));
+  uint32_t a_lane[4];
+#pragma unroll
+  for (int p = 0; p < 4; ++p) a_lane[p] = lds_base + uint32_t(lds_off(wm * (32 * IT) + frow, 2 * p + fhalf));
+  auto read_a = [&](FragSet& f, uint32_t addr, auto tile) {
+    constexpr int I = decltype(tile)::value;
+    __asm__ volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(f.a[I]) : "v"(addr), "n"(I * 4096) : "memory");
   };
-  auto stage = [&](int64_t slice) { return lds + int(uint32_t(slice) % uint32_t(NS)) * S::kStageBytes; };
+  auto landed_a = [&](FragSet& f, int i) {
+    __asm__ volatile("s_waitcnt lgkmcnt(%1)" : "+v"(f.a[i]) : "n"(IT - 1) : "memory");
+  };
+  auto stage_off = [&](int64_t slice) { return uint32_t(uint32_t(slice) % uint32_t(NS)) * uint32_t(S::kStageBytes); };
+  auto stage = [&](int64_t slice) { return lds + stage_off(slice); };
 
   auto prefetch = [&](auto d) {
     constexpr int DD = decltype(d)::value;
@@ -234,8 +249,7 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
   };
   static_for<0, D>(prefetch);                          // register sets are named at compile time
   drain_and_barrier();
-#pragma unroll
-  for (int i = 0; i < IT; ++i) read_a(f0, stage(0), 2 * KH + fhalf, i);
+  static_for<0, IT>([&](auto i) { read_a(f0, a_lane[KH] + stage_off(0), i); });
 #pragma unroll
   for (int j = 0; j < JT; ++j) {
     wr.template half<0, KH>(j, 0, f0.b[j]);
@@ -247,17 +261,18 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
   // fragment read, its share of the 2 * JT halves of the next weights' dequantisation and, in
   // step 0, G/4 direct-to-LDS loads.  Raw nibbles and scales of slice s+2 are fetched in the
   // last step into the register set that the step before finished with.
-  auto kstep = [&](auto par, auto step, const FragSet& cur, FragSet& nxt, const int8_t* ra, int64_t s2, int8_t* nd) {
+  auto kstep = [&](auto par, auto step, FragSet& cur, FragSet& nxt, uint32_t ra, int64_t s2, int8_t* nd) {
     constexpr int PAR = decltype(par)::value, T = decltype(step)::value;
     constexpr bool kLast = T == NK - 1;
     constexpr int NSET = kLast ? (PAR + 1) % D : PAR;  // register set and dword the next k-step's weights come from
     constexpr int NP = kLast ? KH : KH + (T + 1) * KW;
-    const int chunk = 2 * NP + fhalf;
-#pragma unroll
-    for (int c = 0; c < IT; ++c) {
+    const uint32_t raddr = a_lane[NP] + ra;
+    static_for<0, IT>([&](auto cc) {
+      constexpr int c = decltype(cc)::value;
+      landed_a(cur, c);
 #pragma unroll
       for (int j = 0; j < JT; ++j) acc[c][j] = F16Traits::mfma(__builtin_bit_cast(v4i, cur.b[j]), cur.a[c], acc[c][j]);
-      read_a(nxt, ra, chunk, c);
+      read_a(nxt, raddr, cc);
 #pragma unroll
       for (int u = 0; u < 2 * JT; ++u)
         if ((u * IT) / (2 * JT) == c) wr.template half<NSET, NP>(u >> 1, u & 1, nxt.b[u >> 1]);
@@ -271,10 +286,10 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
       }
       if (kLast && c == 0) wr.template fetch<PAR>(s2);
       __builtin_amdgcn_sched_barrier(0);
-    }
+    });
   };
   auto slice_body = [&](auto par, int64_t s) {
-    const int8_t* pa = stage(s);
+    const uint32_t pa = stage_off(s);
     const int64_t s2 = s + D < last ? s + D : last;    // the slice fetched during this one
     int8_t* nd = stage(s + D);
     if (NK == 4) {
@@ -285,9 +300,10 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
       kstep(par, IntC<0>{}, f0, f1, pa, s2, nd);
     }
     // slice s+1 and the registers of slice s+1 have landed; only younger loads may still fly
-    __builtin_amdgcn_s_waitcnt(0x0070 | (kFly & 15) | ((kFly >> 4) << 14));   // vmcnt(kFly) lgkmcnt(0)
+    // (the fragment reads in flight belong to a stage that is not written before the next barrier but one)
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (kFly & 15) | ((kFly >> 4) << 14));   // vmcnt(kFly)
     __asm__ volatile("s_barrier" ::: "memory");
-    kstep(par, IntC<NK - 1>{}, f1, f0, stage(s + 1), s2, nd);
+    kstep(par, IntC<NK - 1>{}, f1, f0, stage_off(s + 1), s2, nd);
   };
 
   int64_t s = 0;
@@ -297,6 +313,9 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
     if (s + decltype(p)::value < slices) slice_body(p, s + decltype(p)::value);
   });
   __builtin_amdgcn_s_waitcnt(0x0070);                  // the surplus loads of the last slices have landed
+  // ... and so have the surplus fragment reads: their registers stay allocated up to here
+#pragma unroll
+  for (int i = 0; i < IT; ++i) __asm__ volatile("s_waitcnt lgkmcnt(0)" ::"v"(f0.a[i]), "v"(f1.a[i]) : "memory");
 
   if (KW == 2) {                                       // second set hands its sums to the first through LDS
     __syncthreads();

@@ -146,10 +146,22 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, int64_t a_row_
     constexpr int SET = decltype(set)::value;
     raw[SET][j][p] = wsrc[j][slice * 256 + p * 64];
   };
-  auto read_a = [&](v4i (&f)[4], const int8_t* pa, int chunk, int i) {
-    f[i] = *reinterpret_cast<const v4i*>(pa + lds_off(wm * 128 + i * 32 + frow, chunk));
+  // Fragment reads are opaque instructions, waited for by count: the reads form one stream (chunk c of a k-step
+  // reads row tile c of the next k-step), so when chunk c needs its fragment exactly three younger reads are
+  // outstanding.  Left to the compiler, every k-step got an s_waitcnt lgkmcnt(0) right behind a read that had
+  // just been issued (one exposed LDS round trip per k-step).  Row tile i sits i * 4096 bytes further; the
+  // swizzle depends on the lane and the k chunk only.
+  const uint32_t lds_base = uint32_t(uintptr_t((lds_void_t*)lds));
+  uint32_t a_lane[4];
+#pragma unroll
+  for (int p = 0; p < 4; ++p) a_lane[p] = lds_base + uint32_t(lds_off(wm * 128 + frow, 2 * p + fhalf));
+  auto read_a = [&](v4i (&f)[4], uint32_t addr, auto tile) {
+    constexpr int I = decltype(tile)::value;
+    __asm__ volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(f[I]) : "v"(addr), "n"(I * 4096) : "memory");
   };
-  auto stage = [&](int64_t slice) { return lds + int(slice & 3) * kStageBytes; };
+  auto landed_a = [&](v4i (&f)[4], int i) { __asm__ volatile("s_waitcnt lgkmcnt(3)" : "+v"(f[i])::"memory"); };
+  auto stage_off = [&](int64_t slice) { return uint32_t(slice & 3) * uint32_t(kStageBytes); };
+  auto stage = [&](int64_t slice) { return lds + stage_off(slice); };
 
   const int64_t one = 1 < last ? 1 : last;
 #pragma unroll
@@ -165,8 +177,10 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, int64_t a_row_
 #pragma unroll
     for (int j = 0; j < JT; ++j) fetch_one(IntC<1>{}, j, one, p);
   drain_and_barrier();
-#pragma unroll
-  for (int i = 0; i < 4; ++i) read_a(fa0, stage(0), fhalf, i);
+  read_a(fa0, a_lane[0] + stage_off(0), IntC<0>{});
+  read_a(fa0, a_lane[0] + stage_off(0), IntC<1>{});
+  read_a(fa0, a_lane[0] + stage_off(0), IntC<2>{});
+  read_a(fa0, a_lane[0] + stage_off(0), IntC<3>{});
 
   // k-step T of slice s (parity PAR): four fenced chunks; chunk c multiplies row tile c by the JT
   // weight fragments of this k-step and carries one A fragment read for the next k-step.  The
@@ -176,25 +190,29 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, int64_t a_row_
   // registers the PREVIOUS k-step finished with: k-step T >= 1 re-fills k-step T-1's registers
   // of this parity for slice s+2, k-step 0 re-fills k-step 3's registers of the other parity for
   // slice s+1.
-  auto kstep = [&](auto par, auto step, const v4i (&cur)[4], v4i (&nxt)[4], const int8_t* ra, int64_t s1, int64_t s2,
-                   int8_t* nd) {
+  auto kstep = [&](auto par, auto step, v4i (&cur)[4], v4i (&nxt)[4], uint32_t ra, int64_t s1, int64_t s2, int8_t* nd) {
     constexpr int PAR = decltype(par)::value, T = decltype(step)::value;
-    const int chunk = 2 * ((T + 1) & 3) + fhalf;
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
+    const uint32_t raddr = a_lane[(T + 1) & 3] + ra;
+    auto chunk = [&](auto cc) {
+      constexpr int c = decltype(cc)::value;
+      landed_a(cur, c);
 #pragma unroll
       for (int j = 0; j < JT; ++j) acc[c][j] = I8Traits::mfma(raw[PAR][j][T], cur[c], acc[c][j]);
-      read_a(nxt, ra, chunk, c);
+      read_a(nxt, raddr, cc);
       if (c == 0) al.dma(s2, nd, T);
       if (c >= 1 && c - 1 < JT) {
         if (T == 0) fetch_one(IntC<PAR ^ 1>{}, c - 1, s1, 3);
         else fetch_one(par, c - 1, s2, T - 1);
       }
       __builtin_amdgcn_sched_barrier(0);
-    }
+    };
+    chunk(IntC<0>{});
+    chunk(IntC<1>{});
+    chunk(IntC<2>{});
+    chunk(IntC<3>{});
   };
   auto slice_body = [&](auto par, int64_t s) {
-    const int8_t* pa = stage(s);
+    const uint32_t pa = stage_off(s);
     const int64_t s1 = s + 1 < last ? s + 1 : last, s2 = s + 2 < last ? s + 2 : last;
     int8_t* nd = stage(s + 2);
     kstep(par, IntC<0>{}, fa0, fa1, pa, s1, s2, nd);
@@ -202,9 +220,10 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, int64_t a_row_
     kstep(par, IntC<2>{}, fa0, fa1, pa, s1, s2, nd);
     // everything issued before this slice has landed (the panel of slice s+1 and its weights for
     // k-steps 0..2); the 3 + 3 * JT loads of this slice's first three k-steps may still fly
-    __builtin_amdgcn_s_waitcnt(0x0070 | (3 + 3 * JT));   // vmcnt(3 + 3 JT) lgkmcnt(0)
+    // (the fragment reads in flight belong to a stage that is not written before the next barrier but one)
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (3 + 3 * JT));   // vmcnt(3 + 3 JT)
     __asm__ volatile("s_barrier" ::: "memory");
-    kstep(par, IntC<3>{}, fa1, fa0, stage(s + 1), s1, s2, nd);
+    kstep(par, IntC<3>{}, fa1, fa0, stage_off(s + 1), s1, s2, nd);
   };
 
   int64_t s = 0;
@@ -214,6 +233,9 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, int64_t a_row_
   }
   if (s < slices) slice_body(IntC<0>{}, s);
   __builtin_amdgcn_s_waitcnt(0x0070);                  // the surplus loads of the last slices have landed
+  // ... and so have the surplus fragment reads: their registers stay allocated up to here
+#pragma unroll
+  for (int i = 0; i < 4; ++i) __asm__ volatile("s_waitcnt lgkmcnt(0)" ::"v"(fa0[i]), "v"(fa1[i]) : "memory");
 
   write_tile<JT, kNWN, kWaves>(acc, epi, y, M, N, m0, n0, lds, slot, true);
 }
