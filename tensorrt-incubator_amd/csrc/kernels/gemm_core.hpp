@@ -93,6 +93,14 @@ struct DmaLoaderT {
   __device__ __forceinline__ void dma(int64_t slice, int8_t* panel, int g) const {
     __builtin_amdgcn_global_load_lds((global_void_t*)(base + slice * BKB + off[g]), (lds_void_t*)(panel + (wave_u * G + g) * 1024), 16, 0, 0);
   }
+  // The same from the slice's (uniform) address: scalar base + 32-bit lane offset in the instruction itself.  The
+  // offset is made opaque at the load so that its widening to 64 bits is not hoisted out of the loop (the load
+  // would then take a vector address pair and one 64-bit vector add per instruction).
+  __device__ __forceinline__ const int8_t* slice_base(uint32_t slice) const { return base + uint64_t(slice) * BKB; }
+  __device__ __forceinline__ void dma_at(const int8_t* sbase, int8_t* panel, int g) {
+    __asm__ volatile("" : "+v"(off[g]));
+    __builtin_amdgcn_global_load_lds((global_void_t*)(sbase + off[g]), (lds_void_t*)(panel + (wave_u * G + g) * 1024), 16, 0, 0);
+  }
 };
 using DmaLoader = DmaLoaderT<8>;
 

@@ -124,26 +124,39 @@ struct PlainEpilogue {
 // D register sets = slices fetched ahead; KEEP: the waves use only part of each vector (see half)
 template <int JT, int D, bool KEEP>
 struct WeightRegs {
-  const uint32_t* wp;
-  const uint16_t* scale;
-  int64_t kblocks, N, tile0;                         // tile0: first 32-column tile of this wave
-  uint32_t slices_per_block;
+  const int8_t* wbase[JT];                           // slice 0 of each of this wave's 32-column tiles (uniform)
+  const int8_t* scale;                               // as bytes (uniform)
+  uint32_t wlane, scol[JT];                          // this lane's byte offsets inside a slice / inside a row of scales
+  int64_t N;
   u4 raw[D][JT];
   uint32_t sc_bits[D][JT];
   uint32_t mask = nibble_pair_mask(), mask_hi = nibble_pair_mask() << 4;
-  template <int SET>
-  __device__ __forceinline__ void fetch(int64_t slice) {
+  // tile0: first 32-column tile of this wave
+  __device__ __forceinline__ void init(const uint32_t* wp, const uint16_t* sc, int64_t kblocks, int64_t n, int64_t tile0) {
     const int lane = threadIdx.x & 63;
-    const int64_t last_tile = (N + 31) / 32 - 1;
-    const int64_t srow = int64_t(uint32_t(slice) / slices_per_block);
+    const int64_t last_tile = (n + 31) / 32 - 1;
+    N = n;
+    scale = reinterpret_cast<const int8_t*>(sc);
+    wlane = uint32_t(lane) * 16;
 #pragma unroll
     for (int j = 0; j < JT; ++j) {
       int64_t tile = tile0 + j;
       tile = tile < last_tile ? tile : last_tile;      // columns past N: some valid data, never stored
       int64_t col = tile * 32 + (lane & 31);
-      col = col < N ? col : N - 1;
-      raw[SET][j] = *reinterpret_cast<const u4*>(wp + ((tile * kblocks + slice) * 64 + lane) * 4);
-      sc_bits[SET][j] = scale[srow * N + col];
+      col = col < n ? col : n - 1;
+      wbase[j] = reinterpret_cast<const int8_t*>(wp) + tile * kblocks * 1024;
+      scol[j] = uint32_t(col) * 2;
+    }
+  }
+  // slice `slice` (its scales in row `srow`): scalar bases, 32-bit lane offsets kept opaque so that the loads take
+  // them as they are (see DmaLoaderT::dma_at)
+  template <int SET>
+  __device__ __forceinline__ void fetch(uint32_t slice, const int8_t* srow_base) {
+#pragma unroll
+    for (int j = 0; j < JT; ++j) {
+      __asm__ volatile("" : "+v"(wlane), "+v"(scol[j]));
+      raw[SET][j] = *reinterpret_cast<const u4*>(wbase[j] + uint64_t(slice) * 1024 + wlane);
+      sc_bits[SET][j] = *reinterpret_cast<const uint16_t*>(srow_base + scol[j]);
     }
   }
   template <int SET, int P>
@@ -192,7 +205,7 @@ __device__ __forceinline__ void static_for(F&& f) {
 
 template <class S, int KH, class Epilogue>
 __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, int64_t a_row_bytes,
-                                                WeightRegs<S::kJT, S::kDepth, (S::kKW > 1)>& wr,
+                                                WeightRegs<S::kJT, S::kDepth, (S::kKW > 1)>& wr, uint32_t slices_per_block,
                                                 Epilogue& epi, uint16_t* __restrict__ y, int64_t M, int64_t N, int64_t slices,
                                                 int64_t m0, int64_t n0, int8_t* lds, int slot) {
   using namespace gemm_core;
@@ -213,9 +226,23 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
 #pragma unroll
     for (int j = 0; j < JT; ++j) acc[i][j] = F16Traits::zero();
 
-  const int64_t last = slices - 1;
+  const uint32_t nslices = uint32_t(slices), last = nslices - 1;
   DmaLoaderT<G> al;
   al.init(a, M, a_row_bytes, m0);
+  // The slice fetched next, its row of scales and its position inside the block; moves on by one per slice until
+  // it reaches the last slice (which is then fetched again into stages and registers that nobody reads).
+  // (plain integer arithmetic instead of selects: it stays on the scalar unit)
+  uint32_t fslice = 0, frem = 0;
+  const int8_t* fsrow = wr.scale;
+  const uint32_t scale_row_bytes = uint32_t(N) * 2;
+  auto advance = [&]() {
+    const uint32_t go = uint32_t(fslice - last) >> 31;                     // fslice < last
+    fslice += go;
+    frem += go;
+    const uint32_t wrap = 1u - (uint32_t(frem - slices_per_block) >> 31);  // frem == slices_per_block (never above)
+    frem &= wrap - 1u;
+    fsrow += wrap * scale_row_bytes;
+  };
   struct FragSet {
     v4i a[IT];
     u4 b[JT];
@@ -237,15 +264,16 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
   auto landed_a = [&](FragSet& f, int i) {
     __asm__ volatile("s_waitcnt lgkmcnt(%1)" : "+v"(f.a[i]) : "n"(IT - 1) : "memory");
   };
-  auto stage_off = [&](int64_t slice) { return uint32_t(uint32_t(slice) % uint32_t(NS)) * uint32_t(S::kStageBytes); };
-  auto stage = [&](int64_t slice) { return lds + stage_off(slice); };
+  auto stage_off = [&](uint32_t slice) { return uint32_t(slice % uint32_t(NS)) * uint32_t(S::kStageBytes); };
+  auto stage = [&](uint32_t slice) { return lds + stage_off(slice); };
 
   auto prefetch = [&](auto d) {
     constexpr int DD = decltype(d)::value;
-    const int64_t sl = DD < last ? DD : last;
+    const int8_t* src = al.slice_base(fslice);
 #pragma unroll
-    for (int g = 0; g < G; ++g) al.dma(sl, stage(DD), g);
-    wr.template fetch<DD>(sl);
+    for (int g = 0; g < G; ++g) al.dma_at(src, stage(DD), g);
+    wr.template fetch<DD>(fslice, fsrow);
+    advance();
   };
   static_for<0, D>(prefetch);                          // register sets are named at compile time
   drain_and_barrier();
@@ -261,7 +289,7 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
   // fragment read, its share of the 2 * JT halves of the next weights' dequantisation and, in
   // step 0, G/4 direct-to-LDS loads.  Raw nibbles and scales of slice s+2 are fetched in the
   // last step into the register set that the step before finished with.
-  auto kstep = [&](auto par, auto step, FragSet& cur, FragSet& nxt, uint32_t ra, int64_t s2, int8_t* nd) {
+  auto kstep = [&](auto par, auto step, FragSet& cur, FragSet& nxt, uint32_t ra, const int8_t* src, int8_t* nd) {
     constexpr int PAR = decltype(par)::value, T = decltype(step)::value;
     constexpr bool kLast = T == NK - 1;
     constexpr int NSET = kLast ? (PAR + 1) % D : PAR;  // register set and dword the next k-step's weights come from
@@ -279,38 +307,39 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
       if (T == 0) {
         if constexpr (G >= IT) {
 #pragma unroll
-          for (int g = 0; g < G / IT; ++g) al.dma(s2, nd, c * (G / IT) + g);
+          for (int g = 0; g < G / IT; ++g) al.dma_at(src, nd, c * (G / IT) + g);
         } else {
-          if (c < G) al.dma(s2, nd, c);
+          if (c < G) al.dma_at(src, nd, c);
         }
       }
-      if (kLast && c == 0) wr.template fetch<PAR>(s2);
+      if (kLast && c == 0) wr.template fetch<PAR>(fslice, fsrow);
       __builtin_amdgcn_sched_barrier(0);
     });
   };
-  auto slice_body = [&](auto par, int64_t s) {
+  auto slice_body = [&](auto par, uint32_t s) {
     const uint32_t pa = stage_off(s);
-    const int64_t s2 = s + D < last ? s + D : last;    // the slice fetched during this one
+    const int8_t* src = al.slice_base(fslice);         // the slice fetched during this one: s + D, or the last
     int8_t* nd = stage(s + D);
     if (NK == 4) {
-      kstep(par, IntC<0>{}, f0, f1, pa, s2, nd);
-      kstep(par, IntC<1>{}, f1, f0, pa, s2, nd);
-      kstep(par, IntC<NK == 4 ? 2 : 0>{}, f0, f1, pa, s2, nd);
+      kstep(par, IntC<0>{}, f0, f1, pa, src, nd);
+      kstep(par, IntC<1>{}, f1, f0, pa, src, nd);
+      kstep(par, IntC<NK == 4 ? 2 : 0>{}, f0, f1, pa, src, nd);
     } else {
-      kstep(par, IntC<0>{}, f0, f1, pa, s2, nd);
+      kstep(par, IntC<0>{}, f0, f1, pa, src, nd);
     }
     // slice s+1 and the registers of slice s+1 have landed; only younger loads may still fly
     // (the fragment reads in flight belong to a stage that is not written before the next barrier but one)
     __builtin_amdgcn_s_waitcnt(0x0F70 | (kFly & 15) | ((kFly >> 4) << 14));   // vmcnt(kFly)
     __asm__ volatile("s_barrier" ::: "memory");
-    kstep(par, IntC<NK - 1>{}, f1, f0, stage_off(s + 1), s2, nd);
+    kstep(par, IntC<NK - 1>{}, f1, f0, stage_off(s + 1), src, nd);
+    advance();
   };
 
-  int64_t s = 0;
-  for (; s + D - 1 < slices; s += D)                   // D slices per trip: one per register set, no branch inside
+  uint32_t s = 0;
+  for (; s + D - 1 < nslices; s += D)                  // D slices per trip: one per register set, no branch inside
     static_for<0, D>([&](auto p) { slice_body(p, s + decltype(p)::value); });
   static_for<0, D - 1>([&](auto p) {
-    if (s + decltype(p)::value < slices) slice_body(p, s + decltype(p)::value);
+    if (s + decltype(p)::value < nslices) slice_body(p, s + decltype(p)::value);
   });
   __builtin_amdgcn_s_waitcnt(0x0070);                  // the surplus loads of the last slices have landed
   // ... and so have the surplus fragment reads: their registers stay allocated up to here
@@ -360,12 +389,12 @@ __device__ __forceinline__ void weight_regs_kernel(const uint16_t* __restrict__ 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int slot = wave % S::kSlots;
   WeightRegs<S::kJT, S::kDepth, (S::kKW > 1)> wr;
-  wr.wp = wp; wr.scale = scale; wr.kblocks = K / BKH; wr.N = N; wr.slices_per_block = uint32_t(block / BKH);
-  wr.tile0 = n0 / 32 + (slot % S::kNWN) * S::kJT;
+  wr.init(wp, scale, K / BKH, N, n0 / 32 + (slot % S::kNWN) * S::kJT);
   PlainEpilogue epi;
   const int8_t* ab = reinterpret_cast<const int8_t*>(a);
-  if (S::kKW == 1 || wave < S::kSlots) run_weight_regs<S, 0>(ab, 2 * K, wr, epi, y, M, N, K / BKH, m0, n0, lds, slot);
-  else run_weight_regs<S, S::kKW - 1>(ab, 2 * K, wr, epi, y, M, N, K / BKH, m0, n0, lds, slot);
+  const uint32_t spb = uint32_t(block / BKH);
+  if (S::kKW == 1 || wave < S::kSlots) run_weight_regs<S, 0>(ab, 2 * K, wr, spb, epi, y, M, N, K / BKH, m0, n0, lds, slot);
+  else run_weight_regs<S, S::kKW - 1>(ab, 2 * K, wr, spb, epi, y, M, N, K / BKH, m0, n0, lds, slot);
 }
 
 // (a [M,K] f16, w_prepacked, scale [K/block, N] f16, y [M,N] f16, M, K, N, block) ; K % 64 == 0, block % 64 == 0,
@@ -395,7 +424,7 @@ extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w4a16_t128x64(
 // activation panel (16 KiB per slice against 2 KiB of weights per 64 columns), and the L1 is what bounds
 // these launches, so the widest tile that still gives every compute unit a workgroup of its own is the
 // fastest.
-using MidWideShape = Shape<1, 4, 1, 2, 4, 5>;          // 128 x 128, 8 waves (two sets of four), four slices ahead
+using MidWideShape = Shape<1, 4, 1, 2, 4, 8>;          // 128 x 128, 8 waves (two sets of four), four slices ahead, ring of eight stages (the stage of a slice is a mask away)
 extern "C" __global__ void __launch_bounds__(512) mtrt_gemm_w4a16_t128x128(
     const uint16_t* __restrict__ a, const uint32_t* __restrict__ wp, const uint16_t* __restrict__ scale,
     uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t block) {
