@@ -130,21 +130,25 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, int64_t a_row_
 #pragma unroll
     for (int j = 0; j < JT; ++j) acc[i][j] = I8Traits::zero();
 
-  const int64_t last = slices - 1;
+  const uint32_t nslices = uint32_t(slices), last = nslices - 1;
   DmaLoaderT<kG> al;
   al.init(a, M, a_row_bytes, m0);
   v4i fa0[4], fa1[4];
   v4i raw[2][JT][4];
-  const v4i* wsrc[JT];                                 // this lane's chunk of slice 0, k-step 0 of each column tile
+  // Every load takes a scalar base and a 32-bit lane offset (kept opaque, so that its widening is not hoisted out
+  // of the loop: the load would then need a vector address pair and a 64-bit vector add of its own).
+  const int8_t* wsrc[JT];                              // slice 0, k-step 0 of each column tile (uniform)
+  uint32_t wlane = uint32_t(lane) * 16;
 #pragma unroll
   for (int j = 0; j < JT; ++j) {
     int64_t tile = n0 / 32 + wn * JT + j;
     tile = tile < ntiles ? tile : ntiles - 1;          // tiles past N: some valid data, never stored
-    wsrc[j] = wfrag + tile * slices * 256 + lane;
+    wsrc[j] = reinterpret_cast<const int8_t*>(wfrag + tile * slices * 256);
   }
-  auto fetch_one = [&](auto set, int j, int64_t slice, int p) {
+  auto fetch_one = [&](auto set, int j, uint32_t slice, int p) {
     constexpr int SET = decltype(set)::value;
-    raw[SET][j][p] = wsrc[j][slice * 256 + p * 64];
+    __asm__ volatile("" : "+v"(wlane));
+    raw[SET][j][p] = *reinterpret_cast<const v4i*>(wsrc[j] + (uint64_t(slice) * 4096 + uint32_t(p) * 1024) + wlane);
   };
   // Fragment reads are opaque instructions, waited for by count: the reads form one stream (chunk c of a k-step
   // reads row tile c of the next k-step), so when chunk c needs its fragment exactly three younger reads are
@@ -160,14 +164,15 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, int64_t a_row_
     __asm__ volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(f[I]) : "v"(addr), "n"(I * 4096) : "memory");
   };
   auto landed_a = [&](v4i (&f)[4], int i) { __asm__ volatile("s_waitcnt lgkmcnt(3)" : "+v"(f[i])::"memory"); };
-  auto stage_off = [&](int64_t slice) { return uint32_t(slice & 3) * uint32_t(kStageBytes); };
-  auto stage = [&](int64_t slice) { return lds + stage_off(slice); };
+  auto stage_off = [&](uint32_t slice) { return uint32_t(slice & 3) * uint32_t(kStageBytes); };
+  auto stage = [&](uint32_t slice) { return lds + stage_off(slice); };
+  auto at_most_last = [&](uint32_t slice) { return slice - ((uint32_t(last - slice) >> 31) * (slice - last)); };  // scalar min
 
-  const int64_t one = 1 < last ? 1 : last;
+  const uint32_t one = at_most_last(1);
 #pragma unroll
-  for (int g = 0; g < kG; ++g) al.dma(0, stage(0), g);
+  for (int g = 0; g < kG; ++g) al.dma_at(al.slice_base(0), stage(0), g);
 #pragma unroll
-  for (int g = 0; g < kG; ++g) al.dma(one, stage(1), g);
+  for (int g = 0; g < kG; ++g) al.dma_at(al.slice_base(one), stage(1), g);
 #pragma unroll
   for (int p = 0; p < 4; ++p)
 #pragma unroll
@@ -190,7 +195,8 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, int64_t a_row_
   // registers the PREVIOUS k-step finished with: k-step T >= 1 re-fills k-step T-1's registers
   // of this parity for slice s+2, k-step 0 re-fills k-step 3's registers of the other parity for
   // slice s+1.
-  auto kstep = [&](auto par, auto step, v4i (&cur)[4], v4i (&nxt)[4], uint32_t ra, int64_t s1, int64_t s2, int8_t* nd) {
+  auto kstep = [&](auto par, auto step, v4i (&cur)[4], v4i (&nxt)[4], uint32_t ra, uint32_t s1, uint32_t s2, const int8_t* src,
+                   int8_t* nd) {
     constexpr int PAR = decltype(par)::value, T = decltype(step)::value;
     const uint32_t raddr = a_lane[(T + 1) & 3] + ra;
     auto chunk = [&](auto cc) {
@@ -199,7 +205,7 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, int64_t a_row_
 #pragma unroll
       for (int j = 0; j < JT; ++j) acc[c][j] = I8Traits::mfma(raw[PAR][j][T], cur[c], acc[c][j]);
       read_a(nxt, raddr, cc);
-      if (c == 0) al.dma(s2, nd, T);
+      if (c == 0) al.dma_at(src, nd, T);
       if (c >= 1 && c - 1 < JT) {
         if (T == 0) fetch_one(IntC<PAR ^ 1>{}, c - 1, s1, 3);
         else fetch_one(par, c - 1, s2, T - 1);
@@ -211,27 +217,28 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, int64_t a_row_
     chunk(IntC<2>{});
     chunk(IntC<3>{});
   };
-  auto slice_body = [&](auto par, int64_t s) {
+  auto slice_body = [&](auto par, uint32_t s) {
     const uint32_t pa = stage_off(s);
-    const int64_t s1 = s + 1 < last ? s + 1 : last, s2 = s + 2 < last ? s + 2 : last;
+    const uint32_t s1 = at_most_last(s + 1), s2 = at_most_last(s + 2);
+    const int8_t* src = al.slice_base(s2);
     int8_t* nd = stage(s + 2);
-    kstep(par, IntC<0>{}, fa0, fa1, pa, s1, s2, nd);
-    kstep(par, IntC<1>{}, fa1, fa0, pa, s1, s2, nd);
-    kstep(par, IntC<2>{}, fa0, fa1, pa, s1, s2, nd);
+    kstep(par, IntC<0>{}, fa0, fa1, pa, s1, s2, src, nd);
+    kstep(par, IntC<1>{}, fa1, fa0, pa, s1, s2, src, nd);
+    kstep(par, IntC<2>{}, fa0, fa1, pa, s1, s2, src, nd);
     // everything issued before this slice has landed (the panel of slice s+1 and its weights for
     // k-steps 0..2); the 3 + 3 * JT loads of this slice's first three k-steps may still fly
     // (the fragment reads in flight belong to a stage that is not written before the next barrier but one)
     __builtin_amdgcn_s_waitcnt(0x0F70 | (3 + 3 * JT));   // vmcnt(3 + 3 JT)
     __asm__ volatile("s_barrier" ::: "memory");
-    kstep(par, IntC<3>{}, fa1, fa0, stage_off(s + 1), s1, s2, nd);
+    kstep(par, IntC<3>{}, fa1, fa0, stage_off(s + 1), s1, s2, src, nd);
   };
 
-  int64_t s = 0;
-  for (; s + 1 < slices; s += 2) {
+  uint32_t s = 0;
+  for (; s + 1 < nslices; s += 2) {
     slice_body(IntC<0>{}, s);
     slice_body(IntC<1>{}, s + 1);
   }
-  if (s < slices) slice_body(IntC<0>{}, s);
+  if (s < nslices) slice_body(IntC<0>{}, s);
   __builtin_amdgcn_s_waitcnt(0x0070);                  // the surplus loads of the last slices have landed
   // ... and so have the surplus fragment reads: their registers stay allocated up to here
 #pragma unroll
