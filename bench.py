@@ -25,6 +25,8 @@ figure is the MEDIAN over ten batches of launches.
 "mfma_sustained" is the matrix-core rate a loop of nothing but MFMAs reaches on the bench's
 own operand data (the published dense peaks hold for idle data only: the clock drops under
 the board's power limit); GEMM entries carry "frac_of_sustained" beside "frac".
+"library_yardsticks" are the vendor library's plain GEMMs (torch.matmul f16, torch._int_mm) at the same shapes,
+timed the same way; they are not part of the step.
 "cpu_baseline" times the CPU oracle (a C++ restatement of the reference's host
 lowering, NOT the reference binary) on a bounded sample, single-threaded like the
 reference interpreter, and extrapolates linearly to the step; "cpu_baseline_all_cores"
@@ -416,6 +418,63 @@ def cache_variants(pkg, torch, wl, which, reps):
     return out
 
 
+def library_yardsticks(torch, which, reps):
+    """The vendor library's plain GEMMs at the benchmark's shapes and on the same kind of data, timed the same way
+    (torch.matmul on f16 operands: the weights already dequantised, so it does less work than the W4A16 cluster;
+    torch._int_mm for int8 x int8 -> int32, without the scale epilogue).  Not part of the step or of `value`: it shows
+    what a tuned library kernel reaches on this chip under the same power limit."""
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev)
+    g.manual_seed(77)
+    out = []
+
+    def timed(fn, n):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        best = None
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(n):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / n
+            best = us if best is None else min(best, us)
+        return best
+
+    if which in ("all", "c5"):
+        K, N, B = 4096, 11008, 128
+        w = torch.randint(-8, 8, (K, N), generator=g, device=dev).half()
+        sc = (torch.rand((K // B, N), generator=g, device=dev) * 0.015 + 0.005).half()
+        wd = (w * sc.repeat_interleave(B, 0)).half()
+        wdt = wd.t().contiguous()
+        del w, sc
+        for M in (16, 256, 4096):
+            a = torch.randn((M, K), generator=g, device=dev).half()
+            y = torch.empty((M, N), dtype=torch.float16, device=dev)
+            n = max(5, reps // (1 if M <= 256 else 4))
+            us = min(timed(lambda: torch.matmul(a, wd, out=y), n), timed(lambda: torch.matmul(a, wdt.t(), out=y), n))
+            out.append(dict(what="torch.matmul f16 (weights dequantised beforehand), better of [K,N] and [N,K] weights",
+                            config="C5 M=%d" % M, us=round(us, 2), achieved=round(2.0 * M * K * N / us / 1e6, 1), unit="TFLOP/s"))
+        del wd, wdt
+    if which in ("all", "c4") and hasattr(torch, "_int_mm"):
+        M, K, N = 2048, 4096, 11008
+
+        def q8(shape):
+            return torch.clamp(torch.round(torch.randn(shape, generator=g, device=dev) * 40.0), -128, 127).to(torch.int8)
+        a, w = q8((M, K)), q8((K, N))
+        wt = w.t().contiguous()
+        try:
+            us = min(timed(lambda: torch._int_mm(a, w), max(5, reps // 4)), timed(lambda: torch._int_mm(a, wt.t()), max(5, reps // 4)))
+            out.append(dict(what="torch._int_mm int8 -> int32 (no scale epilogue, no f16 output), better of [K,N] and [N,K] weights",
+                            config="C4", us=round(us, 2), achieved=round(2.0 * M * K * N / us / 1e6, 1), unit="TOP/s"))
+        except RuntimeError:
+            pass
+    return out
+
+
 def cpu_baseline(which, threads=1):
     """Times the CPU oracle on a bounded sample of each program, with `threads` OpenMP threads (1 = like the
     reference's single-threaded interpreter), and extrapolates linearly to the full configuration; returns
@@ -572,6 +631,10 @@ def main():
     variants = [] if args.no_cache_variants else cache_variants(pkg, torch, wl, args.workload, args.kernel_reps)
     if variants:
         line["cache_variants"] = variants
+    if not args.no_cache_variants:
+        yard = library_yardsticks(torch, args.workload, args.kernel_reps)
+        if yard:
+            line["library_yardsticks"] = yard
     if not args.no_cpu_baseline:
         cpu_s, sample = cpu_baseline(args.workload)
         line["cpu_baseline"] = {"value": round(100.0 * (ideal_us / 1e6) / cpu_s, 6),
