@@ -171,7 +171,7 @@ __device__ __forceinline__ void write_tile(Acc (&acc)[IT][JT], Epilogue& epi, ui
       const u32x4 v = *reinterpret_cast<const u32x4*>(out + lrow * kOutRow + ch * 16);
       if (row < M) {
         if (vec_ok) {
-          if (col < N) *reinterpret_cast<u32x4*>(y + row * N + col) = v;
+          if (col < N) __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(y + row * N + col));
         } else {
 #pragma unroll
           for (int e = 0; e < 8; ++e)
