@@ -140,11 +140,15 @@ __device__ __forceinline__ void write_tile(Acc (&acc)[IT][JT], Epilogue& epi, ui
   if (!active) return;
   int8_t* out = lds + slot * kOutWave;
   const bool vec_ok = (N % 8 == 0) && ((reinterpret_cast<uintptr_t>(y) & 15) == 0);
+  // the whole tile of the workgroup lies inside y (rows of all SLOTS / NWN wave rows, columns of all NWN wave columns)
+  const bool inside = vec_ok && m0 + (SLOTS / NWN) * (32 * IT) <= M && n0 + NWN * WCOLS <= N;
 #pragma unroll
   for (int ib = 0; ib < IT / 4; ++ib)
 #pragma unroll
   for (int half = 0; half < JT / HC; ++half) {
     const int wrow = wm * (32 * IT) + ib * 128;         // first row of this pass inside the workgroup's tile
+    // what the epilogue needs per column (the same for every row of the pass) is fetched once, before the rows
+    epi.template columns<HC>(wn * WCOLS + half * (32 * HC) + fhalf * 4);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int lrow = i * 32 + frow;
@@ -155,7 +159,7 @@ __device__ __forceinline__ void write_tile(Acc (&acc)[IT][JT], Epilogue& epi, ui
         for (int q = 0; q < 4; ++q) {
           const int lcol = jj * 32 + q * 8 + fhalf * 4;  // columns lcol .. lcol+3 of this group <-> r = 4q .. 4q+3
           uint32_t bits[4];
-          epi.convert4(acc[ib * 4 + i][half * HC + jj], q, wn * WCOLS + half * (32 * HC) + lcol, bits);
+          epi.convert4(acc[ib * 4 + i][half * HC + jj], q, jj, bits);
           u32x2 packed;
           packed[0] = bits[0] | (bits[1] << 16);
           packed[1] = bits[2] | (bits[3] << 16);
@@ -163,6 +167,20 @@ __device__ __forceinline__ void write_tile(Acc (&acc)[IT][JT], Epilogue& epi, ui
         }
     }
     // each wave reads back only what it wrote itself: no workgroup barrier needed
+    if (inside) {
+      // every row and column of the tile exists and whole vectors can be stored: no test per store, and the address
+      // moves on by a constant (the general form below costs about ten branches and a 64-bit multiply per store)
+      const int r0 = lane / CHUNKS, ch = lane % CHUNKS;
+      uint16_t* dst = y + (m0 + wrow + r0) * N + (n0 + wn * WCOLS + half * (32 * HC) + ch * 8);
+      const int64_t step = int64_t(64 / CHUNKS) * N;
+#pragma unroll
+      for (int it = 0; it < 128 * CHUNKS / 64; ++it) {
+        const u32x4 v = *reinterpret_cast<const u32x4*>(out + (it * (64 / CHUNKS) + r0) * kOutRow + ch * 16);
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dst));
+        dst += step;
+      }
+      continue;
+    }
 #pragma unroll
     for (int it = 0; it < 128 * CHUNKS / 64; ++it) {
       const int lrow = it * (64 / CHUNKS) + lane / CHUNKS, ch = lane % CHUNKS;
@@ -186,7 +204,8 @@ __device__ __forceinline__ void write_tile(Acc (&acc)[IT][JT], Epilogue& epi, ui
 // 4 waves (2 x 2) compute a 256 x (64 * JT) tile: JT = 4 is the full tile, JT = 2 the half-width
 // tile that fills the last, partial round of a launch.
 // Traits: Acc (16-wide accumulator vector), mfma(first, second, acc), zero().
-// Epilogue: setup(lds scratch, m0, M, n0, N), row(row in tile), convert4(acc, q, col in tile, bits).
+// Epilogue: setup(lds scratch, m0, M, n0, N), columns<HC>(first column of the lane in the tile), row(row in tile),
+// convert4(acc, q, column tile of the pass, bits).
 template <class Traits, int JT, class Epilogue>
 __device__ __forceinline__ void run(const int8_t* __restrict__ a, const int8_t* __restrict__ b, int64_t row_bytes, Epilogue& epi,
                                     uint16_t* __restrict__ y, int64_t M, int64_t N, int64_t slices, int64_t m0,

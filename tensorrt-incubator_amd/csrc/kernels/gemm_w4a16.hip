@@ -102,6 +102,8 @@ struct F16Traits {
 struct PlainEpilogue {
   __device__ __forceinline__ void setup(int8_t*, int64_t, int64_t, int64_t, int64_t) {}
   __device__ __forceinline__ void row(int) {}
+  template <int HC>
+  __device__ __forceinline__ void columns(int) {}
   __device__ __forceinline__ void convert4(const v16f& acc, int q, int, uint32_t (&bits)[4]) const {
 #pragma unroll
     for (int e = 0; e < 4; ++e) bits[e] = f32_to_f16_bits(acc[4 * q + e]);

@@ -47,11 +47,20 @@ struct ScaleEpilogue {
     sw = dst + 256;
   }
   __device__ __forceinline__ void row(int row_in_tile) { as = sa[row_in_tile]; }
-  __device__ __forceinline__ void convert4(const v16i& acc, int q, int col_in_tile, uint32_t (&bits)[4]) const {
-    const f32x4 ws = *reinterpret_cast<const f32x4*>(sw + col_in_tile);
+  // the lane's column scales of one staging pass (HC column tiles of 32, four runs of four columns each), read from LDS
+  // once and kept in registers for the pass's rows
+  template <int HC>
+  __device__ __forceinline__ void columns(int first_col_in_tile) {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) bits[e] = f32_to_f16_bits((float(acc[4 * q + e]) * as) * ws[e]);
+    for (int jj = 0; jj < HC; ++jj)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) wsr[jj][q] = *reinterpret_cast<const f32x4*>(sw + first_col_in_tile + jj * 32 + q * 8);
   }
+  __device__ __forceinline__ void convert4(const v16i& acc, int q, int jj, uint32_t (&bits)[4]) const {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) bits[e] = f32_to_f16_bits((float(acc[4 * q + e]) * as) * wsr[jj][q][e]);
+  }
+  f32x4 wsr[2][4];
 };
 
 // The entry points below have C linkage; they sit inside the namespace only so that
@@ -68,7 +77,7 @@ extern "C" __global__ void __launch_bounds__(gemm_core::THREADS, 1) mtrt_gemm_w8
   __shared__ __attribute__((aligned(16))) int8_t lds[gemm_core::LDS_BYTES];
   const int64_t tiles_m = (M + gemm_core::BM - 1) / gemm_core::BM;
   const int64_t full_blocks = gemm_core::padded_blocks(full_panels, tiles_m);
-  ScaleEpilogue epi{a_scale, w_scale, nullptr, nullptr, 0.0f};
+  ScaleEpilogue epi{a_scale, w_scale, nullptr, nullptr, 0.0f, {}};
   int64_t tile_m, panel;
   if (int64_t(blockIdx.x) < full_blocks) {
     if (!gemm_core::tile_of(blockIdx.x, tiles_m, full_panels, tile_m, panel)) return;
@@ -258,7 +267,7 @@ extern "C" __global__ void __launch_bounds__(frag::kThreads, 1) mtrt_gemm_w8a8_f
   __shared__ __attribute__((aligned(16))) int8_t lds[frag::kLds];
   const int64_t tiles_m = (M + 255) / 256, ntiles = (N + 31) / 32;
   const int64_t full_blocks = gemm_core::padded_blocks(full_panels, tiles_m);
-  ScaleEpilogue epi{a_scale, w_scale, nullptr, nullptr, 0.0f};
+  ScaleEpilogue epi{a_scale, w_scale, nullptr, nullptr, 0.0f, {}};
   int64_t tile_m, panel;
   if (int64_t(blockIdx.x) < full_blocks) {
     if (!gemm_core::tile_of(blockIdx.x, tiles_m, full_panels, tile_m, panel)) return;
