@@ -21,6 +21,9 @@ Every kernel also gets its own line under "workloads" (achieved, peak, fraction)
 timed with HIP events on the launch stream over rotating buffers whose combined
 footprint exceeds the 256 MiB Infinity Cache, so cache hits do not count as HBM; the
 figure is the MEDIAN over ten batches of launches.
+Before the W warm-up steps the step runs `--settle-steps` more times, untimed (default 100, about 70 ms): the
+board's power management takes 10-15 ms of sustained load after an idle period to settle, and the set-up leaves the GPU
+idle; "settle_steps" in the line says how many were run.
 "roofline" repeats the entry of the kernel with the largest share of the step.
 "mfma_sustained" is the matrix-core rate a loop of nothing but MFMAs reaches on the bench's
 own operand data (the published dense peaks hold for idle data only: the clock drops under
@@ -548,6 +551,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="all", choices=["all", "c1", "c2a", "c2b", "c3", "c4", "c5", "nvfp4"])
+    ap.add_argument("--settle-steps", type=int, default=100,
+                    help="untimed steps in front of the warm-up, so that the timed steps run at the settled clocks (0: none)")
     ap.add_argument("--kernel-reps", type=int, default=100, help="launches per kernel for the per-kernel timing")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-cache-variants", action="store_true",
@@ -575,6 +580,13 @@ def main():
         for calls in step_calls:
             calls[k % len(calls)]()
 
+    # Untimed lead-in before the warm-up: after an idle period (the set-up above leaves the GPU idle between its
+    # launches) the board's power management needs some 10-15 ms of sustained load to settle: per-step times of a run
+    # that starts cold read 695 666 675 698 751 778 755 701 709 678 671 668 665 665 ... us, so a window of 20 steps
+    # right after 5 warm-up steps would time that transient, not the step.  The per-kernel figures below are taken in
+    # steady state too (100 launches each, median of ten batches).
+    for k in range(args.settle_steps):
+        run_step(k)
     for k in range(args.warmup):
         run_step(k)
     torch.cuda.synchronize()
@@ -612,7 +624,8 @@ def main():
         "metric": "Q/DQ+reduce HBM GB/s and W8A8/W4A16 GEMM TOPS, as % of MI355X peak, 1 GPU",
         "value": round(value, 2),
         "unit": "% of MI355X peak (time-weighted over the step's kernels)",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "settle_steps": args.settle_steps,
+        "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32 (Q/DQ, LayerNorm, softmax), int8->int32 (W8A8), f16->f32 (W4A16)", "data": "synthetic (seeded)",
         "config": {"workload": {"all": "C1+C2a+C2b+C3+C4+C5 programs of BASELINE.json, one pass each per step"}.get(
