@@ -86,7 +86,7 @@ struct DmaLoaderT {
       const int lrow = (wave_u * G + g) * 8 + (lane >> 3);
       int64_t row = r0 + lrow;
       row = row < rows ? row : rows - 1;               // rows past the edge re-read the last row; never stored
-      off[g] = uint32_t(row * row_bytes + (((lane & 7) ^ ((lrow >> 1) & 7)) << 4));
+      off[g] = uint32_t(row) * uint32_t(row_bytes) + uint32_t(((lane & 7) ^ ((lrow >> 1) & 7)) << 4);   // the operand is below 4 GiB
     }
   }
   // group g (of G) of this wave's share of slice `slice`
@@ -308,11 +308,15 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, const int8_t* 
 // before the next, so a B panel is fetched into one L2 only.  A set of `panels` panels takes
 // padded_blocks(panels, tiles_m) ids; surplus ids get no tile.
 __device__ __host__ __forceinline__ int64_t padded_blocks(int64_t panels, int64_t tiles_m) { return 8 * ((panels + 7) / 8) * tiles_m; }
-__device__ __forceinline__ bool tile_of(int64_t id, int64_t tiles_m, int64_t panels, int64_t& tile_m, int64_t& panel) {
-  const int64_t xcd = id & 7, local = id >> 3;
-  panel = (local / tiles_m) * 8 + xcd;
-  tile_m = local % tiles_m;
-  return panel < panels;
+// (Tile counts fit 32 bits: the index arithmetic is 32-bit on purpose.  As 64-bit divisions, which the hardware does
+// not have, it was some 500 scalar instructions, over a microsecond, in front of the first load of every workgroup.)
+__device__ __forceinline__ bool tile_of(int64_t id64, int64_t tiles_m64, int64_t panels64, int64_t& tile_m, int64_t& panel) {
+  const uint32_t id = uint32_t(id64), tiles_m = uint32_t(tiles_m64), panels = uint32_t(panels64);
+  const uint32_t xcd = id & 7, local = id >> 3;
+  const uint32_t q = local / tiles_m;
+  panel = q * 8 + xcd;
+  tile_m = local - q * tiles_m;
+  return q * 8 + xcd < panels;
 }
 // The same, with the M tiles walked in groups of `group` rows of tiles: an XCD's 32 units then
 // work on `group` M tiles x 32/group panels at a time instead of on all M tiles of a few panels.
@@ -320,13 +324,14 @@ __device__ __forceinline__ bool tile_of(int64_t id, int64_t tiles_m, int64_t pan
 // slice); the group size that minimises it depends on the bytes per row of the two operands
 // (for 4-bit weights under f16 activations a B slice is a quarter of an A slice, so few M tiles and
 // many panels re-read far less).  group >= tiles_m gives tile_of's order.
-__device__ __forceinline__ bool tile_of_grouped(int64_t id, int64_t tiles_m, int64_t panels, int64_t group, int64_t& tile_m,
+__device__ __forceinline__ bool tile_of_grouped(int64_t id64, int64_t tiles_m64, int64_t panels64, int64_t group64, int64_t& tile_m,
                                                 int64_t& panel) {
-  const int64_t xcd = id & 7, local = id >> 3;
-  const int64_t slots = (panels + 7) / 8;                // panel slots of one XCD
-  const int64_t full = tiles_m / group;                  // whole groups; a last group holds the remainder
-  const int64_t per_group = slots * group;
-  int64_t g = local / per_group, r, size;
+  const uint32_t id = uint32_t(id64), tiles_m = uint32_t(tiles_m64), panels = uint32_t(panels64), group = uint32_t(group64);
+  const uint32_t xcd = id & 7, local = id >> 3;
+  const uint32_t slots = (panels + 7) / 8;               // panel slots of one XCD
+  const uint32_t full = tiles_m / group;                 // whole groups; a last group holds the remainder
+  const uint32_t per_group = slots * group;
+  uint32_t g = local / per_group, r, size;
   if (g < full) {
     r = local - g * per_group;
     size = group;
@@ -335,9 +340,10 @@ __device__ __forceinline__ bool tile_of_grouped(int64_t id, int64_t tiles_m, int
     r = local - full * per_group;
     size = tiles_m - full * group;
   }
-  panel = (r / size) * 8 + xcd;
-  tile_m = g * group + r % size;
-  return panel < panels;
+  const uint32_t q = r / size;
+  panel = q * 8 + xcd;
+  tile_m = g * group + (r - q * size);
+  return q * 8 + xcd < panels;
 }
 __device__ __forceinline__ bool tile_origin(int64_t M, int64_t N, int64_t& m0, int64_t& n0) {
   int64_t tile_m, panel;

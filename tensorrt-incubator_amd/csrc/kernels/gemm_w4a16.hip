@@ -223,10 +223,6 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
   const int frow = lane & 31, fhalf = lane >> 5;
 
   v16f acc[IT][JT];
-#pragma unroll
-  for (int i = 0; i < IT; ++i)
-#pragma unroll
-    for (int j = 0; j < JT; ++j) acc[i][j] = F16Traits::zero();
 
   const uint32_t nslices = uint32_t(slices), last = nslices - 1;
   DmaLoaderT<G> al;
@@ -278,7 +274,24 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
     advance();
   };
   static_for<0, D>(prefetch);                          // register sets are named at compile time
-  drain_and_barrier();
+  __builtin_amdgcn_sched_barrier(0);                   // (all of them issued here, none moved behind the barrier)
+  // The accumulators are cleared by the matrix cores themselves (0 x 0 + 0) while the first loads are under way; written
+  // as plain zeros the clearing (one register move per accumulator register) ends up behind the barrier, in front of
+  // the loop, with nothing to overlap.
+  {
+    v4i none = {0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < IT; ++i)
+#pragma unroll
+      for (int j = 0; j < JT; ++j) {
+        __asm__ volatile("" : "+v"(none));             // one MFMA per accumulator, not one result copied around
+        acc[i][j] = F16Traits::mfma(none, none, F16Traits::zero());
+      }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  // slice 0 has landed (the loads of the slices fetched after it may still fly); then meet the other waves
+  __builtin_amdgcn_s_waitcnt(0x0070 | (((D - 1) * (G + 2 * JT)) & 15) | ((((D - 1) * (G + 2 * JT)) >> 4) << 14));
+  __asm__ volatile("s_barrier" ::: "memory");
   static_for<0, IT>([&](auto i) { read_a(f0, a_lane[KH] + stage_off(0), i); });
 #pragma unroll
   for (int j = 0; j < JT; ++j) {

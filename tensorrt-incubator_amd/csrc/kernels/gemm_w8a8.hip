@@ -134,10 +134,6 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, int64_t a_row_
   const int frow = lane & 31, fhalf = lane >> 5;
 
   v16i acc[4][JT];
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int j = 0; j < JT; ++j) acc[i][j] = I8Traits::zero();
 
   const uint32_t nslices = uint32_t(slices), last = nslices - 1;
   DmaLoaderT<kG> al;
@@ -178,19 +174,34 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, int64_t a_row_
   auto at_most_last = [&](uint32_t slice) { return slice - ((uint32_t(last - slice) >> 31) * (slice - last)); };  // scalar min
 
   const uint32_t one = at_most_last(1);
+  // what slice 0 needs first, then slice 1
 #pragma unroll
   for (int g = 0; g < kG; ++g) al.dma_at(al.slice_base(0), stage(0), g);
-#pragma unroll
-  for (int g = 0; g < kG; ++g) al.dma_at(al.slice_base(one), stage(1), g);
 #pragma unroll
   for (int p = 0; p < 4; ++p)
 #pragma unroll
     for (int j = 0; j < JT; ++j) fetch_one(IntC<0>{}, j, 0, p);
 #pragma unroll
+  for (int g = 0; g < kG; ++g) al.dma_at(al.slice_base(one), stage(1), g);
+#pragma unroll
   for (int p = 0; p < 3; ++p)                          // k-step 3 of slice 1 is fetched in k-step 0 of slice 0
 #pragma unroll
     for (int j = 0; j < JT; ++j) fetch_one(IntC<1>{}, j, one, p);
-  drain_and_barrier();
+  __builtin_amdgcn_sched_barrier(0);                   // (all of them issued here, none moved behind the barrier)
+  // The accumulators are cleared by the matrix cores themselves (0 x 0 + 0) while those loads are under way; written as
+  // plain zeros the clearing (one register move per accumulator register) ends up behind the barrier, in front of the loop.
+  {
+    v4i none = {0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < JT; ++j) {
+        __asm__ volatile("" : "+v"(none));             // one MFMA per accumulator, not one result copied around
+        acc[i][j] = I8Traits::mfma(none, none, I8Traits::zero());
+      }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  drain_and_barrier();                                 // (starting on slice 0 while slice 1 is still under way: 3 % slower)
   read_a(fa0, a_lane[0] + stage_off(0), IntC<0>{});
   read_a(fa0, a_lane[0] + stage_off(0), IntC<1>{});
   read_a(fa0, a_lane[0] + stage_off(0), IntC<2>{});
