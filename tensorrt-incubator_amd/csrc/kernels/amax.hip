@@ -108,7 +108,11 @@ __device__ __forceinline__ void amax_body(const typename X::storage* __restrict_
   head = head < n ? head : n;
   const int64_t nvec = (n - head) / A::kPerVec;
   const u32x4* __restrict__ xv = reinterpret_cast<const u32x4*>(x + head);
-  const int64_t per = ((nvec + gridDim.x - 1) / gridDim.x + kStep - 1) / kStep * kStep;   // chunk, whole steps
+  // vectors per workgroup, rounded up; tensors below 2^32 vectors (64 GiB) take the 32-bit division (the 64-bit one is
+  // a hundred scalar instructions in front of the first load)
+  const uint64_t spread = uint64_t(nvec) + gridDim.x - 1;
+  const int64_t share = (spread >> 32) == 0 ? int64_t(uint32_t(spread) / gridDim.x) : int64_t(spread / gridDim.x);
+  const int64_t per = (share + kStep - 1) / kStep * kStep;                                  // chunk, whole steps
   const int64_t c0 = int64_t(blockIdx.x) * per;
   const int64_t c1 = c0 + per < nvec ? c0 + per : nvec;
   uint32_t m = 0;

@@ -782,8 +782,8 @@ __device__ __forceinline__ void strips_chunk(const uint16_t* __restrict__ a, con
 }
 
 // (a [M,K] f16, strip-order weights, scale [K/block, N] f16, y [M,N] f16, M <= 16, K % 128 == 0, N, block % 128 == 0)
-// grid = min(compute units, ceil(N / 16)), block = 256: workgroup g owns the 16-column tiles
-// [g * tiles / grid, (g + 1) * tiles / grid), three at a time.
+// grid = min(compute units, ceil(N / 16)), block = 256: workgroup g owns tiles / grid consecutive 16-column tiles (the first
+// tiles % grid workgroups one more), three at a time.
 // Four waves, one per SIMD.  Measured on M = 16, N = 11008, K = 4096 (rocprofv3 kernel durations): 2 / 4 / 8 waves take
 // 12.7 / 9.6 / 10.7 us; more than one workgroup per compute unit (grids of 344, 512, 688) 11.5-12.6 us.  In-kernel
 // timestamps of the four-wave form: 1.3 us until the loads are issued, first slice landed at 3.9 us, K loop done at
@@ -795,8 +795,11 @@ extern "C" __global__ void __launch_bounds__(64 * kStripWaves) mtrt_gemm_w4a16_s
     const uint16_t* __restrict__ a, const uint32_t* __restrict__ ws, const uint16_t* __restrict__ scale,
     uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t block) {
   __shared__ __attribute__((aligned(16))) int8_t lds[kStripWaves * 4 * 4096];
-  const int64_t tiles = (N + 15) / 16;
-  const int64_t t0 = tiles * blockIdx.x / gridDim.x, t1 = tiles * (int64_t(blockIdx.x) + 1) / gridDim.x;
+  // tiles / grid tiles each, the first tiles % grid workgroups one more (32-bit arithmetic: as 64-bit divisions this was
+  // a microsecond of scalar instructions in front of the first load)
+  const uint32_t tiles = uint32_t((N + 15) / 16), grid = gridDim.x, b = blockIdx.x;
+  const uint32_t per = tiles / grid, rem = tiles - per * grid;
+  const int64_t t0 = int64_t(b * per + (b < rem ? b : rem)), t1 = t0 + per + (b < rem ? 1 : 0);
   for (int64_t t = t0; t < t1; t += 3) {
     const int64_t left = t1 - t;
     if (left >= 3) strips_chunk<kStripWaves, 3>(a, ws, scale, y, M, K, N, block, t, lds);
