@@ -94,11 +94,13 @@ extern "C" __global__ void __launch_bounds__(gemm_core::THREADS, 1) mtrt_gemm_w8
 // are issued only three k-steps before they are needed.  This kernel takes the WEIGHTS from a
 // fragment-order re-layout straight into registers (two register sets, each k-step's registers
 // re-filled seven k-steps before their next use) and leaves LDS to the activations alone: a ring
-// of four 32 KiB stages filled by direct-to-LDS loads two slices ahead.  8 waves (2 x 4, two per
-// SIMD), each 128 rows x 64 columns (JT = 2) or x 32 columns (JT = 1, the half-width tile of a last
-// partial round).
+// of four 32 KiB stages filled by direct-to-LDS loads two slices ahead.  Four waves (2 x 2, one per
+// SIMD), each 128 rows x 128 columns (JT = 4) or x 64 columns (JT = 2, the half-width tile of a last
+// partial round): an activation fragment read from LDS serves four MFMAs.  The loop is written for
+// 2 x NWN waves; with eight (2 x 4, two per SIMD, 128 x 64 each, twice the fragment reads) the launch is
+// 3 % slower on the benchmark's data and 4 % on zero operands, measured in one process.
 //
-// What bounds it (measured on one MI355X at M=2048 K=4096 N=11008, counters per launch):
+// What bounds it (measured on the eight-wave form, one MI355X at M=2048 K=4096 N=11008, counters per launch):
 //   * with every load and LDS read taken out of the loop the launch still needs 164 k cycles per
 //     XCD (ideal for its MFMAs: 98 k), with them 220 k; removing only the LDS reads or only the
 //     barrier changes nothing, removing either operand's loads saves ~13 k, both ~56 k;
@@ -118,16 +120,24 @@ extern "C" __global__ void __launch_bounds__(gemm_core::THREADS, 1) mtrt_gemm_w8
 // contiguous memory.  Columns past N hold zeros.
 namespace frag {
 
-constexpr int kThreads = 512, kWaves = 8, kMW = 2, kNWN = 4;
+constexpr int kMW = 2;                                 // two rows of waves, 128 rows each
 constexpr int kStageBytes = 256 * 128;                 // one slice of the activation panel
-constexpr int kG = 16 * kMW / kWaves;                  // direct-to-LDS loads per wave and slice
-constexpr int kLds = gemm_core::LDS_BYTES_8WAVES;      // output staging of 8 waves; the ring needs 128 KiB
+template <int NWN>
+struct Waves {                                         // kMW x NWN waves
+  static constexpr int kWaves = kMW * NWN, kThreads = 64 * kWaves;
+  static constexpr int kG = 32 / kWaves;               // direct-to-LDS loads per wave and slice
+  static constexpr int kOut = kWaves * gemm_core::kOutWave + 2048;
+  static constexpr int kLds = kOut > 4 * kStageBytes ? kOut : 4 * kStageBytes;   // output staging, or the ring of four stages
+};
 
-template <int JT, class Epilogue>
+template <int NWN, int JT, class Epilogue>
 __device__ __forceinline__ void run(const int8_t* __restrict__ a, int64_t a_row_bytes, const v4i* __restrict__ wfrag,
                                     int64_t ntiles, Epilogue& epi, uint16_t* __restrict__ y, int64_t M, int64_t N,
                                     int64_t slices, int64_t m0, int64_t n0, int8_t* lds) {
   using namespace gemm_core;
+  constexpr int kNWN = NWN, kWaves = Waves<NWN>::kWaves, kG = Waves<NWN>::kG;
+  constexpr int kDmaPerStep = kG / 4;                  // direct-to-LDS loads per wave and k-step
+  static_assert(kG % 4 == 0 && JT <= 4, "loads are dealt to the four chunks of a k-step");
   const int lane = threadIdx.x & 63;
   const int slot = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wm = slot / kNWN, wn = slot % kNWN;
@@ -225,10 +235,11 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, int64_t a_row_
 #pragma unroll
       for (int j = 0; j < JT; ++j) acc[c][j] = I8Traits::mfma(raw[PAR][j][T], cur[c], acc[c][j]);
       read_a(nxt, raddr, cc);
-      if (c == 0) al.dma_at(src, nd, T);
-      if (c >= 1 && c - 1 < JT) {
-        if (T == 0) fetch_one(IntC<PAR ^ 1>{}, c - 1, s1, 3);
-        else fetch_one(par, c - 1, s2, T - 1);
+      if (c % 2 == 0 && c / 2 < kDmaPerStep) al.dma_at(src, nd, T * kDmaPerStep + c / 2);
+      constexpr int j = JT == 4 ? c : c - 1;             // column tile whose weights this chunk fetches
+      if (j >= 0 && j < JT) {
+        if (T == 0) fetch_one(IntC<PAR ^ 1>{}, j, s1, 3);
+        else fetch_one(par, j, s2, T - 1);
       }
       __builtin_amdgcn_sched_barrier(0);
     };
@@ -246,9 +257,10 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, int64_t a_row_
     kstep(par, IntC<1>{}, fa1, fa0, pa, s1, s2, src, nd);
     kstep(par, IntC<2>{}, fa0, fa1, pa, s1, s2, src, nd);
     // everything issued before this slice has landed (the panel of slice s+1 and its weights for
-    // k-steps 0..2); the 3 + 3 * JT loads of this slice's first three k-steps may still fly
+    // k-steps 0..2); the loads of this slice's first three k-steps may still fly
     // (the fragment reads in flight belong to a stage that is not written before the next barrier but one)
-    __builtin_amdgcn_s_waitcnt(0x0F70 | (3 + 3 * JT));   // vmcnt(3 + 3 JT)
+    constexpr int kFly = 3 * kDmaPerStep + 3 * JT;
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (kFly & 15) | ((kFly >> 4) << 14));   // vmcnt(kFly)
     __asm__ volatile("s_barrier" ::: "memory");
     kstep(par, IntC<3>{}, fa1, fa0, stage_off(s + 1), s1, s2, src, nd);
   };
@@ -271,25 +283,32 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, int64_t a_row_
 
 // (a [M,K] i8, w_frag (fragment order), a_scale [M] f32, w_scale [N] f32, y [M,N] f16, M, K, N, full_panels) ;
 // K % 128 == 0, a and w_frag 16-byte aligned, a below 4 GiB.  Tiles and grid as mtrt_gemm_w8a8_nk
-// (256 x 256 for the first full_panels * 256 columns, 256 x 128 after), block = 512.
-extern "C" __global__ void __launch_bounds__(frag::kThreads, 1) mtrt_gemm_w8a8_frag(
-    const int8_t* __restrict__ a, const v4i* __restrict__ w_frag, const float* __restrict__ a_scale,
-    const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t full_panels) {
-  __shared__ __attribute__((aligned(16))) int8_t lds[frag::kLds];
+// (256 x 256 for the first full_panels * 256 columns, 256 x 128 after), block = 64 * 2 * NWN.
+template <int NWN>
+__device__ __forceinline__ void frag_kernel(const int8_t* __restrict__ a, const v4i* __restrict__ w_frag, const float* __restrict__ a_scale,
+                                            const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N,
+                                            int64_t full_panels, int8_t* lds) {
+  constexpr int JT = 8 / NWN;                          // column tiles per wave in a full tile; half of it in a half tile
   const int64_t tiles_m = (M + 255) / 256, ntiles = (N + 31) / 32;
   const int64_t full_blocks = gemm_core::padded_blocks(full_panels, tiles_m);
   ScaleEpilogue epi{a_scale, w_scale, nullptr, nullptr, 0.0f, {}};
   int64_t tile_m, panel;
   if (int64_t(blockIdx.x) < full_blocks) {
     if (!gemm_core::tile_of(blockIdx.x, tiles_m, full_panels, tile_m, panel)) return;
-    frag::run<2>(a, K, w_frag, ntiles, epi, y, M, N, K / 128, tile_m * 256, panel * 256, lds);
+    frag::run<NWN, JT>(a, K, w_frag, ntiles, epi, y, M, N, K / 128, tile_m * 256, panel * 256, lds);
   } else {
     const int64_t n_full = full_panels * 256;
     if (!gemm_core::tile_of(blockIdx.x - full_blocks, tiles_m, (N - n_full + 127) / 128, tile_m, panel)) return;
-    frag::run<1>(a, K, w_frag, ntiles, epi, y, M, N, K / 128, tile_m * 256, n_full + panel * 128, lds);
+    frag::run<NWN, JT / 2>(a, K, w_frag, ntiles, epi, y, M, N, K / 128, tile_m * 256, n_full + panel * 128, lds);
   }
 }
-
+// Four waves, 2 x 2, each 128 rows x 128 columns (one per SIMD): an activation fragment read from LDS serves four MFMAs.
+extern "C" __global__ void __launch_bounds__(frag::Waves<2>::kThreads, 1) mtrt_gemm_w8a8_frag(
+    const int8_t* __restrict__ a, const v4i* __restrict__ w_frag, const float* __restrict__ a_scale,
+    const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t full_panels) {
+  __shared__ __attribute__((aligned(16))) int8_t lds[frag::Waves<2>::kLds];
+  frag_kernel<2>(a, w_frag, a_scale, w_scale, y, M, K, N, full_panels, lds);
+}
 // Weight re-layout into fragment order, from [K,N] (nk = 0) or [N,K] (nk = 1).  One 16-byte chunk per
 // thread.  (w, w_frag, K, N, nk) ; K % 128 == 0 ; w_frag holds 32 * ceil(N/32) * K bytes.
 extern "C" __global__ void __launch_bounds__(256) mtrt_w8_prepack_frag(const int8_t* __restrict__ w, v4i* __restrict__ w_frag,

@@ -638,7 +638,7 @@ int32_t mtrt_hip_gemm_w8a8_fragments(mtrt_stream_t stream, const void *a, const 
   if (grid > int64_t(kMaxGrid) * 1024)
     return set_error(MTRT_INVALID_ARGUMENT, "problem [%lld, %lld] needs too many tiles", (long long)M, (long long)N);
   void *args[] = {&a, &w_frag, &a_scale, &w_scale, &y, &M, &K, &N, &full_panels};
-  return launch(st, KernelName("mtrt_gemm_w8a8_frag"), uint32_t(grid), 512, as_hip(stream), args);
+  return launch(st, KernelName("mtrt_gemm_w8a8_frag"), uint32_t(grid), 256, as_hip(stream), args);
 }
 
 int32_t mtrt_hip_linear_dense(mtrt_stream_t stream, const void *x, const void *w_nk, const void *bias, void *y,
