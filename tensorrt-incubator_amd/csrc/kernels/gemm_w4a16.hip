@@ -343,8 +343,11 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
       kstep(par, IntC<0>{}, f0, f1, pa, src, nd);
     }
     // slice s+1 and the registers of slice s+1 have landed; only younger loads may still fly
-    // (the fragment reads in flight belong to a stage that is not written before the next barrier but one)
-    __builtin_amdgcn_s_waitcnt(0x0F70 | (kFly & 15) | ((kFly >> 4) << 14));   // vmcnt(kFly)
+    // With a ring of at least D + 2 stages the fragment reads in flight belong to a stage that is not written before the
+    // next barrier but one, and they need not be waited for here; with D + 1 stages the stage that the next slice's loads
+    // fill is the one they read, so they are.
+    constexpr int kLgkm = NS >= D + 2 ? 0x0F00 : 0x0000;
+    __builtin_amdgcn_s_waitcnt(0x0070 | kLgkm | (kFly & 15) | ((kFly >> 4) << 14));   // vmcnt(kFly) [lgkmcnt(0)]
     __asm__ volatile("s_barrier" ::: "memory");
     kstep(par, IntC<NK - 1>{}, f1, f0, stage_off(s + 1), src, nd);
     advance();
