@@ -289,8 +289,10 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
       }
     __builtin_amdgcn_sched_barrier(0);
   }
-  // slice 0 has landed (the loads of the slices fetched after it may still fly); then meet the other waves
-  __builtin_amdgcn_s_waitcnt(0x0070 | (((D - 1) * (G + 2 * JT)) & 15) | ((((D - 1) * (G + 2 * JT)) >> 4) << 14));
+  // The activations of slice 0 have landed; then meet the other waves.  Only the direct-to-LDS loads of the later slices
+  // are counted as younger: the compiler may move register loads of the last sets behind this wait (it tracks those
+  // itself), the direct-to-LDS loads stay where they are written, and slice 0's are the oldest of all.
+  __builtin_amdgcn_s_waitcnt(0x0070 | (((D - 1) * G) & 15) | ((((D - 1) * G) >> 4) << 14));
   __asm__ volatile("s_barrier" ::: "memory");
   static_for<0, IT>([&](auto i) { read_a(f0, a_lane[KH] + stage_off(0), i); });
 #pragma unroll
