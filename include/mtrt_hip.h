@@ -308,7 +308,10 @@ MTRT_CAPI_EXPORTED int32_t mtrt_hip_set_wait_limit(int32_t polls);
  * pointer plus (offset, stride0, stride1) in elements, element (r, c) of the [d0, d1] view at
  * base[offset + r * stride0 + c * stride1], which is how the reference hands a dynamic strided memref to a
  * generated kernel (ExpandMemRefArgs.cpp:65-120: base, offset, sizes, strides; order pinned by
- * compiler/test/Passes/1_Core/KernelToCUDA/kernel-to-cuda.mlir:3-48).  Codes are one per byte (MTRT_I8,
+ * compiler/test/Passes/1_Core/KernelToCUDA/kernel-to-cuda.mlir:3-48).  The reference passes only the components
+ * that are dynamic in the memref type (kernel/test/Kernel/Bufferization/expand-memref-args.mlir:1-22: a static
+ * extent, stride or offset is folded into the kernel); the kernels here are the fully dynamic form and take all
+ * of them.  Codes are one per byte (MTRT_I8,
  * MTRT_F8E4M3FN, MTRT_I4); the scale is contiguous and addressed by the logical (r, c) as above.  A view may not
  * reach below its base pointer; that it stays inside the allocation is the caller's responsibility, as it is for
  * generated kernels.  Results equal those of the contiguous entry points on a packed copy of the view. */

@@ -750,17 +750,17 @@ int32_t mtrt_hip_gemm_w4a16(mtrt_stream_t stream, const void *a, const void *w_k
     // from M = 1024 on at N = 11008 they beat the small tiles) and the activations stay inside
     // 32-bit byte offsets; 128 x 64 tiles otherwise.
     const int64_t panels = (N + 255) / 256, tiles_m = (M + 255) / 256;
-    if (panels * tiles_m * 2 >= int64_t(num_compute_units(st)) && M * K * 2 < (int64_t(1) << 32))
-      return launch(st, KernelName("mtrt_gemm_w4a16_t256x256"), uint32_t(8 * ((panels + 7) / 8) * tiles_m), 256, as_hip(stream),
-                    args);
-    if (M * K * 2 < (int64_t(1) << 32)) {
-      // 128-row tiles: 128 columns wide while that leaves every compute unit at most one workgroup, else 64
+    const int64_t big = 8 * ((panels + 7) / 8) * tiles_m;
+    if (panels * tiles_m * 2 >= int64_t(num_compute_units(st)) && M * K * 2 < (int64_t(1) << 32) && big <= int64_t(kMaxGrid) * 1024)
+      return launch(st, KernelName("mtrt_gemm_w4a16_t256x256"), uint32_t(big), 256, as_hip(stream), args);
+    // 128-row tiles: 128 columns wide while that leaves every compute unit at most one workgroup, else 64
+    const int64_t small = 8 * ((((N + 63) / 64) + 7) / 8) * ((M + 127) / 128);
+    if (M * K * 2 < (int64_t(1) << 32) && small <= int64_t(kMaxGrid) * 1024) {
       const int64_t wide_tiles = ((N + 127) / 128) * ((M + 127) / 128);
       if (wide_tiles <= int64_t(num_compute_units(st))) {
         const int64_t wide = 8 * ((((N + 127) / 128) + 7) / 8) * ((M + 127) / 128);
         return launch(st, KernelName("mtrt_gemm_w4a16_t128x128"), uint32_t(wide), 512, as_hip(stream), args);
       }
-      const int64_t small = 8 * ((((N + 63) / 64) + 7) / 8) * ((M + 127) / 128);
       return launch(st, KernelName("mtrt_gemm_w4a16_t128x64"), uint32_t(small), kBlock, as_hip(stream), args);
     }
   }
