@@ -336,7 +336,10 @@ MTRT_CAPI_EXPORTED int32_t mtrt_hip_dequantize_view(mtrt_stream_t stream, const 
  * for f16/bf16 or % 4 for f32), scales [d0/16, d1].  q = f4E2M1FN codes two per byte over the flattened array
  * (element 2i in the low nibble), scales = one f8E4M3FN byte per block, tensor_amax = device pointer to the
  * f32 amax of the whole tensor (mtrt_hip_amax writes it); the second-level scale of the op is
- * tensor_amax / 2688.  x / y: f32, f16 or bf16, 16-byte aligned; q 16-byte aligned; scales 8-byte aligned. */
+ * tensor_amax / 2688.  x / y: f32, f16 or bf16, 16-byte aligned; q 16-byte aligned; scales 8-byte aligned.
+ * NaN elements and all-zero blocks follow the program (code 0).  A tensor_amax below the largest finite |x|
+ * (not what the op computes) lets a block scale exceed the f8 range; the byte stored for such a block is the
+ * hardware conversion's and is not specified here. */
 MTRT_CAPI_EXPORTED int32_t mtrt_hip_nvfp4_quantize(mtrt_stream_t stream, const void *x, int32_t x_dtype,
                                                    void *q_packed, void *scales, const float *tensor_amax,
                                                    int64_t d0, int64_t d1, int32_t block_axis);

@@ -9,7 +9,8 @@
 // Conversions to f4 go through f16, the only f4 truncation the reference defines (RNE, saturation
 // to +-6, inf -> +-6, NaN -> 0: mlir-tensorrt/executor/lib/Passes/ExpandOps.cpp:471-694).  An all-zero
 // block has s8 = 0, S_enc_x = inf and x * S_enc_x = NaN, which that conversion maps to code 0; the
-// same chain is evaluated here, nothing is special-cased.
+// same chain is evaluated here, no block is special-cased.  Only the last step differs by value: the
+// hardware conversion gives a NaN another code than the reference's table, so NaN products take the table.
 //
 // Data movement: as in the quantize/dequantize clusters a lane owns one 128-bit vector of the float
 // operand per trip (4 f32 or 8 f16/bf16), so a block of 16 is held by 4 (or 2) neighbouring lanes
@@ -30,14 +31,6 @@ typedef float f2 __attribute__((ext_vector_type(2)));
 constexpr int kThreads = 256;
 constexpr int kTrips = 8;
 
-// two f32 -> f16 (RNE) -> two f4E2M1FN codes in the low byte.  The hardware conversion is used for
-// ordinary values; NaN (code 0 by the reference's rule) is patched in by the caller per block.
-__device__ __forceinline__ uint32_t f32x2_to_f4(float a, float b) {
-  // f32_to_f16_bits keeps the product's own f32 rounding in front of the f16 rounding (see common.hpp)
-  union { uint32_t u; h2 h; } c;
-  c.u = f32_to_f16_bits(a) | (f32_to_f16_bits(b) << 16);
-  return __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(0u, c.h, 1.0f, 0) & 0xFFu;
-}
 // the reference's table on one f16 bit pattern (exact, slow): used for blocks that contain NaN
 __device__ __forceinline__ uint32_t f16_bits_to_f4_exact(uint32_t h) {
   const uint32_t a = h & 0x7FFFu, sign = (h >> 12) & 8u;
@@ -45,6 +38,71 @@ __device__ __forceinline__ uint32_t f16_bits_to_f4_exact(uint32_t h) {
   const uint32_t code = (a > 0x3400u) + (a >= 0x3A00u) + (a > 0x3D00u) + (a >= 0x3F00u) + (a > 0x4100u) + (a >= 0x4300u) +
                         (a > 0x4500u);
   return code | sign;
+}
+// G products -> G f16 values (RNE), two per word, product k in half k % 2 of word k / 2
+template <int G>
+__device__ __forceinline__ void products_to_f16(float (&w)[G], uint32_t (&h)[G / 2]) {
+#pragma unroll
+  for (int k = 0; k < G; k += 2) {
+    // The empty asm keeps the products' own f32 rounding in front of the f16 rounding (see f32_to_f16_bits in
+    // common.hpp: without it the multiply and the conversion merge into one instruction that rounds once).
+    __asm__("" : "+v"(w[k]), "+v"(w[k + 1]));
+    union { h2 v; uint32_t u; } c;
+    c.v = (h2){(_Float16)w[k], (_Float16)w[k + 1]};
+    h[k / 2] = c.u;
+  }
+}
+// is any of the G values a NaN?  (one unordered compare per pair)
+template <int G>
+__device__ __forceinline__ bool any_nan(const float (&w)[G]) {
+  bool r = false;
+#pragma unroll
+  for (int k = 0; k < G; k += 2) r = r || __builtin_isunordered(w[k], w[k + 1]);
+  return r;
+}
+// G f16 values -> G f4E2M1FN codes, value k in nibble k: the hardware conversion writes one byte of its
+// destination and keeps the others.  Right for ordinary values; NaN (code 0 by the reference's rule) is
+// patched in by the caller per block.
+template <int G>
+__device__ __forceinline__ uint32_t f16_to_f4(const uint32_t (&h)[G / 2]) {
+  union { uint32_t u; h2 v; } c;
+  c.u = h[0];
+  uint32_t codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(0u, c.v, 1.0f, 0);
+  c.u = h[1];
+  codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(codes, c.v, 1.0f, 1);
+  if (G == 8) {
+    c.u = h[2 % (G / 2)];
+    codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(codes, c.v, 1.0f, 2);
+    c.u = h[3 % (G / 2)];
+    codes = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(codes, c.v, 1.0f, 3);
+  }
+  return codes;
+}
+// the reference's table on value k of the packed f16 words
+template <int G>
+__device__ __forceinline__ uint32_t f16_to_f4_exact(const uint32_t (&h)[G / 2], int k) {
+  return f16_bits_to_f4_exact((h[k / 2] >> (16 * (k & 1))) & 0xFFFFu);
+}
+// x / 6 for x >= 0 (a block maximum), correctly rounded, in 5 instructions instead of the 11 of the IEEE divide
+// expansion: q0 = RN(x r), q = RN(q0 + RN(x - 6 q0) r) with r = RN(1/6) (the remainder of a faithful quotient is
+// exact in an FMA; Markstein's correction).  Compared with the IEEE quotient on EVERY non-negative f32 on the
+// CPU: equal for +0 and for all of [2^-125, FLT_MAX]; below (the remainder is no longer exact) and for
+// inf / NaN the lanes take the real divide, in a wave-uniform branch that ordinary data never enters.
+__device__ __forceinline__ float divide_by_six(float x) {
+  const float r = 1.0f / 6.0f;
+  const float q0 = x * r;
+  float q = __builtin_fmaf(__builtin_fmaf(-q0, 6.0f, x), r, q0);
+  // x / 2 is exact, and a positive normal number or +0 exactly where the short form holds: any other class
+  // (0x2BF = all ten classes but those two) takes the divide
+  const bool other = __builtin_amdgcn_classf(x * 0.5f, 0x2BF);
+  if (__builtin_amdgcn_ballot_w64(other) != 0) q = other ? x / 6.0f : q;
+  return q;
+}
+// S_enc / f32(s8) for every scale byte, one IEEE divide per lane of the workgroup (256 lanes): a block's second
+// divide becomes a look-up.  Every lane of the workgroup must get here (there is a barrier inside).
+__device__ __forceinline__ void fill_inverse_scales(float* table, float s_enc) {
+  for (uint32_t b = threadIdx.x; b < 256u; b += blockDim.x) table[b] = s_enc / f8_to_f32<0>(b);
+  __syncthreads();
 }
 
 // (x, q_packed, scales, tensor_amax, nvec) ; nvec 128-bit vectors of x, a multiple of the vectors per block
@@ -61,9 +119,11 @@ __device__ __forceinline__ void quantize_body(const typename X::storage* __restr
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   uint8_t* my_codes = lds + wave * (kSpanCodes + kSpanScales);
   uint8_t* my_scales = my_codes + kSpanCodes;
+  __shared__ float inverse_scale[256];
   const int64_t span = (int64_t(blockIdx.x) * (kThreads / 64) + wave) * (kTrips * 64);   // first vector of this wave
-  if (span >= nvec) return;                            // whole wave
   const float s_enc = 2688.0f / *tensor_amax;
+  fill_inverse_scales(inverse_scale, s_enc);
+  if (span >= nvec) return;                            // whole wave
 
   u32x4 t[kTrips];
 #pragma unroll
@@ -81,23 +141,24 @@ __device__ __forceinline__ void quantize_body(const typename X::storage* __restr
     for (int k = 0; k < G; ++k) amax = fmaxf(amax, fabsf(v[k]));
 #pragma unroll
     for (int off = 1; off < LPB; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off, kWave));
-    const float s_dec_x = amax / 6.0f;
+    const float s_dec_x = divide_by_six(amax);
     uint32_t s8 = f32x2_to_f8_ieee(s_dec_x * s_enc, 0.0f) & 0xFFu;
     s8 = (s8 & 0x7Fu) == 0x7Fu ? 0x7Fu : s8;             // NaN (0 * inf when the tensor amax is 0): 0x7F whatever its sign, as the host class
-    const float s_enc_x = s_enc / f8_to_f32<0>(s8);
+    const float s_enc_x = inverse_scale[s8];             // = s_enc / f32(s8), the same IEEE quotient
     float w[G];
 #pragma unroll
     for (int k = 0; k < G; ++k) w[k] = v[k] * s_enc_x;
-    uint32_t codes = 0;
-#pragma unroll
-    for (int k = 0; k < G; k += 2) codes |= f32x2_to_f4(w[k], w[k + 1]) << (4 * k);
-    // s8 of 0 (or NaN) makes S_enc_x infinite (or NaN) and the products of zeros NaN: those blocks
-    // are converted again by the reference's table (a wave-uniform branch that is rarely taken)
-    const bool special = s8 == 0u || s8 == 0x7Fu;
+    uint32_t h[G / 2];
+    products_to_f16<G>(w, h);
+    uint32_t codes = f16_to_f4<G>(h);
+    // A NaN product (a NaN element; a zero times an infinite S_enc_x, which a scale byte of 0 or a tiny tensor
+    // amax produce; anything times a NaN S_enc_x) has code 0 by the reference's rule, not the hardware's: lanes
+    // that hold one convert again by the reference's table (a wave-uniform branch that is rarely taken)
+    const bool special = any_nan<G>(w);
     if (__builtin_amdgcn_ballot_w64(special) != 0) {
       uint32_t exact = 0;
 #pragma unroll
-      for (int k = 0; k < G; ++k) exact |= f16_bits_to_f4_exact(f32_to_f16_bits(w[k])) << (4 * k);
+      for (int k = 0; k < G; ++k) exact |= f16_to_f4_exact<G>(h, k) << (4 * k);
       codes = special ? exact : codes;
     }
     if (G == 4) *reinterpret_cast<uint16_t*>(my_codes + (j * 64 + lane) * 2) = uint16_t(codes);
@@ -182,11 +243,13 @@ __device__ __forceinline__ void quantize_cols_body(const typename X::storage* __
                                                    uint8_t* __restrict__ scales, const float* __restrict__ tensor_amax,
                                                    int64_t d0, int64_t d1) {
   constexpr int G = FloatGroup<X>::G;
+  __shared__ float inverse_scale[256];
   const int64_t groups = d1 / G, units = (d0 / 16) * groups;
   const int64_t u = int64_t(blockIdx.x) * kThreads + threadIdx.x;
+  const float s_enc = 2688.0f / *tensor_amax;
+  fill_inverse_scales(inverse_scale, s_enc);
   if (u >= units) return;
   const int64_t rb = u / groups, c0 = (u - rb * groups) * G;
-  const float s_enc = 2688.0f / *tensor_amax;
   const typename X::storage* xp = x + rb * 16 * d1 + c0;
   u32x4 t[16];
 #pragma unroll
@@ -203,15 +266,13 @@ __device__ __forceinline__ void quantize_cols_body(const typename X::storage* __
   }
   float s_enc_x[G];
   uint32_t s8[G];
-  bool special = false;
 #pragma unroll
   for (int k = 0; k < G; ++k) {
-    const float s_dec_x = amax[k] / 6.0f;
+    const float s_dec_x = divide_by_six(amax[k]);
     uint32_t b = f32x2_to_f8_ieee(s_dec_x * s_enc, 0.0f) & 0xFFu;
     b = (b & 0x7Fu) == 0x7Fu ? 0x7Fu : b;
     s8[k] = b;
-    special = special || b == 0u || b == 0x7Fu;
-    s_enc_x[k] = s_enc / f8_to_f32<0>(b);
+    s_enc_x[k] = inverse_scale[b];                     // = s_enc / f32(b), the same IEEE quotient
   }
   uint8_t* sp = scales + rb * d1 + c0;
   if (G == 4) {
@@ -221,7 +282,6 @@ __device__ __forceinline__ void quantize_cols_body(const typename X::storage* __
                s8[4 % G] | (s8[5 % G] << 8) | (s8[6 % G] << 16) | (s8[7 % G] << 24)};
     *reinterpret_cast<u32x2*>(sp) = w;
   }
-  const bool any_special = __builtin_amdgcn_ballot_w64(special) != 0;
   uint8_t* qp = q + (rb * 16 * d1 + c0) / 2;
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
@@ -229,18 +289,15 @@ __device__ __forceinline__ void quantize_cols_body(const typename X::storage* __
     FloatGroup<X>::unpack(t[r], v);
 #pragma unroll
     for (int k = 0; k < G; ++k) w[k] = v[k] * s_enc_x[k];
-    uint32_t codes = 0;
-#pragma unroll
-    for (int k = 0; k < G; k += 2) codes |= f32x2_to_f4(w[k], w[k + 1]) << (4 * k);
-    if (any_special) {                                 // columns whose scale byte is 0 or NaN: the exact table
+    uint32_t h[G / 2];
+    products_to_f16<G>(w, h);
+    uint32_t codes = f16_to_f4<G>(h);
+    const bool special = any_nan<G>(w);                // a NaN product: the reference's table (see quantize_body)
+    if (__builtin_amdgcn_ballot_w64(special) != 0) {
       uint32_t exact = 0;
 #pragma unroll
-      for (int k = 0; k < G; ++k) {
-        const bool sk = s8[k] == 0u || s8[k] == 0x7Fu;
-        const uint32_t e = f16_bits_to_f4_exact(f32_to_f16_bits(w[k]));
-        exact |= (sk ? e : ((codes >> (4 * k)) & 0xFu)) << (4 * k);
-      }
-      codes = exact;
+      for (int k = 0; k < G; ++k) exact |= f16_to_f4_exact<G>(h, k) << (4 * k);
+      codes = special ? exact : codes;
     }
     if (G == 4) *reinterpret_cast<uint16_t*>(qp + r * (d1 / 2)) = uint16_t(codes);
     else *reinterpret_cast<uint32_t*>(qp + r * (d1 / 2)) = codes;

@@ -100,6 +100,76 @@ def test_zero_blocks_outliers_and_tiny_blocks(pkg, orc):
     _run(pkg, orc, np.zeros((2, 64), np.float32), "f32")    # amax 0: every scale byte the e4m3 NaN, codes 0
 
 
+def _f8_positive_values():
+    """every finite non-negative f8E4M3FN value (OCP: bias 7, no infinities, 0x7F is NaN)"""
+    out = []
+    for b in range(0x7F):
+        e, m = b >> 3, b & 7
+        out.append(m * 2.0 ** -9 if e == 0 else (1 + m / 8.0) * 2.0 ** (e - 7))
+    return np.array(out, np.float32)
+
+
+def test_block_maxima_whose_sixth_sits_on_a_scale_tie(pkg, orc):
+    """Tensor amax 2688 makes S_enc exactly 1, so a block's scale byte is f8(RN(max / 6)): block maxima are placed so that
+    max / 6 lands on, just below and just above every midpoint between neighbouring f8 values, where one ulp of the
+    quotient changes the byte.  A second tensor walks maxima across 2^-125, where the kernel's short division hands
+    over to the IEEE divide, with a tensor amax small enough that those quotients (f32 denormals) still give ordinary
+    scale bytes."""
+    f8 = _f8_positive_values()
+    mid = (f8[:-1].astype(np.float64) + f8[1:].astype(np.float64)) / 2
+    maxima = []
+    for m in mid:
+        q = np.float32(m)
+        for k in range(-3, 4):
+            t = q
+            for _ in range(abs(k)):
+                t = np.nextafter(t, np.float32(np.inf if k > 0 else 0), dtype=np.float32)
+            x = np.float32(np.float64(t) * 6.0)
+            for j in range(-2, 3):
+                v = x
+                for _ in range(abs(j)):
+                    v = np.nextafter(v, np.float32(np.inf if j > 0 else 0), dtype=np.float32)
+                maxima.append(v)
+    maxima = np.array(maxima, np.float32)
+    maxima = maxima[maxima <= 2688.0]
+    maxima = maxima[:len(maxima) // 8 * 8]              # whole vectors of columns for the second-to-last-axis form
+    x = np.zeros((len(maxima), 16), np.float32)
+    x[:, 0] = maxima
+    x[:, 5] = -maxima / 3
+    for d in ("f32", "f16", "bf16"):       # the 16-bit forms round the maxima first: other quotients, same rule
+        _run(pkg, orc, x, d, amax=2688.0)
+    _run(pkg, orc, x.T.copy().reshape(16, -1), "f32", amax=2688.0, axis=-2)
+
+    g = rng(77)
+    bits = np.concatenate([np.arange(0x00FFFF00, 0x01000100, dtype=np.uint32),                 # across 2^-125
+                           g.integers(0x00000001, 0x03000000, 6000, dtype=np.uint32)])          # denormals to 2^-121
+    tiny = bits.view(np.float32)[:len(bits) // 8 * 8]
+    x = np.zeros((len(tiny), 16), np.float32)
+    x[:, 3] = tiny
+    x[:, 9] = -tiny / 2
+    _run(pkg, orc, x, "f32", amax=float(np.float32(2.0 ** -115)))
+    _run(pkg, orc, x.T.copy().reshape(16, -1), "f32", amax=float(np.float32(2.0 ** -115)), axis=-2)
+
+
+def test_nan_elements_and_an_overflowing_block_scale(pkg, orc):
+    """NaN products take code 0 by the reference's rule wherever they come from: a NaN element of an ordinary block
+    (the block maximum ignores it), and zeros of a block whose S_enc / f32(scale byte) overflows to infinity because
+    the tensor amax is tiny."""
+    g = rng(12)
+    x = g.standard_normal((32, 64)).astype(np.float32)
+    x[2, 5] = np.nan
+    x[2, 40] = -np.nan
+    x[7, 16:32] = np.nan                         # a whole block of NaN: maximum 0, scale byte 0
+    x = np.clip(x, -4.0, 4.0)                    # the tensor amax handed over below bounds every block (NaN stays)
+    for d in ("f32", "f16", "bf16"):
+        _run(pkg, orc, x, d, amax=4.0)
+        _run(pkg, orc, x, d, amax=4.0, axis=-2)
+    z = np.zeros((8, 64), np.float32)
+    z[:, ::7] = (g.standard_normal((8, 10)) * 2.0 ** -118).astype(np.float32)
+    _run(pkg, orc, z, "f32", amax=float(np.float32(2.0 ** -116)))
+    _run(pkg, orc, z.reshape(32, 16), "f32", amax=float(np.float32(2.0 ** -116)), axis=-2)
+
+
 def test_c3_sized_tensor(pkg, orc):
     """bf16 [2048, 8192] (an eighth of BASELINE config 3's tensor, heavy-tail outliers): full bit-exact compare."""
     g = rng(3)
