@@ -146,8 +146,7 @@ __device__ __forceinline__ void dynqdq_body(const typename X::storage* __restric
     if (v < nvec) {
       float f[G];
       FG::unpack(xin[i], f);
-#pragma unroll
-      for (int k = 0; k < G; ++k) f[k] = finish_quotient<Q>(dv.divide(f[k]), flags);
+      quantize_group<Q>(dv, f, flags);
       CodeGroup<Q, G>::store(q, v * G, f, flags);     // leaves f32(code) in f
       if (y) {
 #pragma unroll

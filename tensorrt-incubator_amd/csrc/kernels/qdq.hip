@@ -295,7 +295,39 @@ struct ExactDivisor {
     // has the sign of the true quotient.
     return __builtin_copysignf(q, q0);
   }
+  // The group form of the fast path: quotient, rounding (ROUND) and the target's clamp for G values at once, for
+  // callers that have checked `fast` for the whole wave.  Same values as finish_quotient(divide(x)); the sign of
+  // zero is put back after the clamp (a clamp keeps it), so that the clamp's operands are results of arithmetic
+  // and need no quieting first.
+  template <typename Q, bool ROUND, int G>
+  __device__ __forceinline__ void quantize_fast(float (&v)[G]) const {
+#pragma unroll
+    for (int k = 0; k < G; ++k) {
+      const float xc = fmaxf(fminf(v[k], bound), -bound);
+      const float q0 = xc * r;
+      float q = __builtin_fmaf(__builtin_fmaf(-q0, s, xc), r, q0);
+      q = __builtin_fmaf(__builtin_fmaf(-q, s, xc), r, q);
+      if (ROUND) q = __builtin_rintf(q);
+      q = fmaxf(fminf(q, Codes<Q>::kHi), Codes<Q>::kLo);
+      v[k] = __builtin_copysignf(q, q0);
+    }
+  }
 };
+
+// G values that share one scale -> their clamped (and, where asked for, rounded) quotients.  Both choices, the
+// short division for every lane of the wave or not, and rounding or not, are branches of the whole wave around
+// loops over the group, not selects per element.
+template <typename Q, int G>
+__device__ __forceinline__ void quantize_group(const ExactDivisor& dv, float (&v)[G], int flags) {
+  const bool round = Codes<Q>::kAlwaysRound || (flags & kFlagRoundToInt);
+  if (__builtin_amdgcn_ballot_w64(!dv.fast) == 0) {
+    if (round) dv.template quantize_fast<Q, true>(v);
+    else dv.template quantize_fast<Q, false>(v);
+  } else {
+#pragma unroll
+    for (int k = 0; k < G; ++k) v[k] = finish_quotient<Q>(dv.divide(v[k]), flags);
+  }
+}
 
 enum ScaleKind { kUniform = 0, kRow = 1, kCol = 2 };
 
@@ -366,8 +398,7 @@ __device__ __forceinline__ void qdq_groups(const typename X::storage* __restrict
         } else {
           // one scale for the whole group: exact division through its reciprocal
           const ExactDivisor dv(s[j][0]);
-#pragma unroll
-          for (int k = 0; k < G; ++k) v[j][k] = finish_quotient<Q>(dv.divide(v[j][k]), flags);
+          quantize_group<Q>(dv, v[j], flags);
         }
         CG::store(q, e, v[j], flags);
       }
