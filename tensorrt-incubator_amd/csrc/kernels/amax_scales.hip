@@ -126,6 +126,60 @@ __device__ __forceinline__ void cols_body(const typename X::storage* __restrict_
   }
 }
 
+// col kind, few long blocks (per-channel scales of a [K, N] weight: ONE block of all K rows): the rows of a block are
+// dealt to `parts` workgroups, rows [part * rows_per_part, ...), whose column maxima meet in `stage` (one word per
+// scale element, zero on entry) through atomic max on the bit patterns; mtrt_amax_finish_* turns the words into
+// amax and scale afterwards.  Without the split such a tensor has ceil(d1 / G / 64) workgroups in all.
+template <typename X>
+__device__ __forceinline__ void cols_split_body(const typename X::storage* __restrict__ x, int64_t d0, int64_t d1, int64_t nb,
+                                                int64_t rows_per_part, uint32_t* __restrict__ stage) {
+  using E = AbsEach<X>;
+  constexpr int G = E::G;
+  __shared__ uint32_t part_max[4][kWave][G + 1];
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int64_t nvec = d1 / G, strips = (nvec + kWave - 1) / kWave, parts = (nb + rows_per_part - 1) / rows_per_part;
+  const int64_t part = blockIdx.x % parts, rest = blockIdx.x / parts;
+  const int64_t b = rest / strips, strip = rest % strips;
+  const int64_t vcol = strip * kWave + lane;
+  const int64_t r0 = part * rows_per_part, r1 = r0 + rows_per_part < nb ? r0 + rows_per_part : nb;
+  uint32_t m[G];
+#pragma unroll
+  for (int k = 0; k < G; ++k) m[k] = 0;
+  if (vcol < nvec) {
+    const u32x4* pv = reinterpret_cast<const u32x4*>(x + (b * nb) * d1) + vcol;
+    int64_t r = r0 + wave;
+    for (; r + 12 < r1; r += 16) {                     // four independent loads in flight
+      u32x4 t[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) t[u] = __builtin_nontemporal_load(pv + (r + 4 * u) * nvec);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) E::acc(t[u], m);
+    }
+    for (; r < r1; r += 4) E::acc(__builtin_nontemporal_load(pv + r * nvec), m);
+  }
+#pragma unroll
+  for (int k = 0; k < G; ++k) part_max[wave][lane][k] = m[k];
+  __syncthreads();
+  if (wave == 0 && vcol < nvec) {
+#pragma unroll
+    for (int k = 0; k < G; ++k) {
+      uint32_t r = part_max[0][lane][k];
+#pragma unroll
+      for (int w = 1; w < 4; ++w) r = r > part_max[w][lane][k] ? r : part_max[w][lane][k];
+      // nobody reads the word before the launch has ended: no ordering, no return value
+      __hip_atomic_fetch_max(stage + b * d1 + vcol * G + k, r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+}
+
+// stage word (maximum bit pattern) -> amax and scale; `stage` may be amax_out or scale_out itself
+template <typename X>
+__device__ __forceinline__ void finish_body(const uint32_t* stage, int64_t count, float qmax, float* amax_out, float* scale_out) {
+  const int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  emit(AbsBits<X>::finish(stage[i]), qmax, amax_out, scale_out, i);
+}
+
 // col kind, any shape: one lane per (block, column)
 template <typename X>
 __device__ __forceinline__ void cols_any_body(const typename X::storage* __restrict__ x, int64_t d0, int64_t d1, int64_t nb,
@@ -146,6 +200,9 @@ __device__ __forceinline__ void cols_any_body(const typename X::storage* __restr
 //   rows / rows_any : grid = ceil(nb / 4), block = 256 (one wave per scale)
 //   cols            : grid = (d0 / nb) * ceil(d1 / G / 64), block = 256 ; d1 % G == 0, x 16-byte aligned
 //   cols_any        : grid-stride, block = 256
+// (x, d0, d1, nb, rows_per_part, stage) cols_split : grid = (d0 / nb) * ceil(d1 / G / 64) * ceil(nb / rows_per_part),
+//   block = 256 ; stage = (d0 / nb) * d1 zeroed words ; then (stage, count, qmax, amax_out or null, scale_out or null)
+//   finish : grid = ceil(count / 256), block = 256
 #define MTRT_AMAX_SCALES_KERNELS(XN, XT)                                                                              \
   extern "C" __global__ void __launch_bounds__(256) mtrt_amax_rows_##XN(                                               \
       const XT::storage* x, int64_t d0, int64_t d1, int64_t nb, float qmax, float* amax_out, float* scale_out) {       \
@@ -156,6 +213,12 @@ __device__ __forceinline__ void cols_any_body(const typename X::storage* __restr
   extern "C" __global__ void __launch_bounds__(256) mtrt_amax_cols_##XN(                                               \
       const XT::storage* x, int64_t d0, int64_t d1, int64_t nb, float qmax, float* amax_out, float* scale_out) {       \
     amax_scales_cluster::cols_body<XT>(x, d0, d1, nb, qmax, amax_out, scale_out); }                                    \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_amax_cols_split_##XN(                                         \
+      const XT::storage* x, int64_t d0, int64_t d1, int64_t nb, int64_t rows_per_part, uint32_t* stage) {              \
+    amax_scales_cluster::cols_split_body<XT>(x, d0, d1, nb, rows_per_part, stage); }                                   \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_amax_finish_##XN(                                             \
+      const uint32_t* stage, int64_t count, float qmax, float* amax_out, float* scale_out) {                           \
+    amax_scales_cluster::finish_body<XT>(stage, count, qmax, amax_out, scale_out); }                                   \
   extern "C" __global__ void __launch_bounds__(256) mtrt_amax_cols_any_##XN(                                           \
       const XT::storage* x, int64_t d0, int64_t d1, int64_t nb, float qmax, float* amax_out, float* scale_out) {       \
     amax_scales_cluster::cols_any_body<XT>(x, d0, d1, nb, qmax, amax_out, scale_out); }

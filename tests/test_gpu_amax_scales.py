@@ -69,6 +69,35 @@ def test_every_addressing_on_ragged_shapes(pkg, orc, xname):
         _run(pkg, orc, x, xname, kind, d0, d1, nb, 448.0, kernel)
 
 
+@pytest.mark.parametrize("xname", ["f32", "f16", "bf16"])
+def test_per_channel_scales_of_a_k_by_n_weight(pkg, orc, xname):
+    """Few, long column blocks (per-output-channel scales of a [K, N] weight, nb = K): the rows of a block are dealt
+    to several workgroups that meet by atomic max, then a finishing launch writes amax and scale.  Full-size config-4
+    weight, a block length that is not a multiple of the part length, two blocks, and only one of the two outputs."""
+    import torch
+    grp = 4 if xname == "f32" else 8
+    g = rng(23)
+    orc.set_threads(16)
+    try:
+        cases = [(4096, 11008, 4096), (1000, grp * 33, 1000), (512, grp * 70, 256), (130, grp * 3, 130)]
+        for d0, d1, nb in cases:
+            x = (g.standard_normal(d0 * d1) * 0.3).astype(np.float32)
+            x[g.integers(0, x.size, 50)] *= 40.0
+            xd, scale, s_ref, xs = _run(pkg, orc, x, xname, "col", d0, d1, nb, 127.0, "mtrt_amax_finish_" + xname)
+        # the scales alone (amax_out NULL), then the amax alone: the words the workgroups meet in are the output's own
+        px = {"f32": pkg.F32, "f16": pkg.F16, "bf16": pkg.BF16}[xname]
+        L = pkg.lib()
+        st = torch.cuda.current_stream().cuda_stream
+        only = torch.full((d1,), 7.0, dtype=torch.float32, device="cuda")
+        pkg.check(L.mtrt_hip_amax_scales(st, xd.data_ptr(), px, pkg.SCALE_COL, d0, d1, nb, 127.0, None, only.data_ptr()))
+        assert np.array_equal(f32_bits(only.cpu().numpy()), f32_bits(s_ref))
+        pkg.check(L.mtrt_hip_amax_scales(st, xd.data_ptr(), px, pkg.SCALE_COL, d0, d1, nb, 127.0, only.data_ptr(), None))
+        a_ref, _ = orc.amax_scales(xs, {"f32": orc.F32, "f16": orc.F16, "bf16": orc.BF16}[xname], orc.SCALE_COL, d0, d1, nb, 127.0)
+        assert np.array_equal(f32_bits(only.cpu().numpy()), f32_bits(a_ref))
+    finally:
+        orc.set_threads(1)
+
+
 def test_argument_checks_and_empty(pkg):
     import torch
     L = pkg.lib()
