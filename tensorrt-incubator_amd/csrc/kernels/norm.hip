@@ -15,9 +15,10 @@
 // read from HBM exactly once: ONE WAVE OWNS ONE ROW, the row lives in that wave's
 // registers (NV 128-bit vectors per lane, lane l holding vectors l, l+64, ...: every
 // load instruction of the wave covers 1 KiB of contiguous HBM), and both row
-// reductions are cross-lane exchanges with no LDS and no barrier.  Rows that do not
-// fit that scheme (D not a multiple of the vector width, or D > 64*16 vectors) use
-// the workgroup-per-row "_any" kernels, which re-read the row from cache.
+// reductions are cross-lane exchanges with no LDS and no barrier.  Longer rows (up to
+// 1024 * 16 vectors) are owned by a workgroup in the same way ("_g" kernels); rows that
+// fit neither scheme (D not a multiple of the vector width, or longer still) use the
+// workgroup-per-row "_any" kernels, which re-read the row from cache.
 //
 // All arithmetic is f32 with the operation order above; reductions are trees
 // rather than the host's left-to-right sums, which the float tolerance covers.
@@ -228,6 +229,167 @@ __device__ __forceinline__ void softmax_rows(const typename X::storage* __restri
     softmax_row<X, NV, false>(x, y, row, d);
 }
 
+// ---- rows longer than one wave's registers: one WORKGROUP owns one row ---------------------------
+// THREADS lanes (256 or 1024) hold the row, NV vectors each (lane l the vectors l, l + THREADS, ...), in storage
+// form; the row reductions are a cross-lane exchange per wave and a meeting of the waves' values in LDS.  The row
+// is still read from HBM exactly once.  Covers 64 * 16 < D / E <= 1024 * 16 vectors (hidden sizes above 8192,
+// vocabulary-sized softmax rows).
+template <int THREADS, typename Op>
+__device__ __forceinline__ float group_reduce(float v, Op op, float* lds) {
+  v = wave_reduce(v, op);
+  __syncthreads();                                   // lds may still be read from the previous reduction
+  if ((threadIdx.x & (kWave - 1)) == 0) lds[threadIdx.x / kWave] = v;
+  __syncthreads();
+  float r = lds[0];
+#pragma unroll
+  for (int w = 1; w < THREADS / kWave; ++w) r = op(r, lds[w]);
+  return r;                                          // the same value, combined in the same order, in every lane
+}
+
+template <typename X, int NV, int THREADS, bool FULL>
+__device__ __forceinline__ void layernorm_group_row(const typename X::storage* __restrict__ x,
+                                                    const typename X::storage* __restrict__ gamma,
+                                                    const typename X::storage* __restrict__ beta,
+                                                    typename X::storage* __restrict__ y, int64_t row, int64_t d, float eps,
+                                                    float* lds) {
+  constexpr int E = Vec<X>::kElems;
+  const int nvec = int(d / E);
+  const u32x4* xr = reinterpret_cast<const u32x4*>(x + row * d);
+  u32x4 t[NV];
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int idx = int(threadIdx.x) + THREADS * j;
+    t[j] = __builtin_nontemporal_load(xr + (FULL ? idx : min(idx, nvec - 1)));
+  }
+  const float fd = float(d);
+  float sum = 0.0f;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const bool live = FULL || int(threadIdx.x) + THREADS * j < nvec;
+    float v[E];
+    Vec<X>::unpack(t[j], v);
+#pragma unroll
+    for (int k = 0; k < E; ++k) sum = sum + (live ? v[k] : 0.0f);
+  }
+  const float mu = group_reduce<THREADS>(sum, SumF32(), lds) / fd;
+  float sq = 0.0f;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const bool live = FULL || int(threadIdx.x) + THREADS * j < nvec;
+    float v[E];
+    opaque(t[j]);                                    // widen again instead of keeping pass 1's values live
+    Vec<X>::unpack(t[j], v);
+#pragma unroll
+    for (int k = 0; k < E; ++k) {
+      const float dv = v[k] - mu;
+      sq = sq + (live ? dv * dv : 0.0f);
+    }
+  }
+  const float var = group_reduce<THREADS>(sq, SumF32(), lds) / fd;
+  const float rstd = 1.0f / sqrtf(var + eps);
+  const u32x4* gv = reinterpret_cast<const u32x4*>(gamma);
+  const u32x4* bv = reinterpret_cast<const u32x4*>(beta);
+  u32x4* yr = reinterpret_cast<u32x4*>(y + row * d);
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int idx = int(threadIdx.x) + THREADS * j;
+    const int idc = FULL ? idx : min(idx, nvec - 1);
+    float v[E], g[E], b[E], o[E];
+    opaque(t[j]);
+    Vec<X>::unpack(t[j], v);
+    Vec<X>::unpack(gv[idc], g);
+    Vec<X>::unpack(bv[idc], b);
+#pragma unroll
+    for (int k = 0; k < E; ++k) o[k] = (((v[k] - mu) * rstd) * g[k]) + b[k];
+    if (FULL || idx < nvec) __builtin_nontemporal_store(Vec<X>::pack(o), yr + idx);
+  }
+}
+
+template <typename X, int NV, int THREADS>
+__device__ __forceinline__ void layernorm_group(const typename X::storage* __restrict__ x,
+                                                const typename X::storage* __restrict__ gamma,
+                                                const typename X::storage* __restrict__ beta,
+                                                typename X::storage* __restrict__ y, int64_t rows, int64_t d, float eps) {
+  __shared__ float lds[THREADS / kWave];
+  const int64_t row = blockIdx.x;                    // grid = rows
+  if (d == int64_t(Vec<X>::kElems) * THREADS * NV)
+    layernorm_group_row<X, NV, THREADS, true>(x, gamma, beta, y, row, d, eps, lds);
+  else
+    layernorm_group_row<X, NV, THREADS, false>(x, gamma, beta, y, row, d, eps, lds);
+}
+
+// KEEP: the exponentials stay in registers (f32) between the sum and the output pass; without it they are
+// computed again from the stored row (the 1024-lane form has 128 registers per lane, not enough for both).
+template <typename X, int NV, int THREADS, bool FULL, bool KEEP>
+__device__ __forceinline__ void softmax_group_row(const typename X::storage* __restrict__ x, typename X::storage* __restrict__ y,
+                                                  int64_t row, int64_t d, float* lds) {
+  constexpr int E = Vec<X>::kElems;
+  const int nvec = int(d / E);
+  const u32x4* xr = reinterpret_cast<const u32x4*>(x + row * d);
+  u32x4 t[NV];
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int idx = int(threadIdx.x) + THREADS * j;
+    t[j] = __builtin_nontemporal_load(xr + (FULL ? idx : min(idx, nvec - 1)));
+  }
+  float mx = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const bool live = FULL || int(threadIdx.x) + THREADS * j < nvec;
+    float v[E];
+    Vec<X>::unpack(t[j], v);
+#pragma unroll
+    for (int k = 0; k < E; ++k) mx = fmaxf(mx, live ? v[k] : -INFINITY);
+  }
+  mx = group_reduce<THREADS>(mx, MaxF32(), lds);
+  float e[KEEP ? NV * E : 1];
+  float s = 0.0f;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const bool live = FULL || int(threadIdx.x) + THREADS * j < nvec;
+    float v[E];
+    opaque(t[j]);
+    Vec<X>::unpack(t[j], v);
+#pragma unroll
+    for (int k = 0; k < E; ++k) {
+      const float ev = live ? __expf(v[k] - mx) : 0.0f;
+      if (KEEP) e[j * E + k] = ev;
+      s = s + ev;
+    }
+  }
+  s = group_reduce<THREADS>(s, SumF32(), lds);
+  const float inv = 1.0f / s;                         // e * (1/s), as in softmax_row
+  u32x4* yr = reinterpret_cast<u32x4*>(y + row * d);
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int idx = int(threadIdx.x) + THREADS * j;
+    float o[E];
+    if (KEEP) {
+#pragma unroll
+      for (int k = 0; k < E; ++k) o[k] = e[j * E + k] * inv;
+    } else {
+      float v[E];
+      opaque(t[j]);
+      Vec<X>::unpack(t[j], v);
+#pragma unroll
+      for (int k = 0; k < E; ++k) o[k] = __expf(v[k] - mx) * inv;
+    }
+    if (FULL || idx < nvec) __builtin_nontemporal_store(Vec<X>::pack(o), yr + idx);
+  }
+}
+
+template <typename X, int NV, int THREADS>
+__device__ __forceinline__ void softmax_group(const typename X::storage* __restrict__ x, typename X::storage* __restrict__ y,
+                                              int64_t rows, int64_t d) {
+  __shared__ float lds[THREADS / kWave];
+  constexpr bool kKeep = THREADS <= 256;
+  const int64_t row = blockIdx.x;                    // grid = rows
+  if (d == int64_t(Vec<X>::kElems) * THREADS * NV)
+    softmax_group_row<X, NV, THREADS, true, kKeep>(x, y, row, d, lds);
+  else
+    softmax_group_row<X, NV, THREADS, false, kKeep>(x, y, row, d, lds);
+}
+
 // ---- any D, any alignment: one workgroup per row, row re-read from cache -------------
 template <typename Op>
 __device__ __forceinline__ float block_reduce(float v, Op op, float* lds) {
@@ -318,6 +480,21 @@ using namespace norm_cluster;
   extern "C" __global__ void __launch_bounds__(kNormThreads) mtrt_softmax_##XN##_any(                          \
       const XT::storage* x, XT::storage* y, int64_t rows, int64_t d) { softmax_any<XT>(x, y, rows, d); }
 
+// One workgroup per row: mtrt_layernorm_<t>_g<THREADS>v<NV>(x, gamma, beta, y, rows, d, eps), mtrt_softmax_<t>_g<THREADS>v<NV>(x, y, rows, d)
+//   grid = rows, block = THREADS; d % E == 0, d / E <= THREADS * NV, operands 16-byte aligned.
+#define MTRT_NORM_GROUP_KERNELS(XN, XT, NV, THREADS)                                                           \
+  extern "C" __global__ void __launch_bounds__(THREADS) mtrt_layernorm_##XN##_g##THREADS##v##NV(               \
+      const XT::storage* x, const XT::storage* gamma, const XT::storage* beta, XT::storage* y, int64_t rows,  \
+      int64_t d, float eps) { layernorm_group<XT, NV, THREADS>(x, gamma, beta, y, rows, d, eps); }            \
+  extern "C" __global__ void __launch_bounds__(THREADS) mtrt_softmax_##XN##_g##THREADS##v##NV(                 \
+      const XT::storage* x, XT::storage* y, int64_t rows, int64_t d) { softmax_group<XT, NV, THREADS>(x, y, rows, d); }
+#define MTRT_NORM_GROUPS_FOR_TYPE(XN, XT)                                                                      \
+  MTRT_NORM_GROUP_KERNELS(XN, XT, 8, 256) MTRT_NORM_GROUP_KERNELS(XN, XT, 16, 256)                             \
+  MTRT_NORM_GROUP_KERNELS(XN, XT, 8, 1024) MTRT_NORM_GROUP_KERNELS(XN, XT, 16, 1024)
+
 MTRT_NORM_FOR_TYPE(f32, F32)
 MTRT_NORM_FOR_TYPE(f16, F16)
 MTRT_NORM_FOR_TYPE(bf16, BF16)
+MTRT_NORM_GROUPS_FOR_TYPE(f32, F32)
+MTRT_NORM_GROUPS_FOR_TYPE(f16, F16)
+MTRT_NORM_GROUPS_FOR_TYPE(bf16, BF16)

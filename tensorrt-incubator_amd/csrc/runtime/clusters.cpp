@@ -148,6 +148,19 @@ int32_t pick_nv(int64_t nvec_per_row) {
   return 0;
 }
 
+// Rows too long for one wave: a workgroup of 256 or 1024 lanes with 8 or 16 vectors per lane owns the row.
+// Returns false when the row is longer than 1024 * 16 vectors.
+bool pick_group(int64_t nvec_per_row, int *threads, int *nv) {
+  for (int t : {256, 1024})
+    for (int v : {8, 16})
+      if (nvec_per_row <= int64_t(t) * v) {
+        *threads = t;
+        *nv = v;
+        return true;
+      }
+  return false;
+}
+
 } // namespace
 
 extern "C" {
@@ -510,6 +523,10 @@ int32_t mtrt_hip_layernorm(mtrt_stream_t stream, const void *x, const void *gamm
     return launch(st, KernelName("mtrt_layernorm_") + xn + "_v" + nv + (resident ? "r" : ""),
                   blocks_for(rows, kBlock / 64), kBlock, as_hip(stream), args);
   }
+  int threads, gnv;
+  if (vec_ok && !nv && rows <= int64_t(kMaxGrid) * 1024 && pick_group(d / per_vec, &threads, &gnv))
+    return launch(st, KernelName("mtrt_layernorm_") + xn + "_g" + threads + "v" + gnv, uint32_t(rows), uint32_t(threads),
+                  as_hip(stream), args);
   return launch(st, KernelName("mtrt_layernorm_") + xn + "_any",
                 uint32_t(std::min<int64_t>(rows, int64_t(num_compute_units(st)) * 8)), kBlock, as_hip(stream), args);
 }
@@ -542,6 +559,10 @@ int32_t mtrt_hip_softmax(mtrt_stream_t stream, const void *x, void *y, int32_t d
   if (nv && rows <= kMaxRowsPerWaveKernels)
     return launch(st, KernelName("mtrt_softmax_") + xn + "_v" + nv,
                   blocks_for(rows, kBlock / 64), kBlock, as_hip(stream), args);
+  int threads, gnv;
+  if (vec_ok && !nv && rows <= int64_t(kMaxGrid) * 1024 && pick_group(d / per_vec, &threads, &gnv))
+    return launch(st, KernelName("mtrt_softmax_") + xn + "_g" + threads + "v" + gnv, uint32_t(rows), uint32_t(threads),
+                  as_hip(stream), args);
   return launch(st, KernelName("mtrt_softmax_") + xn + "_any",
                 uint32_t(std::min<int64_t>(rows, int64_t(num_compute_units(st)) * 8)), kBlock, as_hip(stream), args);
 }
