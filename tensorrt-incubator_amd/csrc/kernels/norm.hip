@@ -229,14 +229,22 @@ __device__ __forceinline__ void softmax_rows(const typename X::storage* __restri
     softmax_row<X, NV, false>(x, y, row, d);
 }
 
-// ---- rows longer than one wave's registers: one WORKGROUP owns one row ---------------------------
-// THREADS lanes (256 or 1024) hold the row, NV vectors each (lane l the vectors l, l + THREADS, ...), in storage
-// form; the row reductions are a cross-lane exchange per wave and a meeting of the waves' values in LDS.  The row
-// is still read from HBM exactly once.  Covers 64 * 16 < D / E <= 1024 * 16 vectors (hidden sizes above 8192,
-// vocabulary-sized softmax rows).
+// ---- rows longer than one wave's registers, and rows of any length or alignment: a GROUP of lanes owns one row ----
+// THREADS lanes hold the row, NV vectors each (lane l the vectors l, l + THREADS, ...), in storage form; the row
+// reductions are a cross-lane exchange per wave and, when the group is a whole workgroup (256 or 1024 lanes), a
+// meeting of the waves' values in LDS.  The row is still read from HBM exactly once.  Workgroup-sized groups
+// cover 64 * 16 < D / E <= 1024 * 16 vectors (hidden sizes above 8192, vocabulary-sized softmax rows).
+// RAGGED: D need not be a multiple of the vector width E and nothing need be 16-byte aligned: the D / E whole
+// vectors of a row are moved by 128-bit accesses at element alignment (the hardware splits those that straddle
+// a line), the D % E elements behind them one each by the group's first lanes.  With THREADS = 64 that is the
+// one-wave-per-row scheme for rows such as 197, 1500 or 50257 elements.
+template <bool RAGGED> struct RowVector { typedef u32x4 type; };
+template <> struct RowVector<true> { typedef u32x4 type __attribute__((aligned(2))); };
+
 template <int THREADS, typename Op>
 __device__ __forceinline__ float group_reduce(float v, Op op, float* lds) {
   v = wave_reduce(v, op);
+  if (THREADS == kWave) return v;
   __syncthreads();                                   // lds may still be read from the previous reduction
   if ((threadIdx.x & (kWave - 1)) == 0) lds[threadIdx.x / kWave] = v;
   __syncthreads();
@@ -246,36 +254,41 @@ __device__ __forceinline__ float group_reduce(float v, Op op, float* lds) {
   return r;                                          // the same value, combined in the same order, in every lane
 }
 
-template <typename X, int NV, int THREADS, bool FULL>
+template <typename X, int NV, int THREADS, bool FULL, bool RAGGED>
 __device__ __forceinline__ void layernorm_group_row(const typename X::storage* __restrict__ x,
                                                     const typename X::storage* __restrict__ gamma,
                                                     const typename X::storage* __restrict__ beta,
                                                     typename X::storage* __restrict__ y, int64_t row, int64_t d, float eps,
                                                     float* lds) {
   constexpr int E = Vec<X>::kElems;
-  const int nvec = int(d / E);
-  const u32x4* xr = reinterpret_cast<const u32x4*>(x + row * d);
+  using V = typename RowVector<RAGGED>::type;
+  const int lane = int(threadIdx.x) & (THREADS - 1);
+  const int nvec = int(d / E), tail = RAGGED ? int(d - int64_t(nvec) * E) : 0;
+  const V* xr = reinterpret_cast<const V*>(x + row * d);
   u32x4 t[NV];
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
-    const int idx = int(threadIdx.x) + THREADS * j;
+    const int idx = lane + THREADS * j;
     t[j] = __builtin_nontemporal_load(xr + (FULL ? idx : min(idx, nvec - 1)));
   }
+  const bool extra = RAGGED && lane < tail;          // this lane also owns element nvec * E + lane
+  const int64_t ec = int64_t(nvec) * E + lane;
+  const float xe = extra ? Tile<X>::load1(x + row * d + ec) : 0.0f;
   const float fd = float(d);
-  float sum = 0.0f;
+  float sum = xe;
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
-    const bool live = FULL || int(threadIdx.x) + THREADS * j < nvec;
+    const bool live = FULL || lane + THREADS * j < nvec;
     float v[E];
     Vec<X>::unpack(t[j], v);
 #pragma unroll
     for (int k = 0; k < E; ++k) sum = sum + (live ? v[k] : 0.0f);
   }
   const float mu = group_reduce<THREADS>(sum, SumF32(), lds) / fd;
-  float sq = 0.0f;
+  float sq = extra ? (xe - mu) * (xe - mu) : 0.0f;
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
-    const bool live = FULL || int(threadIdx.x) + THREADS * j < nvec;
+    const bool live = FULL || lane + THREADS * j < nvec;
     float v[E];
     opaque(t[j]);                                    // widen again instead of keeping pass 1's values live
     Vec<X>::unpack(t[j], v);
@@ -287,12 +300,12 @@ __device__ __forceinline__ void layernorm_group_row(const typename X::storage* _
   }
   const float var = group_reduce<THREADS>(sq, SumF32(), lds) / fd;
   const float rstd = 1.0f / sqrtf(var + eps);
-  const u32x4* gv = reinterpret_cast<const u32x4*>(gamma);
-  const u32x4* bv = reinterpret_cast<const u32x4*>(beta);
-  u32x4* yr = reinterpret_cast<u32x4*>(y + row * d);
+  const V* gv = reinterpret_cast<const V*>(gamma);
+  const V* bv = reinterpret_cast<const V*>(beta);
+  V* yr = reinterpret_cast<V*>(y + row * d);
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
-    const int idx = int(threadIdx.x) + THREADS * j;
+    const int idx = lane + THREADS * j;
     const int idc = FULL ? idx : min(idx, nvec - 1);
     float v[E], g[E], b[E], o[E];
     opaque(t[j]);
@@ -303,39 +316,55 @@ __device__ __forceinline__ void layernorm_group_row(const typename X::storage* _
     for (int k = 0; k < E; ++k) o[k] = (((v[k] - mu) * rstd) * g[k]) + b[k];
     if (FULL || idx < nvec) __builtin_nontemporal_store(Vec<X>::pack(o), yr + idx);
   }
+  if (extra)
+    Tile<X>::store1(y + row * d + ec, (((xe - mu) * rstd) * Tile<X>::load1(gamma + ec)) + Tile<X>::load1(beta + ec));
 }
 
-template <typename X, int NV, int THREADS>
+// The group's row: a workgroup-sized group takes row blockIdx.x, wave-sized groups the rows 4 * blockIdx.x + wave.
+template <int THREADS>
+__device__ __forceinline__ int64_t group_row() {
+  if (THREADS == kWave)
+    return int64_t(blockIdx.x) * kRowsPerBlock + __builtin_amdgcn_readfirstlane(int(threadIdx.x / kWave));
+  return blockIdx.x;
+}
+
+template <typename X, int NV, int THREADS, bool RAGGED>
 __device__ __forceinline__ void layernorm_group(const typename X::storage* __restrict__ x,
                                                 const typename X::storage* __restrict__ gamma,
                                                 const typename X::storage* __restrict__ beta,
                                                 typename X::storage* __restrict__ y, int64_t rows, int64_t d, float eps) {
   __shared__ float lds[THREADS / kWave];
-  const int64_t row = blockIdx.x;                    // grid = rows
-  if (d == int64_t(Vec<X>::kElems) * THREADS * NV)
-    layernorm_group_row<X, NV, THREADS, true>(x, gamma, beta, y, row, d, eps, lds);
+  const int64_t row = group_row<THREADS>();
+  if (row >= rows) return;                           // wave-sized groups only (no barrier follows there); grid = rows otherwise
+  if (!RAGGED && d == int64_t(Vec<X>::kElems) * THREADS * NV)
+    layernorm_group_row<X, NV, THREADS, true, false>(x, gamma, beta, y, row, d, eps, lds);
   else
-    layernorm_group_row<X, NV, THREADS, false>(x, gamma, beta, y, row, d, eps, lds);
+    layernorm_group_row<X, NV, THREADS, false, RAGGED>(x, gamma, beta, y, row, d, eps, lds);
 }
 
 // KEEP: the exponentials stay in registers (f32) between the sum and the output pass; without it they are
 // computed again from the stored row (the 1024-lane form has 128 registers per lane, not enough for both).
-template <typename X, int NV, int THREADS, bool FULL, bool KEEP>
+template <typename X, int NV, int THREADS, bool FULL, bool KEEP, bool RAGGED>
 __device__ __forceinline__ void softmax_group_row(const typename X::storage* __restrict__ x, typename X::storage* __restrict__ y,
                                                   int64_t row, int64_t d, float* lds) {
   constexpr int E = Vec<X>::kElems;
-  const int nvec = int(d / E);
-  const u32x4* xr = reinterpret_cast<const u32x4*>(x + row * d);
+  using V = typename RowVector<RAGGED>::type;
+  const int lane = int(threadIdx.x) & (THREADS - 1);
+  const int nvec = int(d / E), tail = RAGGED ? int(d - int64_t(nvec) * E) : 0;
+  const V* xr = reinterpret_cast<const V*>(x + row * d);
   u32x4 t[NV];
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
-    const int idx = int(threadIdx.x) + THREADS * j;
+    const int idx = lane + THREADS * j;
     t[j] = __builtin_nontemporal_load(xr + (FULL ? idx : min(idx, nvec - 1)));
   }
-  float mx = -INFINITY;
+  const bool extra = RAGGED && lane < tail;          // this lane also owns element nvec * E + lane
+  const int64_t ec = int64_t(nvec) * E + lane;
+  const float xe = extra ? Tile<X>::load1(x + row * d + ec) : -INFINITY;
+  float mx = xe;
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
-    const bool live = FULL || int(threadIdx.x) + THREADS * j < nvec;
+    const bool live = FULL || lane + THREADS * j < nvec;
     float v[E];
     Vec<X>::unpack(t[j], v);
 #pragma unroll
@@ -343,10 +372,11 @@ __device__ __forceinline__ void softmax_group_row(const typename X::storage* __r
   }
   mx = group_reduce<THREADS>(mx, MaxF32(), lds);
   float e[KEEP ? NV * E : 1];
-  float s = 0.0f;
+  const float ee = extra ? __expf(xe - mx) : 0.0f;
+  float s = ee;
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
-    const bool live = FULL || int(threadIdx.x) + THREADS * j < nvec;
+    const bool live = FULL || lane + THREADS * j < nvec;
     float v[E];
     opaque(t[j]);
     Vec<X>::unpack(t[j], v);
@@ -359,10 +389,10 @@ __device__ __forceinline__ void softmax_group_row(const typename X::storage* __r
   }
   s = group_reduce<THREADS>(s, SumF32(), lds);
   const float inv = 1.0f / s;                         // e * (1/s), as in softmax_row
-  u32x4* yr = reinterpret_cast<u32x4*>(y + row * d);
+  V* yr = reinterpret_cast<V*>(y + row * d);
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
-    const int idx = int(threadIdx.x) + THREADS * j;
+    const int idx = lane + THREADS * j;
     float o[E];
     if (KEEP) {
 #pragma unroll
@@ -376,18 +406,20 @@ __device__ __forceinline__ void softmax_group_row(const typename X::storage* __r
     }
     if (FULL || idx < nvec) __builtin_nontemporal_store(Vec<X>::pack(o), yr + idx);
   }
+  if (extra) Tile<X>::store1(y + row * d + ec, ee * inv);
 }
 
-template <typename X, int NV, int THREADS>
+template <typename X, int NV, int THREADS, bool RAGGED>
 __device__ __forceinline__ void softmax_group(const typename X::storage* __restrict__ x, typename X::storage* __restrict__ y,
                                               int64_t rows, int64_t d) {
   __shared__ float lds[THREADS / kWave];
   constexpr bool kKeep = THREADS <= 256;
-  const int64_t row = blockIdx.x;                    // grid = rows
-  if (d == int64_t(Vec<X>::kElems) * THREADS * NV)
-    softmax_group_row<X, NV, THREADS, true, kKeep>(x, y, row, d, lds);
+  const int64_t row = group_row<THREADS>();
+  if (row >= rows) return;                           // wave-sized groups only (no barrier follows there); grid = rows otherwise
+  if (!RAGGED && d == int64_t(Vec<X>::kElems) * THREADS * NV)
+    softmax_group_row<X, NV, THREADS, true, kKeep, false>(x, y, row, d, lds);
   else
-    softmax_group_row<X, NV, THREADS, false, kKeep>(x, y, row, d, lds);
+    softmax_group_row<X, NV, THREADS, false, kKeep, RAGGED>(x, y, row, d, lds);
 }
 
 // ---- any D, any alignment: one workgroup per row, row re-read from cache -------------
@@ -482,15 +514,22 @@ using namespace norm_cluster;
 
 // One workgroup per row: mtrt_layernorm_<t>_g<THREADS>v<NV>(x, gamma, beta, y, rows, d, eps), mtrt_softmax_<t>_g<THREADS>v<NV>(x, y, rows, d)
 //   grid = rows, block = THREADS; d % E == 0, d / E <= THREADS * NV, operands 16-byte aligned.
-#define MTRT_NORM_GROUP_KERNELS(XN, XT, NV, THREADS)                                                           \
-  extern "C" __global__ void __launch_bounds__(THREADS) mtrt_layernorm_##XN##_g##THREADS##v##NV(               \
+// Ragged rows: mtrt_{layernorm,softmax}_<t>_u<THREADS>v<NV>, same arguments; any d with 1 <= d / E <= THREADS * NV,
+//   operands aligned to their element; THREADS = 64: grid = ceil(rows / 4), block = 256; else grid = rows, block = THREADS.
+#define MTRT_NORM_GROUP_KERNELS(XN, XT, NV, THREADS, TAG, RAGGED, BLOCK)                                       \
+  extern "C" __global__ void __launch_bounds__(BLOCK) mtrt_layernorm_##XN##_##TAG##THREADS##v##NV(             \
       const XT::storage* x, const XT::storage* gamma, const XT::storage* beta, XT::storage* y, int64_t rows,  \
-      int64_t d, float eps) { layernorm_group<XT, NV, THREADS>(x, gamma, beta, y, rows, d, eps); }            \
-  extern "C" __global__ void __launch_bounds__(THREADS) mtrt_softmax_##XN##_g##THREADS##v##NV(                 \
-      const XT::storage* x, XT::storage* y, int64_t rows, int64_t d) { softmax_group<XT, NV, THREADS>(x, y, rows, d); }
+      int64_t d, float eps) { layernorm_group<XT, NV, THREADS, RAGGED>(x, gamma, beta, y, rows, d, eps); }    \
+  extern "C" __global__ void __launch_bounds__(BLOCK) mtrt_softmax_##XN##_##TAG##THREADS##v##NV(               \
+      const XT::storage* x, XT::storage* y, int64_t rows, int64_t d) { softmax_group<XT, NV, THREADS, RAGGED>(x, y, rows, d); }
 #define MTRT_NORM_GROUPS_FOR_TYPE(XN, XT)                                                                      \
-  MTRT_NORM_GROUP_KERNELS(XN, XT, 8, 256) MTRT_NORM_GROUP_KERNELS(XN, XT, 16, 256)                             \
-  MTRT_NORM_GROUP_KERNELS(XN, XT, 8, 1024) MTRT_NORM_GROUP_KERNELS(XN, XT, 16, 1024)
+  MTRT_NORM_GROUP_KERNELS(XN, XT, 8, 256, g, false, 256) MTRT_NORM_GROUP_KERNELS(XN, XT, 16, 256, g, false, 256)      \
+  MTRT_NORM_GROUP_KERNELS(XN, XT, 8, 1024, g, false, 1024) MTRT_NORM_GROUP_KERNELS(XN, XT, 16, 1024, g, false, 1024)  \
+  MTRT_NORM_GROUP_KERNELS(XN, XT, 1, 64, u, true, 256) MTRT_NORM_GROUP_KERNELS(XN, XT, 2, 64, u, true, 256)           \
+  MTRT_NORM_GROUP_KERNELS(XN, XT, 4, 64, u, true, 256) MTRT_NORM_GROUP_KERNELS(XN, XT, 8, 64, u, true, 256)           \
+  MTRT_NORM_GROUP_KERNELS(XN, XT, 16, 64, u, true, 256)                                                               \
+  MTRT_NORM_GROUP_KERNELS(XN, XT, 8, 256, u, true, 256) MTRT_NORM_GROUP_KERNELS(XN, XT, 16, 256, u, true, 256)        \
+  MTRT_NORM_GROUP_KERNELS(XN, XT, 8, 1024, u, true, 1024) MTRT_NORM_GROUP_KERNELS(XN, XT, 16, 1024, u, true, 1024)
 
 MTRT_NORM_FOR_TYPE(f32, F32)
 MTRT_NORM_FOR_TYPE(f16, F16)

@@ -527,6 +527,16 @@ int32_t mtrt_hip_layernorm(mtrt_stream_t stream, const void *x, const void *gamm
   if (vec_ok && !nv && rows <= int64_t(kMaxGrid) * 1024 && pick_group(d / per_vec, &threads, &gnv))
     return launch(st, KernelName("mtrt_layernorm_") + xn + "_g" + threads + "v" + gnv, uint32_t(rows), uint32_t(threads),
                   as_hip(stream), args);
+  // Row lengths that are not whole vectors, or operands that are not 16-byte aligned: the same two schemes with
+  // 128-bit accesses at element alignment and the last d % per_vec elements of a row moved one by one.
+  if (!vec_ok && d >= per_vec) {
+    const int rnv = pick_nv(d / per_vec);
+    if (rnv && rows <= kMaxRowsPerWaveKernels)
+      return launch(st, KernelName("mtrt_layernorm_") + xn + "_u64v" + rnv, blocks_for(rows, kBlock / 64), kBlock, as_hip(stream), args);
+    if (!rnv && rows <= int64_t(kMaxGrid) * 1024 && pick_group(d / per_vec, &threads, &gnv))
+      return launch(st, KernelName("mtrt_layernorm_") + xn + "_u" + threads + "v" + gnv, uint32_t(rows), uint32_t(threads),
+                    as_hip(stream), args);
+  }
   return launch(st, KernelName("mtrt_layernorm_") + xn + "_any",
                 uint32_t(std::min<int64_t>(rows, int64_t(num_compute_units(st)) * 8)), kBlock, as_hip(stream), args);
 }
@@ -563,6 +573,16 @@ int32_t mtrt_hip_softmax(mtrt_stream_t stream, const void *x, void *y, int32_t d
   if (vec_ok && !nv && rows <= int64_t(kMaxGrid) * 1024 && pick_group(d / per_vec, &threads, &gnv))
     return launch(st, KernelName("mtrt_softmax_") + xn + "_g" + threads + "v" + gnv, uint32_t(rows), uint32_t(threads),
                   as_hip(stream), args);
+  // Row lengths that are not whole vectors, or operands that are not 16-byte aligned: the same two schemes with
+  // 128-bit accesses at element alignment and the last d % per_vec elements of a row moved one by one.
+  if (!vec_ok && d >= per_vec) {
+    const int rnv = pick_nv(d / per_vec);
+    if (rnv && rows <= kMaxRowsPerWaveKernels)
+      return launch(st, KernelName("mtrt_softmax_") + xn + "_u64v" + rnv, blocks_for(rows, kBlock / 64), kBlock, as_hip(stream), args);
+    if (!rnv && rows <= int64_t(kMaxGrid) * 1024 && pick_group(d / per_vec, &threads, &gnv))
+      return launch(st, KernelName("mtrt_softmax_") + xn + "_u" + threads + "v" + gnv, uint32_t(rows), uint32_t(threads),
+                    as_hip(stream), args);
+  }
   return launch(st, KernelName("mtrt_softmax_") + xn + "_any",
                 uint32_t(std::min<int64_t>(rows, int64_t(num_compute_units(st)) * 8)), kBlock, as_hip(stream), args);
 }

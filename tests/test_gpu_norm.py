@@ -184,16 +184,19 @@ def test_layernorm_resident_variant_window_and_bits(pkg, orc):
 
 def test_kernel_selection(pkg, orc):
     import torch
-    for d, k in ((512, "v1"), (1024, "v2"), (2048, "v4"), (4096, "v8"), (8192, "v16"), (8200, "g256v8"), (131080, "any"), (331, "any")):
+    for d, k in ((512, "v1"), (1024, "v2"), (2048, "v4"), (4096, "v8"), (8192, "v16"), (8200, "g256v8"), (131080, "any"), (331, "u64v1"), (5, "any")):
         x = torch.randn(4, d, device="cuda", dtype=torch.bfloat16)
         pkg.softmax(x)
         assert pkg.last_kernel() == "mtrt_softmax_bf16_" + k
         pkg.layernorm(x, torch.ones(d, device="cuda", dtype=torch.bfloat16), torch.zeros(d, device="cuda", dtype=torch.bfloat16), 1e-5)
         assert pkg.last_kernel() == "mtrt_layernorm_bf16_" + k
-    # a row pointer that is not 16-byte aligned falls back to the generic kernel
+    # a row pointer that is not 16-byte aligned takes the kernels that move vectors at element alignment
     buf = torch.randn(4 * 512 + 1, device="cuda", dtype=torch.bfloat16)
-    pkg.softmax(buf[1:].view(4, 512))
-    assert pkg.last_kernel() == "mtrt_softmax_bf16_any"
+    got = pkg.softmax(buf[1:].view(4, 512))
+    assert pkg.last_kernel() == "mtrt_softmax_bf16_u64v1"
+    want = pkg.softmax(buf[1:].view(4, 512).clone())
+    assert pkg.last_kernel() == "mtrt_softmax_bf16_v1"
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
 
 
 def test_softmax_extremes_and_empty(pkg, orc):
@@ -268,3 +271,25 @@ def test_softmax_rows_owned_by_a_workgroup(pkg, orc, name):
     """Vocabulary-sized rows (e.g. 128256 = 8 * 16032 logits): one workgroup per row."""
     for d, suffix in _group_cases(name):
         _run_softmax(pkg, orc, name, 3, d, 70 + d % 89, "mtrt_softmax_" + name + suffix, frac=2e-2 if d <= 40000 else 5e-2)
+
+
+def _ragged_cases(name):
+    """(row length, kernel suffix): lengths that are not whole vectors (attention rows of 77, 197, 1500 keys; a
+    50257-entry vocabulary) in every scheme, from one vector plus one element up to 1024 x 16 vectors plus a tail."""
+    e = 4 if name == "f32" else 8
+    return [(e + 1, "_u64v1"), (77, "_u64v1"), (197, "_u64v1"), (e * 64 + 3, "_u64v1"), (e * 65 + 3, "_u64v2"), (1500 if e == 8 else 1501, "_u64v4" if e == 8 else "_u64v8"),
+            (e * 512 + e - 1, "_u64v8"), (e * 1024 + 1, "_u64v16"), (e * 1025 + 2, "_u256v8"), (e * 4096 + 3, "_u256v16"),
+            (50257, "_u1024v8" if e == 8 else "_u1024v16"), (e * 16384 + e - 1, "_u1024v16"), (e * 16385 + 1, "_any")]
+
+
+@pytest.mark.parametrize("name", ["f32", "f16", "bf16"])
+def test_layernorm_ragged_rows(pkg, orc, name):
+    for d, suffix in _ragged_cases(name):
+        _run_layernorm(pkg, orc, name, 5, d, 80 + d % 89, "mtrt_layernorm_" + name + suffix, frac=2e-2 if d <= 40000 else 5e-2,
+                       oracle_slack=4.0 if d > 40000 else 1.0)
+
+
+@pytest.mark.parametrize("name", ["f32", "f16", "bf16"])
+def test_softmax_ragged_rows(pkg, orc, name):
+    for d, suffix in _ragged_cases(name):
+        _run_softmax(pkg, orc, name, 5, d, 90 + d % 89, "mtrt_softmax_" + name + suffix, frac=2e-2 if d <= 40000 else 5e-2)
