@@ -243,6 +243,11 @@ template <> struct RowVector<true> { typedef u32x4 type __attribute__((aligned(2
 
 template <int THREADS, typename Op>
 __device__ __forceinline__ float group_reduce(float v, Op op, float* lds) {
+  if (THREADS < kWave) {                             // several rows per wave: exchanges stay inside the row's lanes
+#pragma unroll
+    for (int off = THREADS / 2; off > 0; off >>= 1) v = op(v, __shfl_xor(v, off, kWave));
+    return v;
+  }
   v = wave_reduce(v, op);
   if (THREADS == kWave) return v;
   __syncthreads();                                   // lds may still be read from the previous reduction
@@ -320,11 +325,14 @@ __device__ __forceinline__ void layernorm_group_row(const typename X::storage* _
     Tile<X>::store1(y + row * d + ec, (((xe - mu) * rstd) * Tile<X>::load1(gamma + ec)) + Tile<X>::load1(beta + ec));
 }
 
-// The group's row: a workgroup-sized group takes row blockIdx.x, wave-sized groups the rows 4 * blockIdx.x + wave.
+// The group's row: a workgroup-sized group takes row blockIdx.x, wave-sized groups the rows 4 * blockIdx.x + wave,
+// groups of 8, 16 or 32 lanes (short rows, several to a wave) the rows (256 / THREADS) * blockIdx.x + group.
 template <int THREADS>
 __device__ __forceinline__ int64_t group_row() {
   if (THREADS == kWave)
     return int64_t(blockIdx.x) * kRowsPerBlock + __builtin_amdgcn_readfirstlane(int(threadIdx.x / kWave));
+  if (THREADS < kWave)
+    return int64_t(blockIdx.x) * (kNormThreads / THREADS) + int(threadIdx.x) / THREADS;
   return blockIdx.x;
 }
 
@@ -333,9 +341,9 @@ __device__ __forceinline__ void layernorm_group(const typename X::storage* __res
                                                 const typename X::storage* __restrict__ gamma,
                                                 const typename X::storage* __restrict__ beta,
                                                 typename X::storage* __restrict__ y, int64_t rows, int64_t d, float eps) {
-  __shared__ float lds[THREADS / kWave];
+  __shared__ float lds[THREADS >= kWave ? THREADS / kWave : 1];
   const int64_t row = group_row<THREADS>();
-  if (row >= rows) return;                           // wave-sized groups only (no barrier follows there); grid = rows otherwise
+  if (row >= rows) return;                           // groups of a wave or less only (no barrier follows there); grid = rows otherwise
   if (!RAGGED && d == int64_t(Vec<X>::kElems) * THREADS * NV)
     layernorm_group_row<X, NV, THREADS, true, false>(x, gamma, beta, y, row, d, eps, lds);
   else
@@ -412,10 +420,10 @@ __device__ __forceinline__ void softmax_group_row(const typename X::storage* __r
 template <typename X, int NV, int THREADS, bool RAGGED>
 __device__ __forceinline__ void softmax_group(const typename X::storage* __restrict__ x, typename X::storage* __restrict__ y,
                                               int64_t rows, int64_t d) {
-  __shared__ float lds[THREADS / kWave];
+  __shared__ float lds[THREADS >= kWave ? THREADS / kWave : 1];
   constexpr bool kKeep = THREADS <= 256;
   const int64_t row = group_row<THREADS>();
-  if (row >= rows) return;                           // wave-sized groups only (no barrier follows there); grid = rows otherwise
+  if (row >= rows) return;                           // groups of a wave or less only (no barrier follows there); grid = rows otherwise
   if (!RAGGED && d == int64_t(Vec<X>::kElems) * THREADS * NV)
     softmax_group_row<X, NV, THREADS, true, kKeep, false>(x, y, row, d, lds);
   else
@@ -515,7 +523,8 @@ using namespace norm_cluster;
 // One workgroup per row: mtrt_layernorm_<t>_g<THREADS>v<NV>(x, gamma, beta, y, rows, d, eps), mtrt_softmax_<t>_g<THREADS>v<NV>(x, y, rows, d)
 //   grid = rows, block = THREADS; d % E == 0, d / E <= THREADS * NV, operands 16-byte aligned.
 // Ragged rows: mtrt_{layernorm,softmax}_<t>_u<THREADS>v<NV>, same arguments; any d with 1 <= d / E <= THREADS * NV,
-//   operands aligned to their element; THREADS = 64: grid = ceil(rows / 4), block = 256; else grid = rows, block = THREADS.
+//   operands aligned to their element; THREADS <= 64 (NV = 1 below 64): grid = ceil(rows / (256 / THREADS)), block = 256;
+//   else grid = rows, block = THREADS.
 #define MTRT_NORM_GROUP_KERNELS(XN, XT, NV, THREADS, TAG, RAGGED, BLOCK)                                       \
   extern "C" __global__ void __launch_bounds__(BLOCK) mtrt_layernorm_##XN##_##TAG##THREADS##v##NV(             \
       const XT::storage* x, const XT::storage* gamma, const XT::storage* beta, XT::storage* y, int64_t rows,  \
@@ -525,6 +534,8 @@ using namespace norm_cluster;
 #define MTRT_NORM_GROUPS_FOR_TYPE(XN, XT)                                                                      \
   MTRT_NORM_GROUP_KERNELS(XN, XT, 8, 256, g, false, 256) MTRT_NORM_GROUP_KERNELS(XN, XT, 16, 256, g, false, 256)      \
   MTRT_NORM_GROUP_KERNELS(XN, XT, 8, 1024, g, false, 1024) MTRT_NORM_GROUP_KERNELS(XN, XT, 16, 1024, g, false, 1024)  \
+  MTRT_NORM_GROUP_KERNELS(XN, XT, 1, 8, u, true, 256) MTRT_NORM_GROUP_KERNELS(XN, XT, 1, 16, u, true, 256)            \
+  MTRT_NORM_GROUP_KERNELS(XN, XT, 1, 32, u, true, 256)                                                                \
   MTRT_NORM_GROUP_KERNELS(XN, XT, 1, 64, u, true, 256) MTRT_NORM_GROUP_KERNELS(XN, XT, 2, 64, u, true, 256)           \
   MTRT_NORM_GROUP_KERNELS(XN, XT, 4, 64, u, true, 256) MTRT_NORM_GROUP_KERNELS(XN, XT, 8, 64, u, true, 256)           \
   MTRT_NORM_GROUP_KERNELS(XN, XT, 16, 64, u, true, 256)                                                               \

@@ -515,6 +515,11 @@ int32_t mtrt_hip_layernorm(mtrt_stream_t stream, const void *x, const void *gamm
   int64_t rows_arg = rows, d_arg = d;
   float eps_arg = eps;
   void *args[] = {&x, &gamma, &beta, &y, &rows_arg, &d_arg, &eps_arg};
+  // Rows of at most 32 vectors: 8, 16 or 32 lanes per row, several rows to a wave (whatever the alignment).
+  if (d >= per_vec && d / per_vec <= 32 && aligned(x, eb) && rows <= kMaxRowsPerWaveKernels) {
+    const int lanes = d / per_vec <= 8 ? 8 : (d / per_vec <= 16 ? 16 : 32);
+    return launch(st, KernelName("mtrt_layernorm_") + xn + "_u" + lanes + "v1", blocks_for(rows, kBlock / lanes), kBlock, as_hip(stream), args);
+  }
   if (nv && rows <= kMaxRowsPerWaveKernels) {
     // One wave per row.  The eight-vector kernel runs five waves per SIMD; when that leaves a second, partly
     // filled round and eight waves per SIMD would hold every row at once, its 64-register form is faster.
@@ -566,6 +571,11 @@ int32_t mtrt_hip_softmax(mtrt_stream_t stream, const void *x, void *y, int32_t d
   const int nv = vec_ok ? pick_nv(d / per_vec) : 0;
   int64_t rows_arg = rows, d_arg = d;
   void *args[] = {&x, &y, &rows_arg, &d_arg};
+  // Rows of at most 32 vectors: 8, 16 or 32 lanes per row, several rows to a wave (whatever the alignment).
+  if (d >= per_vec && d / per_vec <= 32 && aligned(x, eb) && rows <= kMaxRowsPerWaveKernels) {
+    const int lanes = d / per_vec <= 8 ? 8 : (d / per_vec <= 16 ? 16 : 32);
+    return launch(st, KernelName("mtrt_softmax_") + xn + "_u" + lanes + "v1", blocks_for(rows, kBlock / lanes), kBlock, as_hip(stream), args);
+  }
   if (nv && rows <= kMaxRowsPerWaveKernels)
     return launch(st, KernelName("mtrt_softmax_") + xn + "_v" + nv,
                   blocks_for(rows, kBlock / 64), kBlock, as_hip(stream), args);
