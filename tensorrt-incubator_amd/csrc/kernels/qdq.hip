@@ -278,6 +278,7 @@ __device__ __forceinline__ float quant_value(float x, float s, int flags) {
 struct ExactDivisor {
   float s, r, bound;
   bool fast;
+  ExactDivisor() = default;
   __device__ __forceinline__ explicit ExactDivisor(float scale) : s(scale) {
     const uint32_t e = (f32_to_bits(scale) >> 23) & 0xFFu;
     fast = e >= 127u - 60u && e <= 127u + 60u;
@@ -299,18 +300,20 @@ struct ExactDivisor {
   // callers that have checked `fast` for the whole wave.  Same values as finish_quotient(divide(x)); the sign of
   // zero is put back after the clamp (a clamp keeps it), so that the clamp's operands are results of arithmetic
   // and need no quieting first.
+  template <typename Q, bool ROUND>
+  __device__ __forceinline__ float quantize_fast1(float x) const {
+    const float xc = fmaxf(fminf(x, bound), -bound);
+    const float q0 = xc * r;
+    float q = __builtin_fmaf(__builtin_fmaf(-q0, s, xc), r, q0);
+    q = __builtin_fmaf(__builtin_fmaf(-q, s, xc), r, q);
+    if (ROUND) q = __builtin_rintf(q);
+    q = fmaxf(fminf(q, Codes<Q>::kHi), Codes<Q>::kLo);
+    return __builtin_copysignf(q, q0);
+  }
   template <typename Q, bool ROUND, int G>
   __device__ __forceinline__ void quantize_fast(float (&v)[G]) const {
 #pragma unroll
-    for (int k = 0; k < G; ++k) {
-      const float xc = fmaxf(fminf(v[k], bound), -bound);
-      const float q0 = xc * r;
-      float q = __builtin_fmaf(__builtin_fmaf(-q0, s, xc), r, q0);
-      q = __builtin_fmaf(__builtin_fmaf(-q, s, xc), r, q);
-      if (ROUND) q = __builtin_rintf(q);
-      q = fmaxf(fminf(q, Codes<Q>::kHi), Codes<Q>::kLo);
-      v[k] = __builtin_copysignf(q, q0);
-    }
+    for (int k = 0; k < G; ++k) v[k] = quantize_fast1<Q, ROUND>(v[k]);
   }
 };
 
@@ -330,6 +333,100 @@ __device__ __forceinline__ void quantize_group(const ExactDivisor& dv, float (&v
 }
 
 enum ScaleKind { kUniform = 0, kRow = 1, kCol = 2 };
+
+// Column scales (per-channel on the last axis, blocks of nb rows): in the group loop below every group fetches its
+// own G scales and divides by each once, so the scales cost as many bytes through the vector cache as the tensor
+// and every element an IEEE divide.  Here a wave takes a STRIP of 64 groups of columns and walks kColChunkRows
+// rows of one scale block down it: the lane's G scales are fetched, and their reciprocals formed, once per strip
+// and chunk; every row of the chunk is one contiguous KiB of the float operand per wave, as before.
+// Host guarantees as for qdq_groups<kCol>: d1 % G == 0, n / G < 2^32, operands aligned for group accesses,
+// the scales 16-byte aligned.
+constexpr int kColChunkRows = 32;
+
+template <typename X, typename Q, int MODE>
+__device__ __forceinline__ void qdq_col_strips(const typename X::storage* __restrict__ x, typename Q::storage* __restrict__ q,
+                                               typename X::storage* __restrict__ y, const float* __restrict__ scale,
+                                               int64_t n, int64_t d1, int64_t nb, int flags) {
+  using FG = FloatGroup<X>;
+  constexpr int G = FG::G;
+  constexpr int U = 4;                               // rows in flight per lane
+  using CG = CodeGroup<Q, G>;
+  const uint32_t groups_per_row = uint32_t(d1 / G), strips = (groups_per_row + kWave - 1) / kWave;
+  const int64_t d0 = n / d1, nblocks = d0 / nb;
+  const uint32_t chunks = uint32_t((nb + kColChunkRows - 1) / kColChunkRows);
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t wave = (int64_t(blockIdx.x) * blockDim.x + threadIdx.x) / kWave;
+  const int64_t nwaves = int64_t(gridDim.x) * blockDim.x / kWave;
+  const int64_t items = nblocks * chunks * strips;
+  const bool round = Codes<Q>::kAlwaysRound || (flags & kFlagRoundToInt);
+
+  for (int64_t item = wave; item < items; item += nwaves) {
+    const uint32_t strip = uint32_t(item % strips);
+    const int64_t rest = item / strips;
+    const uint32_t chunk = uint32_t(rest % chunks);
+    const int64_t b = rest / chunks;
+    const uint32_t cg = strip * kWave + lane;
+    const bool live = cg < groups_per_row;
+    const int64_t c0 = int64_t(live ? cg : groups_per_row - 1) * G;     // idle lanes repeat the last group, store nothing
+    float sc[G];
+    const f32x4* sp = reinterpret_cast<const f32x4*>(scale + b * d1 + c0);
+#pragma unroll
+    for (int k = 0; k < G / 4; ++k) {
+      const f32x4 t = sp[k];
+      sc[4 * k] = t.x; sc[4 * k + 1] = t.y; sc[4 * k + 2] = t.z; sc[4 * k + 3] = t.w;
+    }
+    const int64_t r0 = b * nb + int64_t(chunk) * kColChunkRows;
+    const int64_t r1 = r0 + kColChunkRows < (b + 1) * nb ? r0 + kColChunkRows : (b + 1) * nb;
+    ExactDivisor dv[G];
+    bool fast = true;
+#pragma unroll
+    for (int k = 0; k < G; ++k) {
+      if (MODE != 1) dv[k] = ExactDivisor(sc[k]);
+      fast = fast && (MODE == 1 || dv[k].fast);
+    }
+    const bool all_fast = MODE == 1 || __builtin_amdgcn_ballot_w64(!fast) == 0;
+
+    for (int64_t r = r0; r < r1; r += U) {
+      u32x4 xin[U];
+      uint32_t qin[U][2];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int64_t e = (r + u < r1 ? r + u : r1 - 1) * d1 + c0;
+        if (MODE == 1) CG::load_raw(q, e, qin[u]);
+        else xin[u] = FG::load(x + e);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int64_t e = (r + u) * d1 + c0;
+        const bool store = live && r + u < r1;
+        float v[G];
+        if (MODE == 1) {
+          CG::decode(qin[u], v);
+        } else {
+          FG::unpack(xin[u], v);
+          if (all_fast) {
+            if (round) {
+#pragma unroll
+              for (int k = 0; k < G; ++k) v[k] = dv[k].template quantize_fast1<Q, true>(v[k]);
+            } else {
+#pragma unroll
+              for (int k = 0; k < G; ++k) v[k] = dv[k].template quantize_fast1<Q, false>(v[k]);
+            }
+          } else {
+#pragma unroll
+            for (int k = 0; k < G; ++k) v[k] = quant_value<Q>(v[k], sc[k], flags);
+          }
+          if (store) CG::store(q, e, v, flags);       // leaves f32(code) in v
+        }
+        if (MODE != 0 && store) {
+#pragma unroll
+          for (int k = 0; k < G; ++k) v[k] = v[k] * sc[k];
+          FG::store(y + e, v);
+        }
+      }
+    }
+  }
+}
 
 // MODE: 0 = quantize (write q), 1 = dequantize (read q, write y),
 //       2 = fused quantize->dequantize (read x, write q and y)
@@ -502,7 +599,7 @@ using namespace qdq_cluster;
     qdq_groups<XT, QT, kRow, 0>(x, q, nullptr, scale, n, d1, nb, flags); }                                        \
   extern "C" __global__ void __launch_bounds__(256) mtrt_q_col_##XN##_##QN(                                       \
       const XT::storage* x, QT::storage* q, const float* scale, int64_t n, int64_t d1, int64_t nb, int32_t flags) { \
-    qdq_groups<XT, QT, kCol, 0>(x, q, nullptr, scale, n, d1, nb, flags); }                                        \
+    qdq_col_strips<XT, QT, 0>(x, q, nullptr, scale, n, d1, nb, flags); }                                        \
   extern "C" __global__ void __launch_bounds__(256) mtrt_q_any_##XN##_##QN(                                       \
       const XT::storage* x, QT::storage* q, const float* scale, int64_t n, int64_t d1, int64_t nb, int32_t kind,  \
       int32_t flags) { qdq_any<XT, QT, 0>(x, q, nullptr, scale, n, d1, nb, kind, flags); }                        \
@@ -514,7 +611,7 @@ using namespace qdq_cluster;
     qdq_groups<XT, QT, kRow, 1>(nullptr, const_cast<QT::storage*>(q), y, scale, n, d1, nb, 0); }                  \
   extern "C" __global__ void __launch_bounds__(256) mtrt_dq_col_##XN##_##QN(                                      \
       const QT::storage* q, XT::storage* y, const float* scale, int64_t n, int64_t d1, int64_t nb) {              \
-    qdq_groups<XT, QT, kCol, 1>(nullptr, const_cast<QT::storage*>(q), y, scale, n, d1, nb, 0); }                  \
+    qdq_col_strips<XT, QT, 1>(nullptr, const_cast<QT::storage*>(q), y, scale, n, d1, nb, 0); }                  \
   extern "C" __global__ void __launch_bounds__(256) mtrt_dq_any_##XN##_##QN(                                      \
       const QT::storage* q, XT::storage* y, const float* scale, int64_t n, int64_t d1, int64_t nb, int32_t kind) { \
     qdq_any<XT, QT, 1>(nullptr, const_cast<QT::storage*>(q), y, scale, n, d1, nb, kind, 0); }                     \
@@ -526,7 +623,7 @@ using namespace qdq_cluster;
       int32_t flags) { qdq_groups<XT, QT, kRow, 2>(x, q, y, scale, n, d1, nb, flags); }                           \
   extern "C" __global__ void __launch_bounds__(256) mtrt_qdq_col_##XN##_##QN(                                     \
       const XT::storage* x, QT::storage* q, XT::storage* y, const float* scale, int64_t n, int64_t d1, int64_t nb, \
-      int32_t flags) { qdq_groups<XT, QT, kCol, 2>(x, q, y, scale, n, d1, nb, flags); }                           \
+      int32_t flags) { qdq_col_strips<XT, QT, 2>(x, q, y, scale, n, d1, nb, flags); }                           \
   extern "C" __global__ void __launch_bounds__(256) mtrt_qdq_any_##XN##_##QN(                                     \
       const XT::storage* x, QT::storage* q, XT::storage* y, const float* scale, int64_t n, int64_t d1, int64_t nb, \
       int32_t kind, int32_t flags) { qdq_any<XT, QT, 2>(x, q, y, scale, n, d1, nb, kind, flags); }

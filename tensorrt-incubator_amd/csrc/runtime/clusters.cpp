@@ -137,6 +137,11 @@ int32_t qdq_dispatch(int mode, hipStream_t stream, const void *x, int32_t x_dtyp
   if (!tiles) args[na++] = &kind_arg;
   if (mode != 1) args[na++] = &flags_arg;
 
+  if (tiles && kind == MTRT_SCALE_COL) {
+    // one wave per (scale block, chunk of 32 rows of it, strip of 64 groups of columns): see qdq_col_strips
+    const int64_t items = (d0 / nb) * ((nb + 31) / 32) * ((d1 / group + 63) / 64);
+    return launch(st, name, blocks_for(items, kBlock / 64), kBlock, stream, args);
+  }
   const int64_t units = tiles ? (n + kTile - 1) / kTile : (nibbles ? (n + 1) / 2 : n);
   return launch(st, name, blocks_for(units, kBlock), kBlock, stream, args);
 }
