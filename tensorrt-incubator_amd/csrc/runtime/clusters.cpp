@@ -829,22 +829,29 @@ int32_t mtrt_hip_gemm_w4a16(mtrt_stream_t stream, const void *a, const void *w_k
       const uint32_t grid = uint32_t(M > 8 && tiles > cus && tiles <= 2 * cus ? cus : tiles);
       return launch(st, KernelName(M <= 16 ? "mtrt_gemm_w4a16_skinny16" : "mtrt_gemm_w4a16_skinny"), grid, kBlock, as_hip(stream), args);
     }
-    // 256 x 256 tiles (256 threads) once they cover at least half of the compute units (measured:
-    // from M = 1024 on at N = 11008 they beat the small tiles) and the activations stay inside
-    // 32-bit byte offsets; 128 x 64 tiles otherwise.
-    const int64_t panels = (N + 255) / 256, tiles_m = (M + 255) / 256;
-    const int64_t big = 8 * ((panels + 7) / 8) * tiles_m;
-    if (panels * tiles_m * 2 >= int64_t(num_compute_units(st)) && M * K * 2 < (int64_t(1) << 32) && big <= int64_t(kMaxGrid) * 1024)
-      return launch(st, KernelName("mtrt_gemm_w4a16_t256x256"), uint32_t(big), 256, as_hip(stream), args);
-    // 128-row tiles: 128 columns wide while that leaves every compute unit at most one workgroup, else 64
-    const int64_t small = 8 * ((((N + 63) / 64) + 7) / 8) * ((M + 127) / 128);
-    if (M * K * 2 < (int64_t(1) << 32) && small <= int64_t(kMaxGrid) * 1024) {
-      const int64_t wide_tiles = ((N + 127) / 128) * ((M + 127) / 128);
-      if (wide_tiles <= int64_t(num_compute_units(st))) {
-        const int64_t wide = 8 * ((((N + 127) / 128) + 7) / 8) * ((M + 127) / 128);
+    // 256 x 256 tiles (four waves) or 128 x 128 tiles (eight waves), one workgroup per compute unit at a time.  A
+    // launch runs in rounds of one tile per unit; a full round of the large tile takes 3.25 times a full round of
+    // the small one for four times the work, and a partly filled last round is shorter than a full one (fewer
+    // units share the power budget): 0.56 + 0.44 f^2 of it at fill f (measured over M = 48 ... 4096 at (K, N) =
+    // (4096, 4096), (4096, 11008), (11008, 4096), (8192, 8192), (5120, 13824), (4096, 14336), (8192, 28672),
+    // (4096, 2048): the estimate picks the faster kernel in all but near-ties; 128 x 64 tiles were never ahead
+    // by more than 1 % there and only serve matrices at most 64 columns wide).
+    if (M * K * 2 < (int64_t(1) << 32)) {
+      const int64_t units = num_compute_units(st);
+      const int64_t panels = (N + 255) / 256, tiles_m = (M + 255) / 256, big_tiles = panels * tiles_m;
+      const int64_t wide_panels = (N + 127) / 128, wide_m = (M + 127) / 128, wide_tiles = wide_panels * wide_m;
+      auto rounds = [units](int64_t tiles) {
+        const double f = double(tiles % units) / double(units);
+        return double(tiles / units) + (tiles % units ? 0.56 + 0.44 * f * f : 0.0);
+      };
+      const int64_t big = 8 * ((panels + 7) / 8) * tiles_m, wide = 8 * ((wide_panels + 7) / 8) * wide_m;
+      const int64_t narrow = 8 * ((((N + 63) / 64) + 7) / 8) * wide_m;
+      if (3.25 * rounds(big_tiles) < rounds(wide_tiles) && big <= int64_t(kMaxGrid) * 1024)
+        return launch(st, KernelName("mtrt_gemm_w4a16_t256x256"), uint32_t(big), 256, as_hip(stream), args);
+      if (N <= 64 && narrow <= int64_t(kMaxGrid) * 1024)
+        return launch(st, KernelName("mtrt_gemm_w4a16_t128x64"), uint32_t(narrow), kBlock, as_hip(stream), args);
+      if (wide <= int64_t(kMaxGrid) * 1024)
         return launch(st, KernelName("mtrt_gemm_w4a16_t128x128"), uint32_t(wide), 512, as_hip(stream), args);
-      }
-      return launch(st, KernelName("mtrt_gemm_w4a16_t128x64"), uint32_t(small), kBlock, as_hip(stream), args);
     }
   }
   if (!w_kn_packed)

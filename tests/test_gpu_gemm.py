@@ -171,7 +171,8 @@ def test_w4a16_small_shapes(pkg, orc, shape):
     B = 128
     a, w, wp, s = _w4a16_inputs(orc, rng(M + K + N), M, K, N, B)
     y, kernel = _run_w4a16(pkg, a, wp, s, K, N, B)
-    assert kernel == ("mtrt_gemm_w4a16_strips16" if M <= 16 else "mtrt_gemm_w4a16_skinny" if M <= 32 else "mtrt_gemm_w4a16_t128x128")
+    assert kernel == ("mtrt_gemm_w4a16_strips16" if M <= 16 else "mtrt_gemm_w4a16_skinny" if M <= 32 else
+                      "mtrt_gemm_w4a16_t128x64" if N <= 64 else "mtrt_gemm_w4a16_t128x128")
     _check_w4a16(orc, y, a, w, s, K, N, B, orc.gemm_w4a16(a, wp, s, K, N, B))
 
 
@@ -274,9 +275,9 @@ def test_w4a16_strip_kernel(pkg, orc, shape):
 
 
 def test_w4a16_narrow_mid_tile_kernel(pkg, orc):
-    """128 x 64 tiles: more 128-wide tiles than compute units, too few 256-wide ones for the large kernel
-    (M = 600, N = 8480: 5 x 67 = 335 wide tiles; ragged in M and N), K = 320 (five slices: main loop and tail)."""
-    M, K, N, B = 600, 320, 8480, 64
+    """128 x 64 tiles: matrices at most 64 columns wide (M = 600, N = 40: ragged in M and N), K = 320 (five slices:
+    main loop and tail)."""
+    M, K, N, B = 600, 320, 40, 64
     a, w, wp, s = _w4a16_inputs(orc, rng(78), M, K, N, B)
     y, kernel = _run_w4a16(pkg, a, wp, s, K, N, B)
     assert kernel == "mtrt_gemm_w4a16_t128x64"
@@ -295,6 +296,24 @@ def test_w4a16_big_tile_kernel_ragged_edges(pkg, orc):
     y, kernel = _run_w4a16(pkg, a, wp, s, K, N, B)
     assert kernel == "mtrt_gemm_w4a16_t256x256"
     rows = sorted(set([0, 1, 127, 128, 255, 256, 1023, 1791, 1792, 1998, 1999] + list(range(5, M, 97))))
+    orc.set_threads(16)
+    ref = np.concatenate([orc.gemm_w4a16(a, wp, s, K, N, B, m0=r, mcount=1) for r in rows])
+    orc.set_threads(1)
+    _check_w4a16(orc, y[rows].contiguous(), a[rows], w, s, K, N, B, ref)
+
+
+@pytest.mark.parametrize("shape,kernel", [((1536, 4096), "t128x128"), ((600, 8480), "t128x128"), ((2048, 4096), "t128x128"),
+                                          ((768, 11008), "t256x256"), ((1536, 11008), "t128x128"), ((3072, 4096), "t256x256")])
+def test_w4a16_tile_choice_and_results_at_mid_m(pkg, orc, shape, kernel):
+    """The tile is chosen by the estimated number of rounds of one tile per compute unit: 128 x 128 tiles where the
+    256 x 256 ones would fill half of the units or spill a few tiles into another round.  Sampled rows against the
+    oracle for each choice."""
+    M, N = shape
+    K, B = 256, 128
+    a, w, wp, s = _w4a16_inputs(orc, rng(M + N), M, K, N, B)
+    y, k = _run_w4a16(pkg, a, wp, s, K, N, B)
+    assert k == "mtrt_gemm_w4a16_" + kernel
+    rows = sorted(set([0, 1, 127, 128, 255, 256, M - 2, M - 1] + list(range(7, M, 113))))
     orc.set_threads(16)
     ref = np.concatenate([orc.gemm_w4a16(a, wp, s, K, N, B, m0=r, mcount=1) for r in rows])
     orc.set_threads(1)
