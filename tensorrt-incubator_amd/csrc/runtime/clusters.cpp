@@ -811,6 +811,16 @@ int32_t mtrt_hip_gemm_w4a16(mtrt_stream_t stream, const void *a, const void *w_k
   if (!st)
     return MTRT_RUNTIME_ERROR;
   const bool fast = w_prepacked && K > 0 && K % 64 == 0 && block % 64 == 0 && aligned(a, 16) && aligned(w_prepacked, 16);
+  if (fast && M > 32 && M <= 64) {
+    // Between 33 and 64 rows a 128-row tile is at least half padding and the launch lasts as long as one tile's K
+    // loop; two launches of the small-M kernels (rows 0..31, then the rest; the second finds the weights in cache)
+    // are shorter: M = 48 at (K, N) = (4096, 4096) 22.2 us as one tile launch, (11008, 4096) 52.0, (4096, 11008) 23.1.
+    const int32_t rc = mtrt_hip_gemm_w4a16(stream, a, w_kn_packed, w_prepacked, scale, y, 32, K, N, block);
+    if (rc != MTRT_OK)
+      return rc;
+    return mtrt_hip_gemm_w4a16(stream, static_cast<const char *>(a) + 32 * K * 2, w_kn_packed, w_prepacked, scale,
+                               static_cast<char *>(y) + 32 * N * 2, M - 32, K, N, block);
+  }
   if (fast) {
     void *args[] = {&a, &w_prepacked, &scale, &y, &M, &K, &N, &block};
     if (M <= 16 && K % 128 == 0 && block % 128 == 0) {
