@@ -326,6 +326,183 @@ extern "C" __global__ void __launch_bounds__(256) mtrt_w8_prepack_frag(const int
   }
 }
 
+// ---- small M (<= 32): one workgroup per 32 columns, four waves split K -----------------------------------
+// A launch of the tile kernel above lasts one tile's whole K loop however few rows it has (M = 16 at K = 4096,
+// N = 11008: 21.7 us) although all it has to do is read the weights once (45 MB).  Here every workgroup owns one
+// tile of 32 columns (or two, see small_m_tiles) over all of K, its four waves a quarter of K each: a wave keeps
+// a ring of four stages (8 * G rows x 128 k of activations each) of its own in LDS, filled by direct-to-LDS loads
+// three slices ahead as whole 128-byte row segments (a fragment read straight from memory would touch 32 cache
+// lines), and takes the weights from fragment order straight into registers: no barrier until the four partial
+// sums (int32, exact in any order) meet in LDS.  G: groups of 8 activation rows per stage (M <= 8 * G).
+namespace small_m {
+
+template <int G, int WAVES, int JT>
+__device__ __forceinline__ void run(const int8_t* __restrict__ a, const v4i* __restrict__ wfrag, const float* __restrict__ a_scale,
+                                    const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N,
+                                    int8_t* lds) {
+  constexpr int kStages = 4, kStageBytes = 8 * G * 128;
+  constexpr int kLoads = G + 4 * JT;                 // memory instructions per slice and wave
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int frow = lane & 31, fhalf = lane >> 5;
+  const int64_t slices = K / 128;
+  const int64_t kb0 = slices * wave / WAVES, kb1 = slices * (wave + 1) / WAVES;
+  int64_t tile[JT];
+  const v4i* bp[JT];
+#pragma unroll
+  for (int j = 0; j < JT; ++j) {
+    tile[j] = blockIdx.x + int64_t(j) * gridDim.x;
+    bp[j] = wfrag + (tile[j] * slices) * 256 + lane;
+  }
+  int8_t* ring = lds + wave * (kStages * kStageBytes);
+
+  // direct-to-LDS load g (of G) of a slice: rows 8g .. 8g+7, lane l <-> (row l >> 3, LDS chunk l & 7)
+  uint32_t aoff[G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    const int lrow = g * 8 + (lane >> 3);
+    const int64_t row = lrow < M ? lrow : M - 1;     // rows past M repeat the last row; never stored
+    aoff[g] = uint32_t(row * K + (((lane & 7) ^ ((lrow >> 1) & 7)) << 4));
+  }
+  struct Slice {
+    v4i w[JT][4];
+  };
+  // everything slice kb needs from memory: G + 4 JT loads, always, so that the waits can count
+  auto fetch = [&](int64_t kb, int64_t clamp, Slice& dst) {
+    kb = kb < clamp ? kb : clamp;
+    int8_t* st = ring + int(kb & (kStages - 1)) * kStageBytes;
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+      __builtin_amdgcn_global_load_lds((gemm_core::global_void_t*)(a + kb * 128 + aoff[g]),
+                                       (gemm_core::lds_void_t*)(st + g * 1024), 16, 0, 0);
+    // register loads as opaque instructions, the waits placed by hand in `landed` (the compiler's own
+    // bookkeeping drains every load carried around a loop before its first use)
+#pragma unroll
+    for (int j = 0; j < JT; ++j)
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        const v4i* wsrc = bp[j] + kb * 256 + p * 64;
+        __asm__ volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(dst.w[j][p]) : "v"(wsrc) : "memory");
+      }
+  };
+  // four slices issued, the loads of three may fly -> those of the oldest slice have landed
+  auto landed = [&](Slice& sl) {
+#pragma unroll
+    for (int j = 0; j < JT; ++j)
+#pragma unroll
+      for (int p = 0; p < 4; ++p) __asm__ volatile("s_waitcnt vmcnt(%1)" : "+v"(sl.w[j][p]) : "n"(3 * kLoads) : "memory");
+  };
+  auto landed_all = [&](Slice& sl) {
+#pragma unroll
+    for (int j = 0; j < JT; ++j)
+#pragma unroll
+      for (int p = 0; p < 4; ++p) __asm__ volatile("s_waitcnt vmcnt(0)" : "+v"(sl.w[j][p])::"memory");
+  };
+
+  v16i acc[JT];
+#pragma unroll
+  for (int j = 0; j < JT; ++j)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[j][r] = 0;
+  auto multiply = [&](int64_t kb, const Slice& sl) {
+    const int8_t* st = ring + int(kb & (kStages - 1)) * kStageBytes;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const int arow = frow < 8 * G ? frow : 8 * G - 1;   // rows past the ring: any valid data, never stored
+      const v4i fa = *reinterpret_cast<const v4i*>(st + gemm_core::lds_off(arow, 2 * p + fhalf));
+#pragma unroll
+      for (int j = 0; j < JT; ++j) acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa, sl.w[j][p], acc[j], 0, 0, 0);
+    }
+  };
+
+  // Main part: groups of four slices with four register sets, so that nothing is copied (a copy would have
+  // to wait for the load) and the loop has no branch; three slices stay in flight.
+  const int64_t kmain = kb0 + ((kb1 - kb0) & ~int64_t(3));
+  if (kb0 < kmain) {
+    const int64_t clamp = kmain - 1;                   // past the end: the last slice again, into a stage nobody reads
+    Slice s0, s1, s2, s3;
+    fetch(kb0, clamp, s0);
+    fetch(kb0 + 1, clamp, s1);
+    fetch(kb0 + 2, clamp, s2);
+    for (int64_t kb = kb0; kb < kmain; kb += 4) {
+      fetch(kb + 3, clamp, s3);
+      landed(s0);
+      multiply(kb, s0);
+      fetch(kb + 4, clamp, s0);
+      landed(s1);
+      multiply(kb + 1, s1);
+      fetch(kb + 5, clamp, s1);
+      landed(s2);
+      multiply(kb + 2, s2);
+      fetch(kb + 6, clamp, s2);
+      landed(s3);
+      multiply(kb + 3, s3);
+    }
+    // the surplus loads of the last group still target these registers: keep them until they land
+    landed_all(s0);
+    landed_all(s1);
+    landed_all(s2);
+  }
+  for (int64_t kb = kmain; kb < kb1; ++kb) {           // at most three slices, one at a time
+    Slice sl;
+    __builtin_amdgcn_s_waitcnt(0x0070);
+    fetch(kb, kb, sl);
+    landed_all(sl);
+    multiply(kb, sl);
+  }
+  __builtin_amdgcn_s_waitcnt(0x0070);                  // surplus loads have landed before the ring is reused
+  int (*partial)[16][64] = reinterpret_cast<int (*)[16][64]>(lds);
+#pragma unroll
+  for (int j = 0; j < JT; ++j) {
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < 16; ++r) partial[wave][r][lane] = acc[j][r];
+    __syncthreads();
+    for (int e = threadIdx.x; e < 16 * 64; e += 64 * WAVES) {
+      const int r = e >> 6, l = e & 63;
+      int v = partial[0][r][l];
+#pragma unroll
+      for (int w = 1; w < WAVES; ++w) v = v + partial[w][r][l];
+      const int64_t row = (r >> 2) * 8 + (l >> 5) * 4 + (r & 3);
+      const int64_t c = tile[j] * 32 + (l & 31);
+      if (row < M && c < N) y[row * N + c] = uint16_t(f32_to_f16_bits((float(v) * a_scale[row]) * w_scale[c]));
+    }
+  }
+}
+
+// The grid is one workgroup per column tile, or, while that would leave some compute units with two workgroups
+// and the rest with one (tiles between one and two times the compute units), one workgroup per compute unit:
+// workgroup g then also takes tile g + gridDim.x if there is one, and reads the activations once for both.
+template <int G>
+__device__ __forceinline__ void tiles(const int8_t* __restrict__ a, const v4i* __restrict__ wfrag, const float* __restrict__ a_scale,
+                                      const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N,
+                                      int8_t* lds) {
+  const int64_t ntiles = (N + 31) / 32;
+  if (int64_t(blockIdx.x) + gridDim.x < ntiles)
+    run<G, 4, 2>(a, wfrag, a_scale, w_scale, y, M, K, N, lds);
+  else
+    run<G, 4, 1>(a, wfrag, a_scale, w_scale, y, M, K, N, lds);
+}
+
+}  // namespace small_m
+
+// (a [M,K] i8, w_frag (fragment order), a_scale [M] f32, w_scale [N] f32, y [M,N] f16, M, K, N) ; K % 128 == 0, a and
+// w_frag 16-byte aligned, M * K < 2^32; grid = ceil(N / 32) or the number of compute units (see small_m::tiles), block = 256.
+// M <= 16:
+extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w8a8_small16(
+    const int8_t* __restrict__ a, const v4i* __restrict__ w_frag, const float* __restrict__ a_scale,
+    const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N) {
+  __shared__ __attribute__((aligned(16))) int8_t lds[4 * 4 * 2 * 1024];
+  small_m::tiles<2>(a, w_frag, a_scale, w_scale, y, M, K, N, lds);
+}
+// M <= 32:
+extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w8a8_small32(
+    const int8_t* __restrict__ a, const v4i* __restrict__ w_frag, const float* __restrict__ a_scale,
+    const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N) {
+  __shared__ __attribute__((aligned(16))) int8_t lds[4 * 4 * 4 * 1024];
+  small_m::tiles<4>(a, w_frag, a_scale, w_scale, y, M, K, N, lds);
+}
+
 // Any K (no alignment needs): one output element per lane, plain loops.  Serves
 // shapes the MFMA kernel does not take; not a fast path.
 extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w8a8_nk_any(

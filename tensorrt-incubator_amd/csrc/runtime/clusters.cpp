@@ -707,6 +707,24 @@ int32_t mtrt_hip_gemm_w8a8_fragments(mtrt_stream_t stream, const void *a, const 
   DeviceState *st = device_state();
   if (!st)
     return MTRT_RUNTIME_ERROR;
+  if (M > 32 && M <= 64 && (N + 31) / 32 <= int64_t(num_compute_units(st))) {
+    // 33 to 64 rows while every compute unit has at most one 32-column tile: two launches of the small-M kernel
+    // (rows 0..31, then the rest) are shorter than one tile launch, which lasts a whole K loop of a 256-row tile
+    // that is mostly padding (M = 64 at (K, N) = (4096, 4096) 21.0 us, (11008, 4096) 47.0, (8192, 8192) 38.4).
+    const int32_t rc = mtrt_hip_gemm_w8a8_fragments(stream, a, w_frag, a_scale, w_scale, y, 32, K, N);
+    if (rc != MTRT_OK)
+      return rc;
+    return mtrt_hip_gemm_w8a8_fragments(stream, static_cast<const char *>(a) + 32 * K, w_frag, a_scale + 32, w_scale,
+                                        static_cast<char *>(y) + 32 * N * 2, M - 32, K, N);
+  }
+  if (M <= 32) {
+    // one workgroup per 32-column tile, its four waves splitting K; between one and two tiles per compute unit one
+    // workgroup per unit instead, the first ones taking a second tile (as for the int4 weights)
+    const int64_t tiles32 = (N + 31) / 32, cus = num_compute_units(st);
+    const uint32_t grid = uint32_t(M > 8 && tiles32 > cus && tiles32 <= 2 * cus ? cus : tiles32);
+    void *sargs[] = {&a, &w_frag, &a_scale, &w_scale, &y, &M, &K, &N};
+    return launch(st, KernelName(M <= 16 ? "mtrt_gemm_w8a8_small16" : "mtrt_gemm_w8a8_small32"), grid, kBlock, as_hip(stream), sargs);
+  }
   // Tiles and rounds as in mtrt_hip_gemm_w8a8: 256 x 256, one workgroup per compute unit at a time;
   // a last round that would use at most half of the units is cut into 128-wide half tiles.
   const int64_t panels = (N + 255) / 256, tiles_m = (M + 255) / 256, units = num_compute_units(st);

@@ -63,7 +63,26 @@ def test_w8a8_weights_in_registers_kernel(pkg, orc, shape):
     a, w, a_s, w_s = _w8a8_inputs(rng(M + K + N), M, K, N)
     print("case: w8a8 fragments", shape, flush=True)
     y, kernel = _run_w8a8_frag(pkg, a, w, a_s, w_s, from_nk=(M % 2 == 1))
-    assert kernel == "mtrt_gemm_w8a8_frag"
+    # 33..64 rows and at most one 32-column tile per compute unit: two launches of the small-M kernel, the last one for rows 32..M-1
+    assert kernel == ("mtrt_gemm_w8a8_small16" if M <= 16 or (32 < M <= 48 and N <= 8192) else "mtrt_gemm_w8a8_frag")
+    orc.set_threads(16)
+    ref = orc.gemm_w8a8(a, w, a_s, w_s)
+    orc.set_threads(1)
+    assert np.array_equal(bits16(y).reshape(M, N), ref)
+
+
+@pytest.mark.parametrize("shape", [(1, 128, 32), (16, 4096, 11008), (32, 4096, 11008), (17, 384, 200), (9, 1280, 4099), (13, 640, 8240),
+                                   (32, 256, 16384), (25, 512, 16400), (8, 2048, 8209), (16, 128, 40), (64, 512, 4100), (50, 256, 8192)])
+def test_w8a8_small_m_kernel(pkg, orc, shape):
+    """M <= 32: one workgroup per 32-column tile with four waves splitting K.  K = 128 and 384 leave waves without a
+    slice, 1280 gives them 2 or 3 (only the one-at-a-time tail), 4096 eight (two groups of four); N = 11008 gives 344
+    tiles (one workgroup per compute unit, the first 88 with two tiles), 16384 two each, 16400 and 8209 one tile beyond
+    those forms; ragged last tiles; M = 8 stays at one tile per workgroup.  Integer sums: bit-exact."""
+    M, K, N = shape
+    a, w, a_s, w_s = _w8a8_inputs(rng(M + K + N), M, K, N)
+    y, kernel = _run_w8a8_frag(pkg, a, w, a_s, w_s, from_nk=(M % 2 == 1))
+    last = M - 32 if M > 32 else M                       # 33..64 rows run as two launches
+    assert kernel == ("mtrt_gemm_w8a8_small16" if last <= 16 else "mtrt_gemm_w8a8_small32")
     orc.set_threads(16)
     ref = orc.gemm_w8a8(a, w, a_s, w_s)
     orc.set_threads(1)
