@@ -7,7 +7,11 @@
 // (mlir-tensorrt/kernel/test/Kernel/TransformSchedules/fallback-schedule-matmul.mlir:24); this is the same
 // class of kernel, tiled through LDS: 64 x 64 outputs per workgroup, 4 x 4 per lane, K in slices of 16.
 // w is [N,K] (K contiguous), the module's own weight layout; any M, N, K; no alignment needs.
-#include "common.hpp"
+// 16-bit operands whose rows are whole 128-byte slices (K % 64 == 0, 16-byte aligned) go to the matrix cores
+// instead (mtrt_gemm_dense_mfma_*): both operands are K-contiguous per row, which is the form the shared tile
+// loop of gemm_core.hpp takes (both panels through LDS, 256 x 256 tiles, v_mfma_f32_32x32x16_{f16,bf16}; a
+// product of two 16-bit floats is exact in f32), with the bias added to the f32 sum before the one narrowing.
+#include "gemm_core.hpp"
 
 using namespace mtrt_dev;
 
@@ -62,7 +66,105 @@ __device__ __forceinline__ void dense_body(const typename X::storage* __restrict
   }
 }
 
+// ---- matrix-core form for f16 / bf16 --------------------------------------------------------------------
+using gemm_core::v4i;
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef __bf16 v8b __attribute__((ext_vector_type(8)));
+
+template <typename X> struct HalfTraits;
+template <> struct HalfTraits<F16> {
+  using Acc = v16f;
+  static __device__ __forceinline__ Acc zero() {
+    Acc z;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) z[r] = 0.0f;
+    return z;
+  }
+  static __device__ __forceinline__ Acc mfma(v4i a, v4i b, Acc c) {
+    union { v4i i; v8h h; } ua, ub;
+    ua.i = a; ub.i = b;
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(ua.h, ub.h, c, 0, 0, 0);
+  }
+};
+template <> struct HalfTraits<BF16> {
+  using Acc = v16f;
+  static __device__ __forceinline__ Acc zero() { return HalfTraits<F16>::zero(); }
+  static __device__ __forceinline__ Acc mfma(v4i a, v4i b, Acc c) {
+    union { v4i i; v8b h; } ua, ub;
+    ua.i = a; ub.i = b;
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(ua.h, ub.h, c, 0, 0, 0);
+  }
+};
+
+template <typename X> __device__ __forceinline__ uint32_t narrow16(float v);
+template <> __device__ __forceinline__ uint32_t narrow16<F16>(float v) { return f32_to_f16_bits(v); }
+template <> __device__ __forceinline__ uint32_t narrow16<BF16>(float v) { return f32_to_bf16_bits(v); }
+
+// y = narrow(acc + f32(bias[n])) (no addition without a bias, as in the kernel above)
+template <typename X>
+struct BiasEpilogue {
+  const typename X::storage* bias;
+  const float* sb;                                   // bias of this tile's 256 columns as f32, in LDS
+  f32x4 br[2][4];
+  __device__ __forceinline__ void setup(int8_t* scratch, int64_t, int64_t, int64_t n0, int64_t N) {
+    float* dst = reinterpret_cast<float*>(scratch);
+    const int64_t col = n0 + threadIdx.x;             // 256 threads: 256 columns
+    if (threadIdx.x < 256) dst[threadIdx.x] = (bias && col < N) ? Tile<X>::load1(bias + col) : 0.0f;
+    sb = dst;
+  }
+  __device__ __forceinline__ void row(int) {}
+  template <int HC>
+  __device__ __forceinline__ void columns(int first_col_in_tile) {
+#pragma unroll
+    for (int jj = 0; jj < HC; ++jj)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) br[jj][q] = *reinterpret_cast<const f32x4*>(sb + first_col_in_tile + jj * 32 + q * 8);
+  }
+  __device__ __forceinline__ void convert4(const v16f& acc, int q, int jj, uint32_t (&bits)[4]) const {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float v = acc[4 * q + e];
+      if (bias) v = v + br[jj][q][e];
+      bits[e] = narrow16<X>(v);
+    }
+  }
+};
+
+template <typename X>
+__device__ __forceinline__ void dense_mfma_body(const typename X::storage* __restrict__ x, const typename X::storage* __restrict__ w,
+                                                const typename X::storage* __restrict__ bias, uint16_t* __restrict__ y, int64_t M,
+                                                int64_t K, int64_t N, int64_t full_panels, int8_t* lds) {
+  const int64_t tiles_m = (M + gemm_core::BM - 1) / gemm_core::BM;
+  const int64_t full_blocks = gemm_core::padded_blocks(full_panels, tiles_m);
+  BiasEpilogue<X> epi{bias, nullptr, {}};
+  const int8_t* a8 = reinterpret_cast<const int8_t*>(x);
+  const int8_t* w8 = reinterpret_cast<const int8_t*>(w);
+  int64_t tile_m, panel;
+  if (int64_t(blockIdx.x) < full_blocks) {
+    if (!gemm_core::tile_of(blockIdx.x, tiles_m, full_panels, tile_m, panel)) return;
+    gemm_core::run<HalfTraits<X>, 4>(a8, w8, K * 2, epi, y, M, N, K * 2 / gemm_core::BKB, tile_m * 256, panel * 256, lds);
+  } else {
+    const int64_t n_full = full_panels * 256;
+    if (!gemm_core::tile_of(blockIdx.x - full_blocks, tiles_m, (N - n_full + 127) / 128, tile_m, panel)) return;
+    gemm_core::run<HalfTraits<X>, 2>(a8, w8, K * 2, epi, y, M, N, K * 2 / gemm_core::BKB, tile_m * 256, n_full + panel * 128, lds);
+  }
+}
+
 }  // namespace dense_cluster
+
+// (x [M,K], w [N,K], bias [N] or null, y [M,N], M, K, N, full_panels) ; K % 64 == 0, x and w 16-byte aligned and below
+// 4 GiB each; tiles and grid as mtrt_gemm_w8a8_nk (256 x 256 for the first full_panels * 256 columns, 256 x 128 after),
+// block = 256.
+#define MTRT_DENSE_MFMA_KERNEL(XN, XT)                                                                             \
+  extern "C" __global__ void __launch_bounds__(gemm_core::THREADS, 1) mtrt_gemm_dense_mfma_##XN(                   \
+      const XT::storage* __restrict__ x, const XT::storage* __restrict__ w, const XT::storage* __restrict__ bias,  \
+      uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t full_panels) {                            \
+    __shared__ __attribute__((aligned(16))) int8_t lds[gemm_core::LDS_BYTES];                                      \
+    dense_cluster::dense_mfma_body<XT>(x, w, bias, y, M, K, N, full_panels, lds);                                  \
+  }
+MTRT_DENSE_MFMA_KERNEL(f16, F16)
+MTRT_DENSE_MFMA_KERNEL(bf16, BF16)
 
 // (x [M,K], w [N,K], bias [N] or null, y [M,N], M, K, N) ; grid = ceil(M/64) * ceil(N/64), block = 256
 #define MTRT_DENSE_KERNEL(XN, XT)                                                                                  \

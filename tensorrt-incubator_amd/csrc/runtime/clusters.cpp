@@ -764,6 +764,24 @@ int32_t mtrt_hip_linear_dense(mtrt_stream_t stream, const void *x, const void *w
   DeviceState *st = device_state();
   if (!st)
     return MTRT_RUNTIME_ERROR;
+  if (dtype != MTRT_F32 && K > 0 && K % 64 == 0 && aligned(x, 16) && aligned(w_nk, 16) && M * K * 2 < (int64_t(1) << 32) &&
+      N * K * 2 < (int64_t(1) << 32)) {
+    // 16-bit operands in whole 128-byte slices of K: the matrix-core tile loop (tiles and rounds as in
+    // mtrt_hip_gemm_w8a8; f16 [2048, 4096] x [11008, 4096]: 3654 us on the FMA kernel below)
+    const int64_t panels = (N + 255) / 256, tiles_m = (M + 255) / 256, units = num_compute_units(st);
+    const int64_t tiles256 = panels * tiles_m, rest = tiles256 % units;
+    int64_t full_panels = panels;
+    if (tiles256 * 2 <= units)
+      full_panels = 0;
+    else if (rest > 0 && rest * 2 <= units)
+      full_panels = panels - (rest + tiles_m - 1) / tiles_m;
+    const int64_t half_panels = (N - full_panels * 256 + 127) / 128;
+    const int64_t grid = 8 * ((full_panels + 7) / 8) * tiles_m + 8 * ((half_panels + 7) / 8) * tiles_m;
+    if (grid <= int64_t(kMaxGrid) * 1024) {
+      void *margs[] = {&x, &w_nk, &bias, &y, &M, &K, &N, &full_panels};
+      return launch(st, KernelName("mtrt_gemm_dense_mfma_") + xn, uint32_t(grid), kBlock, as_hip(stream), margs);
+    }
+  }
   const int64_t tiles = ((M + 63) / 64) * ((N + 63) / 64);
   if (tiles > int64_t(kMaxGrid) * 1024)
     return set_error(MTRT_INVALID_ARGUMENT, "problem [%lld, %lld] needs too many tiles", (long long)M, (long long)N);

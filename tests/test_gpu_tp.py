@@ -293,14 +293,16 @@ def test_dense_linear_against_float64(tp, pkg, dname):
     d = getattr(tp, dname)
     td = {"float32": torch.float32, "float16": torch.float16, "bfloat16": torch.bfloat16}[dname]
     torch.manual_seed(5)
-    for lead, K, N in (((3, 7), 50, 33), ((130,), 64, 129), ((1,), 1, 1)):
+    for lead, K, N in (((3, 7), 50, 33), ((130,), 64, 129), ((1,), 1, 1), ((2, 300), 256, 520), ((700,), 1024, 8200)):
         x = torch.randn(*lead, K, dtype=torch.float32).to(td)
         w = (torch.randn(N, K, dtype=torch.float32) * 0.2).to(td)
         b = torch.randn(N, dtype=torch.float32).to(td)
         lin = tp.Linear(K, N, dtype=d)
         lin.weight, lin.bias = tp.Tensor(w, dtype=d), tp.Tensor(b, dtype=d)
         out = lin(tp.Tensor(x, dtype=d)).torch()
-        assert pkg.last_kernel() == "mtrt_gemm_dense_" + {"float32": "f32", "float16": "f16", "bfloat16": "bf16"}[dname]
+        # 16-bit operands with K a multiple of 64 run on the matrix cores, everything else on the FMA tiles
+        mfma = dname != "float32" and K % 64 == 0
+        assert pkg.last_kernel() == ("mtrt_gemm_dense_mfma_" if mfma else "mtrt_gemm_dense_") + {"float32": "f32", "float16": "f16", "bfloat16": "bf16"}[dname]
         assert tuple(out.shape) == lead + (N,)
         ref = x.double() @ w.double().T + b.double()
         mag = x.double().abs() @ w.double().abs().T + b.double().abs()
