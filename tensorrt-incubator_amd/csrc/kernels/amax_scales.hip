@@ -172,6 +172,51 @@ __device__ __forceinline__ void cols_split_body(const typename X::storage* __res
   }
 }
 
+// row kind, few scales (a channel axis of a few dozen entries in front of large inner extents, or a handful of very
+// long rows): one wave per scale leaves the chip empty.  The rows of scale s (s, s + nb, ...) are cut into tiles
+// of kRowChunk vectors; `parts` workgroups share the tiles of a scale (workgroup s * parts + p the p-th range of
+// them, its four waves one tile at a time) and meet in stage[s] (zero on entry) by atomic max, one per workgroup;
+// mtrt_amax_finish_* follows.  d1 % G == 0, x 16-byte aligned.
+constexpr int kRowChunk = 1024;                      // vectors per tile: 16 per lane, four loads in flight at a time
+
+template <typename X>
+__device__ __forceinline__ void rows_split_body(const typename X::storage* __restrict__ x, int64_t d0, int64_t d1, int64_t nb,
+                                                int64_t parts, uint32_t* __restrict__ stage) {
+  using A = AbsBits<X>;
+  __shared__ uint32_t wave_max[4];
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int64_t s = blockIdx.x / parts, p = blockIdx.x % parts;
+  const int64_t nvec = d1 / A::kPerVec, chunks = (nvec + kRowChunk - 1) / kRowChunk;
+  const int64_t rows_s = (d0 - s + nb - 1) / nb;     // rows s, s + nb, ... below d0
+  const int64_t tiles = rows_s * chunks;
+  const int64_t t0 = tiles * p / parts, t1 = tiles * (p + 1) / parts;
+  uint32_t m = 0;
+  for (int64_t t = t0 + wave; t < t1; t += 4) {
+    const int64_t i = t / chunks, c = t - i * chunks;
+    const u32x4* pv = reinterpret_cast<const u32x4*>(x + (s + i * nb) * d1);
+    const int64_t v1 = (c + 1) * kRowChunk < nvec ? (c + 1) * kRowChunk : nvec;
+    int64_t v = c * kRowChunk + lane;
+    for (; v + 3 * kWave < v1; v += 4 * kWave) {       // four independent loads in flight
+      u32x4 tt[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) tt[u] = __builtin_nontemporal_load(pv + v + u * kWave);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) { const uint32_t a = A::of(tt[u]); m = m > a ? m : a; }
+    }
+    for (; v < v1; v += kWave) { const uint32_t a = A::of(__builtin_nontemporal_load(pv + v)); m = m > a ? m : a; }
+  }
+  m = wave_reduce(m, MaxU32());
+  if (lane == 0) wave_max[wave] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t r = wave_max[0];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) r = r > wave_max[w] ? r : wave_max[w];
+    // nobody reads the word before the launch has ended: no ordering, no return value
+    __hip_atomic_fetch_max(stage + s, r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
 // stage word (maximum bit pattern) -> amax and scale; `stage` may be amax_out or scale_out itself
 template <typename X>
 __device__ __forceinline__ void finish_body(const uint32_t* stage, int64_t count, float qmax, float* amax_out, float* scale_out) {
@@ -200,6 +245,7 @@ __device__ __forceinline__ void cols_any_body(const typename X::storage* __restr
 //   rows / rows_any : grid = ceil(nb / 4), block = 256 (one wave per scale)
 //   cols            : grid = (d0 / nb) * ceil(d1 / G / 64), block = 256 ; d1 % G == 0, x 16-byte aligned
 //   cols_any        : grid-stride, block = 256
+// (x, d0, d1, nb, parts, stage) rows_split : grid = nb * parts, block = 256 ; stage = nb zeroed words ; then finish
 // (x, d0, d1, nb, rows_per_part, stage) cols_split : grid = (d0 / nb) * ceil(d1 / G / 64) * ceil(nb / rows_per_part),
 //   block = 256 ; stage = (d0 / nb) * d1 zeroed words ; then (stage, count, qmax, amax_out or null, scale_out or null)
 //   finish : grid = ceil(count / 256), block = 256
@@ -216,6 +262,9 @@ __device__ __forceinline__ void cols_any_body(const typename X::storage* __restr
   extern "C" __global__ void __launch_bounds__(256) mtrt_amax_cols_split_##XN(                                         \
       const XT::storage* x, int64_t d0, int64_t d1, int64_t nb, int64_t rows_per_part, uint32_t* stage) {              \
     amax_scales_cluster::cols_split_body<XT>(x, d0, d1, nb, rows_per_part, stage); }                                   \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_amax_rows_split_##XN(                                         \
+      const XT::storage* x, int64_t d0, int64_t d1, int64_t nb, int64_t parts, uint32_t* stage) {                      \
+    amax_scales_cluster::rows_split_body<XT>(x, d0, d1, nb, parts, stage); }                                           \
   extern "C" __global__ void __launch_bounds__(256) mtrt_amax_finish_##XN(                                             \
       const uint32_t* stage, int64_t count, float qmax, float* amax_out, float* scale_out) {                           \
     amax_scales_cluster::finish_body<XT>(stage, count, qmax, amax_out, scale_out); }                                   \

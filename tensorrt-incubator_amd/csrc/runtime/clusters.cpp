@@ -238,6 +238,33 @@ int32_t mtrt_hip_amax_scales(mtrt_stream_t stream, const void *x, int32_t dtype,
   const int group = dtype == MTRT_F32 ? 4 : 8;
   const bool vec = d1 % group == 0 && aligned(x, 16);
   void *args[] = {&x, &d0, &d1, &nb, &qmax, &amax_out, &scale_out};
+  if (scale_kind == MTRT_SCALE_ROW && vec && nb < 4 * int64_t(num_compute_units(st)) && nb <= d0) {
+    // Few scales (one wave each would leave most of the chip idle): the tiles of a scale's rows (1024 vectors each)
+    // are shared by several workgroups that meet in the output word by atomic max, about two workgroups per compute
+    // unit in all; then the finishing launch.  Measured on f16 [65536, 1024]: nb = 64 945.6 us, nb = 8 7684 us as one
+    // wave per scale; [8, 8M] with nb = 8 2387 us.
+    const int64_t units = num_compute_units(st), nvec = d1 / group;
+    const int64_t tiles = ((d0 + nb - 1) / nb) * ((nvec + 1023) / 1024);     // of the scale with the most rows
+    const int64_t parts = std::max<int64_t>(1, std::min<int64_t>((2 * units + nb - 1) / nb, (tiles + 3) / 4));
+    if (parts > 1) {
+      int64_t count = nb;
+      uint32_t *stage = reinterpret_cast<uint32_t *>(amax_out ? amax_out : scale_out);
+      uint8_t *stage_bytes = reinterpret_cast<uint8_t *>(stage);
+      uint32_t zero = 0;
+      int32_t width = 4;
+      void *fill_args[] = {&stage_bytes, &count, &zero, &width};
+      int32_t rc = launch(st, KernelName("mtrt_fill"), blocks_for(count, kBlock), kBlock, as_hip(stream), fill_args);
+      if (rc != MTRT_OK)
+        return rc;
+      int64_t parts_arg = parts;
+      void *split_args[] = {&x, &d0, &d1, &nb, &parts_arg, &stage};
+      rc = launch(st, KernelName("mtrt_amax_rows_split_") + xn, uint32_t(nb * parts), kBlock, as_hip(stream), split_args);
+      if (rc != MTRT_OK)
+        return rc;
+      void *finish_args[] = {&stage, &count, &qmax, &amax_out, &scale_out};
+      return launch(st, KernelName("mtrt_amax_finish_") + xn, blocks_for(count, kBlock), kBlock, as_hip(stream), finish_args);
+    }
+  }
   if (scale_kind == MTRT_SCALE_ROW) {
     const int64_t blocks = (nb + 3) / 4;
     if (blocks > int64_t(kMaxGrid) * 1024)

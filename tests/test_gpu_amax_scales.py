@@ -54,8 +54,8 @@ def test_every_addressing_on_ragged_shapes(pkg, orc, xname):
     grp = 4 if xname == "f32" else 8
     k = "_" + xname
     cases = [
-        ("row", 37, 16 * grp * 9 + grp, 37, "mtrt_amax_rows" + k),          # one scale per row, rows longer than one pass
-        ("row", 60, grp * 5, 12, "mtrt_amax_rows" + k),                      # channel on a middle axis: 5 rows per scale
+        ("row", 37, 16 * grp * 9 + grp, 37, "mtrt_amax_rows" + k),          # one scale per row (one tile each: no sharing)
+        ("row", 60, grp * 5, 12, "mtrt_amax_finish" + k),                    # channel on a middle axis: 5 rows per scale, two workgroups each
         ("row", 9, 131, 9, "mtrt_amax_rows_any" + k),                        # row length not a vector multiple
         ("row", 1, 7, 1, "mtrt_amax_rows_any" + k),
         ("col", 48, grp * 70, 16, "mtrt_amax_cols" + k),                     # two strips of 64 vectors, 16-row blocks
@@ -94,6 +94,23 @@ def test_per_channel_scales_of_a_k_by_n_weight(pkg, orc, xname):
         pkg.check(L.mtrt_hip_amax_scales(st, xd.data_ptr(), px, pkg.SCALE_COL, d0, d1, nb, 127.0, only.data_ptr(), None))
         a_ref, _ = orc.amax_scales(xs, {"f32": orc.F32, "f16": orc.F16, "bf16": orc.BF16}[xname], orc.SCALE_COL, d0, d1, nb, 127.0)
         assert np.array_equal(f32_bits(only.cpu().numpy()), f32_bits(a_ref))
+    finally:
+        orc.set_threads(1)
+
+
+@pytest.mark.parametrize("xname", ["f32", "f16", "bf16"])
+def test_few_row_scales_share_workgroups(pkg, orc, xname):
+    """Row kind with a handful of scales (a short channel axis in front of large inner extents, or a few very long
+    rows): several workgroups per scale meet by atomic max, then the finishing launch.  Rows per scale that differ
+    (37 rows, 5 scales), rows longer than one tile of 1024 vectors, one scale."""
+    grp = 4 if xname == "f32" else 8
+    g = rng(31)
+    orc.set_threads(16)
+    try:
+        for d0, d1, nb in ((512, grp * 300, 8), (8, grp * 5000, 8), (37, grp * 130, 5), (2048, grp * 64, 64), (3, grp * 2049, 1)):
+            x = (g.standard_normal(d0 * d1) * 0.7).astype(np.float32)
+            x[g.integers(0, x.size, 20)] *= 30.0
+            _run(pkg, orc, x, xname, "row", d0, d1, nb, 127.0, "mtrt_amax_finish_" + xname)
     finally:
         orc.set_threads(1)
 
