@@ -200,15 +200,62 @@ __device__ __forceinline__ void write_tile(Acc (&acc)[IT][JT], Epilogue& epi, ui
   }
 }
 
+// The same sub-tiles written as f32, straight from the accumulators: a lane's runs of four consecutive outputs of a
+// row are one 16-byte store each (32-byte pieces of a row per half wave, merged in the write-back cache); no staging.
+// Epilogue: finish4(values of columns col .. col+3, col, N).  For the 2 x 2 waves of `run`.
+template <int JT, class Acc, class Epilogue>
+__device__ __forceinline__ void write_tile_f32(Acc (&acc)[4][JT], Epilogue& epi, float* __restrict__ y, int64_t M, int64_t N,
+                                               int64_t m0, int64_t n0, int wave) {
+  const int lane = threadIdx.x & 63;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int frow = lane & 31, fhalf = lane >> 5;
+  const bool vec_ok = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(y) & 15) == 0);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int64_t row = m0 + wm * 128 + i * 32 + frow;
+    if (row >= M) continue;
+#pragma unroll
+    for (int j = 0; j < JT; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int64_t col = n0 + wn * (32 * JT) + j * 32 + q * 8 + fhalf * 4;
+        if (col >= N) continue;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * q + e];
+        epi.finish4(v, col, N);
+        if (vec_ok && col + 3 < N) {
+          const f32x4 t = {v[0], v[1], v[2], v[3]};
+          __builtin_nontemporal_store(t, reinterpret_cast<f32x4*>(y + row * N + col));
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (col + e < N) y[row * N + col + e] = v[e];
+        }
+      }
+  }
+}
+template <int JT, class Acc, class Epilogue>
+__device__ __forceinline__ void finish_tile(Acc (&acc)[4][JT], Epilogue& epi, uint16_t* __restrict__ y, int64_t M, int64_t N,
+                                            int64_t m0, int64_t n0, int8_t* lds, int wave) {
+  write_tile<JT, 2, 4>(acc, epi, y, M, N, m0, n0, lds, wave, true);
+}
+template <int JT, class Acc, class Epilogue>
+__device__ __forceinline__ void finish_tile(Acc (&acc)[4][JT], Epilogue& epi, float* __restrict__ y, int64_t M, int64_t N,
+                                            int64_t m0, int64_t n0, int8_t*, int wave) {
+  write_tile_f32<JT>(acc, epi, y, M, N, m0, n0, wave);
+}
+
 // Both operands as bytes, K-contiguous per row / per column: a [M, a_row_bytes], b [N, a_row_bytes].
 // 4 waves (2 x 2) compute a 256 x (64 * JT) tile: JT = 4 is the full tile, JT = 2 the half-width
 // tile that fills the last, partial round of a launch.
 // Traits: Acc (16-wide accumulator vector), mfma(first, second, acc), zero().
 // Epilogue: setup(lds scratch, m0, M, n0, N), columns<HC>(first column of the lane in the tile), row(row in tile),
 // convert4(acc, q, column tile of the pass, bits).
-template <class Traits, int JT, class Epilogue>
+// Y: uint16_t (16-bit outputs through the staged epilogue) or float (direct stores, see write_tile_f32).
+template <class Traits, int JT, class Epilogue, typename Y>
 __device__ __forceinline__ void run(const int8_t* __restrict__ a, const int8_t* __restrict__ b, int64_t row_bytes, Epilogue& epi,
-                                    uint16_t* __restrict__ y, int64_t M, int64_t N, int64_t slices, int64_t m0,
+                                    Y* __restrict__ y, int64_t M, int64_t N, int64_t slices, int64_t m0,
                                     int64_t n0, int8_t* lds) {
   using Acc = typename Traits::Acc;
   constexpr int GB = 2 * JT;                           // direct-to-LDS loads per wave and slice for the B panel
@@ -300,7 +347,7 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, const int8_t* 
   }
   if (s < slices) slice_body(IntC<0>{}, s);
 
-  write_tile<JT, 2, 4>(acc, epi, y, M, N, m0, n0, lds, wave, true);
+  finish_tile<JT>(acc, epi, y, M, N, m0, n0, lds, wave);
 }
 
 // Tile order: the hardware deals consecutive workgroup ids round-robin to the 8 XCDs, each with

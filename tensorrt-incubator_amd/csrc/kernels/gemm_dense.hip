@@ -97,6 +97,28 @@ template <> struct HalfTraits<BF16> {
   }
 };
 
+// f32 operands: a 16-byte fragment holds four k values per lane, and v_mfma_f32_32x32x2_f32 takes one per lane (the two
+// halves of the wave supplying its two k values), so a fragment pair is four chained instructions; which k values
+// meet in one instruction does not matter as long as both operands agree.
+struct F32Traits {
+  using Acc = v16f;
+  static __device__ __forceinline__ Acc zero() { return HalfTraits<F16>::zero(); }
+  static __device__ __forceinline__ Acc mfma(v4i a, v4i b, Acc c) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) c = __builtin_amdgcn_mfma_f32_32x32x2f32(bits_to_f32(uint32_t(a[e])), bits_to_f32(uint32_t(b[e])), c, 0, 0, 0);
+    return c;
+  }
+};
+struct BiasF32Epilogue {
+  const float* bias;
+  __device__ __forceinline__ void finish4(float (&v)[4], int64_t col, int64_t N) const {
+    if (!bias) return;
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (col + e < N) v[e] = v[e] + bias[col + e];
+  }
+};
+
 template <typename X> __device__ __forceinline__ uint32_t narrow16(float v);
 template <> __device__ __forceinline__ uint32_t narrow16<F16>(float v) { return f32_to_f16_bits(v); }
 template <> __device__ __forceinline__ uint32_t narrow16<BF16>(float v) { return f32_to_bf16_bits(v); }
@@ -151,7 +173,35 @@ __device__ __forceinline__ void dense_mfma_body(const typename X::storage* __res
   }
 }
 
+__device__ __forceinline__ void dense_mfma_f32_body(const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ bias,
+                                                    float* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t full_panels,
+                                                    int8_t* lds) {
+  const int64_t tiles_m = (M + gemm_core::BM - 1) / gemm_core::BM;
+  const int64_t full_blocks = gemm_core::padded_blocks(full_panels, tiles_m);
+  BiasF32Epilogue epi{bias};
+  const int8_t* a8 = reinterpret_cast<const int8_t*>(x);
+  const int8_t* w8 = reinterpret_cast<const int8_t*>(w);
+  int64_t tile_m, panel;
+  if (int64_t(blockIdx.x) < full_blocks) {
+    if (!gemm_core::tile_of(blockIdx.x, tiles_m, full_panels, tile_m, panel)) return;
+    gemm_core::run<F32Traits, 4>(a8, w8, K * 4, epi, y, M, N, K * 4 / gemm_core::BKB, tile_m * 256, panel * 256, lds);
+  } else {
+    const int64_t n_full = full_panels * 256;
+    if (!gemm_core::tile_of(blockIdx.x - full_blocks, tiles_m, (N - n_full + 127) / 128, tile_m, panel)) return;
+    gemm_core::run<F32Traits, 2>(a8, w8, K * 4, epi, y, M, N, K * 4 / gemm_core::BKB, tile_m * 256, n_full + panel * 128, lds);
+  }
+}
+
 }  // namespace dense_cluster
+
+// f32 operands: (x [M,K], w [N,K], bias [N] or null, y [M,N], M, K, N, full_panels) ; K % 32 == 0, x and w 16-byte aligned
+// and below 4 GiB each; tiles, grid and block as for the 16-bit kernels below.
+extern "C" __global__ void __launch_bounds__(gemm_core::THREADS, 1) mtrt_gemm_dense_mfma_f32(
+    const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ bias, float* __restrict__ y, int64_t M,
+    int64_t K, int64_t N, int64_t full_panels) {
+  __shared__ __attribute__((aligned(16))) int8_t lds[gemm_core::LDS_BYTES];
+  dense_cluster::dense_mfma_f32_body(x, w, bias, y, M, K, N, full_panels, lds);
+}
 
 // (x [M,K], w [N,K], bias [N] or null, y [M,N], M, K, N, full_panels) ; K % 64 == 0, x and w 16-byte aligned and below
 // 4 GiB each; tiles and grid as mtrt_gemm_w8a8_nk (256 x 256 for the first full_panels * 256 columns, 256 x 128 after),

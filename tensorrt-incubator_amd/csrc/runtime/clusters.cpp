@@ -791,10 +791,10 @@ int32_t mtrt_hip_linear_dense(mtrt_stream_t stream, const void *x, const void *w
   DeviceState *st = device_state();
   if (!st)
     return MTRT_RUNTIME_ERROR;
-  if (dtype != MTRT_F32 && K > 0 && K % 64 == 0 && aligned(x, 16) && aligned(w_nk, 16) && M * K * 2 < (int64_t(1) << 32) &&
-      N * K * 2 < (int64_t(1) << 32)) {
-    // 16-bit operands in whole 128-byte slices of K: the matrix-core tile loop (tiles and rounds as in
-    // mtrt_hip_gemm_w8a8; f16 [2048, 4096] x [11008, 4096]: 3654 us on the FMA kernel below)
+  if (K > 0 && (K * eb) % 128 == 0 && aligned(x, 16) && aligned(w_nk, 16) && M * K * eb < (int64_t(1) << 32) &&
+      N * K * eb < (int64_t(1) << 32)) {
+    // operands in whole 128-byte slices of K: the matrix-core tile loop (tiles and rounds as in
+    // mtrt_hip_gemm_w8a8; f16 [2048, 4096] x [11008, 4096]: 3654 us on the FMA kernel below, f32 3835 us)
     const int64_t panels = (N + 255) / 256, tiles_m = (M + 255) / 256, units = num_compute_units(st);
     const int64_t tiles256 = panels * tiles_m, rest = tiles256 % units;
     int64_t full_panels = panels;
