@@ -549,6 +549,107 @@ __device__ __forceinline__ void qdq_groups(const typename X::storage* __restrict
   }
 }
 
+// Row and column scales on rows that are not whole groups (d1 % G != 0) or on operands that are not aligned for group
+// accesses: the element-per-lane kernel below moves one or two bytes per lane and instruction and runs at a sixth of
+// the memory rate.  Here a wave takes 64 consecutive groups of ONE row at a time, with 128-bit accesses at element
+// alignment (the hardware splits those that straddle a cache line) and the codes as unaligned 4- or 8-byte stores;
+// the d1 % G elements behind a row's last whole group go one each to the first lanes.  A group never straddles rows,
+// so a row scale is uniform per group (short exact division, as in qdq_groups) and column scales are G consecutive
+// floats.  Codes one per byte (i8, f8, i4); packed nibbles stay with the kernel below (a byte can straddle rows).
+typedef u32x4 u32x4_unaligned __attribute__((aligned(2)));
+typedef f32x4 f32x4_unaligned __attribute__((aligned(4)));
+typedef uint32_t u32_unaligned __attribute__((aligned(1)));
+
+template <typename X, typename Q, int KIND, int MODE>
+__device__ __forceinline__ void qdq_rows_ragged(const typename X::storage* __restrict__ x, typename Q::storage* __restrict__ q,
+                                                typename X::storage* __restrict__ y, const float* __restrict__ scale,
+                                                int64_t n, int64_t d1, int64_t nb, int flags) {
+  using FG = FloatGroup<X>;
+  constexpr int G = FG::G;
+  const int64_t d0 = n / d1, nvec = d1 / G;
+  const int tail = int(d1 - nvec * G);
+  const int64_t chunks = nvec > 0 ? (nvec + kWave - 1) / kWave : 1;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t wave = (int64_t(blockIdx.x) * blockDim.x + threadIdx.x) / kWave;
+  const int64_t nwaves = int64_t(gridDim.x) * blockDim.x / kWave;
+  const int64_t items = d0 * chunks;
+  for (int64_t item = wave; item < items; item += nwaves) {
+    const int64_t row = item / chunks, c = item - row * chunks;
+    const int64_t v = c * kWave + lane;
+    const int64_t e0 = row * d1 + v * G;
+    const float* srow = KIND == kRow ? scale + row % nb : scale + (row / nb) * d1;
+    if (v < nvec) {
+      float f[G], sc[G];
+      if (KIND == kRow) {
+        const float s = srow[0];
+#pragma unroll
+        for (int k = 0; k < G; ++k) sc[k] = s;
+      } else {
+#pragma unroll
+        for (int k = 0; k < G / 4; ++k) {
+          const f32x4 t = *reinterpret_cast<const f32x4_unaligned*>(srow + v * G + 4 * k);
+          sc[4 * k] = t.x; sc[4 * k + 1] = t.y; sc[4 * k + 2] = t.z; sc[4 * k + 3] = t.w;
+        }
+      }
+      uint32_t w[G / 4];
+      if (MODE == 1) {
+#pragma unroll
+        for (int i = 0; i < G / 4; ++i) {
+          w[i] = *reinterpret_cast<const u32_unaligned*>(q + e0 + 4 * i);
+          unpack4<Q>(w[i], &f[4 * i]);
+        }
+      } else {
+        const u32x4 t = *reinterpret_cast<const u32x4_unaligned*>(x + e0);
+        FG::unpack(t, f);
+        if (KIND == kRow) {
+          const ExactDivisor dv(sc[0]);
+          quantize_group<Q>(dv, f, flags);
+        } else {
+#pragma unroll
+          for (int k = 0; k < G; ++k) f[k] = quant_value<Q>(f[k], sc[k], flags);
+        }
+#pragma unroll
+        for (int i = 0; i < G / 4; ++i) {
+          w[i] = pack4<Q>(&f[4 * i], flags);
+          unpack4<Q>(w[i], &f[4 * i]);                 // f32(code): what a following dequantize multiplies
+          *reinterpret_cast<u32_unaligned*>(q + e0 + 4 * i) = w[i];
+        }
+      }
+      if (MODE != 0) {
+#pragma unroll
+        for (int k = 0; k < G; ++k) f[k] = f[k] * sc[k];
+        u32x4 t;
+        if (G == 4) {
+          t = (u32x4){f32_to_bits(f[0]), f32_to_bits(f[1]), f32_to_bits(f[2]), f32_to_bits(f[3])};
+          *reinterpret_cast<u32x4_unaligned*>(y + e0) = t;
+        } else {
+          // 16-bit outputs: narrowed one by one through the element form, then stored as one vector
+          typename X::storage h[8];
+#pragma unroll
+          for (int k = 0; k < 8; ++k) Tile<X>::store1(&h[k % G], f[k % G]);
+#pragma unroll
+          for (int k = 0; k < 4; ++k) t[k] = uint32_t(uint16_t(h[(2 * k) % G])) | (uint32_t(uint16_t(h[(2 * k + 1) % G])) << 16);
+          *reinterpret_cast<u32x4_unaligned*>(y + e0) = t;
+        }
+      }
+    }
+    if (c == chunks - 1 && lane < tail) {              // the row's last d1 % G elements, one per lane
+      const int64_t col = nvec * G + lane, e = row * d1 + col;
+      const float s = KIND == kRow ? srow[0] : srow[col];
+      float fv;
+      if (MODE == 1) {
+        fv = Codes<Q>::dec(uint32_t(uint8_t(q[e])));
+      } else {
+        fv = quant_value<Q>(Tile<X>::load1(x + e), s, flags);
+        const uint32_t code = Codes<Q>::enc(fv, flags);
+        q[e] = typename Q::storage(code);
+        fv = Codes<Q>::dec(code);
+      }
+      if (MODE != 0) Tile<X>::store1(y + e, fv * s);
+    }
+  }
+}
+
 // Any shape, any alignment: one element per lane (packed int4: one byte = two
 // elements per lane), scale kind chosen at run time.
 template <typename X, typename Q, int MODE>
@@ -638,6 +739,26 @@ using namespace qdq_cluster;
 MTRT_QDQ_FOR_FLOAT(f32, F32)
 MTRT_QDQ_FOR_FLOAT(f16, F16)
 MTRT_QDQ_FOR_FLOAT(bf16, BF16)
+
+// Ragged rows / unaligned operands with row or column scales: mtrt_{q,dq,qdq}_{rowu,colu}_<float type>_<code type>,
+// arguments as the kernels above; grid-stride over (row, chunk of 64 groups), block = 256; codes i8, f8, i4.
+#define MTRT_QDQ_RAGGED_KERNELS(XN, XT, QN, QT, KN, KIND)                                                          \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_q_##KN##_##XN##_##QN(                                     \
+      const XT::storage* x, QT::storage* q, const float* scale, int64_t n, int64_t d1, int64_t nb, int32_t flags) { \
+    qdq_rows_ragged<XT, QT, KIND, 0>(x, q, nullptr, scale, n, d1, nb, flags); }                                    \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_dq_##KN##_##XN##_##QN(                                    \
+      const QT::storage* q, XT::storage* y, const float* scale, int64_t n, int64_t d1, int64_t nb) {              \
+    qdq_rows_ragged<XT, QT, KIND, 1>(nullptr, const_cast<QT::storage*>(q), y, scale, n, d1, nb, 0); }              \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_qdq_##KN##_##XN##_##QN(                                   \
+      const XT::storage* x, QT::storage* q, XT::storage* y, const float* scale, int64_t n, int64_t d1, int64_t nb, \
+      int32_t flags) { qdq_rows_ragged<XT, QT, KIND, 2>(x, q, y, scale, n, d1, nb, flags); }
+#define MTRT_QDQ_RAGGED_FOR_FLOAT(XN, XT)                                                                          \
+  MTRT_QDQ_RAGGED_KERNELS(XN, XT, i8, I8, rowu, kRow) MTRT_QDQ_RAGGED_KERNELS(XN, XT, i8, I8, colu, kCol)          \
+  MTRT_QDQ_RAGGED_KERNELS(XN, XT, f8, F8, rowu, kRow) MTRT_QDQ_RAGGED_KERNELS(XN, XT, f8, F8, colu, kCol)          \
+  MTRT_QDQ_RAGGED_KERNELS(XN, XT, i4, I4, rowu, kRow) MTRT_QDQ_RAGGED_KERNELS(XN, XT, i4, I4, colu, kCol)
+MTRT_QDQ_RAGGED_FOR_FLOAT(f32, F32)
+MTRT_QDQ_RAGGED_FOR_FLOAT(f16, F16)
+MTRT_QDQ_RAGGED_FOR_FLOAT(bf16, BF16)
 
 // ---- strided views ------------------------------------------------------------------
 // The same element-wise programs on rank-2 VIEWS: each tensor operand arrives as the reference expands a fully

@@ -115,10 +115,15 @@ int32_t qdq_dispatch(int mode, hipStream_t stream, const void *x, int32_t x_dtyp
   if (kind == MTRT_SCALE_COL)
     tiles = tiles && aligned(scale, 16);
 
+  // Row or column scales on rows that are not whole groups, or on operands not aligned for group accesses: a wave
+  // per 64 groups of one row with accesses at element alignment (codes one per byte only: a packed byte can
+  // straddle rows).  Everything else that is not `tiles`: one element per lane.
+  const bool ragged = !tiles && kind != MTRT_SCALE_UNIFORM && !nibbles;
   static const char *kModeName[] = {"q", "dq", "qdq"};
   static const char *kKindName[] = {"uniform", "row", "col"};
+  static const char *kRaggedName[] = {"", "rowu", "colu"};
   KernelName name("mtrt_");
-  name + kModeName[mode] + "_" + (tiles ? kKindName[kind] : "any") + "_" + xn + "_" + qn;
+  name + kModeName[mode] + "_" + (tiles ? kKindName[kind] : (ragged ? kRaggedName[kind] : "any")) + "_" + xn + "_" + qn;
 
   int64_t n_arg = n, d1_arg = d1, nb_arg = nb;
   int32_t kind_arg = kind, flags_arg = flags;
@@ -134,13 +139,17 @@ int32_t qdq_dispatch(int mode, hipStream_t stream, const void *x, int32_t x_dtyp
   args[na++] = &n_arg;
   args[na++] = &d1_arg;
   args[na++] = &nb_arg;
-  if (!tiles) args[na++] = &kind_arg;
+  if (!tiles && !ragged) args[na++] = &kind_arg;
   if (mode != 1) args[na++] = &flags_arg;
 
   if (tiles && kind == MTRT_SCALE_COL) {
     // one wave per (scale block, chunk of 32 rows of it, strip of 64 groups of columns): see qdq_col_strips
     const int64_t items = (d0 / nb) * ((nb + 31) / 32) * ((d1 / group + 63) / 64);
     return launch(st, name, blocks_for(items, kBlock / 64), kBlock, stream, args);
+  }
+  if (ragged) {
+    const int64_t chunks = std::max<int64_t>(1, (d1 / group + 63) / 64);
+    return launch(st, name, blocks_for(d0 * chunks, kBlock / 64), kBlock, stream, args);
   }
   const int64_t units = tiles ? (n + kTile - 1) / kTile : (nibbles ? (n + 1) / 2 : n);
   return launch(st, name, blocks_for(units, kBlock), kBlock, stream, args);

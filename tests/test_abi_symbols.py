@@ -78,6 +78,11 @@ def test_embedded_code_object_is_gfx950_and_has_the_kernels(pkg):
             for x in ("f32", "f16", "bf16"):
                 for q in ("i8", "f8", "i4", "i4p", "f4p"):
                     names.append("mtrt_%s_%s_%s_%s" % (mode, kind, x, q))
+    for mode in ("q", "dq", "qdq"):
+        for kind in ("rowu", "colu"):
+            for x in ("f32", "f16", "bf16"):
+                for q in ("i8", "f8", "i4"):
+                    names.append("mtrt_%s_%s_%s_%s" % (mode, kind, x, q))
     for x in ("f32", "f16", "bf16"):
         names.append("mtrt_amax_" + x)
         for v in ("v1", "v2", "v4", "v8", "v16", "any"):

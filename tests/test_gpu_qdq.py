@@ -169,14 +169,29 @@ def test_per_channel(pkg, orc, xname, qname):
     x = g.standard_normal((4, 6, 128), dtype=np.float32)
     s = g.uniform(0.005, 0.05, 6).astype(np.float32)
     _check_all(pkg, orc, x, xname, qname, pkg.SCALE_ROW, 24, 128, 6, s)
-    # ragged inner extent -> generic kernel
+    # ragged inner extent -> the kernels that walk one row at a time with accesses at element alignment
     x = g.standard_normal((7, 5, 9), dtype=np.float32)
     s = g.uniform(0.005, 0.05, 5).astype(np.float32)
     k = _check_all(pkg, orc, x, xname, qname, pkg.SCALE_ROW, 35, 9, 5, s)
-    assert "_any_" in k[0]
+    assert "_rowu_" in k[0] and "_rowu_" in k[1] and "_rowu_" in k[2]
     s = g.uniform(0.005, 0.05, 9).astype(np.float32)
     k = _check_all(pkg, orc, x, xname, qname, pkg.SCALE_COL, 35, 9, 35, s)
-    assert "_any_" in k[0]
+    assert "_colu_" in k[0] and "_colu_" in k[1] and "_colu_" in k[2]
+    # rows longer than one chunk of 64 groups and not whole groups; rows shorter than a group; blocks of 3 rows
+    for d0, d1, nb_row, nb_col in ((21, 1031, 7, 3), (40, 3, 40, 8), (6, 515, 6, 6)):
+        x = g.standard_normal((d0, d1), dtype=np.float32) * np.float32(1.5)
+        x[g.random((d0, d1)) < 0.05] *= np.float32(40.0)
+        s = g.uniform(0.005, 0.05, nb_row).astype(np.float32)
+        k = _check_all(pkg, orc, x, xname, qname, pkg.SCALE_ROW, d0, d1, nb_row, s)
+        assert "_rowu_" in k[0]
+        s = g.uniform(0.005, 0.05, (d0 // nb_col) * d1).astype(np.float32)
+        k = _check_all(pkg, orc, x, xname, qname, pkg.SCALE_COL, d0, d1, nb_col, s)
+        assert "_colu_" in k[0]
+    # aligned shape, misaligned pointers
+    x = g.standard_normal((16, 256), dtype=np.float32)
+    s = g.uniform(0.005, 0.05, 16).astype(np.float32)
+    k = _check_all(pkg, orc, x, xname, qname, pkg.SCALE_ROW, 16, 256, 16, s, misalign=1)
+    assert "_rowu_" in k[0]
 
 
 @pytest.mark.parametrize("xname", ["f32", "f16", "bf16"])
@@ -193,11 +208,12 @@ def test_int4_blockwise(pkg, orc, xname, qname):
     s = g.uniform(0.005, 0.02, (64, 4)).astype(np.float32)
     k = _check_all(pkg, orc, x, xname, qname, pkg.SCALE_ROW, 64 * 4, 128, 64 * 4, s.ravel())
     assert "_row_" in k[0]
-    # tiny blocks, odd column count -> generic kernel (pairs of nibbles straddle rows)
+    # tiny blocks, odd column count: packed codes -> generic kernel (pairs of nibbles straddle rows), one code per byte ->
+    # the row-walking kernel
     x = g.standard_normal((6, 7), dtype=np.float32)
     s = g.uniform(0.1, 0.3, (3, 7)).astype(np.float32)
     k = _check_all(pkg, orc, x, xname, qname, pkg.SCALE_COL, 6, 7, 2, s.ravel())
-    assert "_any_" in k[0]
+    assert ("_colu_" if qname == "i4" else "_any_") in k[0]
 
 
 @pytest.mark.parametrize("seed", range(48))
