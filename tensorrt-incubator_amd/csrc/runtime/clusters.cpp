@@ -118,7 +118,13 @@ int32_t qdq_dispatch(int mode, hipStream_t stream, const void *x, int32_t x_dtyp
   // Row or column scales on rows that are not whole groups, or on operands not aligned for group accesses: a wave
   // per 64 groups of one row with accesses at element alignment (codes one per byte only: a packed byte can
   // straddle rows).  Everything else that is not `tiles`: one element per lane.
-  const bool ragged = !tiles && kind != MTRT_SCALE_UNIFORM && !nibbles;
+  // A per-tensor scale on unaligned operands is the row kind on one row of n elements.
+  const bool ragged = !tiles && !nibbles;
+  if (ragged && kind == MTRT_SCALE_UNIFORM) {
+    kind = MTRT_SCALE_ROW;
+    d0 = 1;
+    d1 = n;
+  }
   static const char *kModeName[] = {"q", "dq", "qdq"};
   static const char *kKindName[] = {"uniform", "row", "col"};
   static const char *kRaggedName[] = {"", "rowu", "colu"};
