@@ -78,39 +78,76 @@ __device__ __forceinline__ void rows_body(const typename X::storage* __restrict_
       }
       for (; v < nvec; v += kWave) { const uint32_t a = A::of(__builtin_nontemporal_load(pv + v)); m = m > a ? m : a; }
     } else {
-      for (int64_t c = lane; c < d1; c += kWave) { const uint32_t a = A::one(p + c); m = m > a ? m : a; }
+      // any row length and alignment: the row's whole vectors by 128-bit loads at element alignment (the hardware
+      // splits those that straddle a cache line), the d1 % G elements behind them one per lane
+      typedef u32x4 u32x4_unaligned __attribute__((aligned(2)));
+      const u32x4_unaligned* pv = reinterpret_cast<const u32x4_unaligned*>(p);
+      const int64_t nvec = d1 / A::kPerVec;
+      int64_t v = lane;
+      for (; v + 3 * kWave < nvec; v += 4 * kWave) {
+        u32x4 t[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) t[u] = pv[v + u * kWave];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) { const uint32_t a = A::of(t[u]); m = m > a ? m : a; }
+      }
+      for (; v < nvec; v += kWave) { const uint32_t a = A::of(pv[v]); m = m > a ? m : a; }
+      for (int64_t c = nvec * A::kPerVec + lane; c < d1; c += kWave) { const uint32_t a = A::one(p + c); m = m > a ? m : a; }
     }
   }
   m = wave_reduce(m, MaxU32());
   if (lane == 0) emit(A::finish(m), qmax, amax_out, scale_out, s);
 }
 
+// The vector of columns vcol * G .. of row `row` for the column kernels.  UNALIGNED: any d1 and any alignment of x: whole
+// vectors by 128-bit loads at element alignment, and the d1 % G columns behind the last whole vector gathered one
+// by one into a vector of their own (index d1 / G), zeros in the lanes beyond.
+__device__ __forceinline__ uint32_t raw_bits(float v) { return f32_to_bits(v); }
+__device__ __forceinline__ uint32_t raw_bits(uint16_t v) { return v; }
+template <typename X, bool UNALIGNED>
+__device__ __forceinline__ u32x4 column_vector(const typename X::storage* __restrict__ x, int64_t row, int64_t vcol, int64_t d1) {
+  constexpr int G = AbsEach<X>::G;
+  if (!UNALIGNED) return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(x + row * d1) + vcol);
+  typedef u32x4 u32x4_unaligned __attribute__((aligned(2)));
+  const typename X::storage* p = x + row * d1 + vcol * G;
+  if ((vcol + 1) * G <= d1) return *reinterpret_cast<const u32x4_unaligned*>(p);
+  u32x4 t = {0u, 0u, 0u, 0u};
+  const int tail = int(d1 - vcol * G);
+#pragma unroll
+  for (int k = 0; k < G - 1; ++k)
+    if (k < tail) {
+      if (G == 4) t[k & 3] = raw_bits(p[k]);
+      else t[(k >> 1) & 3] |= raw_bits(p[k]) << (16 * (k & 1));
+    }
+  return t;
+}
+
 // col kind, vector form: workgroup = (block b, strip of 64 vectors of columns); wave w takes rows w, w + 4, ... of
 // the block, lane l the vector column strip * 64 + l; the four waves' partial maxima meet in LDS.
-template <typename X>
+template <typename X, bool UNALIGNED>
 __device__ __forceinline__ void cols_body(const typename X::storage* __restrict__ x, int64_t d0, int64_t d1, int64_t nb,
                                           float qmax, float* __restrict__ amax_out, float* __restrict__ scale_out) {
   using E = AbsEach<X>;
   constexpr int G = E::G;
   __shared__ uint32_t part[4][kWave][G + 1];
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-  const int64_t nvec = d1 / G, strips = (nvec + kWave - 1) / kWave;
+  const int64_t nvec = (d1 + (UNALIGNED ? G - 1 : 0)) / G, strips = (nvec + kWave - 1) / kWave;   // a last partial vector counts when UNALIGNED
   const int64_t b = blockIdx.x / strips, strip = blockIdx.x % strips;
   const int64_t vcol = strip * kWave + lane;
   uint32_t m[G];
 #pragma unroll
   for (int k = 0; k < G; ++k) m[k] = 0;
   if (vcol < nvec) {
-    const u32x4* pv = reinterpret_cast<const u32x4*>(x + (b * nb) * d1) + vcol;
+    const int64_t row0 = b * nb;
     int64_t r = wave;
     for (; r + 12 < nb; r += 16) {                     // four independent loads in flight
       u32x4 t[4];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) t[u] = __builtin_nontemporal_load(pv + (r + 4 * u) * nvec);
+      for (int u = 0; u < 4; ++u) t[u] = column_vector<X, UNALIGNED>(x, row0 + r + 4 * u, vcol, d1);
 #pragma unroll
       for (int u = 0; u < 4; ++u) E::acc(t[u], m);
     }
-    for (; r < nb; r += 4) E::acc(__builtin_nontemporal_load(pv + r * nvec), m);
+    for (; r < nb; r += 4) E::acc(column_vector<X, UNALIGNED>(x, row0 + r, vcol, d1), m);
   }
 #pragma unroll
   for (int k = 0; k < G; ++k) part[wave][lane][k] = m[k];
@@ -121,7 +158,7 @@ __device__ __forceinline__ void cols_body(const typename X::storage* __restrict_
       uint32_t r = part[0][lane][k];
 #pragma unroll
       for (int w = 1; w < 4; ++w) r = r > part[w][lane][k] ? r : part[w][lane][k];
-      emit(AbsBits<X>::finish(r), qmax, amax_out, scale_out, b * d1 + vcol * G + k);
+      if (vcol * G + k < d1) emit(AbsBits<X>::finish(r), qmax, amax_out, scale_out, b * d1 + vcol * G + k);
     }
   }
 }
@@ -130,14 +167,15 @@ __device__ __forceinline__ void cols_body(const typename X::storage* __restrict_
 // dealt to `parts` workgroups, rows [part * rows_per_part, ...), whose column maxima meet in `stage` (one word per
 // scale element, zero on entry) through atomic max on the bit patterns; mtrt_amax_finish_* turns the words into
 // amax and scale afterwards.  Without the split such a tensor has ceil(d1 / G / 64) workgroups in all.
-template <typename X>
+template <typename X, bool UNALIGNED>
 __device__ __forceinline__ void cols_split_body(const typename X::storage* __restrict__ x, int64_t d0, int64_t d1, int64_t nb,
                                                 int64_t rows_per_part, uint32_t* __restrict__ stage) {
   using E = AbsEach<X>;
   constexpr int G = E::G;
   __shared__ uint32_t part_max[4][kWave][G + 1];
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-  const int64_t nvec = d1 / G, strips = (nvec + kWave - 1) / kWave, parts = (nb + rows_per_part - 1) / rows_per_part;
+  const int64_t nvec = (d1 + (UNALIGNED ? G - 1 : 0)) / G, strips = (nvec + kWave - 1) / kWave;
+  const int64_t parts = (nb + rows_per_part - 1) / rows_per_part;
   const int64_t part = blockIdx.x % parts, rest = blockIdx.x / parts;
   const int64_t b = rest / strips, strip = rest % strips;
   const int64_t vcol = strip * kWave + lane;
@@ -146,16 +184,16 @@ __device__ __forceinline__ void cols_split_body(const typename X::storage* __res
 #pragma unroll
   for (int k = 0; k < G; ++k) m[k] = 0;
   if (vcol < nvec) {
-    const u32x4* pv = reinterpret_cast<const u32x4*>(x + (b * nb) * d1) + vcol;
+    const int64_t row0 = b * nb;
     int64_t r = r0 + wave;
     for (; r + 12 < r1; r += 16) {                     // four independent loads in flight
       u32x4 t[4];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) t[u] = __builtin_nontemporal_load(pv + (r + 4 * u) * nvec);
+      for (int u = 0; u < 4; ++u) t[u] = column_vector<X, UNALIGNED>(x, row0 + r + 4 * u, vcol, d1);
 #pragma unroll
       for (int u = 0; u < 4; ++u) E::acc(t[u], m);
     }
-    for (; r < r1; r += 4) E::acc(__builtin_nontemporal_load(pv + r * nvec), m);
+    for (; r < r1; r += 4) E::acc(column_vector<X, UNALIGNED>(x, row0 + r, vcol, d1), m);
   }
 #pragma unroll
   for (int k = 0; k < G; ++k) part_max[wave][lane][k] = m[k];
@@ -167,7 +205,7 @@ __device__ __forceinline__ void cols_split_body(const typename X::storage* __res
 #pragma unroll
       for (int w = 1; w < 4; ++w) r = r > part_max[w][lane][k] ? r : part_max[w][lane][k];
       // nobody reads the word before the launch has ended: no ordering, no return value
-      __hip_atomic_fetch_max(stage + b * d1 + vcol * G + k, r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (vcol * G + k < d1) __hip_atomic_fetch_max(stage + b * d1 + vcol * G + k, r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   }
 }
@@ -244,6 +282,7 @@ __device__ __forceinline__ void cols_any_body(const typename X::storage* __restr
 // (x, d0, d1, nb, qmax, amax_out or null, scale_out or null)
 //   rows / rows_any : grid = ceil(nb / 4), block = 256 (one wave per scale)
 //   cols            : grid = (d0 / nb) * ceil(d1 / G / 64), block = 256 ; d1 % G == 0, x 16-byte aligned
+//   cols_u, cols_split_u : the same two for any d1 and alignment, grid with ceil(d1 / G) vectors per row
 //   cols_any        : grid-stride, block = 256
 // (x, d0, d1, nb, parts, stage) rows_split : grid = nb * parts, block = 256 ; stage = nb zeroed words ; then finish
 // (x, d0, d1, nb, rows_per_part, stage) cols_split : grid = (d0 / nb) * ceil(d1 / G / 64) * ceil(nb / rows_per_part),
@@ -258,10 +297,16 @@ __device__ __forceinline__ void cols_any_body(const typename X::storage* __restr
     amax_scales_cluster::rows_body<XT, false>(x, d0, d1, nb, qmax, amax_out, scale_out); }                             \
   extern "C" __global__ void __launch_bounds__(256) mtrt_amax_cols_##XN(                                               \
       const XT::storage* x, int64_t d0, int64_t d1, int64_t nb, float qmax, float* amax_out, float* scale_out) {       \
-    amax_scales_cluster::cols_body<XT>(x, d0, d1, nb, qmax, amax_out, scale_out); }                                    \
+    amax_scales_cluster::cols_body<XT, false>(x, d0, d1, nb, qmax, amax_out, scale_out); }                             \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_amax_cols_u_##XN(                                             \
+      const XT::storage* x, int64_t d0, int64_t d1, int64_t nb, float qmax, float* amax_out, float* scale_out) {       \
+    amax_scales_cluster::cols_body<XT, true>(x, d0, d1, nb, qmax, amax_out, scale_out); }                              \
   extern "C" __global__ void __launch_bounds__(256) mtrt_amax_cols_split_##XN(                                         \
       const XT::storage* x, int64_t d0, int64_t d1, int64_t nb, int64_t rows_per_part, uint32_t* stage) {              \
-    amax_scales_cluster::cols_split_body<XT>(x, d0, d1, nb, rows_per_part, stage); }                                   \
+    amax_scales_cluster::cols_split_body<XT, false>(x, d0, d1, nb, rows_per_part, stage); }                            \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_amax_cols_split_u_##XN(                                       \
+      const XT::storage* x, int64_t d0, int64_t d1, int64_t nb, int64_t rows_per_part, uint32_t* stage) {              \
+    amax_scales_cluster::cols_split_body<XT, true>(x, d0, d1, nb, rows_per_part, stage); }                             \
   extern "C" __global__ void __launch_bounds__(256) mtrt_amax_rows_split_##XN(                                         \
       const XT::storage* x, int64_t d0, int64_t d1, int64_t nb, int64_t parts, uint32_t* stage) {                      \
     amax_scales_cluster::rows_split_body<XT>(x, d0, d1, nb, parts, stage); }                                           \

@@ -287,8 +287,14 @@ int32_t mtrt_hip_amax_scales(mtrt_stream_t stream, const void *x, int32_t dtype,
     return launch(st, KernelName(vec ? "mtrt_amax_rows_" : "mtrt_amax_rows_any_") + xn, uint32_t(blocks), kBlock,
                   as_hip(stream), args);
   }
-  if (vec) {
-    const int64_t blocks = (d0 / nb) * ((d1 / group + 63) / 64), units = num_compute_units(st);
+  // A row length that is not whole vectors, or an unaligned operand: one lane per (block, column) while that gives
+  // every compute unit a thousand lanes (f16 [8192, 8190], blocks of 128 rows: 44.7 us against 51.1 us for the
+  // vector form at element alignment); with fewer, longer blocks the `_u` kernels, which move whole vectors at
+  // element alignment, count a last partial vector and can share a block's rows (one block of 8192 rows: 2085 us
+  // as one lane per column, 112.6 us shared).
+  if (vec || (d0 / nb) * d1 < int64_t(num_compute_units(st)) * 1024) {
+    const char *u = vec ? "" : "u_";
+    const int64_t blocks = (d0 / nb) * (((d1 + group - 1) / group + 63) / 64), units = num_compute_units(st);
     if (blocks < 2 * units && nb >= 128 && (d0 / nb) * d1 < (int64_t(1) << 31)) {
       // Few, long blocks (one per-channel scale per column of a [K, N] weight): too few workgroups to pull the
       // tensor through.  Each block's rows are dealt to several workgroups (at least 32 rows each, about two
@@ -310,14 +316,14 @@ int32_t mtrt_hip_amax_scales(mtrt_stream_t stream, const void *x, int32_t dtype,
         return rc;
       int64_t rpp = rows_per_part;
       void *split_args[] = {&x, &d0, &d1, &nb, &rpp, &stage};
-      rc = launch(st, KernelName("mtrt_amax_cols_split_") + xn, uint32_t(blocks * parts), kBlock, as_hip(stream), split_args);
+      rc = launch(st, KernelName("mtrt_amax_cols_split_") + u + xn, uint32_t(blocks * parts), kBlock, as_hip(stream), split_args);
       if (rc != MTRT_OK)
         return rc;
       void *finish_args[] = {&stage, &count, &qmax, &amax_out, &scale_out};
       return launch(st, KernelName("mtrt_amax_finish_") + xn, blocks_for(count, kBlock), kBlock, as_hip(stream), finish_args);
     }
     if (blocks <= int64_t(kMaxGrid) * 1024)
-      return launch(st, KernelName("mtrt_amax_cols_") + xn, uint32_t(blocks), kBlock, as_hip(stream), args);
+      return launch(st, KernelName("mtrt_amax_cols_") + u + xn, uint32_t(blocks), kBlock, as_hip(stream), args);
   }
   return launch(st, KernelName("mtrt_amax_cols_any_") + xn, blocks_for((d0 / nb) * d1, kBlock), kBlock, as_hip(stream), args);
 }

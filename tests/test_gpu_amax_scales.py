@@ -61,7 +61,9 @@ def test_every_addressing_on_ragged_shapes(pkg, orc, xname):
         ("col", 48, grp * 70, 16, "mtrt_amax_cols" + k),                     # two strips of 64 vectors, 16-row blocks
         ("col", 40, grp * 3, 40, "mtrt_amax_cols" + k),                      # per channel on the last axis
         ("col", 6, grp * 2, 1, "mtrt_amax_cols" + k),                        # block of one row: amax = |x|
-        ("col", 30, 77, 5, "mtrt_amax_cols_any" + k),
+        ("col", 30, 77, 5, "mtrt_amax_cols_u" + k),                         # row length not a vector multiple: vectors at element alignment
+        ("col", 8, grp * 70 + 3, 4, "mtrt_amax_cols_u" + k),                  # two strips and a partial last vector
+        ("col", 260, grp * 2 + 1, 130, "mtrt_amax_finish" + k),               # long ragged blocks: rows dealt to several workgroups
         ("uniform", 11, 100, 1, "mtrt_amax" + k),
     ]
     for kind, d0, d1, nb, kernel in cases:
