@@ -274,7 +274,8 @@ __device__ __forceinline__ void layernorm_group_row(const typename X::storage* _
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
     const int idx = lane + THREADS * j;
-    t[j] = __builtin_nontemporal_load(xr + (FULL ? idx : min(idx, nvec - 1)));
+    if (RAGGED && nvec == 0) t[j] = (u32x4){0u, 0u, 0u, 0u};   // a row shorter than one vector: only the scalar elements below
+    else t[j] = __builtin_nontemporal_load(xr + (FULL ? idx : min(idx, nvec - 1)));
   }
   const bool extra = RAGGED && lane < tail;          // this lane also owns element nvec * E + lane
   const int64_t ec = int64_t(nvec) * E + lane;
@@ -312,6 +313,7 @@ __device__ __forceinline__ void layernorm_group_row(const typename X::storage* _
   for (int j = 0; j < NV; ++j) {
     const int idx = lane + THREADS * j;
     const int idc = FULL ? idx : min(idx, nvec - 1);
+    if (RAGGED && nvec == 0) continue;               // no whole vector: nothing to read or store here
     float v[E], g[E], b[E], o[E];
     opaque(t[j]);
     Vec<X>::unpack(t[j], v);
@@ -364,7 +366,8 @@ __device__ __forceinline__ void softmax_group_row(const typename X::storage* __r
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
     const int idx = lane + THREADS * j;
-    t[j] = __builtin_nontemporal_load(xr + (FULL ? idx : min(idx, nvec - 1)));
+    if (RAGGED && nvec == 0) t[j] = (u32x4){0u, 0u, 0u, 0u};   // a row shorter than one vector: only the scalar elements below
+    else t[j] = __builtin_nontemporal_load(xr + (FULL ? idx : min(idx, nvec - 1)));
   }
   const bool extra = RAGGED && lane < tail;          // this lane also owns element nvec * E + lane
   const int64_t ec = int64_t(nvec) * E + lane;
@@ -522,7 +525,7 @@ using namespace norm_cluster;
 
 // One workgroup per row: mtrt_layernorm_<t>_g<THREADS>v<NV>(x, gamma, beta, y, rows, d, eps), mtrt_softmax_<t>_g<THREADS>v<NV>(x, y, rows, d)
 //   grid = rows, block = THREADS; d % E == 0, d / E <= THREADS * NV, operands 16-byte aligned.
-// Ragged rows: mtrt_{layernorm,softmax}_<t>_u<THREADS>v<NV>, same arguments; any d with 1 <= d / E <= THREADS * NV,
+// Ragged rows: mtrt_{layernorm,softmax}_<t>_u<THREADS>v<NV>, same arguments; any d >= 1 with d / E <= THREADS * NV,
 //   operands aligned to their element; THREADS <= 64 (NV = 1 below 64): grid = ceil(rows / (256 / THREADS)), block = 256;
 //   else grid = rows, block = THREADS.
 #define MTRT_NORM_GROUP_KERNELS(XN, XT, NV, THREADS, TAG, RAGGED, BLOCK)                                       \

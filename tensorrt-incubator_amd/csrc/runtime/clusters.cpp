@@ -569,7 +569,7 @@ int32_t mtrt_hip_layernorm(mtrt_stream_t stream, const void *x, const void *gamm
   float eps_arg = eps;
   void *args[] = {&x, &gamma, &beta, &y, &rows_arg, &d_arg, &eps_arg};
   // Rows of at most 32 vectors: 8, 16 or 32 lanes per row, several rows to a wave (whatever the alignment).
-  if (d >= per_vec && d / per_vec <= 32 && aligned(x, eb) && rows <= kMaxRowsPerWaveKernels) {
+  if (d / per_vec <= 32 && rows <= kMaxRowsPerWaveKernels) {
     const int lanes = d / per_vec <= 8 ? 8 : (d / per_vec <= 16 ? 16 : 32);
     return launch(st, KernelName("mtrt_layernorm_") + xn + "_u" + lanes + "v1", blocks_for(rows, kBlock / lanes), kBlock, as_hip(stream), args);
   }
@@ -625,7 +625,7 @@ int32_t mtrt_hip_softmax(mtrt_stream_t stream, const void *x, void *y, int32_t d
   int64_t rows_arg = rows, d_arg = d;
   void *args[] = {&x, &y, &rows_arg, &d_arg};
   // Rows of at most 32 vectors: 8, 16 or 32 lanes per row, several rows to a wave (whatever the alignment).
-  if (d >= per_vec && d / per_vec <= 32 && aligned(x, eb) && rows <= kMaxRowsPerWaveKernels) {
+  if (d / per_vec <= 32 && rows <= kMaxRowsPerWaveKernels) {
     const int lanes = d / per_vec <= 8 ? 8 : (d / per_vec <= 16 ? 16 : 32);
     return launch(st, KernelName("mtrt_softmax_") + xn + "_u" + lanes + "v1", blocks_for(rows, kBlock / lanes), kBlock, as_hip(stream), args);
   }

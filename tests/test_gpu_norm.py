@@ -184,7 +184,7 @@ def test_layernorm_resident_variant_window_and_bits(pkg, orc):
 
 def test_kernel_selection(pkg, orc):
     import torch
-    for d, k in ((512, "v1"), (1024, "v2"), (2048, "v4"), (4096, "v8"), (8192, "v16"), (8200, "g256v8"), (131080, "any"), (331, "u64v1"), (5, "any")):
+    for d, k in ((512, "v1"), (1024, "v2"), (2048, "v4"), (4096, "v8"), (8192, "v16"), (8200, "g256v8"), (131080, "any"), (331, "u64v1"), (5, "u8v1"), (1, "u8v1")):
         x = torch.randn(4, d, device="cuda", dtype=torch.bfloat16)
         pkg.softmax(x)
         assert pkg.last_kernel() == "mtrt_softmax_bf16_" + k
@@ -278,7 +278,7 @@ def _ragged_cases(name):
     50257-entry vocabulary) in every scheme, from one vector plus one element up to 1024 x 16 vectors plus a tail;
     rows of at most 32 vectors share a wave (8, 16 or 32 lanes each) whether or not they are whole vectors."""
     e = 4 if name == "f32" else 8
-    return [(e + 1, "_u8v1"), (77, "_u16v1" if e == 8 else "_u32v1"), (197, "_u32v1" if e == 8 else "_u64v1"), (e * 8, "_u8v1"),
+    return [(1, "_u8v1"), (2, "_u8v1"), (e - 1, "_u8v1"), (e + 1, "_u8v1"), (77, "_u16v1" if e == 8 else "_u32v1"), (197, "_u32v1" if e == 8 else "_u64v1"), (e * 8, "_u8v1"),
             (e * 32, "_u32v1"), (e * 32 + 1, "_u32v1"), (e * 33 + 1, "_u64v1"), (e * 64 + 3, "_u64v1"), (e * 65 + 3, "_u64v2"), (1500 if e == 8 else 1501, "_u64v4" if e == 8 else "_u64v8"),
             (e * 512 + e - 1, "_u64v8"), (e * 1024 + 1, "_u64v16"), (e * 1025 + 2, "_u256v8"), (e * 4096 + 3, "_u256v16"),
             (50257, "_u1024v8" if e == 8 else "_u1024v16"), (e * 16384 + e - 1, "_u1024v16"), (e * 16385 + 1, "_any")]
