@@ -447,22 +447,52 @@ __device__ __forceinline__ float block_reduce(float v, Op op, float* lds) {
   return r;
 }
 
+// Rows of any length and alignment: whole vectors by 128-bit accesses at element alignment, the d % E elements behind
+// them one per lane; the row is read three times (the second and third time from cache).
 template <typename X>
 __device__ __forceinline__ void layernorm_any(const typename X::storage* __restrict__ x,
                                               const typename X::storage* __restrict__ gamma,
                                               const typename X::storage* __restrict__ beta,
                                               typename X::storage* __restrict__ y, int64_t rows, int64_t d, float eps) {
+  constexpr int E = Vec<X>::kElems;
+  using V = typename RowVector<true>::type;
   __shared__ float lds[kNormThreads / kWave];
+  const int64_t nvec = d / E, tail0 = nvec * E;
+  const V* gv = reinterpret_cast<const V*>(gamma);
+  const V* bv = reinterpret_cast<const V*>(beta);
   for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
     const typename X::storage* xr = x + row * d;
+    const V* xv = reinterpret_cast<const V*>(xr);
     float sum = 0.0f;
-    for (int64_t c = threadIdx.x; c < d; c += kNormThreads) sum = sum + Tile<X>::load1(xr + c);
+    for (int64_t v = threadIdx.x; v < nvec; v += kNormThreads) {
+      float f[E];
+      Vec<X>::unpack(xv[v], f);
+#pragma unroll
+      for (int k = 0; k < E; ++k) sum = sum + f[k];
+    }
+    for (int64_t c = tail0 + threadIdx.x; c < d; c += kNormThreads) sum = sum + Tile<X>::load1(xr + c);
     const float mu = block_reduce(sum, SumF32(), lds) / float(d);
     float sq = 0.0f;
-    for (int64_t c = threadIdx.x; c < d; c += kNormThreads) { const float dv = Tile<X>::load1(xr + c) - mu; sq = sq + dv * dv; }
+    for (int64_t v = threadIdx.x; v < nvec; v += kNormThreads) {
+      float f[E];
+      Vec<X>::unpack(xv[v], f);
+#pragma unroll
+      for (int k = 0; k < E; ++k) { const float dv = f[k] - mu; sq = sq + dv * dv; }
+    }
+    for (int64_t c = tail0 + threadIdx.x; c < d; c += kNormThreads) { const float dv = Tile<X>::load1(xr + c) - mu; sq = sq + dv * dv; }
     const float var = block_reduce(sq, SumF32(), lds) / float(d);
     const float rstd = 1.0f / sqrtf(var + eps);
-    for (int64_t c = threadIdx.x; c < d; c += kNormThreads) {
+    V* yv = reinterpret_cast<V*>(y + row * d);
+    for (int64_t v = threadIdx.x; v < nvec; v += kNormThreads) {
+      float f[E], g[E], b[E], o[E];
+      Vec<X>::unpack(xv[v], f);
+      Vec<X>::unpack(gv[v], g);
+      Vec<X>::unpack(bv[v], b);
+#pragma unroll
+      for (int k = 0; k < E; ++k) o[k] = (((f[k] - mu) * rstd) * g[k]) + b[k];
+      yv[v] = Vec<X>::pack(o);
+    }
+    for (int64_t c = tail0 + threadIdx.x; c < d; c += kNormThreads) {
       const float dv = Tile<X>::load1(xr + c) - mu;
       Tile<X>::store1(y + row * d + c, ((dv * rstd) * Tile<X>::load1(gamma + c)) + Tile<X>::load1(beta + c));
     }
@@ -472,17 +502,41 @@ __device__ __forceinline__ void layernorm_any(const typename X::storage* __restr
 template <typename X>
 __device__ __forceinline__ void softmax_any(const typename X::storage* __restrict__ x, typename X::storage* __restrict__ y,
                                             int64_t rows, int64_t d) {
+  constexpr int E = Vec<X>::kElems;
+  using V = typename RowVector<true>::type;
   __shared__ float lds[kNormThreads / kWave];
+  const int64_t nvec = d / E, tail0 = nvec * E;
   for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
     const typename X::storage* xr = x + row * d;
+    const V* xv = reinterpret_cast<const V*>(xr);
     float mx = -INFINITY;
-    for (int64_t c = threadIdx.x; c < d; c += kNormThreads) mx = fmaxf(mx, Tile<X>::load1(xr + c));
+    for (int64_t v = threadIdx.x; v < nvec; v += kNormThreads) {
+      float f[E];
+      Vec<X>::unpack(xv[v], f);
+#pragma unroll
+      for (int k = 0; k < E; ++k) mx = fmaxf(mx, f[k]);
+    }
+    for (int64_t c = tail0 + threadIdx.x; c < d; c += kNormThreads) mx = fmaxf(mx, Tile<X>::load1(xr + c));
     mx = block_reduce(mx, MaxF32(), lds);
     float s = 0.0f;
-    for (int64_t c = threadIdx.x; c < d; c += kNormThreads) s = s + __expf(Tile<X>::load1(xr + c) - mx);
+    for (int64_t v = threadIdx.x; v < nvec; v += kNormThreads) {
+      float f[E];
+      Vec<X>::unpack(xv[v], f);
+#pragma unroll
+      for (int k = 0; k < E; ++k) s = s + __expf(f[k] - mx);
+    }
+    for (int64_t c = tail0 + threadIdx.x; c < d; c += kNormThreads) s = s + __expf(Tile<X>::load1(xr + c) - mx);
     s = block_reduce(s, SumF32(), lds);
     const float inv = 1.0f / s;
-    for (int64_t c = threadIdx.x; c < d; c += kNormThreads)
+    V* yv = reinterpret_cast<V*>(y + row * d);
+    for (int64_t v = threadIdx.x; v < nvec; v += kNormThreads) {
+      float f[E], o[E];
+      Vec<X>::unpack(xv[v], f);
+#pragma unroll
+      for (int k = 0; k < E; ++k) o[k] = __expf(f[k] - mx) * inv;
+      yv[v] = Vec<X>::pack(o);
+    }
+    for (int64_t c = tail0 + threadIdx.x; c < d; c += kNormThreads)
       Tile<X>::store1(y + row * d + c, __expf(Tile<X>::load1(xr + c) - mx) * inv);
   }
 }
