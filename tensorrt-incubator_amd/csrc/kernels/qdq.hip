@@ -563,7 +563,7 @@ typedef uint32_t u32_unaligned __attribute__((aligned(1)));
 template <typename X, typename Q, int KIND, int MODE>
 __device__ __forceinline__ void qdq_rows_ragged(const typename X::storage* __restrict__ x, typename Q::storage* __restrict__ q,
                                                 typename X::storage* __restrict__ y, const float* __restrict__ scale,
-                                                int64_t n, int64_t d1, int64_t nb, int flags) {
+                                                int64_t n, int64_t d1, int64_t nb, int64_t fpitch, int64_t qpitch, int flags) {
   using FG = FloatGroup<X>;
   constexpr int G = FG::G;
   const int64_t d0 = n / d1, nvec = d1 / G;
@@ -576,7 +576,7 @@ __device__ __forceinline__ void qdq_rows_ragged(const typename X::storage* __res
   for (int64_t item = wave; item < items; item += nwaves) {
     const int64_t row = item / chunks, c = item - row * chunks;
     const int64_t v = c * kWave + lane;
-    const int64_t e0 = row * d1 + v * G;
+    const int64_t fe0 = row * fpitch + v * G, qe0 = row * qpitch + v * G;   // row pitches in elements: d1 unless the operand is a view
     const float* srow = KIND == kRow ? scale + row % nb : scale + (row / nb) * d1;
     if (v < nvec) {
       float f[G], sc[G];
@@ -595,11 +595,11 @@ __device__ __forceinline__ void qdq_rows_ragged(const typename X::storage* __res
       if (MODE == 1) {
 #pragma unroll
         for (int i = 0; i < G / 4; ++i) {
-          w[i] = *reinterpret_cast<const u32_unaligned*>(q + e0 + 4 * i);
+          w[i] = *reinterpret_cast<const u32_unaligned*>(q + qe0 + 4 * i);
           unpack4<Q>(w[i], &f[4 * i]);
         }
       } else {
-        const u32x4 t = *reinterpret_cast<const u32x4_unaligned*>(x + e0);
+        const u32x4 t = *reinterpret_cast<const u32x4_unaligned*>(x + fe0);
         FG::unpack(t, f);
         if (KIND == kRow) {
           const ExactDivisor dv(sc[0]);
@@ -612,7 +612,7 @@ __device__ __forceinline__ void qdq_rows_ragged(const typename X::storage* __res
         for (int i = 0; i < G / 4; ++i) {
           w[i] = pack4<Q>(&f[4 * i], flags);
           unpack4<Q>(w[i], &f[4 * i]);                 // f32(code): what a following dequantize multiplies
-          *reinterpret_cast<u32_unaligned*>(q + e0 + 4 * i) = w[i];
+          *reinterpret_cast<u32_unaligned*>(q + qe0 + 4 * i) = w[i];
         }
       }
       if (MODE != 0) {
@@ -621,7 +621,7 @@ __device__ __forceinline__ void qdq_rows_ragged(const typename X::storage* __res
         u32x4 t;
         if (G == 4) {
           t = (u32x4){f32_to_bits(f[0]), f32_to_bits(f[1]), f32_to_bits(f[2]), f32_to_bits(f[3])};
-          *reinterpret_cast<u32x4_unaligned*>(y + e0) = t;
+          *reinterpret_cast<u32x4_unaligned*>(y + fe0) = t;
         } else {
           // 16-bit outputs: narrowed one by one through the element form, then stored as one vector
           typename X::storage h[8];
@@ -629,23 +629,23 @@ __device__ __forceinline__ void qdq_rows_ragged(const typename X::storage* __res
           for (int k = 0; k < 8; ++k) Tile<X>::store1(&h[k % G], f[k % G]);
 #pragma unroll
           for (int k = 0; k < 4; ++k) t[k] = uint32_t(uint16_t(h[(2 * k) % G])) | (uint32_t(uint16_t(h[(2 * k + 1) % G])) << 16);
-          *reinterpret_cast<u32x4_unaligned*>(y + e0) = t;
+          *reinterpret_cast<u32x4_unaligned*>(y + fe0) = t;
         }
       }
     }
     if (c == chunks - 1 && lane < tail) {              // the row's last d1 % G elements, one per lane
-      const int64_t col = nvec * G + lane, e = row * d1 + col;
+      const int64_t col = nvec * G + lane, fe = row * fpitch + col, qe = row * qpitch + col;
       const float s = KIND == kRow ? srow[0] : srow[col];
       float fv;
       if (MODE == 1) {
-        fv = Codes<Q>::dec(uint32_t(uint8_t(q[e])));
+        fv = Codes<Q>::dec(uint32_t(uint8_t(q[qe])));
       } else {
-        fv = quant_value<Q>(Tile<X>::load1(x + e), s, flags);
+        fv = quant_value<Q>(Tile<X>::load1(x + fe), s, flags);
         const uint32_t code = Codes<Q>::enc(fv, flags);
-        q[e] = typename Q::storage(code);
+        q[qe] = typename Q::storage(code);
         fv = Codes<Q>::dec(code);
       }
-      if (MODE != 0) Tile<X>::store1(y + e, fv * s);
+      if (MODE != 0) Tile<X>::store1(y + fe, fv * s);
     }
   }
 }
@@ -741,17 +741,19 @@ MTRT_QDQ_FOR_FLOAT(f16, F16)
 MTRT_QDQ_FOR_FLOAT(bf16, BF16)
 
 // Ragged rows / unaligned operands with row or column scales: mtrt_{q,dq,qdq}_{rowu,colu}_<float type>_<code type>,
-// arguments as the kernels above; grid-stride over (row, chunk of 64 groups), block = 256; codes i8, f8, i4.
+// arguments as the kernels above plus, behind nb, the row pitches in elements of the float operand(s) and of the codes
+// (d1 for contiguous tensors; views with unit inner stride pass their row strides); grid-stride over (row, chunk of
+// 64 groups), block = 256; codes i8, f8, i4.
 #define MTRT_QDQ_RAGGED_KERNELS(XN, XT, QN, QT, KN, KIND)                                                          \
   extern "C" __global__ void __launch_bounds__(256) mtrt_q_##KN##_##XN##_##QN(                                     \
-      const XT::storage* x, QT::storage* q, const float* scale, int64_t n, int64_t d1, int64_t nb, int32_t flags) { \
-    qdq_rows_ragged<XT, QT, KIND, 0>(x, q, nullptr, scale, n, d1, nb, flags); }                                    \
+      const XT::storage* x, QT::storage* q, const float* scale, int64_t n, int64_t d1, int64_t nb, int64_t fpitch, \
+      int64_t qpitch, int32_t flags) { qdq_rows_ragged<XT, QT, KIND, 0>(x, q, nullptr, scale, n, d1, nb, fpitch, qpitch, flags); } \
   extern "C" __global__ void __launch_bounds__(256) mtrt_dq_##KN##_##XN##_##QN(                                    \
-      const QT::storage* q, XT::storage* y, const float* scale, int64_t n, int64_t d1, int64_t nb) {              \
-    qdq_rows_ragged<XT, QT, KIND, 1>(nullptr, const_cast<QT::storage*>(q), y, scale, n, d1, nb, 0); }              \
+      const QT::storage* q, XT::storage* y, const float* scale, int64_t n, int64_t d1, int64_t nb, int64_t fpitch, \
+      int64_t qpitch) { qdq_rows_ragged<XT, QT, KIND, 1>(nullptr, const_cast<QT::storage*>(q), y, scale, n, d1, nb, fpitch, qpitch, 0); } \
   extern "C" __global__ void __launch_bounds__(256) mtrt_qdq_##KN##_##XN##_##QN(                                   \
       const XT::storage* x, QT::storage* q, XT::storage* y, const float* scale, int64_t n, int64_t d1, int64_t nb, \
-      int32_t flags) { qdq_rows_ragged<XT, QT, KIND, 2>(x, q, y, scale, n, d1, nb, flags); }
+      int64_t fpitch, int64_t qpitch, int32_t flags) { qdq_rows_ragged<XT, QT, KIND, 2>(x, q, y, scale, n, d1, nb, fpitch, qpitch, flags); }
 #define MTRT_QDQ_RAGGED_FOR_FLOAT(XN, XT)                                                                          \
   MTRT_QDQ_RAGGED_KERNELS(XN, XT, i8, I8, rowu, kRow) MTRT_QDQ_RAGGED_KERNELS(XN, XT, i8, I8, colu, kCol)          \
   MTRT_QDQ_RAGGED_KERNELS(XN, XT, f8, F8, rowu, kRow) MTRT_QDQ_RAGGED_KERNELS(XN, XT, f8, F8, colu, kCol)          \

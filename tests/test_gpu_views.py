@@ -63,6 +63,49 @@ def test_views_equal_packed_copies_and_the_oracle(pkg, orc, xname, qname):
             assert np.array_equal(got, y_ref.view(np.uint32) if ox == orc.F32 else y_ref), (name, kind)
 
 
+@pytest.mark.parametrize("xname", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("qname", ["i8", "f8", "i4"])
+def test_views_with_contiguous_rows_take_the_row_walking_kernels(pkg, orc, xname, qname):
+    """Row and column slices and offset sub-tensors keep their inner stride of one: both operands of such a call are
+    walked row by row with vector accesses, the views' row strides as pitches.  Results against the oracle, nothing
+    outside the destination views written; widths that are and are not whole vectors, a row step of two."""
+    import torch
+    td = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}[xname]
+    ox = {"f32": orc.F32, "bf16": orc.BF16, "f16": orc.F16}[xname]
+    pq, oq = {"i8": (pkg.I8, orc.I8), "f8": (pkg.F8E4M3FN, orc.F8E4M3FN), "i4": (pkg.I4, orc.I4)}[qname]
+    torch.manual_seed(11)
+    parent = (torch.randn(70, 1200, device="cuda") * 2).to(td)
+    views = {"offset block": parent[3:27, 8:40], "wide ragged slice": parent[1:60, 5:1136], "every other row": parent[1::2, 16:528],
+             "whole": parent, "one column": parent[:, 7:8]}
+    for name, xv in views.items():
+        d0, d1 = xv.shape
+        xc = xv.contiguous()
+        xs = xc.cpu().numpy().ravel() if ox == orc.F32 else bits16(xc)
+        for kind, okind, nb, ns, tag in ((pkg.SCALE_UNIFORM, orc.SCALE_UNIFORM, 1, 1, "rowu"), (pkg.SCALE_ROW, orc.SCALE_ROW, d0, d0, "rowu"),
+                                         (pkg.SCALE_COL, orc.SCALE_COL, d0, d1, "colu")):
+            scale = (torch.rand(ns, device="cuda") * 0.05 + 0.01)
+            qbuf = torch.full((d0 + 2, d1 + 9), 0x55, dtype=torch.uint8, device="cuda")
+            qv = qbuf[1:1 + d0, 5:5 + d1]
+            pkg.quantize_view(xv, scale, pq, qv, kind, nb)
+            assert pkg.last_kernel() == "mtrt_q_%s_%s_%s" % (tag, xname, qname), (name, pkg.last_kernel())
+            q_ref = orc.quantize(xs, ox, oq, scale.cpu().numpy(), okind, d0, d1, nb)
+            assert np.array_equal(qv.contiguous().cpu().numpy().ravel(), q_ref.view(np.uint8)), (name, kind)
+            untouched = qbuf.clone()
+            untouched[1:1 + d0, 5:5 + d1] = 0x55
+            assert bool((untouched == 0x55).all()), "bytes outside the view were written (%s)" % name
+            ybuf = torch.full((d0 + 1, d1 + 3), 7.0, dtype=td, device="cuda")
+            yv = ybuf[1:, 2:2 + d1]
+            pkg.dequantize_view(qv, scale, pq, yv, kind, nb)
+            assert pkg.last_kernel() == "mtrt_dq_%s_%s_%s" % (tag, xname, qname)
+            y_ref = orc.dequantize(q_ref, oq, ox, scale.cpu().numpy(), okind, d0, d1, nb)
+            got = yv.contiguous()
+            got = got.cpu().numpy().ravel().view(np.uint32) if ox == orc.F32 else bits16(got)
+            assert np.array_equal(got, y_ref.view(np.uint32) if ox == orc.F32 else y_ref), (name, kind)
+            rest = ybuf.clone()
+            rest[1:, 2:2 + d1] = 7.0
+            assert bool((rest == 7.0).all()), "values outside the destination view were written (%s)" % name
+
+
 def test_view_kernel_launched_by_hand_in_the_expanded_argument_order(pkg, orc):
     """memref<?x?xf32, strided<[?, ?], offset: ?>> -> (base, offset, size0, size1, stride0, stride1), per operand."""
     import torch
