@@ -731,6 +731,13 @@ int32_t mtrt_hip_gemm_w8a8(mtrt_stream_t stream, const void *a, const void *w_nk
       return launch(st, KernelName("mtrt_gemm_w8a8_nk"), uint32_t(grid), kBlock, as_hip(stream), fast_args);
     }
   }
+  if (K > 0) {
+    // Any other K or alignment still goes to the matrix cores: 128 x 128 tiles with byte-aligned loads and a
+    // zero-padded last k-step (M=4096 K=4100 N=11008: 1.2 s on the one-element-per-lane kernel below).
+    const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
+    return launch(st, KernelName("mtrt_gemm_w8a8_nk_edge"), uint32_t(std::min<int64_t>(tiles, int64_t(kMaxGrid) * 1024)), kBlock,
+                  as_hip(stream), args);
+  }
   return launch(st, KernelName("mtrt_gemm_w8a8_nk_any"), blocks_for(M * N, kBlock), kBlock, as_hip(stream), args);
 }
 

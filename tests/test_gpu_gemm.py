@@ -89,12 +89,46 @@ def test_w8a8_small_m_kernel(pkg, orc, shape):
     assert np.array_equal(bits16(y).reshape(M, N), ref)
 
 
-@pytest.mark.parametrize("shape", [(5, 7, 3), (33, 100, 65), (2, 130, 4)])
-def test_w8a8_generic_kernel(pkg, orc, shape):
+@pytest.mark.parametrize("shape", [(5, 7, 3), (33, 100, 65), (2, 130, 4), (300, 1, 140), (129, 15, 257), (128, 16, 128), (130, 271, 131),
+                                   (64, 4100, 520), (257, 1153, 385), (100, 4160, 264)])
+def test_w8a8_any_k_kernel(pkg, orc, shape):
+    """K that is not a whole number of 128-byte slices: the 128 x 128 tile kernel with byte-aligned loads and a
+    zero-padded last k-step.  K below one chunk, one byte over a chunk / a k-step, several k-steps, ragged M and N,
+    several tiles per axis.  Integer sums: bit-exact."""
     M, K, N = shape
     a, w, a_s, w_s = _w8a8_inputs(rng(M * K + N), M, K, N)
+    print("case: w8a8 any K", shape, flush=True)
     y, kernel = _run_w8a8(pkg, a, w, a_s, w_s)
-    assert kernel == "mtrt_gemm_w8a8_nk_any"
+    assert kernel == "mtrt_gemm_w8a8_nk_edge"
+    assert np.array_equal(bits16(y).reshape(M, N), orc.gemm_w8a8(a, w, a_s, w_s))
+
+
+def test_w8a8_operands_off_alignment_and_outputs_inside_a_larger_buffer(pkg, orc):
+    """Operands one and three bytes off 16-byte alignment with K a multiple of 128, an output one element off 4-byte
+    alignment: same kernel, nothing written outside y."""
+    import torch
+    M, K, N = 200, 256, 136
+    a, w, a_s, w_s = _w8a8_inputs(rng(77), M, K, N)
+    abuf = torch.zeros(M * K + 16, dtype=torch.int8, device="cuda")
+    wbuf = torch.zeros(N * K + 16, dtype=torch.int8, device="cuda")
+    ybuf = torch.full((M * N + 9,), 7.0, dtype=torch.float16, device="cuda")
+    ad, wd, yd = abuf[1:1 + M * K].view(M, K), wbuf[3:3 + N * K].view(N, K), ybuf[1:1 + M * N].view(M, N)
+    ad.copy_(torch.from_numpy(a))
+    wd.copy_(torch.from_numpy(np.ascontiguousarray(w.T)))
+    pkg.gemm_w8a8(ad, wd, torch.from_numpy(a_s).cuda(), torch.from_numpy(w_s).cuda(), out=yd)
+    assert pkg.last_kernel() == "mtrt_gemm_w8a8_nk_edge"
+    assert np.array_equal(bits16(yd.contiguous()).reshape(M, N), orc.gemm_w8a8(a, w, a_s, w_s))
+    assert float(ybuf[0]) == 7.0 and bool((ybuf[1 + M * N:] == 7.0).all())
+
+
+def test_w8a8_empty_reduction_is_zero(pkg, orc):
+    """K = 0: every sum is empty, the outputs are the scaled zero; the one-element-per-lane kernel."""
+    M, K, N = 5, 0, 9
+    a, w, a_s, w_s = _w8a8_inputs(rng(5), M, K, N)
+    import torch
+    y = pkg.gemm_w8a8(torch.from_numpy(a).cuda(), torch.zeros((N, 0), dtype=torch.int8, device="cuda"),
+                      torch.from_numpy(a_s).cuda(), torch.from_numpy(w_s).cuda())
+    assert pkg.last_kernel() == "mtrt_gemm_w8a8_nk_any"
     assert np.array_equal(bits16(y).reshape(M, N), orc.gemm_w8a8(a, w, a_s, w_s))
 
 
