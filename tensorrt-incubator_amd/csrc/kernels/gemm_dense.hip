@@ -6,7 +6,8 @@
 // reference's own generator emits an FMA loop nest for such a matmul
 // (mlir-tensorrt/kernel/test/Kernel/TransformSchedules/fallback-schedule-matmul.mlir:24); this is the same
 // class of kernel, tiled through LDS: 64 x 64 outputs per workgroup, 4 x 4 per lane, K in slices of 16.
-// w is [N,K] (K contiguous), the module's own weight layout; any M, N, K; no alignment needs.
+// w is [N,K] (K contiguous), the module's own weight layout; any M, N, K; no alignment needs.  It only serves
+// K = 0 now: every other shape runs on the matrix cores (mtrt_gemm_dense_edge_* for rows that are not whole slices).
 // 16-bit operands whose rows are whole 128-byte slices (K % 64 == 0, 16-byte aligned) go to the matrix cores
 // instead (mtrt_gemm_dense_mfma_*): both operands are K-contiguous per row, which is the form the shared tile
 // loop of gemm_core.hpp takes (both panels through LDS, 256 x 256 tiles, v_mfma_f32_32x32x16_{f16,bf16}; a
@@ -192,6 +193,22 @@ __device__ __forceinline__ void dense_mfma_f32_body(const float* __restrict__ x,
   }
 }
 
+// Epilogues of the any-shape tile loop (gemm_core::edge): the same sum + bias, one narrowing.
+template <typename X>
+struct EdgeBiasEpilogue {
+  const typename X::storage* bias;
+  __device__ __forceinline__ void row(int64_t, bool) {}
+  __device__ __forceinline__ uint32_t finish(float acc, int64_t col, bool valid) const {
+    if (bias && valid) acc = acc + Tile<X>::load1(bias + col);
+    return narrow16<X>(acc);
+  }
+};
+struct EdgeBiasF32Epilogue {
+  const float* bias;
+  __device__ __forceinline__ void row(int64_t, bool) {}
+  __device__ __forceinline__ float finish(float acc, int64_t col, bool valid) const { return bias && valid ? acc + bias[col] : acc; }
+};
+
 }  // namespace dense_cluster
 
 // f32 operands: (x [M,K], w [N,K], bias [N] or null, y [M,N], M, K, N, full_panels) ; K % 32 == 0, x and w 16-byte aligned
@@ -215,6 +232,27 @@ extern "C" __global__ void __launch_bounds__(gemm_core::THREADS, 1) mtrt_gemm_de
   }
 MTRT_DENSE_MFMA_KERNEL(f16, F16)
 MTRT_DENSE_MFMA_KERNEL(bf16, BF16)
+
+// Any K and any alignment on the matrix cores: (x [M,K], w [N,K], bias [N] or null, y [M,N], M, K, N) ; grid: any
+// (128 x 128 tiles dealt round-robin), block = 256.
+extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_dense_edge_f32(
+    const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ bias, float* __restrict__ y, int64_t M,
+    int64_t K, int64_t N) {
+  __shared__ __attribute__((aligned(16))) int8_t lds[gemm_core::edge::kLdsBytes];
+  dense_cluster::EdgeBiasF32Epilogue epi{bias};
+  gemm_core::edge::run<dense_cluster::F32Traits>(reinterpret_cast<const int8_t*>(x), reinterpret_cast<const int8_t*>(w), K * 4, epi, y, M, N, lds);
+}
+#define MTRT_DENSE_EDGE_KERNEL(XN, XT)                                                                             \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_dense_edge_##XN(                                     \
+      const XT::storage* __restrict__ x, const XT::storage* __restrict__ w, const XT::storage* __restrict__ bias,  \
+      uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N) {                                                 \
+    __shared__ __attribute__((aligned(16))) int8_t lds[gemm_core::edge::kLdsBytes];                                \
+    dense_cluster::EdgeBiasEpilogue<XT> epi{bias};                                                                 \
+    gemm_core::edge::run<dense_cluster::HalfTraits<XT>>(reinterpret_cast<const int8_t*>(x), reinterpret_cast<const int8_t*>(w), K * 2, epi, y, \
+                                                        M, N, lds);                                                \
+  }
+MTRT_DENSE_EDGE_KERNEL(f16, F16)
+MTRT_DENSE_EDGE_KERNEL(bf16, BF16)
 
 // (x [M,K], w [N,K], bias [N] or null, y [M,N], M, K, N) ; grid = ceil(M/64) * ceil(N/64), block = 256
 #define MTRT_DENSE_KERNEL(XN, XT)                                                                                  \

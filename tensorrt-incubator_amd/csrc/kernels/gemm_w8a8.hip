@@ -518,136 +518,25 @@ extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w8a8_nk_any(
 }
 
 // Any K and any operand alignment on the matrix cores, for the shapes the kernels above do not take (K not a
-// multiple of 128, operands off 16-byte alignment, operands of 4 GiB and more).  128 x 128 tiles, four waves (2 x 2)
-// of 64 x 64; a k-step of 128 bytes per row goes through registers into one LDS stage (row pitch 144 bytes: the
-// sixteen rows of a fragment read start in sixteen different groups of four banks), the next k-step's global
-// loads in flight while the MFMAs of this one run.  Global accesses are 16 bytes at byte alignment; the chunk that
-// straddles K is read byte by byte and padded with zeros, rows past M / N read as zeros.  The finished tile is
-// staged through the same LDS so that the stores are whole 128-byte row pieces.
-// (a [M,K] i8, w_nk [N,K] i8, a_scale [M] f32, w_scale [N] f32, y [M,N] f16, M, K, N) grid: any, tiles are dealt
-// round-robin (all row tiles of one 128-column panel next to each other), block = 256.
-namespace edge {
-constexpr int kTile = 128, kStep = 128, kPitch = 144;
-typedef u32x4 u32x4_bytes __attribute__((aligned(1)));
-typedef u32x4 u32x4_halves __attribute__((aligned(2)));
-
-__device__ __forceinline__ u32x4 load_chunk(const int8_t* __restrict__ base, int64_t row, int64_t rows, int64_t K, int64_t k) {
-  u32x4 v = {0u, 0u, 0u, 0u};
-  if (row >= rows || k >= K) return v;
-  const int8_t* p = base + row * K + k;
-  if (k + 16 <= K) return *reinterpret_cast<const u32x4_bytes*>(p);
-  const int left = int(K - k);                         // 1 .. 15 bytes: the one chunk of a row that straddles K
-  uint64_t lo = 0, hi = 0;
-#pragma unroll 1
-  for (int b = 0; b < left; ++b) {
-    const uint64_t byte = uint8_t(p[b]);
-    if (b < 8) lo |= byte << (8 * b);
-    else hi |= byte << (8 * (b - 8));
+// multiple of 128, operands off 16-byte alignment, operands of 4 GiB and more): the 128 x 128 tile loop of
+// gemm_core::edge.  (a [M,K] i8, w_nk [N,K] i8, a_scale [M] f32, w_scale [N] f32, y [M,N] f16, M, K, N)
+// grid: any (tiles are dealt round-robin), block = 256.
+struct EdgeScaleEpilogue {
+  const float* a_scale;
+  const float* w_scale;
+  float as;
+  __device__ __forceinline__ void row(int64_t row, bool valid) { as = valid ? a_scale[row] : 0.0f; }
+  __device__ __forceinline__ uint32_t finish(int acc, int64_t col, bool valid) const {
+    return f32_to_f16_bits((float(acc) * as) * (valid ? w_scale[col] : 0.0f));
   }
-  v[0] = uint32_t(lo); v[1] = uint32_t(lo >> 32); v[2] = uint32_t(hi); v[3] = uint32_t(hi >> 32);
-  return v;
-}
-}  // namespace edge
+};
 
 extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w8a8_nk_edge(
     const int8_t* __restrict__ a, const int8_t* __restrict__ w, const float* __restrict__ a_scale,
     const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N) {
-  using namespace edge;
-  __shared__ __attribute__((aligned(16))) int8_t lds[2 * kTile * kPitch];
-  int8_t* sa = lds;
-  int8_t* sw = lds + kTile * kPitch;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
-  const int frow = lane & 31, fhalf = lane >> 5;
-  const int64_t tiles_m = (M + kTile - 1) / kTile, tiles_n = (N + kTile - 1) / kTile;
-  const int64_t steps = (K + kStep - 1) / kStep;
-  // the four chunks of each operand this lane moves per k-step: rows crow + 32 i, bytes ccol .. ccol + 15
-  const int crow = threadIdx.x >> 3, ccol = (threadIdx.x & 7) * 16;
-  for (int64_t tile = blockIdx.x; tile < tiles_m * tiles_n; tile += gridDim.x) {
-    const int64_t m0 = (tile % tiles_m) * kTile, n0 = (tile / tiles_m) * kTile;
-    v16i acc[2][2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-      for (int j = 0; j < 2; ++j) acc[i][j] = I8Traits::zero();
-    u32x4 ra[4], rw[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      ra[i] = load_chunk(a, m0 + crow + 32 * i, M, K, ccol);
-      rw[i] = load_chunk(w, n0 + crow + 32 * i, N, K, ccol);
-    }
-    for (int64_t s = 0; s < steps; ++s) {
-      __syncthreads();                                 // the previous k-step's (or tile's) LDS reads are done
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        *reinterpret_cast<u32x4*>(sa + (crow + 32 * i) * kPitch + ccol) = ra[i];
-        *reinterpret_cast<u32x4*>(sw + (crow + 32 * i) * kPitch + ccol) = rw[i];
-      }
-      __syncthreads();
-      if (s + 1 < steps) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          ra[i] = load_chunk(a, m0 + crow + 32 * i, M, K, (s + 1) * kStep + ccol);
-          rw[i] = load_chunk(w, n0 + crow + 32 * i, N, K, (s + 1) * kStep + ccol);
-        }
-      }
-#pragma unroll
-      for (int p = 0; p < kStep / 32; ++p) {
-        v4i fa[2], fw[2];
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-          fa[i] = *reinterpret_cast<const v4i*>(sa + (wm * 64 + i * 32 + frow) * kPitch + p * 32 + fhalf * 16);
-          fw[i] = *reinterpret_cast<const v4i*>(sw + (wn * 64 + i * 32 + frow) * kPitch + p * 32 + fhalf * 16);
-        }
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-          for (int j = 0; j < 2; ++j) acc[i][j] = I8Traits::mfma(fw[j], fa[i], acc[i][j]);
-      }
-    }
-    __syncthreads();                                   // all fragment reads done: the stage becomes the output staging
-    // lane (frow, fhalf) holds row frow of each 32 x 32 block, columns 8 q + 4 fhalf + e in register 4 q + e
-    int8_t* out = lds + wave * (64 * kPitch);
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int64_t row = m0 + wm * 64 + i * 32 + frow;
-      const float as = row < M ? a_scale[row] : 0.0f;
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int lcol = j * 32 + q * 8 + fhalf * 4;
-          const int64_t col = n0 + wn * 64 + lcol;
-          uint32_t bits[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const float ws = col + e < N ? w_scale[col + e] : 0.0f;
-            bits[e] = f32_to_f16_bits((float(acc[i][j][4 * q + e]) * as) * ws);
-          }
-          u32x2 packed;
-          packed[0] = bits[0] | (bits[1] << 16);
-          packed[1] = bits[2] | (bits[3] << 16);
-          *reinterpret_cast<u32x2*>(out + (i * 32 + frow) * kPitch + lcol * 2) = packed;
-        }
-    }
-    // a wave reads back only what it wrote, and its own LDS accesses complete in order: no workgroup barrier
-    __builtin_amdgcn_wave_barrier();
-#pragma unroll
-    for (int r = 0; r < 8; ++r) {
-      const int lrow = r * 8 + (lane >> 3), lcol = (lane & 7) * 8;
-      const int64_t row = m0 + wm * 64 + lrow, col = n0 + wn * 64 + lcol;
-      if (row >= M || col >= N) continue;
-      const u32x4 v = *reinterpret_cast<const u32x4*>(out + lrow * kPitch + lcol * 2);
-      uint16_t* dst = y + row * N + col;
-      if (col + 8 <= N) {
-        *reinterpret_cast<u32x4_halves*>(dst) = v;
-      } else {
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (col + e < N) dst[e] = uint16_t(v[e >> 1] >> (16 * (e & 1)));
-      }
-    }
-  }
+  __shared__ __attribute__((aligned(16))) int8_t lds[gemm_core::edge::kLdsBytes];
+  EdgeScaleEpilogue epi{a_scale, w_scale, 0.0f};
+  gemm_core::edge::run<I8Traits>(a, w, K, epi, y, M, N, lds);
 }
 
 // Weight re-layout [K,N] -> [N,K], bytes.  64 x 64 tiles through LDS; both the global
