@@ -406,8 +406,8 @@ __device__ __forceinline__ bool tile_origin(int64_t M, int64_t N, int64_t& m0, i
 // b [N, row_bytes].  128 x 128 tiles, four waves (2 x 2) of 64 x 64; a k-step of 128 bytes per row goes through
 // registers into one LDS stage (row pitch 144 bytes: the sixteen rows of a fragment read start in sixteen different
 // groups of four banks), the next k-step's global loads in flight while the MFMAs of this one run.  Global
-// accesses are 16 bytes at byte alignment; the chunk that straddles the end of a row is read byte by byte and padded
-// with zeros (a zero in both operands: the padded products are exact zeros for integers and floats alike), rows
+// accesses are 16 bytes at byte alignment; the chunk that straddles the end of a row is read byte by byte (in the last
+// k-step only, so that no other step's loads wait on that loop) and padded with zeros (a zero in both operands: the padded products are exact zeros for integers and floats alike), rows
 // past M / N read as zeros.  16-bit outputs are staged through the same LDS so that the stores are whole 128-byte
 // row pieces; 32-bit outputs go out as 16-byte pieces straight from the accumulators.
 // Traits as for `run`.  Epilogue: row(row, row < M) once per output row of the lane, then finish(sum, col, col < N)
@@ -420,12 +420,19 @@ typedef u32x4 u32x4_bytes __attribute__((aligned(1)));
 typedef u32x4 u32x4_halves __attribute__((aligned(2)));
 typedef f32x4 f32x4_words __attribute__((aligned(4)));
 
+// A 16-byte chunk that lies wholly inside its row; zeros otherwise (rows past the last one, the chunk that straddles
+// the end of a row: see finish_chunk).  No loop in here: the callers' loads stay in flight together.
 __device__ __forceinline__ u32x4 load_chunk(const int8_t* __restrict__ base, int64_t row, int64_t rows, int64_t row_bytes, int64_t k) {
   u32x4 v = {0u, 0u, 0u, 0u};
-  if (row >= rows || k >= row_bytes) return v;
+  if (row < rows && k + 16 <= row_bytes) v = *reinterpret_cast<const u32x4_bytes*>(base + row * row_bytes + k);
+  return v;
+}
+// The chunk that straddles the end of its row (1 .. 15 bytes inside), byte by byte; any other chunk is returned as it
+// is.  Only the last k-step of rows that are not whole chunks has such a chunk: callers test that first.
+__device__ __forceinline__ u32x4 finish_chunk(u32x4 v, const int8_t* __restrict__ base, int64_t row, int64_t rows, int64_t row_bytes, int64_t k) {
+  if (row >= rows || k >= row_bytes || k + 16 <= row_bytes) return v;
   const int8_t* p = base + row * row_bytes + k;
-  if (k + 16 <= row_bytes) return *reinterpret_cast<const u32x4_bytes*>(p);
-  const int left = int(row_bytes - k);                 // 1 .. 15 bytes: the one chunk of a row that straddles its end
+  const int left = int(row_bytes - k);
   uint64_t lo = 0, hi = 0;
 #pragma unroll 1
   for (int b = 0; b < left; ++b) {
@@ -436,6 +443,115 @@ __device__ __forceinline__ u32x4 load_chunk(const int8_t* __restrict__ base, int
   v[0] = uint32_t(lo); v[1] = uint32_t(lo >> 32); v[2] = uint32_t(hi); v[3] = uint32_t(hi >> 32);
   return v;
 }
+// The four chunks of one operand a lane moves per k-step: rows r0 + crow + 32 i, bytes k .. k + 15.
+__device__ __forceinline__ void load_chunks(u32x4 (&r)[4], const int8_t* __restrict__ base, int64_t r0, int64_t rows, int64_t row_bytes,
+                                            int64_t k, bool last_step) {
+  const int crow = threadIdx.x >> 3;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) r[i] = load_chunk(base, r0 + crow + 32 * i, rows, row_bytes, k);
+  if (last_step && (row_bytes & 15)) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r[i] = finish_chunk(r[i], base, r0 + crow + 32 * i, rows, row_bytes, k);
+  }
+}
+
+// One k-step of the four waves from the two operand stages (128 rows of kPitch bytes each, kStep bytes of k per row).
+template <class Traits>
+__device__ __forceinline__ void multiply_stage(typename Traits::Acc (&acc)[2][2], const int8_t* sa, const int8_t* sb) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int frow = lane & 31, fhalf = lane >> 5;
+#pragma unroll
+  for (int p = 0; p < kStep / 32; ++p) {
+    v4i fa[2], fb[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      fa[i] = *reinterpret_cast<const v4i*>(sa + (wm * 64 + i * 32 + frow) * kPitch + p * 32 + fhalf * 16);
+      fb[i] = *reinterpret_cast<const v4i*>(sb + (wn * 64 + i * 32 + frow) * kPitch + p * 32 + fhalf * 16);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) acc[i][j] = Traits::mfma(fb[j], fa[i], acc[i][j]);
+  }
+}
+
+// The finished 128 x 128 tile of the four waves (acc[i][j]: rows 64 wm + 32 i, columns 64 wn + 32 j) out to y through
+// the epilogue; `lds` (at least kLdsBytes) is the staging of 16-bit outputs and must no longer be read as operands
+// by any wave when a wave's stores begin (the barrier below), nor written again before the caller's next barrier.
+template <class Acc, class Epilogue, typename Y>
+__device__ __forceinline__ void write_tile(Acc (&acc)[2][2], Epilogue& epi, Y* __restrict__ y, int64_t M, int64_t N, int64_t m0,
+                                           int64_t n0, int8_t* lds) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int frow = lane & 31, fhalf = lane >> 5;
+  // lane (frow, fhalf) holds row frow of each 32 x 32 block, columns 8 q + 4 fhalf + e in register 4 q + e
+  if constexpr (sizeof(Y) == 2) {
+    __syncthreads();                                 // all fragment reads done: the stage becomes the output staging
+    int8_t* out = lds + wave * (64 * kPitch);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int64_t row = m0 + wm * 64 + i * 32 + frow;
+      epi.row(row, row < M);
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int lcol = j * 32 + q * 8 + fhalf * 4;
+          const int64_t col = n0 + wn * 64 + lcol;
+          uint32_t bits[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) bits[e] = epi.finish(acc[i][j][4 * q + e], col + e, col + e < N);
+          u32x2 packed;
+          packed[0] = bits[0] | (bits[1] << 16);
+          packed[1] = bits[2] | (bits[3] << 16);
+          *reinterpret_cast<u32x2*>(out + (i * 32 + frow) * kPitch + lcol * 2) = packed;
+        }
+    }
+    // a wave reads back only what it wrote, and its own LDS accesses complete in order: no workgroup barrier
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const int lrow = r * 8 + (lane >> 3), lcol = (lane & 7) * 8;
+      const int64_t row = m0 + wm * 64 + lrow, col = n0 + wn * 64 + lcol;
+      if (row >= M || col >= N) continue;
+      const u32x4 v = *reinterpret_cast<const u32x4*>(out + lrow * kPitch + lcol * 2);
+      uint16_t* dst = y + row * N + col;
+      if (col + 8 <= N) {
+        *reinterpret_cast<u32x4_halves*>(dst) = v;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (col + e < N) dst[e] = uint16_t(v[e >> 1] >> (16 * (e & 1)));
+      }
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int64_t row = m0 + wm * 64 + i * 32 + frow;
+      epi.row(row, row < M);
+      if (row >= M) continue;
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int64_t col = n0 + wn * 64 + j * 32 + q * 8 + fhalf * 4;
+          if (col >= N) continue;
+          f32x4 v;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = epi.finish(acc[i][j][4 * q + e], col + e, col + e < N);
+          float* dst = y + row * N + col;
+          if (col + 4 <= N) {
+            *reinterpret_cast<f32x4_words*>(dst) = v;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (col + e < N) dst[e] = v[e];
+          }
+        }
+    }
+  }
+}
 
 template <class Traits, class Epilogue, typename Y>
 __device__ __forceinline__ void run(const int8_t* __restrict__ a, const int8_t* __restrict__ b, int64_t row_bytes, Epilogue& epi,
@@ -443,9 +559,6 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, const int8_t* 
   using Acc = typename Traits::Acc;
   int8_t* sa = lds;
   int8_t* sb = lds + kTile * kPitch;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
-  const int frow = lane & 31, fhalf = lane >> 5;
   const int64_t tiles_m = (M + kTile - 1) / kTile, tiles_n = (N + kTile - 1) / kTile;
   const int64_t steps = (row_bytes + kStep - 1) / kStep;
   // the four chunks of each operand this lane moves per k-step: rows crow + 32 i, bytes ccol .. ccol + 15
@@ -458,11 +571,8 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, const int8_t* 
 #pragma unroll
       for (int j = 0; j < 2; ++j) acc[i][j] = Traits::zero();
     u32x4 ra[4], rb[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      ra[i] = load_chunk(a, m0 + crow + 32 * i, M, row_bytes, ccol);
-      rb[i] = load_chunk(b, n0 + crow + 32 * i, N, row_bytes, ccol);
-    }
+    load_chunks(ra, a, m0, M, row_bytes, ccol, steps == 1);
+    load_chunks(rb, b, n0, N, row_bytes, ccol, steps == 1);
     for (int64_t s = 0; s < steps; ++s) {
       __syncthreads();                                 // the previous k-step's (or tile's) LDS reads are done
 #pragma unroll
@@ -472,92 +582,12 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, const int8_t* 
       }
       __syncthreads();
       if (s + 1 < steps) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          ra[i] = load_chunk(a, m0 + crow + 32 * i, M, row_bytes, (s + 1) * kStep + ccol);
-          rb[i] = load_chunk(b, n0 + crow + 32 * i, N, row_bytes, (s + 1) * kStep + ccol);
-        }
+        load_chunks(ra, a, m0, M, row_bytes, (s + 1) * kStep + ccol, s + 2 == steps);
+        load_chunks(rb, b, n0, N, row_bytes, (s + 1) * kStep + ccol, s + 2 == steps);
       }
-#pragma unroll
-      for (int p = 0; p < kStep / 32; ++p) {
-        v4i fa[2], fb[2];
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-          fa[i] = *reinterpret_cast<const v4i*>(sa + (wm * 64 + i * 32 + frow) * kPitch + p * 32 + fhalf * 16);
-          fb[i] = *reinterpret_cast<const v4i*>(sb + (wn * 64 + i * 32 + frow) * kPitch + p * 32 + fhalf * 16);
-        }
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-          for (int j = 0; j < 2; ++j) acc[i][j] = Traits::mfma(fb[j], fa[i], acc[i][j]);
-      }
+      multiply_stage<Traits>(acc, sa, sb);
     }
-    // lane (frow, fhalf) holds row frow of each 32 x 32 block, columns 8 q + 4 fhalf + e in register 4 q + e
-    if constexpr (sizeof(Y) == 2) {
-      __syncthreads();                                 // all fragment reads done: the stage becomes the output staging
-      int8_t* out = lds + wave * (64 * kPitch);
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        const int64_t row = m0 + wm * 64 + i * 32 + frow;
-        epi.row(row, row < M);
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const int lcol = j * 32 + q * 8 + fhalf * 4;
-            const int64_t col = n0 + wn * 64 + lcol;
-            uint32_t bits[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) bits[e] = epi.finish(acc[i][j][4 * q + e], col + e, col + e < N);
-            u32x2 packed;
-            packed[0] = bits[0] | (bits[1] << 16);
-            packed[1] = bits[2] | (bits[3] << 16);
-            *reinterpret_cast<u32x2*>(out + (i * 32 + frow) * kPitch + lcol * 2) = packed;
-          }
-      }
-      // a wave reads back only what it wrote, and its own LDS accesses complete in order: no workgroup barrier
-      __builtin_amdgcn_wave_barrier();
-#pragma unroll
-      for (int r = 0; r < 8; ++r) {
-        const int lrow = r * 8 + (lane >> 3), lcol = (lane & 7) * 8;
-        const int64_t row = m0 + wm * 64 + lrow, col = n0 + wn * 64 + lcol;
-        if (row >= M || col >= N) continue;
-        const u32x4 v = *reinterpret_cast<const u32x4*>(out + lrow * kPitch + lcol * 2);
-        uint16_t* dst = y + row * N + col;
-        if (col + 8 <= N) {
-          *reinterpret_cast<u32x4_halves*>(dst) = v;
-        } else {
-#pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (col + e < N) dst[e] = uint16_t(v[e >> 1] >> (16 * (e & 1)));
-        }
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        const int64_t row = m0 + wm * 64 + i * 32 + frow;
-        epi.row(row, row < M);
-        if (row >= M) continue;
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const int64_t col = n0 + wn * 64 + j * 32 + q * 8 + fhalf * 4;
-            if (col >= N) continue;
-            f32x4 v;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] = epi.finish(acc[i][j][4 * q + e], col + e, col + e < N);
-            float* dst = y + row * N + col;
-            if (col + 4 <= N) {
-              *reinterpret_cast<f32x4_words*>(dst) = v;
-            } else {
-#pragma unroll
-              for (int e = 0; e < 4; ++e)
-                if (col + e < N) dst[e] = v[e];
-            }
-          }
-      }
-    }
+    write_tile(acc, epi, y, M, N, m0, n0, lds);
   }
 }
 }  // namespace edge

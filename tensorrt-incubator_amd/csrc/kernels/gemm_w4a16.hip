@@ -842,6 +842,156 @@ extern "C" __global__ void __launch_bounds__(256) mtrt_w4_prepack_strips(const u
   }
 }
 
+// Any K, N and block on the matrix cores, reading the ORIGINAL packed [K,N] nibbles: for shapes the kernels above do
+// not take (blocks that are not multiples of 64, K that is not, no re-laid weights, operands off alignment).  The
+// 128 x 128 tile loop of gemm_core::edge with the weight stage produced here: a k-step of 64 rows x 128 columns of
+// nibbles (65 bytes a row when a row starts on an odd nibble) goes through registers into a raw LDS stage of 17
+// dwords per row; then every lane dequantises 8 consecutive k of one column at a time (nibble -> f32, times the
+// block's scale, one rounding to f16; the group's first scale is fetched a k-step ahead with the nibbles, another one
+// only when a block ends inside the group) and stores them as one
+// 16-byte piece of the [column][k] stage the fragments are read from.  Rows at and past K and columns at and past
+// N become zeros without touching their scales.
+// (a [M,K] f16, w_kn_packed, scale [K/block, N] f16, y [M,N] f16, M, K, N, block) grid: any, block = 256.
+namespace edge4 {
+constexpr int kRawRow = 68;                            // bytes of a raw row: 17 dwords cover 65 bytes from any byte offset
+constexpr int kRawBytes = 64 * kRawRow;
+typedef uint32_t u32_bytes __attribute__((aligned(1)));
+
+struct HalfEpilogue {
+  __device__ __forceinline__ void row(int64_t, bool) {}
+  __device__ __forceinline__ uint32_t finish(float acc, int64_t, bool) const { return f32_to_f16_bits(acc); }
+};
+
+// dword `dw` of the raw row of k: the bytes holding nibbles (k, n0 ...) onwards; zeros past K.  The last bytes of the
+// weights can end inside a dword: that dword is zero here and read byte by byte by finish_raw.
+__device__ __forceinline__ uint32_t load_raw(const uint8_t* __restrict__ w, int64_t k, int64_t K, int64_t N, int64_t n0, int dw,
+                                             int64_t total_bytes) {
+  const int64_t at = ((k * N + n0) >> 1) + 4 * dw;
+  uint32_t v = 0;
+  if (k < K && at + 4 <= total_bytes) v = *reinterpret_cast<const u32_bytes*>(w + at);
+  return v;
+}
+__device__ __forceinline__ uint32_t finish_raw(uint32_t v, const uint8_t* __restrict__ w, int64_t k, int64_t K, int64_t N, int64_t n0,
+                                               int dw, int64_t total_bytes) {
+  const int64_t at = ((k * N + n0) >> 1) + 4 * dw;
+  if (k >= K || at + 4 <= total_bytes) return v;
+#pragma unroll 1
+  for (int b = 0; b < 4; ++b)
+    if (at + b < total_bytes) v |= uint32_t(w[at + b]) << (8 * b);
+  return v;
+}
+// the five dwords of the raw stage a lane moves per k-step (17 per row, 64 rows from k0 on)
+__device__ __forceinline__ void load_raws(uint32_t (&r)[5], const uint8_t* __restrict__ w, int64_t k0, int64_t K, int64_t N, int64_t n0,
+                                          int64_t total_bytes) {
+#pragma unroll
+  for (int i = 0; i < 5; ++i) {
+    const int idx = threadIdx.x + 256 * i;
+    r[i] = idx < 64 * 17 ? load_raw(w, k0 + idx / 17, K, N, n0, idx % 17, total_bytes) : 0u;
+  }
+  // only the rows next to the end of the weights can have such a dword (the same test for the whole workgroup)
+  const int64_t k_hi = k0 + 63 < K ? k0 + 63 : K - 1;
+  if (((k_hi * N + n0) >> 1) + 4 * 17 > total_bytes) {
+#pragma unroll
+    for (int i = 0; i < 5; ++i) {
+      const int idx = threadIdx.x + 256 * i;
+      if (idx < 64 * 17) r[i] = finish_raw(r[i], w, k0 + idx / 17, K, N, n0, idx % 17, total_bytes);
+    }
+  }
+}
+
+// the scale of (k, n) as its f16 bits (widened where it is used, so that a load a k-step ahead is not waited for
+// where it is issued); 0 where the element does not exist
+__device__ __forceinline__ uint32_t first_scale(const uint16_t* __restrict__ scale, int64_t k, int64_t K, int64_t N, int64_t n, uint32_t blk) {
+  return (k < K && n < N) ? uint32_t(scale[int64_t(uint32_t(k) / blk) * N + n]) : 0u;
+}
+}  // namespace edge4
+
+extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w4a16_edge(
+    const uint16_t* __restrict__ a, const uint8_t* __restrict__ w_kn_packed, const uint16_t* __restrict__ scale,
+    uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t block) {
+  namespace ge = gemm_core::edge;
+  using namespace edge4;
+  __shared__ __attribute__((aligned(16))) int8_t lds[ge::kLdsBytes + kRawBytes];
+  int8_t* sa = lds;
+  int8_t* sb = lds + ge::kTile * ge::kPitch;
+  uint8_t* raw = reinterpret_cast<uint8_t*>(lds + ge::kLdsBytes);
+  const int8_t* a8 = reinterpret_cast<const int8_t*>(a);
+  const int64_t row_bytes = K * 2, total_bytes = (K * N + 1) >> 1;
+  const int64_t tiles_m = (M + ge::kTile - 1) / ge::kTile, tiles_n = (N + ge::kTile - 1) / ge::kTile;
+  const int64_t steps = (K + 63) / 64;
+  const int crow = threadIdx.x >> 3, ccol = (threadIdx.x & 7) * 16;
+  const int dcol = threadIdx.x & 127, dgroup = threadIdx.x >> 7;     // dequantise: column of the tile, k groups dgroup + 2 i
+  const uint32_t blk = uint32_t(block);
+  HalfEpilogue epi;
+  for (int64_t tile = blockIdx.x; tile < tiles_m * tiles_n; tile += gridDim.x) {
+    const int64_t m0 = (tile % tiles_m) * ge::kTile, n0 = (tile / tiles_m) * ge::kTile;
+    v16f acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) acc[i][j] = F16Traits::zero();
+    u32x4 ra[4];
+    uint32_t rw[5];
+    uint32_t rs[4];                                    // the scale (f16 bits) of the first k of each of the lane's four groups
+    const int64_t n = n0 + dcol;
+    ge::load_chunks(ra, a8, m0, M, row_bytes, ccol, steps == 1);
+    load_raws(rw, w_kn_packed, 0, K, N, n0, total_bytes);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) rs[i] = first_scale(scale, (dgroup + 2 * i) * 8, K, N, n, blk);
+    for (int64_t s = 0; s < steps; ++s) {
+      __syncthreads();                                 // the previous k-step's (or tile's) LDS reads are done
+#pragma unroll
+      for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(sa + (crow + 32 * i) * ge::kPitch + ccol) = ra[i];
+#pragma unroll
+      for (int i = 0; i < 5; ++i) {
+        const int idx = threadIdx.x + 256 * i;
+        if (idx < 64 * 17) *reinterpret_cast<uint32_t*>(raw + 4 * idx) = rw[i];
+      }
+      __syncthreads();
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int g = dgroup + 2 * i;                  // the same for the whole wave
+        const int64_t k0 = s * 64 + g * 8;
+        const uint32_t kb0 = uint32_t(k0) / blk, rem0 = uint32_t(k0) - kb0 * blk;
+        // the eight bytes first, then the arithmetic: rows at and past K hold zeros, every address is inside the stage
+        uint32_t byte[8];
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) {
+          const uint32_t pos = uint32_t(dcol) + uint32_t(((k0 + kk) & N) & 1);  // n0 is even: the row starts at nibble (k N) mod 2
+          byte[kk] = uint32_t(raw[(g * 8 + kk) * kRawRow + (pos >> 1)]) >> (4 * (pos & 1));
+        }
+        float sc[8];
+        if (rem0 + 8 <= blk) {                         // one block for the group (wave-uniform): the scale fetched ahead
+#pragma unroll
+          for (int kk = 0; kk < 8; ++kk) sc[kk] = f16_bits_to_f32(rs[i]);
+        } else {
+#pragma unroll
+          for (int kk = 0; kk < 8; ++kk) sc[kk] = f16_bits_to_f32(first_scale(scale, k0 + kk, K, N, n, blk));
+        }
+        uint32_t h[8];
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) {
+          const uint32_t bits = f32_to_f16_bits(float(int(byte[kk] << 28) >> 28) * sc[kk]);
+          h[kk] = (k0 + kk < K && n < N) ? bits : 0u;   // no NaN from a scale that does not exist or is not finite
+        }
+        u32x4 packed;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) packed[e] = h[2 * e] | (h[2 * e + 1] << 16);
+        *reinterpret_cast<u32x4*>(sb + dcol * ge::kPitch + g * 16) = packed;
+      }
+      __syncthreads();
+      if (s + 1 < steps) {
+        ge::load_chunks(ra, a8, m0, M, row_bytes, (s + 1) * ge::kStep + ccol, s + 2 == steps);
+        load_raws(rw, w_kn_packed, (s + 1) * 64, K, N, n0, total_bytes);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) rs[i] = first_scale(scale, (s + 1) * 64 + (dgroup + 2 * i) * 8, K, N, n, blk);
+      }
+      ge::multiply_stage<F16Traits>(acc, sa, sb);
+    }
+    ge::write_tile(acc, epi, y, M, N, m0, n0, lds);
+  }
+}
+
 // Any shape: one output per lane, reading the ORIGINAL packed [K,N] nibbles; not a fast path.
 extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w4a16_any(
     const uint16_t* __restrict__ a, const uint8_t* __restrict__ w_kn_packed, const uint16_t* __restrict__ scale,

@@ -989,6 +989,13 @@ int32_t mtrt_hip_gemm_w4a16(mtrt_stream_t stream, const void *a, const void *w_k
     return set_error(MTRT_INVALID_ARGUMENT, "this shape needs the original packed weights (K=%lld block=%lld)",
                      (long long)K, (long long)block);
   void *args[] = {&a, &w_kn_packed, &scale, &y, &M, &K, &N, &block};
+  if (K > 0) {
+    // any block, K, N and alignment from the original nibbles, still on the matrix cores: 128 x 128 tiles whose
+    // weight stage is dequantised in the kernel (M = 256, K = N = 4096, block 32: 3660 us on the kernel below)
+    const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
+    return launch(st, KernelName("mtrt_gemm_w4a16_edge"), uint32_t(std::min<int64_t>(tiles, int64_t(kMaxGrid) * 1024)), kBlock,
+                  as_hip(stream), args);
+  }
   return launch(st, KernelName("mtrt_gemm_w4a16_any"), blocks_for(M * N, kBlock), kBlock, as_hip(stream), args);
 }
 

@@ -97,7 +97,7 @@ def test_embedded_code_object_is_gfx950_and_has_the_kernels(pkg):
     names += ["mtrt_fill", "mtrt_gemm_dense_f32", "mtrt_gemm_dense_f16", "mtrt_gemm_dense_bf16", "mtrt_gemm_dense_mfma_f16", "mtrt_gemm_dense_mfma_bf16", "mtrt_gemm_dense_mfma_f32", "mtrt_gemm_dense_edge_f32", "mtrt_gemm_dense_edge_f16", "mtrt_gemm_dense_edge_bf16", "mtrt_gemm_w8a8_frag",
               "mtrt_gemm_w8a8_small16", "mtrt_gemm_w8a8_small32", "mtrt_gemm_w8a8_nk", "mtrt_gemm_w8a8_nk_edge", "mtrt_gemm_w8a8_nk_any", "mtrt_gemm_w4a16_t256x256",
               "mtrt_gemm_w4a16_t128x128", "mtrt_gemm_w4a16_t128x64", "mtrt_gemm_w4a16_skinny", "mtrt_gemm_w4a16_skinny16",
-              "mtrt_gemm_w4a16_strips16"]
+              "mtrt_gemm_w4a16_strips16", "mtrt_gemm_w4a16_edge", "mtrt_gemm_w4a16_any"]
     for n in names:
         assert n.encode() + b"\x00" in blob, "kernel %s is not in the code object" % n
     # measurement yardsticks and launch-ABI fixtures live in their own module, not in the product code object

@@ -247,13 +247,43 @@ def test_w4a16_dequantised_weights_are_bit_exact(pkg, orc):
         assert np.array_equal(bits16(y).reshape(-1, N), wd[rows]), kernel
 
 
-def test_w4a16_generic_kernel(pkg, orc):
-    for (M, K, N, B) in ((5, 48, 7, 16), (9, 100, 33, 20), (3, 128, 6, 128)):
-        a, w, wp, s = _w4a16_inputs(orc, rng(M * K + N), M, K, N, B)
-        y, kernel = _run_w4a16(pkg, a, wp, s, K, N, B, prepack=False)
-        assert kernel == "mtrt_gemm_w4a16_any"
-        # same left-to-right f32 accumulation as the host: bit-identical
-        assert np.array_equal(bits16(y).reshape(M, N), orc.gemm_w4a16(a, wp, s, K, N, B))
+@pytest.mark.parametrize("case", [(5, 48, 7, 16), (9, 100, 33, 20), (3, 128, 6, 128), (130, 256, 200, 32), (70, 192, 131, 16),
+                                  (256, 520, 129, 8), (33, 77, 300, 7), (140, 1024, 257, 1024), (64, 4096, 130, 32), (3, 65, 1, 65), (4, 70, 3, 5), (2, 129, 7, 43)])
+def test_w4a16_any_shape_kernel(pkg, orc, case):
+    """Blocks that are not multiples of 64, K that is not, odd N (rows of nibbles that start in the middle of a byte),
+    no re-laid weights: the 128 x 128 tile kernel that dequantises the original nibbles.  f32 sums in the matrix
+    cores' order: within the bound of the tile kernels, against the oracle and against float64."""
+    M, K, N, B = case
+    a, w, wp, s = _w4a16_inputs(orc, rng(M * K + N), M, K, N, B)
+    print("case: w4a16 any shape", case, flush=True)
+    y, kernel = _run_w4a16(pkg, a, wp, s, K, N, B, prepack=False)
+    assert kernel == "mtrt_gemm_w4a16_edge"
+    _check_w4a16(orc, y, a, w, s, K, N, B, orc.gemm_w4a16(a, wp, s, K, N, B))
+
+
+@pytest.mark.parametrize("case", [(200, 131, 8), (136, 257, 17), (128, 130, 32)])
+def test_w4a16_any_shape_kernel_dequantises_bit_exactly(pkg, orc, case):
+    """One-hot activations read the dequantised weights back unchanged: pins the nibble of every (k, n) for odd and
+    even N, the block index of the scale when a group of eight k crosses blocks, and the single f16 rounding."""
+    K, N, B = case
+    g = rng(K + N)
+    w = g.integers(-8, 8, (K, N)).astype(np.int8)
+    s = orc.narrow(g.uniform(0.005, 0.02, (K // B, N)).astype(np.float32), orc.F16)
+    eye = np.zeros((K, K), np.float32)
+    np.fill_diagonal(eye, 1.0)
+    wd = (w.astype(np.float16) * np.repeat(s.view(np.float16), B, axis=0)).view(np.uint16)
+    y, kernel = _run_w4a16(pkg, orc.narrow(eye, orc.F16), orc.pack_int4(w), s, K, N, B, prepack=False)
+    assert kernel == "mtrt_gemm_w4a16_edge"
+    assert np.array_equal(bits16(y).reshape(K, N), wd)
+
+
+def test_w4a16_block_of_32_with_re_laid_weights_present(pkg, orc):
+    """A block the tile kernels do not take, with both weight layouts passed: the original nibbles are used."""
+    M, K, N, B = 100, 512, 192, 32
+    a, w, wp, s = _w4a16_inputs(orc, rng(9), M, K, N, B)
+    y, kernel = _run_w4a16(pkg, a, wp, s, K, N, B)
+    assert kernel == "mtrt_gemm_w4a16_edge"
+    _check_w4a16(orc, y, a, w, s, K, N, B, orc.gemm_w4a16(a, wp, s, K, N, B))
 
 
 @pytest.mark.parametrize("M", [16, 256, 4096])
