@@ -364,7 +364,9 @@ MTRT_CAPI_EXPORTED int32_t mtrt_hip_softmax(mtrt_stream_t stream, const void *x,
  * TransformSchedules/fallback-schedule-matmul.mlir:24).  Weights are program constants: they are
  * re-laid ONCE from the program's [K,N] into [N,K] (K contiguous, what the matrix cores read) by
  * the prepack call; the GEMM takes the re-laid weights.  a: int8 [M,K]; a_scale: f32 [M];
- * w_scale: f32 [N]; y: f16 [M,N]. */
+ * w_scale: f32 [N]; y: f16 [M,N].  Any M, K, N and any operand alignment run on the matrix cores (K that
+ * is a multiple of 128 with 16-byte aligned operands on the faster tile loop); the sums are integers, so
+ * every kernel gives the same bits. */
 MTRT_CAPI_EXPORTED int32_t mtrt_hip_gemm_w8a8_prepack(mtrt_stream_t stream, const void *w_kn,
                                                       void *w_nk, int64_t K, int64_t N);
 MTRT_CAPI_EXPORTED int32_t mtrt_hip_gemm_w8a8(mtrt_stream_t stream, const void *a, const void *w_nk,
@@ -395,9 +397,10 @@ MTRT_CAPI_EXPORTED int32_t mtrt_hip_gemm_w8a8_fragments(mtrt_stream_t stream, co
  * prepack call, mtrt_hip_gemm_w4a16_prepacked_bytes(K, N) bytes, needs K % 64 == 0; it holds the weights in
  * the fragment order of the 32-column kernels and, when K % 128 == 0, once more in the strip order of the
  * M <= 16 kernel, so it is about K * N bytes); they are
- * used when w_prepacked is given and K % 64 == 0, block % 64 == 0, K % block == 0.  Otherwise the
- * generic kernel reads w_kn_packed directly (any shape, slow).  Either weight pointer may be NULL
- * if the other path applies. */
+ * used when w_prepacked is given and K % 64 == 0, block % 64 == 0, K % block == 0.  Otherwise a
+ * matrix-core kernel that dequantises the original nibbles tile by tile reads w_kn_packed directly
+ * (any block that divides K, any K and N; several times slower than the re-laid form).  Either weight
+ * pointer may be NULL if the other path applies. */
 MTRT_CAPI_EXPORTED int64_t mtrt_hip_gemm_w4a16_prepacked_bytes(int64_t K, int64_t N);
 MTRT_CAPI_EXPORTED int32_t mtrt_hip_gemm_w4a16_prepack(mtrt_stream_t stream, const void *w_kn_packed,
                                                        void *w_prepacked, int64_t K, int64_t N);
@@ -410,8 +413,9 @@ MTRT_CAPI_EXPORTED int32_t mtrt_hip_gemm_w4a16(mtrt_stream_t stream, const void 
  * accumulation; bias may be NULL.  The float matmul of the fake-quant Linear (linear.py:112-151:
  * out = x' @ W'^T + b on dequantized operands) for the parameter combinations the two matrix-core clusters
  * above do not express, and of the unquantized module; w_nk is the module's own [out_features, in_features]
- * weight.  A tiled FMA kernel, the class of code the reference generates for a matmul
- * (fallback-schedule-matmul.mlir:24); any shape, no alignment needs. */
+ * weight.  The reference generates a tiled FMA loop nest for such a matmul
+ * (fallback-schedule-matmul.mlir:24); here every shape with K > 0 runs on the matrix cores (f16 / bf16 / f32
+ * MFMA with f32 accumulation), any shape, no alignment needs beyond the element size. */
 MTRT_CAPI_EXPORTED int32_t mtrt_hip_linear_dense(mtrt_stream_t stream, const void *x, const void *w_nk,
                                                  const void *bias, void *y, int32_t dtype, int64_t M,
                                                  int64_t K, int64_t N);

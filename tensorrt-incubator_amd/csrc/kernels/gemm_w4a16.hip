@@ -960,19 +960,20 @@ extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w4a16_edge(
           const uint32_t pos = uint32_t(dcol) + uint32_t(((k0 + kk) & N) & 1);  // n0 is even: the row starts at nibble (k N) mod 2
           byte[kk] = uint32_t(raw[(g * 8 + kk) * kRawRow + (pos >> 1)]) >> (4 * (pos & 1));
         }
-        float sc[8];
-        if (rem0 + 8 <= blk) {                         // one block for the group (wave-uniform): the scale fetched ahead
+        uint32_t h[8];
+        if (rem0 + 8 <= blk && k0 + 8 <= K) {
+          // one block for the group and all of it below K (the same for the whole wave): the scale fetched ahead; it is
+          // zero in the lanes of columns at and past N, whose nibbles belong to the next row
+          const float sc = f16_bits_to_f32(rs[i]);
 #pragma unroll
-          for (int kk = 0; kk < 8; ++kk) sc[kk] = f16_bits_to_f32(rs[i]);
+          for (int kk = 0; kk < 8; ++kk) h[kk] = f32_to_f16_bits(float(int(byte[kk] << 28) >> 28) * sc);
         } else {
 #pragma unroll
-          for (int kk = 0; kk < 8; ++kk) sc[kk] = f16_bits_to_f32(first_scale(scale, k0 + kk, K, N, n, blk));
-        }
-        uint32_t h[8];
-#pragma unroll
-        for (int kk = 0; kk < 8; ++kk) {
-          const uint32_t bits = f32_to_f16_bits(float(int(byte[kk] << 28) >> 28) * sc[kk]);
-          h[kk] = (k0 + kk < K && n < N) ? bits : 0u;   // no NaN from a scale that does not exist or is not finite
+          for (int kk = 0; kk < 8; ++kk) {
+            const float sc = f16_bits_to_f32(first_scale(scale, k0 + kk, K, N, n, blk));
+            const uint32_t bits = f32_to_f16_bits(float(int(byte[kk] << 28) >> 28) * sc);
+            h[kk] = (k0 + kk < K && n < N) ? bits : 0u; // no NaN from a scale that is not finite times the zeros past K
+          }
         }
         u32x4 packed;
 #pragma unroll
