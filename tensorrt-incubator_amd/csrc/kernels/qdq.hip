@@ -144,9 +144,26 @@ __device__ __forceinline__ uint32_t pack4(const float* v, int flags) {
 }
 template <>
 __device__ __forceinline__ uint32_t pack4<F8>(const float* v, int flags) {
-  if (flags & kFlagF8RefHost)
-    return f32_to_f8_refhost(v[0]) | (f32_to_f8_refhost(v[1]) << 8) | (f32_to_f8_refhost(v[2]) << 16) |
-           (f32_to_f8_refhost(v[3]) << 24);
+  if (flags & kFlagF8RefHost) {
+    // The host class (f32_to_f8_refhost) equals the hardware's round-to-nearest-even except that every result with
+    // the top exponent (256 .. 448) becomes 448, and that it rounds differently below the normal range
+    // (2^-10 <= |v| < 2^-6; smaller values are zero both ways).  So: the hardware conversion, the top exponent
+    // fixed up on the four bytes at once, and the software form only for the elements, and in the waves, where a lane
+    // holds such a small value (with scales derived from amax about one value in 10^4).
+    int hw = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], 0, false);
+    hw = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], hw, true);
+    uint32_t codes = uint32_t(hw);
+    const uint32_t top = (((codes & 0x7F7F7F7Fu) + 0x08080808u) >> 7) & 0x01010101u;   // magnitude >= 0x78, per byte
+    codes = (codes | (top * 0x7Eu)) & ~top;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const bool small = ((f32_to_bits(v[k]) & 0x7FFFFFFFu) - 0x3A800000u) < 0x02000000u;
+      if (__builtin_amdgcn_ballot_w64(small)) {
+        if (small) codes = (codes & ~(0xFFu << (8 * k))) | (f32_to_f8_refhost(v[k]) << (8 * k));
+      }
+    }
+    return codes;
+  }
   // The reference's generated GPU code never converts f32 to f8 directly: it truncates to f16 first and
   // converts that (mlir-tensorrt/kernel/lib/Kernel/Transforms/NormalizeQuantizedConversions.cpp:38-118,
   // cvt.rn.satfinite.e4m3x2.f16x2 in LowerToNVVM.cpp:281-339).  Both steps round to nearest even, so a value
