@@ -846,10 +846,9 @@ extern "C" __global__ void __launch_bounds__(256) mtrt_w4_prepack_strips(const u
 // not take (blocks that are not multiples of 64, K that is not, no re-laid weights, operands off alignment).  The
 // 128 x 128 tile loop of gemm_core::edge with the weight stage produced here: a k-step of 64 rows x 128 columns of
 // nibbles (65 bytes a row when a row starts on an odd nibble) goes through registers into a raw LDS stage of 17
-// dwords per row; then every lane dequantises 8 consecutive k of one column at a time (nibble -> f32, times the
-// block's scale, one rounding to f16; the group's first scale is fetched a k-step ahead with the nibbles, another one
-// only when a block ends inside the group) and stores them as one
-// 16-byte piece of the [column][k] stage the fragments are read from.  Rows at and past K and columns at and past
+// dwords per row; then every lane takes one k row of the step and dequantises eight columns at a time (one dword of
+// nibbles -> f32, times the eight scales of the row's block fetched a k-step ahead, one rounding to f16 each) into
+// 16-bit pieces of the [column][k] stage the fragments are read from.  Rows at and past K and columns at and past
 // N become zeros without touching their scales.
 // (a [M,K] f16, w_kn_packed, scale [K/block, N] f16, y [M,N] f16, M, K, N, block) grid: any, block = 256.
 namespace edge4 {
@@ -899,10 +898,19 @@ __device__ __forceinline__ void load_raws(uint32_t (&r)[5], const uint8_t* __res
   }
 }
 
-// the scale of (k, n) as its f16 bits (widened where it is used, so that a load a k-step ahead is not waited for
-// where it is issued); 0 where the element does not exist
-__device__ __forceinline__ uint32_t first_scale(const uint16_t* __restrict__ scale, int64_t k, int64_t K, int64_t N, int64_t n, uint32_t blk) {
-  return (k < K && n < N) ? uint32_t(scale[int64_t(uint32_t(k) / blk) * N + n]) : 0u;
+// the f16 scales of columns n .. n + 7 in the block of row k, as four words of two; zeros where the element does not
+// exist.  Fetched a k-step ahead and widened only where they are used, so that the load is not waited for where it
+// is issued; all lanes of a wave whose rows share a block read the same 16 bytes.
+typedef u32x4 u32x4_halves __attribute__((aligned(2)));
+__device__ __forceinline__ u32x4 load_scales8(const uint16_t* __restrict__ scale, int64_t k, int64_t K, int64_t N, int64_t n, uint32_t blk) {
+  u32x4 v = {0u, 0u, 0u, 0u};
+  if (k >= K || n >= N) return v;
+  const uint16_t* p = scale + int64_t(uint32_t(k) / blk) * N + n;
+  if (n + 8 <= N) return *reinterpret_cast<const u32x4_halves*>(p);
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+    if (n + j < N) v[j >> 1] |= uint32_t(p[j]) << (16 * (j & 1));
+  return v;
 }
 }  // namespace edge4
 
@@ -920,7 +928,7 @@ extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w4a16_edge(
   const int64_t tiles_m = (M + ge::kTile - 1) / ge::kTile, tiles_n = (N + ge::kTile - 1) / ge::kTile;
   const int64_t steps = (K + 63) / 64;
   const int crow = threadIdx.x >> 3, ccol = (threadIdx.x & 7) * 16;
-  const int dcol = threadIdx.x & 127, dgroup = threadIdx.x >> 7;     // dequantise: column of the tile, k groups dgroup + 2 i
+  const int drow = threadIdx.x & 63, dwave = threadIdx.x >> 6;       // dequantise: k row of the step, column groups 4 dwave + i
   const uint32_t blk = uint32_t(block);
   HalfEpilogue epi;
   for (int64_t tile = blockIdx.x; tile < tiles_m * tiles_n; tile += gridDim.x) {
@@ -932,12 +940,11 @@ extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w4a16_edge(
       for (int j = 0; j < 2; ++j) acc[i][j] = F16Traits::zero();
     u32x4 ra[4];
     uint32_t rw[5];
-    uint32_t rs[4];                                    // the scale (f16 bits) of the first k of each of the lane's four groups
-    const int64_t n = n0 + dcol;
+    u32x4 rs[4];                                       // the eight scales (f16 bits) of each of the lane's four column groups
     ge::load_chunks(ra, a8, m0, M, row_bytes, ccol, steps == 1);
     load_raws(rw, w_kn_packed, 0, K, N, n0, total_bytes);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) rs[i] = first_scale(scale, (dgroup + 2 * i) * 8, K, N, n, blk);
+    for (int i = 0; i < 4; ++i) rs[i] = load_scales8(scale, drow, K, N, n0 + (4 * dwave + i) * 8, blk);
     for (int64_t s = 0; s < steps; ++s) {
       __syncthreads();                                 // the previous k-step's (or tile's) LDS reads are done
 #pragma unroll
@@ -948,44 +955,33 @@ extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w4a16_edge(
         if (idx < 64 * 17) *reinterpret_cast<uint32_t*>(raw + 4 * idx) = rw[i];
       }
       __syncthreads();
+      {
+        // lane = k row of the step: its eight nibbles of a column group are one aligned dword of the raw row (plus
+        // the next byte when the row starts on an odd nibble), its stores are 16-bit pieces of eight columns' rows of
+        // the [column][k] stage, 64 lanes side by side in k.  Rows at and past K hold zero nibbles and get zero
+        // scales, columns at and past N zero scales.
+        const uint8_t* rrow = raw + drow * kRawRow;
+        const uint32_t shift = 4u * uint32_t(((s * 64 + drow) & N) & 1);   // n0 is even: the row starts at nibble (k N) mod 2
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int g = dgroup + 2 * i;                  // the same for the whole wave
-        const int64_t k0 = s * 64 + g * 8;
-        const uint32_t kb0 = uint32_t(k0) / blk, rem0 = uint32_t(k0) - kb0 * blk;
-        // the eight bytes first, then the arithmetic: rows at and past K hold zeros, every address is inside the stage
-        uint32_t byte[8];
+        for (int i = 0; i < 4; ++i) {
+          const int cg = 4 * dwave + i;
+          const uint32_t lo = *reinterpret_cast<const uint32_t*>(rrow + 4 * cg), hi = rrow[4 * cg + 4];
+          const uint32_t nibbles = uint32_t(((uint64_t(hi) << 32) | lo) >> shift);
+          int8_t* dst = sb + (cg * 8) * ge::kPitch + drow * 2;
 #pragma unroll
-        for (int kk = 0; kk < 8; ++kk) {
-          const uint32_t pos = uint32_t(dcol) + uint32_t(((k0 + kk) & N) & 1);  // n0 is even: the row starts at nibble (k N) mod 2
-          byte[kk] = uint32_t(raw[(g * 8 + kk) * kRawRow + (pos >> 1)]) >> (4 * (pos & 1));
-        }
-        uint32_t h[8];
-        if (rem0 + 8 <= blk && k0 + 8 <= K) {
-          // one block for the group and all of it below K (the same for the whole wave): the scale fetched ahead; it is
-          // zero in the lanes of columns at and past N, whose nibbles belong to the next row
-          const float sc = f16_bits_to_f32(rs[i]);
-#pragma unroll
-          for (int kk = 0; kk < 8; ++kk) h[kk] = f32_to_f16_bits(float(int(byte[kk] << 28) >> 28) * sc);
-        } else {
-#pragma unroll
-          for (int kk = 0; kk < 8; ++kk) {
-            const float sc = f16_bits_to_f32(first_scale(scale, k0 + kk, K, N, n, blk));
-            const uint32_t bits = f32_to_f16_bits(float(int(byte[kk] << 28) >> 28) * sc);
-            h[kk] = (k0 + kk < K && n < N) ? bits : 0u; // no NaN from a scale that is not finite times the zeros past K
+          for (int j = 0; j < 8; ++j) {
+            const float sc = f16_bits_to_f32((rs[i][j >> 1] >> (16 * (j & 1))) & 0xFFFFu);
+            const uint32_t bits = f32_to_f16_bits(float(int(nibbles << (28 - 4 * j)) >> 28) * sc);
+            *reinterpret_cast<uint16_t*>(dst + j * ge::kPitch) = uint16_t(bits);
           }
         }
-        u32x4 packed;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) packed[e] = h[2 * e] | (h[2 * e + 1] << 16);
-        *reinterpret_cast<u32x4*>(sb + dcol * ge::kPitch + g * 16) = packed;
       }
       __syncthreads();
       if (s + 1 < steps) {
         ge::load_chunks(ra, a8, m0, M, row_bytes, (s + 1) * ge::kStep + ccol, s + 2 == steps);
         load_raws(rw, w_kn_packed, (s + 1) * 64, K, N, n0, total_bytes);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) rs[i] = first_scale(scale, (s + 1) * 64 + (dgroup + 2 * i) * 8, K, N, n, blk);
+        for (int i = 0; i < 4; ++i) rs[i] = load_scales8(scale, (s + 1) * 64 + drow, K, N, n0 + (4 * dwave + i) * 8, blk);
       }
       ge::multiply_stage<F16Traits>(acc, sa, sb);
     }
