@@ -405,6 +405,15 @@ int32_t view_dispatch(bool quantize, hipStream_t stream, const void *f, int32_t 
   if (kind == MTRT_SCALE_UNIFORM)
     nb = 1;
   int64_t fo = fv->offset, fs0 = fv->stride0, fs1 = fv->stride1, qo = qv->offset, qs0 = qv->stride0, qs1 = qv->stride1;
+  if (fs1 == 1 && qs1 == 1 && (d0 == 1 || (fs0 == d1 && qs0 == d1))) {
+    // Dense in both operands (what a launch with whole row-major tensors passes): the contiguous entry points' own
+    // dispatch on the offset pointers, tile kernels when aligned (f16 [8192, 8192] to i8: 56 us row by row, 41 us so).
+    void *fp = const_cast<char *>(static_cast<const char *>(f)) + fo * float_bytes(f_dtype);
+    void *qp = const_cast<char *>(static_cast<const char *>(q)) + qo;
+    if (quantize)
+      return qdq_dispatch(0, stream, fp, f_dtype, qp, q_dtype, nullptr, scale, kind, d0, d1, nb, flags);
+    return qdq_dispatch(1, stream, nullptr, f_dtype, qp, q_dtype, fp, scale, kind, d0, d1, nb, flags);
+  }
   if (fs1 == 1 && qs1 == 1) {
     // Rows that are contiguous in both operands (row and column slices of row-major tensors, offset sub-tensors): the
     // row-walking kernels of the contiguous entry points, with the views' row strides as pitches (f16 [8192, 8192]

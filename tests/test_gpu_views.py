@@ -106,6 +106,40 @@ def test_views_with_contiguous_rows_take_the_row_walking_kernels(pkg, orc, xname
             assert bool((rest == 7.0).all()), "values outside the destination view were written (%s)" % name
 
 
+@pytest.mark.parametrize("xname", ["f32", "bf16"])
+def test_dense_views_take_the_contiguous_kernels(pkg, orc, xname):
+    """Views that are dense in both operands (whole row-major tensors with an offset, what a launch with memref
+    descriptors usually passes) run the kernels of the contiguous entry points: the tile kernels when the offset
+    pointers are aligned, the row-walking ones otherwise.  Same results as the oracle either way."""
+    import torch
+    td = {"f32": torch.float32, "bf16": torch.bfloat16}[xname]
+    ox = {"f32": orc.F32, "bf16": orc.BF16}[xname]
+    torch.manual_seed(12)
+    d0, d1 = 96, 1024
+    for off, tags in ((0, ("uniform", "row", "col")), (64, ("uniform", "row", "col")), (3, ("rowu", "rowu", "colu"))):
+        xbuf = (torch.randn(off + d0 * d1, device="cuda") * 2).to(td)
+        xv = xbuf[off:].view(d0, d1)
+        xs = xv.cpu().numpy().ravel() if ox == orc.F32 else bits16(xv.contiguous())
+        for (kind, okind, nb, ns), tag in zip(((pkg.SCALE_UNIFORM, orc.SCALE_UNIFORM, 1, 1), (pkg.SCALE_ROW, orc.SCALE_ROW, d0, d0),
+                                              (pkg.SCALE_COL, orc.SCALE_COL, d0 // 32, 32 * d1)), tags):
+            scale = torch.rand(ns, device="cuda") * 0.05 + 0.01
+            qbuf = torch.full((off + d0 * d1 + 5,), 0x55, dtype=torch.uint8, device="cuda")
+            qv = qbuf[off:off + d0 * d1].view(d0, d1)
+            pkg.quantize_view(xv, scale, pkg.I8, qv, kind, nb)
+            assert pkg.last_kernel() == "mtrt_q_%s_%s_i8" % (tag, xname), (off, kind, pkg.last_kernel())
+            q_ref = orc.quantize(xs, ox, orc.I8, scale.cpu().numpy(), okind, d0, d1, nb)
+            assert np.array_equal(qv.cpu().numpy().ravel(), q_ref.view(np.uint8))
+            assert bool((qbuf[:off] == 0x55).all()) and bool((qbuf[off + d0 * d1:] == 0x55).all())
+            ybuf = torch.full((off + d0 * d1 + 5,), 7.0, dtype=td, device="cuda")
+            yv = ybuf[off:off + d0 * d1].view(d0, d1)
+            pkg.dequantize_view(qv, scale, pkg.I8, yv, kind, nb)
+            assert pkg.last_kernel() == "mtrt_dq_%s_%s_i8" % (tag, xname), (off, kind, pkg.last_kernel())
+            y_ref = orc.dequantize(q_ref, orc.I8, ox, scale.cpu().numpy(), okind, d0, d1, nb)
+            got = yv.cpu().numpy().ravel().view(np.uint32) if ox == orc.F32 else bits16(yv.contiguous())
+            assert np.array_equal(got, y_ref.view(np.uint32) if ox == orc.F32 else y_ref)
+            assert bool((ybuf[:off] == 7.0).all()) and bool((ybuf[off + d0 * d1:] == 7.0).all())
+
+
 def test_view_kernel_launched_by_hand_in_the_expanded_argument_order(pkg, orc):
     """memref<?x?xf32, strided<[?, ?], offset: ?>> -> (base, offset, size0, size1, stride0, stride1), per operand."""
     import torch
