@@ -809,11 +809,60 @@ __device__ __forceinline__ void qdq_view(typename X::storage* __restrict__ xb, i
   }
 }
 
+// The same program in 64 x 64 tiles through LDS, for views whose operands run fastest along different dimensions (a
+// transposed source into a row-major destination and the like): one element per lane moves a few bytes per cache
+// line on the side it walks against the grain (f16 [8192, 8192] transposed to i8: 0.9 TB/s).  Here each side is
+// walked along its own fastest dimension: the source side fills the tile (floats, or decoded codes), the
+// destination side empties it, applying the scale of the element's logical (r, c).  The pitch of 65 floats keeps
+// both walks free of bank conflicts.  Grid: any (tiles are dealt round-robin), block = 256.
+template <typename X, typename Q, int MODE>
+__device__ __forceinline__ void qdq_view_tiles(typename X::storage* __restrict__ xb, int64_t xo, int64_t xs0, int64_t xs1,
+                                               typename Q::storage* __restrict__ qb, int64_t qo, int64_t qs0, int64_t qs1,
+                                               const float* __restrict__ scale, int64_t d0, int64_t d1, int64_t nb, int kind,
+                                               int flags) {
+  __shared__ float tile[64][65];
+  auto magnitude = [](int64_t v) { return v < 0 ? -v : v; };
+  const bool x_d0_fast = magnitude(xs0) < magnitude(xs1), q_d0_fast = magnitude(qs0) < magnitude(qs1);
+  const bool src_d0_fast = MODE == 0 ? x_d0_fast : q_d0_fast, dst_d0_fast = MODE == 0 ? q_d0_fast : x_d0_fast;
+  const int64_t tiles_c = (d1 + 63) / 64, tiles = ((d0 + 63) / 64) * tiles_c;
+  const int a = threadIdx.x & 63, b0 = threadIdx.x >> 6;
+  for (int64_t t = blockIdx.x; t < tiles; t += gridDim.x) {
+    const int64_t r0 = (t / tiles_c) * 64, c0 = (t % tiles_c) * 64;
+#pragma unroll 4
+    for (int i = 0; i < 16; ++i) {
+      const int b = b0 + 4 * i;
+      const int lr = src_d0_fast ? a : b, lc = src_d0_fast ? b : a;
+      const int64_t r = r0 + lr, c = c0 + lc;
+      if (r < d0 && c < d1)
+        tile[lr][lc] = MODE == 0 ? Tile<X>::load1(xb + xo + r * xs0 + c * xs1)
+                                 : Codes<Q>::dec(uint32_t(uint8_t(qb[qo + r * qs0 + c * qs1])));
+    }
+    __syncthreads();
+#pragma unroll 4
+    for (int i = 0; i < 16; ++i) {
+      const int b = b0 + 4 * i;
+      const int lr = dst_d0_fast ? a : b, lc = dst_d0_fast ? b : a;
+      const int64_t r = r0 + lr, c = c0 + lc;
+      if (r < d0 && c < d1) {
+        const float s = kind == kUniform ? scale[0] : (kind == kRow ? scale[r % nb] : scale[(r / nb) * d1 + c]);
+        if (MODE == 0) {
+          const float v = quant_value<Q>(tile[lr][lc], s, flags);
+          qb[qo + r * qs0 + c * qs1] = typename Q::storage(Codes<Q>::enc(v, flags));
+        } else {
+          Tile<X>::store1(xb + xo + r * xs0 + c * xs1, tile[lr][lc] * s);
+        }
+      }
+    }
+    __syncthreads();
+  }
+}
+
 }  // namespace qdq_cluster
 
 //   q_view  (x: base, offset, size0, size1, stride0, stride1 ; q: the same six ; scale, nb, kind, flags)
 //   dq_view (q: six ; y: six ; scale, nb, kind)
-// The two operands of a call have equal sizes; the kernel reads them from the first one.
+// The two operands of a call have equal sizes; the kernel reads them from the first one.  The _viewt_ forms take the
+// same arguments and walk 64 x 64 tiles (see qdq_view_tiles).
 #define MTRT_QDQ_VIEW_KERNELS(XN, XT, QN, QT)                                                                        \
   extern "C" __global__ void __launch_bounds__(256) mtrt_q_view_##XN##_##QN(                                         \
       const XT::storage* x, int64_t xo, int64_t d0, int64_t d1, int64_t xs0, int64_t xs1, QT::storage* q, int64_t qo, \
@@ -822,7 +871,15 @@ __device__ __forceinline__ void qdq_view(typename X::storage* __restrict__ xb, i
   extern "C" __global__ void __launch_bounds__(256) mtrt_dq_view_##XN##_##QN(                                        \
       const QT::storage* q, int64_t qo, int64_t d0, int64_t d1, int64_t qs0, int64_t qs1, XT::storage* y, int64_t yo, \
       int64_t, int64_t, int64_t ys0, int64_t ys1, const float* scale, int64_t nb, int32_t kind) {                    \
-    qdq_view<XT, QT, 1>(y, yo, ys0, ys1, const_cast<QT::storage*>(q), qo, qs0, qs1, scale, d0, d1, nb, kind, 0); }
+    qdq_view<XT, QT, 1>(y, yo, ys0, ys1, const_cast<QT::storage*>(q), qo, qs0, qs1, scale, d0, d1, nb, kind, 0); }   \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_q_viewt_##XN##_##QN(                                        \
+      const XT::storage* x, int64_t xo, int64_t d0, int64_t d1, int64_t xs0, int64_t xs1, QT::storage* q, int64_t qo, \
+      int64_t, int64_t, int64_t qs0, int64_t qs1, const float* scale, int64_t nb, int32_t kind, int32_t flags) {     \
+    qdq_view_tiles<XT, QT, 0>(const_cast<XT::storage*>(x), xo, xs0, xs1, q, qo, qs0, qs1, scale, d0, d1, nb, kind, flags); } \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_dq_viewt_##XN##_##QN(                                       \
+      const QT::storage* q, int64_t qo, int64_t d0, int64_t d1, int64_t qs0, int64_t qs1, XT::storage* y, int64_t yo, \
+      int64_t, int64_t, int64_t ys0, int64_t ys1, const float* scale, int64_t nb, int32_t kind) {                    \
+    qdq_view_tiles<XT, QT, 1>(y, yo, ys0, ys1, const_cast<QT::storage*>(q), qo, qs0, qs1, scale, d0, d1, nb, kind, 0); }
 #define MTRT_QDQ_VIEW_FOR_X(XN, XT)  \
   MTRT_QDQ_VIEW_KERNELS(XN, XT, i8, I8) MTRT_QDQ_VIEW_KERNELS(XN, XT, f8, F8) MTRT_QDQ_VIEW_KERNELS(XN, XT, i4, I4)
 MTRT_QDQ_VIEW_FOR_X(f32, F32)

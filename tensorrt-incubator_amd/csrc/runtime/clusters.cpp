@@ -433,9 +433,14 @@ int32_t view_dispatch(bool quantize, hipStream_t stream, const void *f, int32_t 
     void *rargs[] = {&qp, &fp, &scale, &n, &d1, &nb, &fs0, &qs0};
     return launch(st, rname, rgrid, kBlock, stream, rargs);
   }
-  KernelName name(quantize ? "mtrt_q_view_" : "mtrt_dq_view_");
+  // An operand that runs fastest along its first dimension (a transpose): 64 x 64 tiles through LDS, each side walked
+  // along its own grain.  Otherwise one element per lane.
+  auto magnitude = [](int64_t v) { return v < 0 ? -v : v; };
+  const bool tiled = magnitude(fs0) < magnitude(fs1) || magnitude(qs0) < magnitude(qs1);
+  KernelName name(quantize ? (tiled ? "mtrt_q_viewt_" : "mtrt_q_view_") : (tiled ? "mtrt_dq_viewt_" : "mtrt_dq_view_"));
   name + xn + "_" + code_name(q_dtype);
-  const uint32_t grid = blocks_for(n, kBlock);
+  const uint32_t grid = tiled ? uint32_t(std::min<int64_t>(((d0 + 63) / 64) * ((d1 + 63) / 64), int64_t(kMaxGrid) * 1024))
+                              : blocks_for(n, kBlock);
   if (quantize) {
     void *args[] = {&f, &fo, &d0, &d1, &fs0, &fs1, &q, &qo, &d0, &d1, &qs0, &qs1, &scale, &nb, &kind, &flags};
     return launch(st, name, grid, kBlock, stream, args);

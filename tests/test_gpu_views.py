@@ -45,7 +45,8 @@ def test_views_equal_packed_copies_and_the_oracle(pkg, orc, xname, qname):
             qbuf = torch.full((d0 + 2, 2 * d1 + 3), 0x55, dtype=torch.uint8, device="cuda")
             qv = qbuf[1:1 + d0, 3::2][:, :d1]
             pkg.quantize_view(xv, scale, pq, qv, kind, nb)
-            assert pkg.last_kernel() == "mtrt_q_view_%s_%s" % (xname, qname)
+            # a source that runs fastest along its first dimension goes through 64 x 64 tiles, the rest one element per lane
+            assert pkg.last_kernel() == "mtrt_q_view%s_%s_%s" % ("t" if name == "transpose" else "", xname, qname)
             q_ref = orc.quantize(xs, ox, oq, scale.cpu().numpy(), okind, d0, d1, nb)
             assert np.array_equal(qv.contiguous().cpu().numpy().ravel(), q_ref.view(np.uint8)), (name, kind)
             untouched = qbuf.clone()
@@ -56,11 +57,19 @@ def test_views_equal_packed_copies_and_the_oracle(pkg, orc, xname, qname):
             # dequantize the strided codes into a transposed destination
             ybuf = torch.zeros(d1, d0, dtype=td, device="cuda")
             pkg.dequantize_view(qv, scale, pq, ybuf.t(), kind, nb)
-            assert pkg.last_kernel() == "mtrt_dq_view_%s_%s" % (xname, qname)
+            assert pkg.last_kernel() == "mtrt_dq_viewt_%s_%s" % (xname, qname)
             y_ref = orc.dequantize(q_ref, oq, ox, scale.cpu().numpy(), okind, d0, d1, nb)
             got = ybuf.t().contiguous()
             got = got.cpu().numpy().ravel().view(np.uint32) if ox == orc.F32 else bits16(got)
             assert np.array_equal(got, y_ref.view(np.uint32) if ox == orc.F32 else y_ref), (name, kind)
+            # ... and into every second column of a row-major buffer (no operand against the grain: one element per lane)
+            ybuf2 = torch.full((d0, 2 * d1), 7.0, dtype=td, device="cuda")
+            pkg.dequantize_view(qv, scale, pq, ybuf2[:, ::2], kind, nb)
+            assert pkg.last_kernel() == "mtrt_dq_view_%s_%s" % (xname, qname)
+            got2 = ybuf2[:, ::2].contiguous()
+            got2 = got2.cpu().numpy().ravel().view(np.uint32) if ox == orc.F32 else bits16(got2)
+            assert np.array_equal(got2, y_ref.view(np.uint32) if ox == orc.F32 else y_ref), (name, kind)
+            assert bool((ybuf2[:, 1::2] == 7.0).all())
 
 
 @pytest.mark.parametrize("xname", ["f32", "bf16", "f16"])
@@ -138,6 +147,50 @@ def test_dense_views_take_the_contiguous_kernels(pkg, orc, xname):
             got = yv.cpu().numpy().ravel().view(np.uint32) if ox == orc.F32 else bits16(yv.contiguous())
             assert np.array_equal(got, y_ref.view(np.uint32) if ox == orc.F32 else y_ref)
             assert bool((ybuf[:off] == 7.0).all()) and bool((ybuf[off + d0 * d1:] == 7.0).all())
+
+
+@pytest.mark.parametrize("xname", ["f32", "f16"])
+@pytest.mark.parametrize("qname", ["i8", "f8"])
+def test_transposed_views_go_through_tiles(pkg, orc, xname, qname):
+    """Transposed sources into row-major codes, row-major codes into transposed destinations, both transposed, and a
+    transposed slice with an offset: several 64 x 64 tiles with ragged edges, every scale kind, against the oracle;
+    nothing outside the destination is written."""
+    import torch
+    td = {"f32": torch.float32, "f16": torch.float16}[xname]
+    ox = {"f32": orc.F32, "f16": orc.F16}[xname]
+    pq, oq = {"i8": (pkg.I8, orc.I8), "f8": (pkg.F8E4M3FN, orc.F8E4M3FN)}[qname]
+    torch.manual_seed(21)
+    parent = (torch.randn(200, 301, device="cuda") * 2).to(td)
+    for name, xv in (("transpose", parent.t()), ("transposed slice", parent[5:133, 17:230].t()), ("row-major", parent)):
+        d0, d1 = xv.shape
+        xc = xv.contiguous()
+        xs = xc.cpu().numpy().ravel() if ox == orc.F32 else bits16(xc)
+        for kind, okind, nb, ns in ((pkg.SCALE_UNIFORM, orc.SCALE_UNIFORM, 1, 1), (pkg.SCALE_ROW, orc.SCALE_ROW, 7, 7),
+                                    (pkg.SCALE_COL, orc.SCALE_COL, d0, d1)):
+            scale = (torch.rand(ns, device="cuda") * 0.05 + 0.01)
+            for q_transposed in (False, True):
+                if name == "row-major" and not q_transposed:
+                    continue                                     # dense on both sides: not a view kernel
+                qbuf = torch.full((d1 + 2, d0 + 3) if q_transposed else (d0 + 2, d1 + 3), 0x55, dtype=torch.uint8, device="cuda")
+                qv = qbuf[1:1 + d1, 2:2 + d0].t() if q_transposed else qbuf[1:1 + d0, 2:2 + d1]
+                pkg.quantize_view(xv, scale, pq, qv, kind, nb)
+                assert pkg.last_kernel() == "mtrt_q_viewt_%s_%s" % (xname, qname), (name, pkg.last_kernel())
+                q_ref = orc.quantize(xs, ox, oq, scale.cpu().numpy(), okind, d0, d1, nb)
+                assert np.array_equal(qv.contiguous().cpu().numpy().ravel(), q_ref.view(np.uint8)), (name, kind, q_transposed)
+                rest = qbuf.clone()
+                (rest[1:1 + d1, 2:2 + d0] if q_transposed else rest[1:1 + d0, 2:2 + d1])[:] = 0x55
+                assert bool((rest == 0x55).all()), "bytes outside the view were written (%s)" % name
+                ybuf = torch.full((d1 + 1, d0 + 2), 7.0, dtype=td, device="cuda")
+                yv = ybuf[1:, 1:1 + d0].t()
+                pkg.dequantize_view(qv, scale, pq, yv, kind, nb)
+                assert pkg.last_kernel() == "mtrt_dq_viewt_%s_%s" % (xname, qname)
+                y_ref = orc.dequantize(q_ref, oq, ox, scale.cpu().numpy(), okind, d0, d1, nb)
+                got = yv.contiguous()
+                got = got.cpu().numpy().ravel().view(np.uint32) if ox == orc.F32 else bits16(got)
+                assert np.array_equal(got, y_ref.view(np.uint32) if ox == orc.F32 else y_ref), (name, kind, q_transposed)
+                rest = ybuf.clone()
+                rest[1:, 1:1 + d0] = 7.0
+                assert bool((rest == 7.0).all())
 
 
 def test_view_kernel_launched_by_hand_in_the_expanded_argument_order(pkg, orc):
