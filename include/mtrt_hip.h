@@ -365,8 +365,9 @@ MTRT_CAPI_EXPORTED int32_t mtrt_hip_softmax(mtrt_stream_t stream, const void *x,
  * re-laid ONCE from the program's [K,N] into [N,K] (K contiguous, what the matrix cores read) by
  * the prepack call; the GEMM takes the re-laid weights.  a: int8 [M,K]; a_scale: f32 [M];
  * w_scale: f32 [N]; y: f16 [M,N].  Any M, K, N and any operand alignment run on the matrix cores (K that
- * is a multiple of 128 with 16-byte aligned operands on the faster tile loop); the sums are integers, so
- * every kernel gives the same bits. */
+ * is a multiple of 128 with 16-byte aligned operands on the faster tile loop; up to 32 rows with weights
+ * of moderate size on a kernel bound by reading the weights once); the sums are integers, so every kernel
+ * gives the same bits. */
 MTRT_CAPI_EXPORTED int32_t mtrt_hip_gemm_w8a8_prepack(mtrt_stream_t stream, const void *w_kn,
                                                       void *w_nk, int64_t K, int64_t N);
 MTRT_CAPI_EXPORTED int32_t mtrt_hip_gemm_w8a8(mtrt_stream_t stream, const void *a, const void *w_nk,

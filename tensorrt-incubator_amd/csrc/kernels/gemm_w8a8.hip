@@ -336,10 +336,15 @@ extern "C" __global__ void __launch_bounds__(256) mtrt_w8_prepack_frag(const int
 // sums (int32, exact in any order) meet in LDS.  G: groups of 8 activation rows per stage (M <= 8 * G).
 namespace small_m {
 
-template <int G, int WAVES, int JT>
+// ROWS: the weights are the [N,K] array itself instead of its fragment-order re-layout.  A lane's 16 bytes of k-step
+// p of slice kb are then bytes 128 kb + 32 p + 16 h of row n (instead of chunk p * 64 + lane of block kb): the same
+// fragment, read as 32-byte pieces of 32 rows per instruction, the four k-steps of a slice covering one 128-byte
+// line of each row.  Rows past N repeat the last row; their columns are never stored.
+template <int G, int WAVES, int JT, bool ROWS = false>
 __device__ __forceinline__ void run(const int8_t* __restrict__ a, const v4i* __restrict__ wfrag, const float* __restrict__ a_scale,
                                     const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N,
                                     int8_t* lds) {
+  constexpr int kSliceStride = ROWS ? 8 : 256, kStepStride = ROWS ? 2 : 64;   // in 16-byte chunks
   constexpr int kStages = 4, kStageBytes = 8 * G * 128;
   constexpr int kLoads = G + 4 * JT;                 // memory instructions per slice and wave
   const int lane = threadIdx.x & 63;
@@ -352,7 +357,12 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, const v4i* __r
 #pragma unroll
   for (int j = 0; j < JT; ++j) {
     tile[j] = blockIdx.x + int64_t(j) * gridDim.x;
-    bp[j] = wfrag + (tile[j] * slices) * 256 + lane;
+    if (ROWS) {
+      const int64_t n = tile[j] * 32 + frow;
+      bp[j] = reinterpret_cast<const v4i*>(reinterpret_cast<const int8_t*>(wfrag) + (n < N ? n : N - 1) * K) + fhalf;
+    } else {
+      bp[j] = wfrag + (tile[j] * slices) * 256 + lane;
+    }
   }
   int8_t* ring = lds + wave * (kStages * kStageBytes);
 
@@ -381,7 +391,7 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, const v4i* __r
     for (int j = 0; j < JT; ++j)
 #pragma unroll
       for (int p = 0; p < 4; ++p) {
-        const v4i* wsrc = bp[j] + kb * 256 + p * 64;
+        const v4i* wsrc = bp[j] + kb * kSliceStride + p * kStepStride;
         __asm__ volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(dst.w[j][p]) : "v"(wsrc) : "memory");
       }
   };
@@ -473,15 +483,15 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, const v4i* __r
 // The grid is one workgroup per column tile, or, while that would leave some compute units with two workgroups
 // and the rest with one (tiles between one and two times the compute units), one workgroup per compute unit:
 // workgroup g then also takes tile g + gridDim.x if there is one, and reads the activations once for both.
-template <int G>
+template <int G, bool ROWS = false>
 __device__ __forceinline__ void tiles(const int8_t* __restrict__ a, const v4i* __restrict__ wfrag, const float* __restrict__ a_scale,
                                       const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N,
                                       int8_t* lds) {
   const int64_t ntiles = (N + 31) / 32;
   if (int64_t(blockIdx.x) + gridDim.x < ntiles)
-    run<G, 4, 2>(a, wfrag, a_scale, w_scale, y, M, K, N, lds);
+    run<G, 4, 2, ROWS>(a, wfrag, a_scale, w_scale, y, M, K, N, lds);
   else
-    run<G, 4, 1>(a, wfrag, a_scale, w_scale, y, M, K, N, lds);
+    run<G, 4, 1, ROWS>(a, wfrag, a_scale, w_scale, y, M, K, N, lds);
 }
 
 }  // namespace small_m
@@ -515,6 +525,22 @@ extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w8a8_nk_any(
     for (int64_t k = 0; k < K; ++k) acc += int(a[m * K + k]) * int(w[n * K + k]);
     y[e] = uint16_t(f32_to_f16_bits((float(acc) * a_scale[m]) * w_scale[n]));
   }
+}
+
+// The same two kernels on [N,K] weights as they are (callers that hold no fragment-order re-layout):
+// (a [M,K] i8, w_nk [N,K] i8, a_scale, w_scale, y, M, K, N) ; K % 128 == 0, a and w_nk 16-byte aligned, M * K < 2^32; grid and
+// block as above.
+extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w8a8_nk_small16(
+    const int8_t* __restrict__ a, const int8_t* __restrict__ w_nk, const float* __restrict__ a_scale,
+    const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N) {
+  __shared__ __attribute__((aligned(16))) int8_t lds[4 * 4 * 2 * 1024];
+  small_m::tiles<2, true>(a, reinterpret_cast<const v4i*>(w_nk), a_scale, w_scale, y, M, K, N, lds);
+}
+extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w8a8_nk_small32(
+    const int8_t* __restrict__ a, const int8_t* __restrict__ w_nk, const float* __restrict__ a_scale,
+    const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N) {
+  __shared__ __attribute__((aligned(16))) int8_t lds[4 * 4 * 4 * 1024];
+  small_m::tiles<4, true>(a, reinterpret_cast<const v4i*>(w_nk), a_scale, w_scale, y, M, K, N, lds);
 }
 
 // Any K and any operand alignment on the matrix cores, for the shapes the kernels above do not take (K not a

@@ -727,6 +727,17 @@ int32_t mtrt_hip_gemm_w8a8(mtrt_stream_t stream, const void *a, const void *w_nk
   // The matrix-core kernel moves 128-byte K slices with 16-byte accesses.
   if (K > 0 && K % 128 == 0 && aligned(a, 16) && aligned(w_nk, 16) && M * K < (int64_t(1) << 32) &&
       N * K < (int64_t(1) << 32)) {
+    const double tile_rounds = double(((N + 255) / 256 + num_compute_units(st) - 1) / num_compute_units(st));
+    if (M <= 32 && 3.0 + double(N) * double(K) / 2.2e6 < (8.0 + 0.006 * double(K)) * tile_rounds) {
+      // decode-sized calls: the small-M kernels of the fragment-order entry point, reading the [N,K] rows as they are.
+      // A tile launch lasts one 256-row tile's whole K loop per round whatever M is (about 8 us + 6 ns per k: M = 16,
+      // K = 4096, N = 11008 32.7 us; M = 32, K = N = 8192 57.1 us); these kernels read 32-byte pieces of 32 rows per
+      // instruction and stream the weights at 2.2 TB/s only (fragment order: 4 TB/s), which is shorter while the
+      // weights are small enough (24.9 and 28.0 us at those shapes, K = N = 4096 at M = 1: 27.6 -> 10.5 us).
+      const int64_t tiles32 = (N + 31) / 32, cus = num_compute_units(st);
+      const uint32_t sgrid = uint32_t(M > 8 && tiles32 > cus && tiles32 <= 2 * cus ? cus : tiles32);
+      return launch(st, KernelName(M <= 16 ? "mtrt_gemm_w8a8_nk_small16" : "mtrt_gemm_w8a8_nk_small32"), sgrid, kBlock, as_hip(stream), args);
+    }
     // 256 x 256 tiles, one workgroup per compute unit at a time, N panels dealt round-robin to the
     // 8 XCDs (gemm_core.hpp), so each set of panels takes 8 * ceil(panels / 8) * tiles_m workgroup
     // ids.  The launch runs in rounds of one tile per unit; when the last round would use at most
