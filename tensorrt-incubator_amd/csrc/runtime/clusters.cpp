@@ -728,7 +728,17 @@ int32_t mtrt_hip_gemm_w8a8(mtrt_stream_t stream, const void *a, const void *w_nk
   if (K > 0 && K % 128 == 0 && aligned(a, 16) && aligned(w_nk, 16) && M * K < (int64_t(1) << 32) &&
       N * K < (int64_t(1) << 32)) {
     const double tile_rounds = double(((N + 255) / 256 + num_compute_units(st) - 1) / num_compute_units(st));
-    if (M <= 32 && 3.0 + double(N) * double(K) / 2.2e6 < (8.0 + 0.006 * double(K)) * tile_rounds) {
+    const double small_us = 3.0 + double(N) * double(K) / 2.2e6, tile_us = (8.0 + 0.006 * double(K)) * tile_rounds;
+    if (M > 32 && M <= 64 && 2.0 * small_us < tile_us) {
+      // 33 to 64 rows: two launches of those kernels (rows 0..31, then the rest) while that is still shorter than the
+      // one tile launch (M = 64, K = N = 4096: 27.4 us; a tile launch at K = 4096 takes 33)
+      const int32_t rc = mtrt_hip_gemm_w8a8(stream, a, w_nk, a_scale, w_scale, y, 32, K, N);
+      if (rc != MTRT_OK)
+        return rc;
+      return mtrt_hip_gemm_w8a8(stream, static_cast<const char *>(a) + 32 * K, w_nk, a_scale + 32, w_scale,
+                                static_cast<char *>(y) + 32 * N * 2, M - 32, K, N);
+    }
+    if (M <= 32 && small_us < tile_us) {
       // decode-sized calls: the small-M kernels of the fragment-order entry point, reading the [N,K] rows as they are.
       // A tile launch lasts one 256-row tile's whole K loop per round whatever M is (about 8 us + 6 ns per k: M = 16,
       // K = 4096, N = 11008 32.7 us; M = 32, K = N = 8192 57.1 us); these kernels read 32-byte pieces of 32 rows per

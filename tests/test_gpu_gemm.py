@@ -43,7 +43,9 @@ def test_w8a8_mfma_kernel_small_shapes(pkg, orc, shape):
     M, K, N = shape
     a, w, a_s, w_s = _w8a8_inputs(rng(M + K + N), M, K, N)
     y, kernel = _run_w8a8(pkg, a, w, a_s, w_s)
-    assert kernel == ("mtrt_gemm_w8a8_nk_small16" if M <= 16 else "mtrt_gemm_w8a8_nk")
+    # up to 32 rows, and 33 .. 64 as two launches, take the small-M kernels at these sizes
+    last = M - 32 if 32 < M <= 64 else M
+    assert kernel == ("mtrt_gemm_w8a8_nk_small16" if last <= 16 else "mtrt_gemm_w8a8_nk_small32" if last <= 32 else "mtrt_gemm_w8a8_nk")
     assert np.array_equal(bits16(y).reshape(M, N), orc.gemm_w8a8(a, w, a_s, w_s))
 
 
@@ -64,6 +66,15 @@ def test_w8a8_small_m_kernel_on_row_major_weights(pkg, orc, shape):
     ref = orc.gemm_w8a8(a, w, a_s, w_s)
     orc.set_threads(1)
     assert np.array_equal(bits16(y).reshape(M, N), ref)
+
+
+@pytest.mark.parametrize("shape", [(64, 512, 4096), (33, 1024, 520), (50, 256, 8209)])
+def test_w8a8_33_to_64_rows_on_row_major_weights_run_as_two_launches(pkg, orc, shape):
+    M, K, N = shape
+    a, w, a_s, w_s = _w8a8_inputs(rng(M + K + N), M, K, N)
+    y, kernel = _run_w8a8(pkg, a, w, a_s, w_s)
+    assert kernel == ("mtrt_gemm_w8a8_nk_small16" if M - 32 <= 16 else "mtrt_gemm_w8a8_nk_small32")   # the launch of rows 32 .. M - 1
+    assert np.array_equal(bits16(y).reshape(M, N), orc.gemm_w8a8(a, w, a_s, w_s))
 
 
 def _run_w8a8_frag(pkg, a, w, a_s, w_s, from_nk=False):
