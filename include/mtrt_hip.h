@@ -416,7 +416,8 @@ MTRT_CAPI_EXPORTED int32_t mtrt_hip_gemm_w4a16(mtrt_stream_t stream, const void 
  * above do not express, and of the unquantized module; w_nk is the module's own [out_features, in_features]
  * weight.  The reference generates a tiled FMA loop nest for such a matmul
  * (fallback-schedule-matmul.mlir:24); here every shape with K > 0 runs on the matrix cores (f16 / bf16 / f32
- * MFMA with f32 accumulation), any shape, no alignment needs beyond the element size. */
+ * MFMA with f32 accumulation), any shape, no alignment needs beyond the element size.  Up to 32 rows (64 as two
+ * launches) with rows in whole 128-byte slices take a kernel bound by reading the weights once. */
 MTRT_CAPI_EXPORTED int32_t mtrt_hip_linear_dense(mtrt_stream_t stream, const void *x, const void *w_nk,
                                                  const void *bias, void *y, int32_t dtype, int64_t M,
                                                  int64_t K, int64_t N);

@@ -76,6 +76,7 @@ typedef __bf16 v8b __attribute__((ext_vector_type(8)));
 template <typename X> struct HalfTraits;
 template <> struct HalfTraits<F16> {
   using Acc = v16f;
+  using Scalar = float;
   static __device__ __forceinline__ Acc zero() {
     Acc z;
 #pragma unroll
@@ -90,6 +91,7 @@ template <> struct HalfTraits<F16> {
 };
 template <> struct HalfTraits<BF16> {
   using Acc = v16f;
+  using Scalar = float;
   static __device__ __forceinline__ Acc zero() { return HalfTraits<F16>::zero(); }
   static __device__ __forceinline__ Acc mfma(v4i a, v4i b, Acc c) {
     union { v4i i; v8b h; } ua, ub;
@@ -103,6 +105,7 @@ template <> struct HalfTraits<BF16> {
 // meet in one instruction does not matter as long as both operands agree.
 struct F32Traits {
   using Acc = v16f;
+  using Scalar = float;
   static __device__ __forceinline__ Acc zero() { return HalfTraits<F16>::zero(); }
   static __device__ __forceinline__ Acc mfma(v4i a, v4i b, Acc c) {
 #pragma unroll
@@ -209,6 +212,20 @@ struct EdgeBiasF32Epilogue {
   __device__ __forceinline__ float finish(float acc, int64_t col, bool valid) const { return bias && valid ? acc + bias[col] : acc; }
 };
 
+// Epilogues of the up-to-32-rows kernel (gemm_core::rows32)
+template <typename X>
+struct RowsBiasEpilogue {
+  const typename X::storage* bias;
+  __device__ __forceinline__ uint32_t finish(float sum, int64_t, int64_t col) const {
+    if (bias) sum = sum + Tile<X>::load1(bias + col);
+    return narrow16<X>(sum);
+  }
+};
+struct RowsBiasF32Epilogue {
+  const float* bias;
+  __device__ __forceinline__ float finish(float sum, int64_t, int64_t col) const { return bias ? sum + bias[col] : sum; }
+};
+
 }  // namespace dense_cluster
 
 // f32 operands: (x [M,K], w [N,K], bias [N] or null, y [M,N], M, K, N, full_panels) ; K % 32 == 0, x and w 16-byte aligned
@@ -232,6 +249,27 @@ extern "C" __global__ void __launch_bounds__(gemm_core::THREADS, 1) mtrt_gemm_de
   }
 MTRT_DENSE_MFMA_KERNEL(f16, F16)
 MTRT_DENSE_MFMA_KERNEL(bf16, BF16)
+
+// Up to 32 rows, weights read once as whole rows (gemm_core::rows32): (x [M,K], w [N,K], bias or null, y, M <= 32, K, N) ;
+// rows in whole 128-byte slices, x and w 16-byte aligned; grid: any, block = 512.
+extern "C" __global__ void __launch_bounds__(512) mtrt_gemm_dense_rows32_f32(
+    const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ bias, float* __restrict__ y, int64_t M,
+    int64_t K, int64_t N) {
+  __shared__ __attribute__((aligned(16))) int8_t lds[gemm_core::rows32::lds_bytes<8>()];
+  dense_cluster::RowsBiasF32Epilogue epi{bias};
+  gemm_core::rows32::run<dense_cluster::F32Traits, 8>(reinterpret_cast<const int8_t*>(x), reinterpret_cast<const int8_t*>(w), K * 4, epi, y, M, N, lds);
+}
+#define MTRT_DENSE_ROWS32_KERNEL(XN, XT)                                                                           \
+  extern "C" __global__ void __launch_bounds__(512) mtrt_gemm_dense_rows32_##XN(                                   \
+      const XT::storage* __restrict__ x, const XT::storage* __restrict__ w, const XT::storage* __restrict__ bias,  \
+      uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N) {                                                 \
+    __shared__ __attribute__((aligned(16))) int8_t lds[gemm_core::rows32::lds_bytes<8>()];                         \
+    dense_cluster::RowsBiasEpilogue<XT> epi{bias};                                                                 \
+    gemm_core::rows32::run<dense_cluster::HalfTraits<XT>, 8>(reinterpret_cast<const int8_t*>(x), reinterpret_cast<const int8_t*>(w), K * 2, \
+                                                             epi, y, M, N, lds);                                   \
+  }
+MTRT_DENSE_ROWS32_KERNEL(f16, F16)
+MTRT_DENSE_ROWS32_KERNEL(bf16, BF16)
 
 // Any K and any alignment on the matrix cores: (x [M,K], w [N,K], bias [N] or null, y [M,N], M, K, N) ; grid: any
 // (128 x 128 tiles dealt round-robin), block = 256.

@@ -21,6 +21,7 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 
 struct I8Traits {
   using Acc = v16i;
+  using Scalar = int;
   static __device__ __forceinline__ Acc zero() {
     Acc z;
 #pragma unroll
@@ -336,15 +337,10 @@ extern "C" __global__ void __launch_bounds__(256) mtrt_w8_prepack_frag(const int
 // sums (int32, exact in any order) meet in LDS.  G: groups of 8 activation rows per stage (M <= 8 * G).
 namespace small_m {
 
-// ROWS: the weights are the [N,K] array itself instead of its fragment-order re-layout.  A lane's 16 bytes of k-step
-// p of slice kb are then bytes 128 kb + 32 p + 16 h of row n (instead of chunk p * 64 + lane of block kb): the same
-// fragment, read as 32-byte pieces of 32 rows per instruction, the four k-steps of a slice covering one 128-byte
-// line of each row.  Rows past N repeat the last row; their columns are never stored.
-template <int G, int WAVES, int JT, bool ROWS = false>
+template <int G, int WAVES, int JT>
 __device__ __forceinline__ void run(const int8_t* __restrict__ a, const v4i* __restrict__ wfrag, const float* __restrict__ a_scale,
                                     const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N,
                                     int8_t* lds) {
-  constexpr int kSliceStride = ROWS ? 8 : 256, kStepStride = ROWS ? 2 : 64;   // in 16-byte chunks
   constexpr int kStages = 4, kStageBytes = 8 * G * 128;
   constexpr int kLoads = G + 4 * JT;                 // memory instructions per slice and wave
   const int lane = threadIdx.x & 63;
@@ -357,12 +353,7 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, const v4i* __r
 #pragma unroll
   for (int j = 0; j < JT; ++j) {
     tile[j] = blockIdx.x + int64_t(j) * gridDim.x;
-    if (ROWS) {
-      const int64_t n = tile[j] * 32 + frow;
-      bp[j] = reinterpret_cast<const v4i*>(reinterpret_cast<const int8_t*>(wfrag) + (n < N ? n : N - 1) * K) + fhalf;
-    } else {
-      bp[j] = wfrag + (tile[j] * slices) * 256 + lane;
-    }
+    bp[j] = wfrag + (tile[j] * slices) * 256 + lane;
   }
   int8_t* ring = lds + wave * (kStages * kStageBytes);
 
@@ -391,7 +382,7 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, const v4i* __r
     for (int j = 0; j < JT; ++j)
 #pragma unroll
       for (int p = 0; p < 4; ++p) {
-        const v4i* wsrc = bp[j] + kb * kSliceStride + p * kStepStride;
+        const v4i* wsrc = bp[j] + kb * 256 + p * 64;
         __asm__ volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(dst.w[j][p]) : "v"(wsrc) : "memory");
       }
   };
@@ -483,15 +474,15 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, const v4i* __r
 // The grid is one workgroup per column tile, or, while that would leave some compute units with two workgroups
 // and the rest with one (tiles between one and two times the compute units), one workgroup per compute unit:
 // workgroup g then also takes tile g + gridDim.x if there is one, and reads the activations once for both.
-template <int G, bool ROWS = false>
+template <int G>
 __device__ __forceinline__ void tiles(const int8_t* __restrict__ a, const v4i* __restrict__ wfrag, const float* __restrict__ a_scale,
                                       const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N,
                                       int8_t* lds) {
   const int64_t ntiles = (N + 31) / 32;
   if (int64_t(blockIdx.x) + gridDim.x < ntiles)
-    run<G, 4, 2, ROWS>(a, wfrag, a_scale, w_scale, y, M, K, N, lds);
+    run<G, 4, 2>(a, wfrag, a_scale, w_scale, y, M, K, N, lds);
   else
-    run<G, 4, 1, ROWS>(a, wfrag, a_scale, w_scale, y, M, K, N, lds);
+    run<G, 4, 1>(a, wfrag, a_scale, w_scale, y, M, K, N, lds);
 }
 
 }  // namespace small_m
@@ -527,20 +518,21 @@ extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w8a8_nk_any(
   }
 }
 
-// The same two kernels on [N,K] weights as they are (callers that hold no fragment-order re-layout):
-// (a [M,K] i8, w_nk [N,K] i8, a_scale, w_scale, y, M, K, N) ; K % 128 == 0, a and w_nk 16-byte aligned, M * K < 2^32; grid and
-// block as above.
-extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w8a8_nk_small16(
+// Up to 32 rows on [N,K] weights read as whole rows (gemm_core::rows32): (a [M,K] i8, w_nk [N,K] i8, a_scale, w_scale, y,
+// M <= 32, K, N) ; K % 128 == 0, a and w_nk 16-byte aligned; grid: any, block = 512.
+struct RowsScaleEpilogue {
+  const float* a_scale;
+  const float* w_scale;
+  __device__ __forceinline__ uint32_t finish(int sum, int64_t row, int64_t col) const {
+    return f32_to_f16_bits((float(sum) * a_scale[row]) * w_scale[col]);
+  }
+};
+extern "C" __global__ void __launch_bounds__(512) mtrt_gemm_w8a8_nk_rows32(
     const int8_t* __restrict__ a, const int8_t* __restrict__ w_nk, const float* __restrict__ a_scale,
     const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N) {
-  __shared__ __attribute__((aligned(16))) int8_t lds[4 * 4 * 2 * 1024];
-  small_m::tiles<2, true>(a, reinterpret_cast<const v4i*>(w_nk), a_scale, w_scale, y, M, K, N, lds);
-}
-extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w8a8_nk_small32(
-    const int8_t* __restrict__ a, const int8_t* __restrict__ w_nk, const float* __restrict__ a_scale,
-    const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N) {
-  __shared__ __attribute__((aligned(16))) int8_t lds[4 * 4 * 4 * 1024];
-  small_m::tiles<4, true>(a, reinterpret_cast<const v4i*>(w_nk), a_scale, w_scale, y, M, K, N, lds);
+  __shared__ __attribute__((aligned(16))) int8_t lds[gemm_core::rows32::lds_bytes<8>()];
+  RowsScaleEpilogue epi{a_scale, w_scale};
+  gemm_core::rows32::run<I8Traits, 8>(a, w_nk, K, epi, y, M, N, lds);
 }
 
 // Any K and any operand alignment on the matrix cores, for the shapes the kernels above do not take (K not a

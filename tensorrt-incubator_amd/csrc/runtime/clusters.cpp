@@ -727,11 +727,15 @@ int32_t mtrt_hip_gemm_w8a8(mtrt_stream_t stream, const void *a, const void *w_nk
   // The matrix-core kernel moves 128-byte K slices with 16-byte accesses.
   if (K > 0 && K % 128 == 0 && aligned(a, 16) && aligned(w_nk, 16) && M * K < (int64_t(1) << 32) &&
       N * K < (int64_t(1) << 32)) {
+    // Up to 32 rows are bound by reading the weights once: one workgroup per 32 weight rows, its eight waves splitting K
+    // and reading whole rows (3.4 TB/s of weights; the fragment-order entry point reaches 4).  A tile launch lasts
+    // one 256-row tile's whole K loop per round whatever M is (about 8 us + 6 ns per k: M = 16, K = 4096, N = 11008
+    // 32.7 us against 13.4; M = 32, K = N = 8192 57.1 against 18.6; M = 1, K = N = 4096 27.6 against 11.2), so it
+    // only wins on very large weights.  33 to 64 rows run as two such launches while that is shorter (M = 64,
+    // K = N = 4096: 16.1 us against 33).
     const double tile_rounds = double(((N + 255) / 256 + num_compute_units(st) - 1) / num_compute_units(st));
-    const double small_us = 3.0 + double(N) * double(K) / 2.2e6, tile_us = (8.0 + 0.006 * double(K)) * tile_rounds;
+    const double small_us = 3.0 + double(N) * double(K) / 3.4e6, tile_us = (8.0 + 0.006 * double(K)) * tile_rounds;
     if (M > 32 && M <= 64 && 2.0 * small_us < tile_us) {
-      // 33 to 64 rows: two launches of those kernels (rows 0..31, then the rest) while that is still shorter than the
-      // one tile launch (M = 64, K = N = 4096: 27.4 us; a tile launch at K = 4096 takes 33)
       const int32_t rc = mtrt_hip_gemm_w8a8(stream, a, w_nk, a_scale, w_scale, y, 32, K, N);
       if (rc != MTRT_OK)
         return rc;
@@ -739,14 +743,9 @@ int32_t mtrt_hip_gemm_w8a8(mtrt_stream_t stream, const void *a, const void *w_nk
                                 static_cast<char *>(y) + 32 * N * 2, M - 32, K, N);
     }
     if (M <= 32 && small_us < tile_us) {
-      // decode-sized calls: the small-M kernels of the fragment-order entry point, reading the [N,K] rows as they are.
-      // A tile launch lasts one 256-row tile's whole K loop per round whatever M is (about 8 us + 6 ns per k: M = 16,
-      // K = 4096, N = 11008 32.7 us; M = 32, K = N = 8192 57.1 us); these kernels read 32-byte pieces of 32 rows per
-      // instruction and stream the weights at 2.2 TB/s only (fragment order: 4 TB/s), which is shorter while the
-      // weights are small enough (24.9 and 28.0 us at those shapes, K = N = 4096 at M = 1: 27.6 -> 10.5 us).
-      const int64_t tiles32 = (N + 31) / 32, cus = num_compute_units(st);
-      const uint32_t sgrid = uint32_t(M > 8 && tiles32 > cus && tiles32 <= 2 * cus ? cus : tiles32);
-      return launch(st, KernelName(M <= 16 ? "mtrt_gemm_w8a8_nk_small16" : "mtrt_gemm_w8a8_nk_small32"), sgrid, kBlock, as_hip(stream), args);
+      const int64_t tiles32 = (N + 31) / 32;
+      return launch(st, KernelName("mtrt_gemm_w8a8_nk_rows32"), uint32_t(std::min<int64_t>(tiles32, int64_t(kMaxGrid) * 1024)), 512,
+                    as_hip(stream), args);
     }
     // 256 x 256 tiles, one workgroup per compute unit at a time, N panels dealt round-robin to the
     // 8 XCDs (gemm_core.hpp), so each set of panels takes 8 * ceil(panels / 8) * tiles_m workgroup
@@ -877,6 +876,26 @@ int32_t mtrt_hip_linear_dense(mtrt_stream_t stream, const void *x, const void *w
   DeviceState *st = device_state();
   if (!st)
     return MTRT_RUNTIME_ERROR;
+  // Decode-sized calls are bound by reading the weights once: up to 32 rows take one workgroup per 32 weight rows, its
+  // eight waves splitting K (f16 M = 16, K = 4096, N = 11008: 55 us on the tile loop, 23.3 so, 3.9 TB/s of weights; f32
+  // 473 -> 50 us); 33 to 64 rows two such launches; the tile loop (about 8 us + 6 ns per byte of a row, per round)
+  // only wins on very large weights.
+  const bool whole_slices = K > 0 && (K * eb) % 128 == 0 && aligned(x, 16) && aligned(w_nk, 16);
+  const double tile_us = (8.0 + 0.006 * double(K * eb)) * double(((N + 255) / 256 + num_compute_units(st) - 1) / num_compute_units(st));
+  const double small_us = 3.0 + double(N) * double(K * eb) / 4.0e6;
+  if (whole_slices && M > 32 && M <= 64 && 2.0 * small_us < tile_us) {
+    const int32_t rc = mtrt_hip_linear_dense(stream, x, w_nk, bias, y, dtype, 32, K, N);
+    if (rc != MTRT_OK)
+      return rc;
+    return mtrt_hip_linear_dense(stream, static_cast<const char *>(x) + 32 * K * eb, w_nk, bias, static_cast<char *>(y) + 32 * N * eb,
+                                 dtype, M - 32, K, N);
+  }
+  if (whole_slices && M <= 32 && small_us < tile_us) {
+    const int64_t tiles32 = (N + 31) / 32;
+    void *rargs[] = {&x, &w_nk, &bias, &y, &M, &K, &N};
+    return launch(st, KernelName("mtrt_gemm_dense_rows32_") + xn, uint32_t(std::min<int64_t>(tiles32, int64_t(kMaxGrid) * 1024)), 512,
+                  as_hip(stream), rargs);
+  }
   if (K > 0 && (K * eb) % 128 == 0 && aligned(x, 16) && aligned(w_nk, 16) && M * K * eb < (int64_t(1) << 32) &&
       N * K * eb < (int64_t(1) << 32)) {
     // operands in whole 128-byte slices of K: the matrix-core tile loop (tiles and rounds as in

@@ -45,23 +45,23 @@ def test_w8a8_mfma_kernel_small_shapes(pkg, orc, shape):
     y, kernel = _run_w8a8(pkg, a, w, a_s, w_s)
     # up to 32 rows, and 33 .. 64 as two launches, take the small-M kernels at these sizes
     last = M - 32 if 32 < M <= 64 else M
-    assert kernel == ("mtrt_gemm_w8a8_nk_small16" if last <= 16 else "mtrt_gemm_w8a8_nk_small32" if last <= 32 else "mtrt_gemm_w8a8_nk")
+    assert kernel == ("mtrt_gemm_w8a8_nk_rows32" if last <= 32 else "mtrt_gemm_w8a8_nk")
     assert np.array_equal(bits16(y).reshape(M, N), orc.gemm_w8a8(a, w, a_s, w_s))
 
 
 @pytest.mark.parametrize("shape", [(1, 128, 32), (16, 4096, 11008), (32, 4096, 11008), (17, 384, 200), (9, 1280, 4099), (13, 640, 8240),
-                                   (32, 256, 16384), (25, 512, 16400), (8, 2048, 8209), (16, 128, 40), (16, 4096, 4096), (32, 4096, 6144), (5, 8192, 8192), (3, 512, 65000)])
+                                   (32, 256, 16384), (25, 512, 16400), (8, 2048, 8209), (16, 128, 40), (16, 4096, 4096), (32, 4096, 6144), (5, 8192, 8192), (3, 512, 65000), (2, 128, 200000)])
 def test_w8a8_small_m_kernel_on_row_major_weights(pkg, orc, shape):
-    """M <= 32 with [N,K] weights as they are: the small-M kernels reading 32-byte pieces of 32 weight rows per
-    instruction instead of fragment order; the shapes of the fragment-order test (waves without a slice, one and two
-    tiles per workgroup, ragged last tiles whose missing rows repeat row N - 1).  Integer sums: bit-exact."""
+    """M <= 32 with [N,K] weights as they are: one workgroup per 32 weight rows, eight waves splitting K and reading
+    whole rows; K = 128 and 384 leave waves without a slice, 640 and 1280 give them uneven shares; ragged last tiles
+    whose missing rows repeat row N - 1; very wide weights stay on the tile loop.  Integer sums: bit-exact."""
     M, K, N = shape
     a, w, a_s, w_s = _w8a8_inputs(rng(M + K + N), M, K, N)
     print("case: w8a8 small M, row-major weights", shape, flush=True)
     y, kernel = _run_w8a8(pkg, a, w, a_s, w_s)
     # while streaming the weights at this kernel's rate is shorter than one tile's K loop
-    small = 3.0 + N * K / 2.2e6 < (8.0 + 0.006 * K) * -(-((N + 255) // 256) // 256)
-    assert kernel == (("mtrt_gemm_w8a8_nk_small16" if M <= 16 else "mtrt_gemm_w8a8_nk_small32") if small else "mtrt_gemm_w8a8_nk")
+    small = 3.0 + N * K / 3.4e6 < (8.0 + 0.006 * K) * -(-((N + 255) // 256) // 256)
+    assert kernel == ("mtrt_gemm_w8a8_nk_rows32" if small else "mtrt_gemm_w8a8_nk")
     orc.set_threads(16)
     ref = orc.gemm_w8a8(a, w, a_s, w_s)
     orc.set_threads(1)
@@ -73,7 +73,7 @@ def test_w8a8_33_to_64_rows_on_row_major_weights_run_as_two_launches(pkg, orc, s
     M, K, N = shape
     a, w, a_s, w_s = _w8a8_inputs(rng(M + K + N), M, K, N)
     y, kernel = _run_w8a8(pkg, a, w, a_s, w_s)
-    assert kernel == ("mtrt_gemm_w8a8_nk_small16" if M - 32 <= 16 else "mtrt_gemm_w8a8_nk_small32")   # the launch of rows 32 .. M - 1
+    assert kernel == "mtrt_gemm_w8a8_nk_rows32"
     assert np.array_equal(bits16(y).reshape(M, N), orc.gemm_w8a8(a, w, a_s, w_s))
 
 
