@@ -593,7 +593,7 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, const int8_t* 
 }  // namespace edge
 
 // ---- up to 32 rows against K-contiguous weights -----------------------------------------------------------
-// a [M <= 32, row_bytes], w [N, row_bytes], both in whole 128-byte slices and 16-byte aligned.  With so few rows a
+// a [M <= 32 MT, row_bytes], w [N, row_bytes], both in whole 128-byte slices and 16-byte aligned.  With so few rows a
 // call is bound by reading the weights once, and a tile of the loops above would spend a whole K loop on padding.
 // One workgroup per 32 weight rows (output columns); its WAVES waves split K.  Each wave works alone, without
 // workgroup barriers: per 128-byte slice it reads its 32 weight rows and the 32 activation rows as whole rows (eight
@@ -607,79 +607,89 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, const int8_t* 
 // pattern (Y = uint16_t) or the float (Y = float) of y[row, col].  Grid: any (tiles dealt round-robin), block = 64 WAVES.
 namespace rows32 {
 constexpr int kPitch = 144, kStageBytes = 32 * kPitch;
-template <int WAVES> constexpr int lds_bytes() { return WAVES * 2 * kStageBytes; }
+// MT: activation row tiles of 32 (1: M <= 32, 2: M <= 64, the weight fragments of a k-step serving both)
+template <int WAVES, int MT = 1> constexpr int lds_bytes() { return WAVES * (MT + 1) * kStageBytes; }
 
-template <class Traits, int WAVES, class Epilogue, typename Y>
+template <class Traits, int WAVES, int MT = 1, class Epilogue, typename Y>
 __device__ __forceinline__ void run(const int8_t* __restrict__ a, const int8_t* __restrict__ w, int64_t row_bytes, Epilogue& epi,
                                     Y* __restrict__ y, int64_t M, int64_t N, int8_t* lds) {
   using Acc = typename Traits::Acc;
   using Scalar = typename Traits::Scalar;
-  static_assert(2 * kStageBytes >= 16 * 64 * int(sizeof(Scalar)), "a wave's stages also hold its partial sums");
+  constexpr int kWaveBytes = (MT + 1) * kStageBytes;
+  static_assert(kWaveBytes >= MT * 16 * 64 * int(sizeof(Scalar)), "a wave's stages also hold its partial sums");
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int frow = lane & 31, fhalf = lane >> 5;
   const int lrow = lane >> 3, lchunk = (lane & 7) * 16;
   const int64_t slices = row_bytes / 128;
   const int64_t kb0 = slices * wave / WAVES, kb1 = slices * (wave + 1) / WAVES;
-  int8_t* sa = lds + wave * (2 * kStageBytes);
-  int8_t* sw = sa + kStageBytes;
+  int8_t* sa = lds + wave * kWaveBytes;
+  int8_t* sw = sa + MT * kStageBytes;
   const int64_t tiles = (N + 31) / 32;
   for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
-    const int8_t* ap[4];
+    const int8_t* ap[4 * MT];
     const int8_t* wp[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int64_t m = lrow + 8 * i, n = tile * 32 + lrow + 8 * i;
+    for (int i = 0; i < 4 * MT; ++i) {
+      const int64_t m = lrow + 8 * i;
       ap[i] = a + (m < M ? m : M - 1) * row_bytes + lchunk;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int64_t n = tile * 32 + lrow + 8 * i;
       wp[i] = w + (n < N ? n : N - 1) * row_bytes + lchunk;
     }
-    Acc acc = Traits::zero();
-    u32x4 ra[2][4], rw[2][4];
+    Acc acc[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[t] = Traits::zero();
+    u32x4 ra[2][4 * MT], rw[2][4];
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
-      // a slice past the wave's last one is the last one again (kb0 itself for a wave without slices; slices >= 1)
+      // a slice past the wave's last one is the last one again (slice 0 for a wave without slices; slices >= 1)
       int64_t kb = kb0 + p < kb1 ? kb0 + p : kb1 - 1;
       kb = kb < 0 ? 0 : kb;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        ra[p][i] = *reinterpret_cast<const u32x4*>(ap[i] + kb * 128);
-        rw[p][i] = *reinterpret_cast<const u32x4*>(wp[i] + kb * 128);
-      }
+      for (int i = 0; i < 4 * MT; ++i) ra[p][i] = *reinterpret_cast<const u32x4*>(ap[i] + kb * 128);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) rw[p][i] = *reinterpret_cast<const u32x4*>(wp[i] + kb * 128);
     }
     for (int64_t kb = kb0; kb < kb1; kb += 2) {
 #pragma unroll
       for (int p = 0; p < 2; ++p) {
         if (kb + p < kb1) {
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            *reinterpret_cast<u32x4*>(sa + (lrow + 8 * i) * kPitch + lchunk) = ra[p][i];
-            *reinterpret_cast<u32x4*>(sw + (lrow + 8 * i) * kPitch + lchunk) = rw[p][i];
-          }
+          for (int i = 0; i < 4 * MT; ++i) *reinterpret_cast<u32x4*>(sa + (lrow + 8 * i) * kPitch + lchunk) = ra[p][i];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(sw + (lrow + 8 * i) * kPitch + lchunk) = rw[p][i];
           const int64_t next = kb + p + 2 < kb1 ? kb + p + 2 : kb1 - 1;   // always a load: the waits stay countable
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            ra[p][i] = *reinterpret_cast<const u32x4*>(ap[i] + next * 128);
-            rw[p][i] = *reinterpret_cast<const u32x4*>(wp[i] + next * 128);
-          }
+          for (int i = 0; i < 4 * MT; ++i) ra[p][i] = *reinterpret_cast<const u32x4*>(ap[i] + next * 128);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) rw[p][i] = *reinterpret_cast<const u32x4*>(wp[i] + next * 128);
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
-            const v4i fa = *reinterpret_cast<const v4i*>(sa + frow * kPitch + q * 32 + fhalf * 16);
             const v4i fw = *reinterpret_cast<const v4i*>(sw + frow * kPitch + q * 32 + fhalf * 16);
-            acc = Traits::mfma(fa, fw, acc);
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+              const v4i fa = *reinterpret_cast<const v4i*>(sa + (t * 32 + frow) * kPitch + q * 32 + fhalf * 16);
+              acc[t] = Traits::mfma(fa, fw, acc[t]);
+            }
           }
         }
       }
     }
-    // lane (n = lane % 32, h = lane / 32) holds rows 8 (r / 4) + 4 h + r % 4 of column n in register r
+    // lane (n = lane % 32, h = lane / 32) holds rows 32 t + 8 (r / 4) + 4 h + r % 4 of column n in register r of acc[t]
     Scalar* mine = reinterpret_cast<Scalar*>(sa);
 #pragma unroll
-    for (int r = 0; r < 16; ++r) mine[r * 64 + lane] = acc[r];
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mine[(t * 16 + r) * 64 + lane] = acc[t][r];
     __syncthreads();
-    for (int e = threadIdx.x; e < 16 * 64; e += 64 * WAVES) {
-      const int r = e >> 6, l = e & 63;
+    for (int e = threadIdx.x; e < MT * 16 * 64; e += 64 * WAVES) {
+      const int t = e >> 10, r = (e >> 6) & 15, l = e & 63;
       Scalar v = reinterpret_cast<const Scalar*>(lds)[e];
 #pragma unroll
-      for (int k = 1; k < WAVES; ++k) v = v + reinterpret_cast<const Scalar*>(lds + k * (2 * kStageBytes))[e];
-      const int64_t row = (r >> 2) * 8 + (l >> 5) * 4 + (r & 3);
+      for (int k = 1; k < WAVES; ++k) v = v + reinterpret_cast<const Scalar*>(lds + k * kWaveBytes)[e];
+      const int64_t row = t * 32 + (r >> 2) * 8 + (l >> 5) * 4 + (r & 3);
       const int64_t c = tile * 32 + (l & 31);
       if (row < M && c < N) y[row * N + c] = Y(epi.finish(v, row, c));
     }

@@ -731,21 +731,13 @@ int32_t mtrt_hip_gemm_w8a8(mtrt_stream_t stream, const void *a, const void *w_nk
     // and reading whole rows (3.4 TB/s of weights; the fragment-order entry point reaches 4).  A tile launch lasts
     // one 256-row tile's whole K loop per round whatever M is (about 8 us + 6 ns per k: M = 16, K = 4096, N = 11008
     // 32.7 us against 13.4; M = 32, K = N = 8192 57.1 against 18.6; M = 1, K = N = 4096 27.6 against 11.2), so it
-    // only wins on very large weights.  33 to 64 rows run as two such launches while that is shorter (M = 64,
-    // K = N = 4096: 16.1 us against 33).
+    // only wins on very large weights.  33 to 64 rows take the form with two activation row tiles per weight fragment.
     const double tile_rounds = double(((N + 255) / 256 + num_compute_units(st) - 1) / num_compute_units(st));
     const double small_us = 3.0 + double(N) * double(K) / 3.4e6, tile_us = (8.0 + 0.006 * double(K)) * tile_rounds;
-    if (M > 32 && M <= 64 && 2.0 * small_us < tile_us) {
-      const int32_t rc = mtrt_hip_gemm_w8a8(stream, a, w_nk, a_scale, w_scale, y, 32, K, N);
-      if (rc != MTRT_OK)
-        return rc;
-      return mtrt_hip_gemm_w8a8(stream, static_cast<const char *>(a) + 32 * K, w_nk, a_scale + 32, w_scale,
-                                static_cast<char *>(y) + 32 * N * 2, M - 32, K, N);
-    }
-    if (M <= 32 && small_us < tile_us) {
+    if (M <= 64 && small_us < tile_us) {
       const int64_t tiles32 = (N + 31) / 32;
-      return launch(st, KernelName("mtrt_gemm_w8a8_nk_rows32"), uint32_t(std::min<int64_t>(tiles32, int64_t(kMaxGrid) * 1024)), 512,
-                    as_hip(stream), args);
+      return launch(st, KernelName(M <= 32 ? "mtrt_gemm_w8a8_nk_rows32" : "mtrt_gemm_w8a8_nk_rows64"),
+                    uint32_t(std::min<int64_t>(tiles32, int64_t(kMaxGrid) * 1024)), 512, as_hip(stream), args);
     }
     // 256 x 256 tiles, one workgroup per compute unit at a time, N panels dealt round-robin to the
     // 8 XCDs (gemm_core.hpp), so each set of panels takes 8 * ceil(panels / 8) * tiles_m workgroup
@@ -878,22 +870,15 @@ int32_t mtrt_hip_linear_dense(mtrt_stream_t stream, const void *x, const void *w
     return MTRT_RUNTIME_ERROR;
   // Decode-sized calls are bound by reading the weights once: up to 32 rows take one workgroup per 32 weight rows, its
   // eight waves splitting K (f16 M = 16, K = 4096, N = 11008: 55 us on the tile loop, 23.3 so, 3.9 TB/s of weights; f32
-  // 473 -> 50 us); 33 to 64 rows two such launches; the tile loop (about 8 us + 6 ns per byte of a row, per round)
+  // 473 -> 50 us); 33 to 64 rows the form with two activation row tiles per weight fragment; the tile loop (about 8 us + 6 ns per byte of a row, per round)
   // only wins on very large weights.
   const bool whole_slices = K > 0 && (K * eb) % 128 == 0 && aligned(x, 16) && aligned(w_nk, 16);
   const double tile_us = (8.0 + 0.006 * double(K * eb)) * double(((N + 255) / 256 + num_compute_units(st) - 1) / num_compute_units(st));
   const double small_us = 3.0 + double(N) * double(K * eb) / 4.0e6;
-  if (whole_slices && M > 32 && M <= 64 && 2.0 * small_us < tile_us) {
-    const int32_t rc = mtrt_hip_linear_dense(stream, x, w_nk, bias, y, dtype, 32, K, N);
-    if (rc != MTRT_OK)
-      return rc;
-    return mtrt_hip_linear_dense(stream, static_cast<const char *>(x) + 32 * K * eb, w_nk, bias, static_cast<char *>(y) + 32 * N * eb,
-                                 dtype, M - 32, K, N);
-  }
-  if (whole_slices && M <= 32 && small_us < tile_us) {
+  if (whole_slices && M <= 64 && small_us < tile_us) {
     const int64_t tiles32 = (N + 31) / 32;
     void *rargs[] = {&x, &w_nk, &bias, &y, &M, &K, &N};
-    return launch(st, KernelName("mtrt_gemm_dense_rows32_") + xn, uint32_t(std::min<int64_t>(tiles32, int64_t(kMaxGrid) * 1024)), 512,
+    return launch(st, KernelName(M <= 32 ? "mtrt_gemm_dense_rows32_" : "mtrt_gemm_dense_rows64_") + xn, uint32_t(std::min<int64_t>(tiles32, int64_t(kMaxGrid) * 1024)), 512,
                   as_hip(stream), rargs);
   }
   if (K > 0 && (K * eb) % 128 == 0 && aligned(x, 16) && aligned(w_nk, 16) && M * K * eb < (int64_t(1) << 32) &&

@@ -279,7 +279,7 @@ def test_quant_linear_int4_weight_only_runs_on_the_w4a16_cluster(tp, orc, pkg):
     lin32.load_state_dict({"weight": tp.Tensor(w.astype(np.float32)), "weight_scale": tp.Tensor(s_w.astype(np.float32))})
     assert lin32.route() == "dense"
     o32 = lin32(tp.Tensor(x.astype(np.float32))).torch().cpu().numpy().astype(np.float64)
-    assert pkg.last_kernel() == (("mtrt_gemm_dense_rows32_f32" if M <= 64 else "mtrt_gemm_dense_mfma_f32") if K % 32 == 0 else "mtrt_gemm_dense_edge_f32")
+    assert pkg.last_kernel() == (("mtrt_gemm_dense_rows32_f32" if M <= 32 else "mtrt_gemm_dense_rows64_f32" if M <= 64 else "mtrt_gemm_dense_mfma_f32") if K % 32 == 0 else "mtrt_gemm_dense_edge_f32")
     wd32 = (sgn.reshape(N, K).astype(np.float32) * s_w.astype(np.float32)[:, None]).astype(np.float64)
     ex32 = x.astype(np.float64) @ wd32.T
     assert np.all(np.abs(o32 - ex32) <= 1e-5 * (np.abs(x.astype(np.float64)) @ np.abs(wd32.T)) + 1e-6)
@@ -303,8 +303,9 @@ def test_dense_linear_against_float64(tp, pkg, dname):
         # operands whose rows are whole 128-byte slices of K run the 256 x 256 tile loop, everything else 128 x 128 tiles
         # with element-aligned loads; both on the matrix cores
         mfma = K % (32 if dname == "float32" else 64) == 0
-        rows = int(np.prod(lead))                          # up to 32 rows, and 33 .. 64 as two launches, read the weights once
-        assert pkg.last_kernel() == ("mtrt_gemm_dense_rows32_" if mfma and rows <= 64 else "mtrt_gemm_dense_mfma_" if mfma else "mtrt_gemm_dense_edge_") + {"float32": "f32", "float16": "f16", "bfloat16": "bf16"}[dname]
+        rows = int(np.prod(lead))                          # up to 64 rows read the weights once
+        assert pkg.last_kernel() == ("mtrt_gemm_dense_rows32_" if mfma and rows <= 32 else "mtrt_gemm_dense_rows64_" if mfma and rows <= 64 else
+                                     "mtrt_gemm_dense_mfma_" if mfma else "mtrt_gemm_dense_edge_") + {"float32": "f32", "float16": "f16", "bfloat16": "bf16"}[dname]
         assert tuple(out.shape) == lead + (N,)
         ref = x.double() @ w.double().T + b.double()
         mag = x.double().abs() @ w.double().abs().T + b.double().abs()
