@@ -365,8 +365,8 @@ MTRT_CAPI_EXPORTED int32_t mtrt_hip_softmax(mtrt_stream_t stream, const void *x,
  * re-laid ONCE from the program's [K,N] into [N,K] (K contiguous, what the matrix cores read) by
  * the prepack call; the GEMM takes the re-laid weights.  a: int8 [M,K]; a_scale: f32 [M];
  * w_scale: f32 [N]; y: f16 [M,N].  Any M, K, N and any operand alignment run on the matrix cores (K that
- * is a multiple of 128 with 16-byte aligned operands on the faster tile loop; up to 64 rows with weights
- * of moderate size on a kernel bound by reading the weights once); the sums are integers, so every kernel
+ * is a multiple of 128 with 16-byte aligned operands on the faster tile loop; up to 128 rows with weights
+ * of moderate size on kernels bound by reading the weights once); the sums are integers, so every kernel
  * gives the same bits. */
 MTRT_CAPI_EXPORTED int32_t mtrt_hip_gemm_w8a8_prepack(mtrt_stream_t stream, const void *w_kn,
                                                       void *w_nk, int64_t K, int64_t N);
@@ -416,8 +416,8 @@ MTRT_CAPI_EXPORTED int32_t mtrt_hip_gemm_w4a16(mtrt_stream_t stream, const void 
  * above do not express, and of the unquantized module; w_nk is the module's own [out_features, in_features]
  * weight.  The reference generates a tiled FMA loop nest for such a matmul
  * (fallback-schedule-matmul.mlir:24); here every shape with K > 0 runs on the matrix cores (f16 / bf16 / f32
- * MFMA with f32 accumulation), any shape, no alignment needs beyond the element size.  Up to 64 rows with rows
- * in whole 128-byte slices take a kernel bound by reading the weights once. */
+ * MFMA with f32 accumulation), any shape, no alignment needs beyond the element size.  Up to 128 rows with rows
+ * in whole 128-byte slices take kernels bound by reading the weights once. */
 MTRT_CAPI_EXPORTED int32_t mtrt_hip_linear_dense(mtrt_stream_t stream, const void *x, const void *w_nk,
                                                  const void *bias, void *y, int32_t dtype, int64_t M,
                                                  int64_t K, int64_t N);

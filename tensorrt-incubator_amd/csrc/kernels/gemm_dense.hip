@@ -289,6 +289,25 @@ extern "C" __global__ void __launch_bounds__(512) mtrt_gemm_dense_rows64_f32(
   }
 MTRT_DENSE_ROWS64_KERNEL(f16, F16)
 MTRT_DENSE_ROWS64_KERNEL(bf16, BF16)
+// ... and up to 128 rows: four row tiles, four waves (block = 256)
+extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_dense_rows128_f32(
+    const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ bias, float* __restrict__ y, int64_t M,
+    int64_t K, int64_t N) {
+  __shared__ __attribute__((aligned(16))) int8_t lds[gemm_core::rows32::lds_bytes<4, 4>()];
+  dense_cluster::RowsBiasF32Epilogue epi{bias};
+  gemm_core::rows32::run<dense_cluster::F32Traits, 4, 4>(reinterpret_cast<const int8_t*>(x), reinterpret_cast<const int8_t*>(w), K * 4, epi, y, M, N, lds);
+}
+#define MTRT_DENSE_ROWS128_KERNEL(XN, XT)                                                                          \
+  extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_dense_rows128_##XN(                                  \
+      const XT::storage* __restrict__ x, const XT::storage* __restrict__ w, const XT::storage* __restrict__ bias,  \
+      uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N) {                                                 \
+    __shared__ __attribute__((aligned(16))) int8_t lds[gemm_core::rows32::lds_bytes<4, 4>()];                      \
+    dense_cluster::RowsBiasEpilogue<XT> epi{bias};                                                                 \
+    gemm_core::rows32::run<dense_cluster::HalfTraits<XT>, 4, 4>(reinterpret_cast<const int8_t*>(x), reinterpret_cast<const int8_t*>(w),     \
+                                                                K * 2, epi, y, M, N, lds);                         \
+  }
+MTRT_DENSE_ROWS128_KERNEL(f16, F16)
+MTRT_DENSE_ROWS128_KERNEL(bf16, BF16)
 
 // Any K and any alignment on the matrix cores: (x [M,K], w [N,K], bias [N] or null, y [M,N], M, K, N) ; grid: any
 // (128 x 128 tiles dealt round-robin), block = 256.

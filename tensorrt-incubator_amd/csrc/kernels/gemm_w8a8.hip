@@ -542,6 +542,14 @@ extern "C" __global__ void __launch_bounds__(512) mtrt_gemm_w8a8_nk_rows64(
   RowsScaleEpilogue epi{a_scale, w_scale};
   gemm_core::rows32::run<I8Traits, 8, 2>(a, w_nk, K, epi, y, M, N, lds);
 }
+// ... and up to 128 rows: four row tiles, four waves (block = 256)
+extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w8a8_nk_rows128(
+    const int8_t* __restrict__ a, const int8_t* __restrict__ w_nk, const float* __restrict__ a_scale,
+    const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N) {
+  __shared__ __attribute__((aligned(16))) int8_t lds[gemm_core::rows32::lds_bytes<4, 4>()];
+  RowsScaleEpilogue epi{a_scale, w_scale};
+  gemm_core::rows32::run<I8Traits, 4, 4>(a, w_nk, K, epi, y, M, N, lds);
+}
 
 // Any K and any operand alignment on the matrix cores, for the shapes the kernels above do not take (K not a
 // multiple of 128, operands off 16-byte alignment, operands of 4 GiB and more): the 128 x 128 tile loop of

@@ -734,10 +734,14 @@ int32_t mtrt_hip_gemm_w8a8(mtrt_stream_t stream, const void *a, const void *w_nk
     // only wins on very large weights.  33 to 64 rows take the form with two activation row tiles per weight fragment.
     const double tile_rounds = double(((N + 255) / 256 + num_compute_units(st) - 1) / num_compute_units(st));
     const double small_us = 3.0 + double(N) * double(K) / 3.4e6, tile_us = (8.0 + 0.006 * double(K)) * tile_rounds;
-    if (M <= 64 && small_us < tile_us) {
-      const int64_t tiles32 = (N + 31) / 32;
-      return launch(st, KernelName(M <= 32 ? "mtrt_gemm_w8a8_nk_rows32" : "mtrt_gemm_w8a8_nk_rows64"),
-                    uint32_t(std::min<int64_t>(tiles32, int64_t(kMaxGrid) * 1024)), 512, as_hip(stream), args);
+    // 65 to 128 rows: four row tiles per weight fragment, one workgroup of four waves per compute unit at a time, so
+    // the launch runs in rounds of about 3.7 ns per k (M = 128, K = N = 4096: 33 -> 18.4 us; K = N = 8192: 57 -> 30.7;
+    // N = 11008 needs two rounds and equals the tile launch)
+    const int64_t tiles32 = (N + 31) / 32;
+    const double mid_us = 3.0 + 0.0037 * double(K) * double((tiles32 + num_compute_units(st) - 1) / num_compute_units(st));
+    if (M <= 64 ? small_us < tile_us : M <= 128 && mid_us < tile_us) {
+      return launch(st, KernelName(M <= 32 ? "mtrt_gemm_w8a8_nk_rows32" : M <= 64 ? "mtrt_gemm_w8a8_nk_rows64" : "mtrt_gemm_w8a8_nk_rows128"),
+                    uint32_t(std::min<int64_t>(tiles32, int64_t(kMaxGrid) * 1024)), M <= 64 ? 512 : 256, as_hip(stream), args);
     }
     // 256 x 256 tiles, one workgroup per compute unit at a time, N panels dealt round-robin to the
     // 8 XCDs (gemm_core.hpp), so each set of panels takes 8 * ceil(panels / 8) * tiles_m workgroup
@@ -870,16 +874,19 @@ int32_t mtrt_hip_linear_dense(mtrt_stream_t stream, const void *x, const void *w
     return MTRT_RUNTIME_ERROR;
   // Decode-sized calls are bound by reading the weights once: up to 32 rows take one workgroup per 32 weight rows, its
   // eight waves splitting K (f16 M = 16, K = 4096, N = 11008: 55 us on the tile loop, 23.3 so, 3.9 TB/s of weights; f32
-  // 473 -> 50 us); 33 to 64 rows the form with two activation row tiles per weight fragment; the tile loop (about 8 us + 6 ns per byte of a row, per round)
-  // only wins on very large weights.
+  // 473 -> 50 us); 33 to 64 rows the form with two activation row tiles per weight fragment; the tile loop (about
+  // 8 us + 6 ns per byte of a row, per round) only wins on very large weights.
   const bool whole_slices = K > 0 && (K * eb) % 128 == 0 && aligned(x, 16) && aligned(w_nk, 16);
   const double tile_us = (8.0 + 0.006 * double(K * eb)) * double(((N + 255) / 256 + num_compute_units(st) - 1) / num_compute_units(st));
   const double small_us = 3.0 + double(N) * double(K * eb) / 4.0e6;
-  if (whole_slices && M <= 64 && small_us < tile_us) {
-    const int64_t tiles32 = (N + 31) / 32;
+  const int64_t tiles32 = (N + 31) / 32;
+  // 65 to 128 rows: four row tiles per weight fragment, rounds of one workgroup per compute unit (3.7 ns per byte of a row);
+  // f32 operands are bound by their matrix instructions there, which the tile loop is as well, at eight times the rows
+  const double mid_us = 3.0 + 0.0037 * double(K * eb) * double((tiles32 + num_compute_units(st) - 1) / num_compute_units(st));
+  if (whole_slices && (M <= 64 ? small_us < tile_us : M <= 128 && (dtype == MTRT_F32 || mid_us < tile_us))) {
     void *rargs[] = {&x, &w_nk, &bias, &y, &M, &K, &N};
-    return launch(st, KernelName(M <= 32 ? "mtrt_gemm_dense_rows32_" : "mtrt_gemm_dense_rows64_") + xn, uint32_t(std::min<int64_t>(tiles32, int64_t(kMaxGrid) * 1024)), 512,
-                  as_hip(stream), rargs);
+    return launch(st, KernelName(M <= 32 ? "mtrt_gemm_dense_rows32_" : M <= 64 ? "mtrt_gemm_dense_rows64_" : "mtrt_gemm_dense_rows128_") + xn,
+                  uint32_t(std::min<int64_t>(tiles32, int64_t(kMaxGrid) * 1024)), M <= 64 ? 512 : 256, as_hip(stream), rargs);
   }
   if (K > 0 && (K * eb) % 128 == 0 && aligned(x, 16) && aligned(w_nk, 16) && M * K * eb < (int64_t(1) << 32) &&
       N * K * eb < (int64_t(1) << 32)) {

@@ -44,7 +44,8 @@ def test_w8a8_mfma_kernel_small_shapes(pkg, orc, shape):
     a, w, a_s, w_s = _w8a8_inputs(rng(M + K + N), M, K, N)
     y, kernel = _run_w8a8(pkg, a, w, a_s, w_s)
     # up to 64 rows take the kernels that read the weights once at these sizes
-    assert kernel == ("mtrt_gemm_w8a8_nk_rows32" if M <= 32 else "mtrt_gemm_w8a8_nk_rows64" if M <= 64 else "mtrt_gemm_w8a8_nk")
+    assert kernel == ("mtrt_gemm_w8a8_nk_rows32" if M <= 32 else "mtrt_gemm_w8a8_nk_rows64" if M <= 64 else
+                      "mtrt_gemm_w8a8_nk_rows128" if M <= 128 else "mtrt_gemm_w8a8_nk")
     assert np.array_equal(bits16(y).reshape(M, N), orc.gemm_w8a8(a, w, a_s, w_s))
 
 
@@ -67,14 +68,15 @@ def test_w8a8_small_m_kernel_on_row_major_weights(pkg, orc, shape):
     assert np.array_equal(bits16(y).reshape(M, N), ref)
 
 
-@pytest.mark.parametrize("shape", [(64, 512, 4096), (33, 1024, 520), (50, 256, 8209), (64, 4096, 4100), (41, 128, 31)])
-def test_w8a8_33_to_64_rows_on_row_major_weights(pkg, orc, shape):
-    """Two activation row tiles against each weight fragment: every row of both tiles, ragged M and N, waves with and
-    without slices.  Integer sums: bit-exact."""
+@pytest.mark.parametrize("shape", [(64, 512, 4096), (33, 1024, 520), (50, 256, 8209), (64, 4096, 4100), (41, 128, 31),
+                                   (128, 512, 4096), (65, 1024, 520), (100, 256, 8209), (128, 4096, 1030), (97, 128, 31)])
+def test_w8a8_33_to_128_rows_on_row_major_weights(pkg, orc, shape):
+    """Two (up to 64 rows) or four (up to 128) activation row tiles against each weight fragment: every row of every
+    tile, ragged M and N, waves with and without slices.  Integer sums: bit-exact."""
     M, K, N = shape
     a, w, a_s, w_s = _w8a8_inputs(rng(M + K + N), M, K, N)
     y, kernel = _run_w8a8(pkg, a, w, a_s, w_s)
-    assert kernel == "mtrt_gemm_w8a8_nk_rows64"
+    assert kernel == ("mtrt_gemm_w8a8_nk_rows64" if M <= 64 else "mtrt_gemm_w8a8_nk_rows128")
     assert np.array_equal(bits16(y).reshape(M, N), orc.gemm_w8a8(a, w, a_s, w_s))
 
 

@@ -293,7 +293,7 @@ def test_dense_linear_against_float64(tp, pkg, dname):
     d = getattr(tp, dname)
     td = {"float32": torch.float32, "float16": torch.float16, "bfloat16": torch.bfloat16}[dname]
     torch.manual_seed(5)
-    for lead, K, N in (((3, 7), 50, 33), ((130,), 64, 129), ((1,), 1, 1), ((2, 300), 256, 520), ((700,), 1024, 8200), ((260,), 1031, 300), ((1,), 256, 40), ((2, 8), 4096, 1000), ((32,), 1024, 8209), ((5,), 64, 33), ((17,), 6144, 100), ((40,), 512, 300), ((64,), 128, 70)):
+    for lead, K, N in (((3, 7), 50, 33), ((130,), 64, 129), ((1,), 1, 1), ((2, 300), 256, 520), ((700,), 1024, 8200), ((260,), 1031, 300), ((1,), 256, 40), ((2, 8), 4096, 1000), ((32,), 1024, 8209), ((5,), 64, 33), ((17,), 6144, 100), ((40,), 512, 300), ((64,), 128, 70), ((100,), 512, 300), ((2, 64), 256, 1000), ((65,), 2048, 33)):
         x = torch.randn(*lead, K, dtype=torch.float32).to(td)
         w = (torch.randn(N, K, dtype=torch.float32) * 0.2).to(td)
         b = torch.randn(N, dtype=torch.float32).to(td)
@@ -303,8 +303,9 @@ def test_dense_linear_against_float64(tp, pkg, dname):
         # operands whose rows are whole 128-byte slices of K run the 256 x 256 tile loop, everything else 128 x 128 tiles
         # with element-aligned loads; both on the matrix cores
         mfma = K % (32 if dname == "float32" else 64) == 0
-        rows = int(np.prod(lead))                          # up to 64 rows read the weights once
+        rows = int(np.prod(lead))                          # up to 128 rows read the weights once
         assert pkg.last_kernel() == ("mtrt_gemm_dense_rows32_" if mfma and rows <= 32 else "mtrt_gemm_dense_rows64_" if mfma and rows <= 64 else
+                                     "mtrt_gemm_dense_rows128_" if mfma and rows <= 128 else
                                      "mtrt_gemm_dense_mfma_" if mfma else "mtrt_gemm_dense_edge_") + {"float32": "f32", "float16": "f16", "bfloat16": "bf16"}[dname]
         assert tuple(out.shape) == lead + (N,)
         ref = x.double() @ w.double().T + b.double()
