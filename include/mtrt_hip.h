@@ -379,7 +379,8 @@ MTRT_CAPI_EXPORTED int32_t mtrt_hip_gemm_w8a8(mtrt_stream_t stream, const void *
  * in that form only).  `w` is the program's [K,N] constant (w_is_nk = 0) or an [N,K] array (w_is_nk = 1);
  * w_frag holds mtrt_hip_gemm_w8a8_fragments_bytes(K, N) bytes (0 = shape not supported: K % 128 != 0)
  * and must be 16-byte aligned.  Same results, bit for bit.  Up to 32 rows (decode) take a kernel of their own
- * that is bound by reading the weights once, not by a tile's K loop; 33 to 64 rows may run as two launches. */
+ * that is bound by reading the weights once, not by a tile's K loop, and so do 33 to 128 rows while that is
+ * shorter than a tile launch. */
 MTRT_CAPI_EXPORTED int64_t mtrt_hip_gemm_w8a8_fragments_bytes(int64_t K, int64_t N);
 MTRT_CAPI_EXPORTED int32_t mtrt_hip_gemm_w8a8_prepack_fragments(mtrt_stream_t stream, const void *w,
                                                                 int32_t w_is_nk, void *w_frag, int64_t K,

@@ -610,7 +610,10 @@ constexpr int kPitch = 144, kStageBytes = 32 * kPitch;
 // MT: activation row tiles of 32 (1: M <= 32, 2: M <= 64, the weight fragments of a k-step serving both)
 template <int WAVES, int MT = 1> constexpr int lds_bytes() { return WAVES * (MT + 1) * kStageBytes; }
 
-template <class Traits, int WAVES, int MT = 1, class Epilogue, typename Y>
+// FRAG: `w` is not the [N,K] array but its fragment-order re-layout (per 32 rows and 128-byte slice four 1 KiB blocks,
+// lane l of block q holding the 16 bytes of k-step q of its row: exactly the second MFMA operand).  The weight
+// fragments then go from memory to registers and into the MFMA without passing LDS, 1 KiB contiguous per instruction.
+template <class Traits, int WAVES, int MT = 1, bool FRAG = false, class Epilogue, typename Y>
 __device__ __forceinline__ void run(const int8_t* __restrict__ a, const int8_t* __restrict__ w, int64_t row_bytes, Epilogue& epi,
                                     Y* __restrict__ y, int64_t M, int64_t N, int8_t* lds) {
   using Acc = typename Traits::Acc;
@@ -636,8 +639,10 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, const int8_t* 
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int64_t n = tile * 32 + lrow + 8 * i;
-      wp[i] = w + (n < N ? n : N - 1) * row_bytes + lchunk;
+      // fragment order: block i of a slice (the re-layout holds zeros for rows past N); else: row n of the array
+      wp[i] = FRAG ? w + tile * slices * 4096 + i * 1024 + lane * 16 : w + (n < N ? n : N - 1) * row_bytes + lchunk;
     }
+    constexpr int64_t kSliceBytes = FRAG ? 4096 : 128;   // from one slice of a lane's weight pieces to the next
     Acc acc[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[t] = Traits::zero();
@@ -650,7 +655,7 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, const int8_t* 
 #pragma unroll
       for (int i = 0; i < 4 * MT; ++i) ra[p][i] = *reinterpret_cast<const u32x4*>(ap[i] + kb * 128);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) rw[p][i] = *reinterpret_cast<const u32x4*>(wp[i] + kb * 128);
+      for (int i = 0; i < 4; ++i) rw[p][i] = *reinterpret_cast<const u32x4*>(wp[i] + kb * kSliceBytes);
     }
     for (int64_t kb = kb0; kb < kb1; kb += 2) {
 #pragma unroll
@@ -658,16 +663,25 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, const int8_t* 
         if (kb + p < kb1) {
 #pragma unroll
           for (int i = 0; i < 4 * MT; ++i) *reinterpret_cast<u32x4*>(sa + (lrow + 8 * i) * kPitch + lchunk) = ra[p][i];
+          u32x4 held[4];                               // fragment order: this slice's fragments stay in registers
 #pragma unroll
-          for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(sw + (lrow + 8 * i) * kPitch + lchunk) = rw[p][i];
+          for (int i = 0; i < 4; ++i) {
+            if (FRAG) held[i] = rw[p][i];
+            else *reinterpret_cast<u32x4*>(sw + (lrow + 8 * i) * kPitch + lchunk) = rw[p][i];
+          }
           const int64_t next = kb + p + 2 < kb1 ? kb + p + 2 : kb1 - 1;   // always a load: the waits stay countable
 #pragma unroll
           for (int i = 0; i < 4 * MT; ++i) ra[p][i] = *reinterpret_cast<const u32x4*>(ap[i] + next * 128);
 #pragma unroll
-          for (int i = 0; i < 4; ++i) rw[p][i] = *reinterpret_cast<const u32x4*>(wp[i] + next * 128);
+          for (int i = 0; i < 4; ++i) rw[p][i] = *reinterpret_cast<const u32x4*>(wp[i] + next * kSliceBytes);
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
-            const v4i fw = *reinterpret_cast<const v4i*>(sw + frow * kPitch + q * 32 + fhalf * 16);
+            v4i fw;
+            if (FRAG) {
+              fw = v4i{int(held[q][0]), int(held[q][1]), int(held[q][2]), int(held[q][3])};
+            } else {
+              fw = *reinterpret_cast<const v4i*>(sw + frow * kPitch + q * 32 + fhalf * 16);
+            }
 #pragma unroll
             for (int t = 0; t < MT; ++t) {
               const v4i fa = *reinterpret_cast<const v4i*>(sa + (t * 32 + frow) * kPitch + q * 32 + fhalf * 16);

@@ -551,6 +551,24 @@ extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w8a8_nk_rows128(
   gemm_core::rows32::run<I8Traits, 4, 4>(a, w_nk, K, epi, y, M, N, lds);
 }
 
+// 33 to 64 and 65 to 128 rows on fragment-order weights: the same kernels with the weight fragments straight from
+// memory into registers.  (a [M,K] i8, w_frag, a_scale, w_scale, y, M, K, N) ; K % 128 == 0, a and w_frag 16-byte
+// aligned; grid: any, block = 512 (rows64) / 256 (rows128).
+extern "C" __global__ void __launch_bounds__(512) mtrt_gemm_w8a8_frag_rows64(
+    const int8_t* __restrict__ a, const int8_t* __restrict__ w_frag, const float* __restrict__ a_scale,
+    const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N) {
+  __shared__ __attribute__((aligned(16))) int8_t lds[gemm_core::rows32::lds_bytes<8, 2>()];
+  RowsScaleEpilogue epi{a_scale, w_scale};
+  gemm_core::rows32::run<I8Traits, 8, 2, true>(a, w_frag, K, epi, y, M, N, lds);
+}
+extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w8a8_frag_rows128(
+    const int8_t* __restrict__ a, const int8_t* __restrict__ w_frag, const float* __restrict__ a_scale,
+    const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N) {
+  __shared__ __attribute__((aligned(16))) int8_t lds[gemm_core::rows32::lds_bytes<4, 4>()];
+  RowsScaleEpilogue epi{a_scale, w_scale};
+  gemm_core::rows32::run<I8Traits, 4, 4, true>(a, w_frag, K, epi, y, M, N, lds);
+}
+
 // Any K and any operand alignment on the matrix cores, for the shapes the kernels above do not take (K not a
 // multiple of 128, operands off 16-byte alignment, operands of 4 GiB and more): the 128 x 128 tile loop of
 // gemm_core::edge.  (a [M,K] i8, w_nk [N,K] i8, a_scale [M] f32, w_scale [N] f32, y [M,N] f16, M, K, N)

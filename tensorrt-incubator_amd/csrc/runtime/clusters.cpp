@@ -815,15 +815,23 @@ int32_t mtrt_hip_gemm_w8a8_fragments(mtrt_stream_t stream, const void *a, const 
   DeviceState *st = device_state();
   if (!st)
     return MTRT_RUNTIME_ERROR;
-  if (M > 32 && M <= 64 && (N + 31) / 32 <= int64_t(num_compute_units(st))) {
-    // 33 to 64 rows while every compute unit has at most one 32-column tile: two launches of the small-M kernel
-    // (rows 0..31, then the rest) are shorter than one tile launch, which lasts a whole K loop of a 256-row tile
-    // that is mostly padding (M = 64 at (K, N) = (4096, 4096) 21.0 us, (11008, 4096) 47.0, (8192, 8192) 38.4).
-    const int32_t rc = mtrt_hip_gemm_w8a8_fragments(stream, a, w_frag, a_scale, w_scale, y, 32, K, N);
-    if (rc != MTRT_OK)
-      return rc;
-    return mtrt_hip_gemm_w8a8_fragments(stream, static_cast<const char *>(a) + 32 * K, w_frag, a_scale + 32, w_scale,
-                                        static_cast<char *>(y) + 32 * N * 2, M - 32, K, N);
+  if (M > 32 && M <= 128) {
+    // 33 to 128 rows: a tile launch lasts one 256-row tile's whole K loop per round (about 5 us + 4 ns per k, and no less
+    // than reading the weights at 4.5 TB/s) and is mostly padding.  The wave-private kernels of gemm_core::rows32 with the
+    // weight fragments straight into registers read the weights once with two (up to 64 rows) or four row tiles per
+    // fragment: 64 rows about 5 us + 1 us per 4 MB of weights (K = N = 4096: 17.1 -> 10.2 us, K = 11008, N = 4096
+    // 34.1 -> 17.5, K = N = 8192 29.3 -> 19.0), 128 rows one workgroup per compute unit at a time, rounds of about
+    // 3.2 ns per k (K = N = 4096: 21.6 -> 16.0 us, K = N = 8192 38.0 -> 27.1; N = 11008 needs two rounds, 30.5 us, and
+    // stays on the tiles at 23.9).
+    const int64_t tiles32 = (N + 31) / 32, units = num_compute_units(st);
+    const double weights = double(N) * double(K);
+    const double tile_us = std::max(5.0 + 0.004 * double(K), weights / 4.5e6) * double(((N + 255) / 256 + units - 1) / units);
+    const double rows_us = M <= 64 ? 5.0 + weights / 4.0e6 : 3.0 + 0.0032 * double(K) * double((tiles32 + units - 1) / units);
+    if (rows_us < tile_us) {
+      void *rargs[] = {&a, &w_frag, &a_scale, &w_scale, &y, &M, &K, &N};
+      return launch(st, KernelName(M <= 64 ? "mtrt_gemm_w8a8_frag_rows64" : "mtrt_gemm_w8a8_frag_rows128"),
+                    uint32_t(std::min<int64_t>(tiles32, int64_t(kMaxGrid) * 1024)), M <= 64 ? 512 : 256, as_hip(stream), rargs);
+    }
   }
   if (M <= 32) {
     // one workgroup per 32-column tile, its four waves splitting K; between one and two tiles per compute unit one

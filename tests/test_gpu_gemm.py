@@ -96,8 +96,7 @@ def test_w8a8_weights_in_registers_kernel(pkg, orc, shape):
     a, w, a_s, w_s = _w8a8_inputs(rng(M + K + N), M, K, N)
     print("case: w8a8 fragments", shape, flush=True)
     y, kernel = _run_w8a8_frag(pkg, a, w, a_s, w_s, from_nk=(M % 2 == 1))
-    # 33..64 rows and at most one 32-column tile per compute unit: two launches of the small-M kernel, the last one for rows 32..M-1
-    assert kernel == ("mtrt_gemm_w8a8_small16" if M <= 16 or (32 < M <= 48 and N <= 8192) else "mtrt_gemm_w8a8_frag")
+    assert kernel == ("mtrt_gemm_w8a8_small16" if M <= 16 else "mtrt_gemm_w8a8_frag_rows64" if 32 < M <= 64 else "mtrt_gemm_w8a8_frag")
     orc.set_threads(16)
     ref = orc.gemm_w8a8(a, w, a_s, w_s)
     orc.set_threads(1)
@@ -105,7 +104,7 @@ def test_w8a8_weights_in_registers_kernel(pkg, orc, shape):
 
 
 @pytest.mark.parametrize("shape", [(1, 128, 32), (16, 4096, 11008), (32, 4096, 11008), (17, 384, 200), (9, 1280, 4099), (13, 640, 8240),
-                                   (32, 256, 16384), (25, 512, 16400), (8, 2048, 8209), (16, 128, 40), (64, 512, 4100), (50, 256, 8192)])
+                                   (32, 256, 16384), (25, 512, 16400), (8, 2048, 8209), (16, 128, 40)])
 def test_w8a8_small_m_kernel(pkg, orc, shape):
     """M <= 32: one workgroup per 32-column tile with four waves splitting K.  K = 128 and 384 leave waves without a
     slice, 1280 gives them 2 or 3 (only the one-at-a-time tail), 4096 eight (two groups of four); N = 11008 gives 344
@@ -114,8 +113,32 @@ def test_w8a8_small_m_kernel(pkg, orc, shape):
     M, K, N = shape
     a, w, a_s, w_s = _w8a8_inputs(rng(M + K + N), M, K, N)
     y, kernel = _run_w8a8_frag(pkg, a, w, a_s, w_s, from_nk=(M % 2 == 1))
-    last = M - 32 if M > 32 else M                       # 33..64 rows run as two launches
-    assert kernel == ("mtrt_gemm_w8a8_small16" if last <= 16 else "mtrt_gemm_w8a8_small32")
+    assert kernel == ("mtrt_gemm_w8a8_small16" if M <= 16 else "mtrt_gemm_w8a8_small32")
+    orc.set_threads(16)
+    ref = orc.gemm_w8a8(a, w, a_s, w_s)
+    orc.set_threads(1)
+    assert np.array_equal(bits16(y).reshape(M, N), ref)
+
+
+def _frag_rows_estimates(M, K, N, units=256):
+    tile = max(5.0 + 0.004 * K, N * K / 4.5e6) * -(-((N + 255) // 256) // units)
+    rows = 5.0 + N * K / 4.0e6 if M <= 64 else 3.0 + 0.0032 * K * -(-((N + 31) // 32) // units)
+    return rows, tile
+
+
+@pytest.mark.parametrize("shape", [(64, 512, 4100), (50, 256, 8192), (33, 1024, 520), (64, 4096, 4096), (41, 128, 31), (48, 4096, 11008),
+                                   (128, 512, 4096), (65, 1024, 520), (100, 256, 8209), (128, 4096, 1030), (97, 128, 31), (96, 4096, 11008),
+                                   (40, 128, 150000)])
+def test_w8a8_33_to_128_rows_on_fragment_order_weights(pkg, orc, shape):
+    """Two (up to 64 rows) or four activation row tiles against weight fragments that go from memory straight into
+    registers: every row of every tile, ragged M and N (the re-layout holds zeros past N), waves with and without
+    slices; shapes whose estimate favours the tile launch stay there.  Integer sums: bit-exact."""
+    M, K, N = shape
+    a, w, a_s, w_s = _w8a8_inputs(rng(M + K + N), M, K, N)
+    print("case: w8a8 fragments, 33..128 rows", shape, flush=True)
+    y, kernel = _run_w8a8_frag(pkg, a, w, a_s, w_s, from_nk=(M % 2 == 1))
+    rows_us, tile_us = _frag_rows_estimates(M, K, N)
+    assert kernel == (("mtrt_gemm_w8a8_frag_rows64" if M <= 64 else "mtrt_gemm_w8a8_frag_rows128") if rows_us < tile_us else "mtrt_gemm_w8a8_frag")
     orc.set_threads(16)
     ref = orc.gemm_w8a8(a, w, a_s, w_s)
     orc.set_threads(1)

@@ -212,7 +212,7 @@ def test_quant_linear_int8_runs_on_the_w8a8_cluster(tp, orc, pkg):
     (fragment-order weights prepared once): against a float64 product of the oracle's dequantized operands,
     1e-3 relative (f16 result)."""
     r = rng(77)
-    for M, K, N, kernel in ((96, 256, 160, "mtrt_gemm_w8a8_frag"), (5, 72, 33, "mtrt_gemm_w8a8_nk_edge")):
+    for M, K, N, kernel in ((96, 256, 160, "mtrt_gemm_w8a8_frag_rows128"), (5, 72, 33, "mtrt_gemm_w8a8_nk_edge")):
         x = r.standard_normal((M, K)).astype(np.float32)
         w = (r.standard_normal((N, K)) * 0.05).astype(np.float32)
         b = r.standard_normal(N).astype(np.float32)
