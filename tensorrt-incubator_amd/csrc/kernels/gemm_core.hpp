@@ -608,7 +608,7 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, const int8_t* 
 namespace rows32 {
 constexpr int kPitch = 144, kStageBytes = 32 * kPitch;
 // MT: activation row tiles of 32 (1: M <= 32, 2: M <= 64, the weight fragments of a k-step serving both)
-template <int WAVES, int MT = 1> constexpr int lds_bytes() { return WAVES * (MT + 1) * kStageBytes; }
+template <int WAVES, int MT = 1, bool FRAG = false> constexpr int lds_bytes() { return WAVES * (MT + (FRAG ? 0 : 1)) * kStageBytes; }
 
 // FRAG: `w` is not the [N,K] array but its fragment-order re-layout (per 32 rows and 128-byte slice four 1 KiB blocks,
 // lane l of block q holding the 16 bytes of k-step q of its row: exactly the second MFMA operand).  The weight
@@ -618,7 +618,7 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, const int8_t* 
                                     Y* __restrict__ y, int64_t M, int64_t N, int8_t* lds) {
   using Acc = typename Traits::Acc;
   using Scalar = typename Traits::Scalar;
-  constexpr int kWaveBytes = (MT + 1) * kStageBytes;
+  constexpr int kWaveBytes = (MT + (FRAG ? 0 : 1)) * kStageBytes;   // fragment-order weights need no stage
   static_assert(kWaveBytes >= MT * 16 * 64 * int(sizeof(Scalar)), "a wave's stages also hold its partial sums");
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int frow = lane & 31, fhalf = lane >> 5;

@@ -557,14 +557,14 @@ extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w8a8_nk_rows128(
 extern "C" __global__ void __launch_bounds__(512) mtrt_gemm_w8a8_frag_rows64(
     const int8_t* __restrict__ a, const int8_t* __restrict__ w_frag, const float* __restrict__ a_scale,
     const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N) {
-  __shared__ __attribute__((aligned(16))) int8_t lds[gemm_core::rows32::lds_bytes<8, 2>()];
+  __shared__ __attribute__((aligned(16))) int8_t lds[gemm_core::rows32::lds_bytes<8, 2, true>()];
   RowsScaleEpilogue epi{a_scale, w_scale};
   gemm_core::rows32::run<I8Traits, 8, 2, true>(a, w_frag, K, epi, y, M, N, lds);
 }
 extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w8a8_frag_rows128(
     const int8_t* __restrict__ a, const int8_t* __restrict__ w_frag, const float* __restrict__ a_scale,
     const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N) {
-  __shared__ __attribute__((aligned(16))) int8_t lds[gemm_core::rows32::lds_bytes<4, 4>()];
+  __shared__ __attribute__((aligned(16))) int8_t lds[gemm_core::rows32::lds_bytes<4, 4, true>()];
   RowsScaleEpilogue epi{a_scale, w_scale};
   gemm_core::rows32::run<I8Traits, 4, 4, true>(a, w_frag, K, epi, y, M, N, lds);
 }
