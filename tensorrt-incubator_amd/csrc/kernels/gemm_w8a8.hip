@@ -496,16 +496,8 @@ extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w8a8_small16(
   __shared__ __attribute__((aligned(16))) int8_t lds[4 * 4 * 2 * 1024];
   small_m::tiles<2>(a, w_frag, a_scale, w_scale, y, M, K, N, lds);
 }
-// M <= 32:
-extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w8a8_small32(
-    const int8_t* __restrict__ a, const v4i* __restrict__ w_frag, const float* __restrict__ a_scale,
-    const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N) {
-  __shared__ __attribute__((aligned(16))) int8_t lds[4 * 4 * 4 * 1024];
-  small_m::tiles<4>(a, w_frag, a_scale, w_scale, y, M, K, N, lds);
-}
-
-// Any K (no alignment needs): one output element per lane, plain loops.  Serves
-// shapes the MFMA kernel does not take; not a fast path.
+// Any K (no alignment needs): one output element per lane, plain loops.  Only K = 0 is left to it (every
+// other shape runs on the matrix cores).
 extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w8a8_nk_any(
     const int8_t* __restrict__ a, const int8_t* __restrict__ w, const float* __restrict__ a_scale,
     const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N) {
@@ -551,9 +543,16 @@ extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w8a8_nk_rows128(
   gemm_core::rows32::run<I8Traits, 4, 4>(a, w_nk, K, epi, y, M, N, lds);
 }
 
-// 33 to 64 and 65 to 128 rows on fragment-order weights: the same kernels with the weight fragments straight from
+// Up to 32, 64 and 128 rows on fragment-order weights: the same kernels with the weight fragments straight from
 // memory into registers.  (a [M,K] i8, w_frag, a_scale, w_scale, y, M, K, N) ; K % 128 == 0, a and w_frag 16-byte
-// aligned; grid: any, block = 512 (rows64) / 256 (rows128).
+// aligned; grid: any, block = 512 (rows32, rows64) / 256 (rows128).
+extern "C" __global__ void __launch_bounds__(512) mtrt_gemm_w8a8_frag_rows32(
+    const int8_t* __restrict__ a, const int8_t* __restrict__ w_frag, const float* __restrict__ a_scale,
+    const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N) {
+  __shared__ __attribute__((aligned(16))) int8_t lds[gemm_core::rows32::lds_bytes<8, 1, true>()];
+  RowsScaleEpilogue epi{a_scale, w_scale};
+  gemm_core::rows32::run<I8Traits, 8, 1, true>(a, w_frag, K, epi, y, M, N, lds);
+}
 extern "C" __global__ void __launch_bounds__(512) mtrt_gemm_w8a8_frag_rows64(
     const int8_t* __restrict__ a, const int8_t* __restrict__ w_frag, const float* __restrict__ a_scale,
     const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N) {

@@ -833,13 +833,23 @@ int32_t mtrt_hip_gemm_w8a8_fragments(mtrt_stream_t stream, const void *a, const 
                     uint32_t(std::min<int64_t>(tiles32, int64_t(kMaxGrid) * 1024)), M <= 64 ? 512 : 256, as_hip(stream), rargs);
     }
   }
-  if (M <= 32) {
+  if (M <= 32 && (M > 16 || 2 * ((N + 31) / 32) <= int64_t(num_compute_units(st)))) {
+    // 17 to 32 rows, and fewer rows when at most half of the compute units would get a 32-column tile: the wave-private
+    // kernel, eight waves splitting K (M = 32 at (K, N) = (11008, 4096) 18.6 -> 12.9 us, (4096, 11008) 14.3 -> 13.5,
+    // (8192, 8192) 15.8 -> 14.9; M = 16 at (11008, 4096) 15.1 -> 11.7).  With more tiles and up to 16 rows the
+    // four-wave kernel below with its hand-counted waits stays ahead (M = 1 at (4096, 11008): 10.7 against 12.5 us).
+    const int64_t tiles32 = (N + 31) / 32;
+    void *rargs[] = {&a, &w_frag, &a_scale, &w_scale, &y, &M, &K, &N};
+    return launch(st, KernelName("mtrt_gemm_w8a8_frag_rows32"), uint32_t(std::min<int64_t>(tiles32, int64_t(kMaxGrid) * 1024)), 512,
+                  as_hip(stream), rargs);
+  }
+  if (M <= 16) {
     // one workgroup per 32-column tile, its four waves splitting K; between one and two tiles per compute unit one
     // workgroup per unit instead, the first ones taking a second tile (as for the int4 weights)
     const int64_t tiles32 = (N + 31) / 32, cus = num_compute_units(st);
     const uint32_t grid = uint32_t(M > 8 && tiles32 > cus && tiles32 <= 2 * cus ? cus : tiles32);
     void *sargs[] = {&a, &w_frag, &a_scale, &w_scale, &y, &M, &K, &N};
-    return launch(st, KernelName(M <= 16 ? "mtrt_gemm_w8a8_small16" : "mtrt_gemm_w8a8_small32"), grid, kBlock, as_hip(stream), sargs);
+    return launch(st, KernelName("mtrt_gemm_w8a8_small16"), grid, kBlock, as_hip(stream), sargs);
   }
   // Tiles and rounds as in mtrt_hip_gemm_w8a8: 256 x 256, one workgroup per compute unit at a time;
   // a last round that would use at most half of the units is cut into 128-wide half tiles.

@@ -80,6 +80,12 @@ def test_w8a8_33_to_128_rows_on_row_major_weights(pkg, orc, shape):
     assert np.array_equal(bits16(y).reshape(M, N), orc.gemm_w8a8(a, w, a_s, w_s))
 
 
+def _frag_small_kernel(M, N, units=256):
+    """Up to 32 rows on fragment-order weights: the four-wave kernel with hand-counted waits for up to 16 rows and more
+    32-column tiles than half the compute units, the wave-private eight-wave kernel otherwise."""
+    return "mtrt_gemm_w8a8_frag_rows32" if M > 16 or 2 * ((N + 31) // 32) <= units else "mtrt_gemm_w8a8_small16"
+
+
 def _run_w8a8_frag(pkg, a, w, a_s, w_s, from_nk=False):
     import torch
     ad, wd = torch.from_numpy(a).cuda(), torch.from_numpy(w).cuda()
@@ -96,7 +102,7 @@ def test_w8a8_weights_in_registers_kernel(pkg, orc, shape):
     a, w, a_s, w_s = _w8a8_inputs(rng(M + K + N), M, K, N)
     print("case: w8a8 fragments", shape, flush=True)
     y, kernel = _run_w8a8_frag(pkg, a, w, a_s, w_s, from_nk=(M % 2 == 1))
-    assert kernel == ("mtrt_gemm_w8a8_small16" if M <= 16 else "mtrt_gemm_w8a8_frag_rows64" if 32 < M <= 64 else "mtrt_gemm_w8a8_frag")
+    assert kernel == (_frag_small_kernel(M, N) if M <= 32 else "mtrt_gemm_w8a8_frag_rows64" if M <= 64 else "mtrt_gemm_w8a8_frag")
     orc.set_threads(16)
     ref = orc.gemm_w8a8(a, w, a_s, w_s)
     orc.set_threads(1)
@@ -106,14 +112,14 @@ def test_w8a8_weights_in_registers_kernel(pkg, orc, shape):
 @pytest.mark.parametrize("shape", [(1, 128, 32), (16, 4096, 11008), (32, 4096, 11008), (17, 384, 200), (9, 1280, 4099), (13, 640, 8240),
                                    (32, 256, 16384), (25, 512, 16400), (8, 2048, 8209), (16, 128, 40)])
 def test_w8a8_small_m_kernel(pkg, orc, shape):
-    """M <= 32: one workgroup per 32-column tile with four waves splitting K.  K = 128 and 384 leave waves without a
+    """M <= 32: one workgroup per 32-column tile with four or eight waves splitting K.  K = 128 and 384 leave waves without a
     slice, 1280 gives them 2 or 3 (only the one-at-a-time tail), 4096 eight (two groups of four); N = 11008 gives 344
     tiles (one workgroup per compute unit, the first 88 with two tiles), 16384 two each, 16400 and 8209 one tile beyond
     those forms; ragged last tiles; M = 8 stays at one tile per workgroup.  Integer sums: bit-exact."""
     M, K, N = shape
     a, w, a_s, w_s = _w8a8_inputs(rng(M + K + N), M, K, N)
     y, kernel = _run_w8a8_frag(pkg, a, w, a_s, w_s, from_nk=(M % 2 == 1))
-    assert kernel == ("mtrt_gemm_w8a8_small16" if M <= 16 else "mtrt_gemm_w8a8_small32")
+    assert kernel == _frag_small_kernel(M, N)
     orc.set_threads(16)
     ref = orc.gemm_w8a8(a, w, a_s, w_s)
     orc.set_threads(1)
