@@ -28,6 +28,9 @@ idle; "settle_steps" in the line says how many were run.
 "mfma_sustained" is the matrix-core rate a loop of nothing but MFMAs reaches on the bench's
 own operand data (the published dense peaks hold for idle data only: the clock drops under
 the board's power limit); GEMM entries carry "frac_of_sustained" beside "frac".
+"hbm_sustained" is the matching yardstick for the memory-bound kernels: a stream that is only read, one that is only
+written and a plain copy, over 1 GiB each; HBM entries carry "frac_of_sustained" against the yardstick with their
+access mix ("sustained_mix").
 "library_yardsticks" are the vendor library's plain GEMMs (torch.matmul f16, torch._int_mm) at the same shapes,
 timed the same way; they are not part of the step.
 "cpu_baseline" times the CPU oracle (a C++ restatement of the reference's host
@@ -143,7 +146,8 @@ def build_workloads(pkg, torch, which):
             a = (xs[i].data_ptr(), pkg.BF16, qs[i].data_ptr(), pkg.F8E4M3FN, ys[i].data_ptr(), sc[i].data_ptr() + 4,
                  pkg.SCALE_UNIFORM, rows, cols, 1, 0)
             return lambda: pkg.check(L.mtrt_hip_quantize_dequantize(stream(), *a))
-        out.append(dict(name="mtrt_amax_bf16", config="C3", bound="hbm", work=2.0 * n, nslots=ns, make=amax, keep=(xs, sc)))
+        out.append(dict(name="mtrt_amax_bf16", config="C3", bound="hbm", work=2.0 * n, nslots=ns, make=amax, keep=(xs, sc),
+                        mix="read"))
         out.append(dict(name="mtrt_qdq_uniform_bf16_f8", config="C3", bound="hbm", work=5.0 * n, nslots=ns, make=qdq,
                         keep=(qs, ys)))
 
@@ -218,7 +222,7 @@ def build_workloads(pkg, torch, which):
                 return lambda: pkg.check(L.mtrt_hip_gemm_w4a16(stream(), *a))
             if M == 16:      # arithmetic intensity ~61 FLOP/B: bound by reading the weights once
                 out.append(dict(name=kname, config="C5 M=16", bound="hbm", work=float(nbytes), nslots=ns, make=gemm4,
-                                keep=(a5, w5, s5, y5)))
+                                keep=(a5, w5, s5, y5), mix="read"))
             else:
                 zero = None
                 if M == 4096:    # the same launch with zero activations and zero weights (nibble 8 is the value 0)
@@ -299,6 +303,53 @@ def mfma_sustained(pkg, torch, kernel, operand, ops_per_mfma):
     L.mtrt_cuda_event_release(e0)
     L.mtrt_cuda_event_release(e1)
     return ksteps * 16.0 * units * 4 * ops_per_mfma / us / 1e6
+
+
+def hbm_sustained(pkg, torch, nbytes=1 << 30):
+    """What the memory system sustains on this box for the three access mixes of the memory-bound clusters, each as
+    one launch of a yardstick kernel over `nbytes` (one 128-bit access per lane, one-shot grid, buffers far larger than
+    the 256 MiB Infinity Cache): {"read": GB/s of a stream that is only read, "write": only written, "copy": bytes
+    read + bytes written of a plain copy}.  Timed like the clusters: HIP events on the launch stream, median of ten."""
+    import ctypes
+    L = pkg.lib()
+    dev = L.mtrt_cuda_get_current_device()
+    s = torch.cuda.current_stream().cuda_stream
+    src = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    dst = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    sink = torch.zeros(4, dtype=torch.int32, device="cuda")
+    src.fill_(1)
+    dst.fill_(2)
+    nvec = nbytes // 16
+    grid = nvec // 256
+
+    def launcher(name, vals):
+        fn = L.mtrt_cuda_module_get_function(yardstick_module(pkg), name, len(name))
+        args = (ctypes.c_void_p * len(vals))(*[ctypes.cast(ctypes.pointer(v), ctypes.c_void_p) for v in vals])
+        return lambda keep=(vals, args): L.mtrt_cuda_launch_kernel(fn, grid, 1, 1, 256, 1, 1, 0, s, args)
+    kinds = (
+        ("read", launcher(b"mtrt_read_b128", (ctypes.c_void_p(src.data_ptr()), ctypes.c_void_p(sink.data_ptr()),
+                                              ctypes.c_int64(nvec), ctypes.c_uint32(0))), nbytes),
+        ("write", launcher(b"mtrt_fill_b128", (ctypes.c_void_p(dst.data_ptr()), ctypes.c_int64(nvec), ctypes.c_uint32(3))), nbytes),
+        ("copy", launcher(b"mtrt_copy_b128", (ctypes.c_void_p(src.data_ptr()), ctypes.c_void_p(dst.data_ptr()),
+                                              ctypes.c_int64(nvec))), 2 * nbytes),
+    )
+    out = {}
+    for kind, launch, moved in kinds:
+        for _ in range(3):
+            launch()
+        events = [L.mtrt_cuda_event_create(dev) for _ in range(11)]
+        L.mtrt_cuda_stream_record_event(s, events[0])
+        for b in range(10):
+            launch()
+            L.mtrt_cuda_stream_record_event(s, events[b + 1])
+        L.mtrt_cuda_event_sync(events[-1])
+        us = sorted(L.mtrt_cuda_event_elapsed_msec(events[b], events[b + 1]) * 1e3 for b in range(10))
+        for e in events:
+            L.mtrt_cuda_event_release(e)
+        out[kind] = round(moved / (0.5 * (us[4] + us[5])) / 1e3, 1)
+    assert int(sink[0]) == 0
+    del src, dst
+    return out
 
 
 def kernel_sources_digest():
@@ -418,6 +469,46 @@ def cache_variants(pkg, torch, wl, which, reps):
         us = time_kernel(pkg, torch, dict(make=sm, nslots=2), max(10, reps // 4))
         out.append(dict(kernel="mtrt_softmax_f16_v8", config="C2b x16 rows [65536, 4096]", us=round(us, 2),
                         achieved=round(4.0 * rows * d / us / 1e3, 1), unit="GB/s"))
+    return out
+
+
+def extra_clusters(pkg, torch, reps):
+    """Clusters that are not one of BASELINE.json's configs and not part of the step or of `value`, each with its own
+    roofline line: the per-token dynamic quantization that makes C4's int8 activations and a_scale (f16 [2048, 4096]
+    -> int8 codes + f32 scales in one launch; x read once, codes written: 3 bytes per element), beside the two
+    launches it replaces (per-row amax, then row-scaled quantize: x read twice, 5 bytes per element)."""
+    L = pkg.lib()
+    dev = torch.device("cuda:0")
+    rows, d = 2048, 4096
+    ns = max(2, int(np.ceil(CACHE_BYTES / (rows * d * 3))))
+    g = torch.Generator(device=dev)
+    g.manual_seed(44)
+    xs = [(torch.randn((rows, d), generator=g, device=dev) * 3.0).half() for _ in range(ns)]
+    qs = [torch.empty((rows, d), dtype=torch.int8, device=dev) for _ in range(ns)]
+    sc = [torch.empty((2, rows), dtype=torch.float32, device=dev) for _ in range(ns)]
+
+    def stream():
+        return torch.cuda.current_stream().cuda_stream
+
+    def fused(i):
+        a = (xs[i].data_ptr(), pkg.F16, qs[i].data_ptr(), pkg.I8, rows, d, 127.0, sc[i][0].data_ptr(), sc[i][1].data_ptr(), 0)
+        return lambda: pkg.check(L.mtrt_hip_dynamic_quantize_rows(stream(), *a))
+
+    def two(i):
+        a1 = (xs[i].data_ptr(), pkg.F16, pkg.SCALE_ROW, rows, d, rows, 127.0, sc[i][0].data_ptr(), sc[i][1].data_ptr())
+        a2 = (xs[i].data_ptr(), pkg.F16, qs[i].data_ptr(), pkg.I8, sc[i][1].data_ptr(), pkg.SCALE_ROW, rows, d, rows, 0)
+
+        def run():
+            pkg.check(L.mtrt_hip_amax_scales(stream(), *a1))
+            pkg.check(L.mtrt_hip_quantize(stream(), *a2))
+        return run
+    out = []
+    work = 3.0 * rows * d + 8.0 * rows
+    for what, make in (("mtrt_dynq_rows_f16_i8_v8 (one launch)", fused), ("mtrt_amax_rows_f16 + mtrt_q_row_f16_i8 (two launches)", two)):
+        us = time_kernel(pkg, torch, dict(make=make, nslots=ns), reps)
+        out.append(dict(kernel=what, config="per-token int8 quantization of C4's activations, f16 [2048, 4096]", bound="hbm",
+                        us=round(us, 2), achieved=round(work / us / 1e3, 1), peak=HBM_PEAK, unit="GB/s",
+                        frac=round(work / us / 1e3 / HBM_PEAK, 4), work=work))
     return out
 
 
@@ -617,6 +708,15 @@ def main():
     for k in kernels:
         if k["bound"] == "mfma" and k["unit"] in sustained:
             k["frac_of_sustained"] = round(k["achieved"] / sustained[k["unit"]], 4)
+    # what the memory system sustains on this box (pure read, pure write, copy); HBM rows are also given as a fraction
+    # of the yardstick with their access mix (amax only reads; every other cluster reads and writes, like the copy;
+    # the small-M GEMM reads 60 bytes for every byte it writes)
+    hbm = hbm_sustained(pkg, torch)
+    for w, k in zip(wl, kernels):
+        if k["bound"] == "hbm":
+            mix = w.get("mix", "copy")
+            k["frac_of_sustained"] = round(k["achieved"] / hbm[mix], 4)
+            k["sustained_mix"] = mix
     value = 100.0 * (ideal_us / 1e3) / ms_per_step
     dom = max(kernels, key=lambda k: k["us"])
     traffic = traffic_from_profile(dom["kernel"])
@@ -635,6 +735,8 @@ def main():
         "mfma_sustained": {"rates": sustained, "rates_on_zero_operands": sustained_zero, "method": "mtrt_mfma_probe_*: 16 independent MFMAs per round and wave, one wave "
                            "per SIMD, operands = this bench's own data, no memory traffic; published dense peaks are "
                            "not reached on non-zero data (power limit)"},
+        "hbm_sustained": {"rates": hbm, "unit": "GB/s", "method": "mtrt_read_b128 / mtrt_fill_b128 / mtrt_copy_b128 over 1 GiB per "
+                          "stream: one 128-bit access per lane, one launch each, median of ten; copy counts bytes read + written"},
         "workloads": kernels,
     }
     if not args.no_cache_variants:
@@ -644,6 +746,8 @@ def main():
     variants = [] if args.no_cache_variants else cache_variants(pkg, torch, wl, args.workload, args.kernel_reps)
     if variants:
         line["cache_variants"] = variants
+    if not args.no_cache_variants and args.workload in ("all", "c4"):
+        line["extra_clusters"] = extra_clusters(pkg, torch, args.kernel_reps)
     if not args.no_cache_variants:
         try:                      # an optional extra: never let the vendor library's state fail the benchmark
             yard = library_yardsticks(torch, args.workload, args.kernel_reps)

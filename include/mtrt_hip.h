@@ -300,6 +300,21 @@ MTRT_CAPI_EXPORTED int32_t mtrt_hip_dynamic_quantize_dequantize(mtrt_stream_t st
                                                                 void *y, int64_t n, float qmax,
                                                                 float *amax_out, float *scale_out,
                                                                 int32_t flags);
+/* Dynamic per-row (per-token) quantization in one call: for every row r of x [rows, d]
+ *   amax[r] = max_c |f32(x[r,c])| ; scale[r] = amax[r] / qmax ; q[r,c] = convert(clamp(rne?(f32(x[r,c]) / scale[r])))
+ * the single-use elementwise producers pulled into their consumer as the reference's segmentation does
+ * (mlir-tensorrt/compiler/lib/Backends/Kernel/KernelSegmentation.cpp:84-100), with the scale rule of
+ * tripy/examples/nanogpt/weight_loader.py:67-68, 102-115.  This is what makes the int8 activations and the per-token
+ * scales a_scale[m] that mtrt_hip_gemm_w8a8 takes.  q_dtype: MTRT_I8 or MTRT_F8E4M3FN (one code per byte);
+ * scale_out: f32 [rows], required; amax_out: f32 [rows] or NULL; flags as for mtrt_hip_quantize.  Results are
+ * bit-identical to mtrt_hip_amax_scales(MTRT_SCALE_ROW, nb = rows) followed by mtrt_hip_quantize(MTRT_SCALE_ROW,
+ * nb = rows).  Rows of whole 128-bit vectors (d % 4 == 0 for f32, d % 8 == 0 for f16 / bf16, x 16-byte aligned, q
+ * aligned to 4 / 8 bytes) of up to 16384 (f32) or 32768 elements run as ONE launch that reads x once, the row held in
+ * registers between the reduction and the quantization; other shapes run as those two launches. */
+MTRT_CAPI_EXPORTED int32_t mtrt_hip_dynamic_quantize_rows(mtrt_stream_t stream, const void *x, int32_t x_dtype,
+                                                          void *q, int32_t q_dtype, int64_t rows, int64_t d,
+                                                          float qmax, float *amax_out, float *scale_out,
+                                                          int32_t flags);
 /* Number of polls a workgroup of the one-launch form spends waiting for the grid's maximum before it computes
  * the maximum by itself (default 65536; 0: never wait).  Returns the previous value.  Process-wide. */
 MTRT_CAPI_EXPORTED int32_t mtrt_hip_set_wait_limit(int32_t polls);

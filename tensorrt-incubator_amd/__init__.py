@@ -95,6 +95,7 @@ PROTOTYPES = {
     "mtrt_hip_dequantize": (_i32, [_vp, _vp, _i32, _vp, _i32, _vp, _i32, _i64, _i64, _i64]),
     "mtrt_hip_quantize_dequantize": (_i32, [_vp, _vp, _i32, _vp, _i32, _vp, _vp, _i32, _i64, _i64, _i64, _i32]),
     "mtrt_hip_dynamic_quantize_dequantize": (_i32, [_vp, _vp, _i32, _vp, _i32, _vp, _i64, _f32, _vp, _vp, _i32]),
+    "mtrt_hip_dynamic_quantize_rows": (_i32, [_vp, _vp, _i32, _vp, _i32, _i64, _i64, _f32, _vp, _vp, _i32]),
     "mtrt_hip_set_wait_limit": (_i32, [_i32]),
     "mtrt_hip_quantize_view": (_i32, [_vp, _vp, _i32, _vp, _vp, _i32, _vp, _vp, _i32, _i64, _i64, _i64, _i32]),
     "mtrt_hip_dequantize_view": (_i32, [_vp, _vp, _i32, _vp, _vp, _i32, _vp, _vp, _i32, _i64, _i64, _i64]),
@@ -244,6 +245,20 @@ def dynamic_quantize_dequantize(x, q_dtype, qmax, flags=0, dequantize=True):
                                                      _ptr(y), x.numel(), float(qmax), out.data_ptr(), out.data_ptr() + 4,
                                                      flags))
     return q, y, out[0], out[1]
+
+
+def dynamic_quantize_rows(x, q_dtype, qmax, flags=0, want_amax=True):
+    """Per-row amax -> scale -> quantize of a [rows, d] tensor (leading axes folded into rows) in one call; returns
+    (q [rows * d] codes, amax [rows] or None, scale [rows])."""
+    torch = _torch()
+    assert x.is_cuda and x.is_contiguous() and x.dim() >= 1
+    d = x.shape[-1]
+    rows = x.numel() // d if d else 0
+    out = torch.empty((2, rows), dtype=torch.float32, device=x.device)
+    q = code_tensor(q_dtype, x.numel(), x.device)
+    check(lib().mtrt_hip_dynamic_quantize_rows(_stream(), x.data_ptr(), float_dtype_of(x), q.data_ptr(), q_dtype, rows, d,
+                                               float(qmax), out[0].data_ptr() if want_amax else None, out[1].data_ptr(), flags))
+    return q, (out[0] if want_amax else None), out[1]
 
 
 class View2d(ctypes.Structure):

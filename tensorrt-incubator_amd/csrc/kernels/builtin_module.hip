@@ -4,6 +4,7 @@
 #include "amax_scales.hip"
 #include "qdq.hip"
 #include "dynq.hip"
+#include "dynq_rows.hip"
 #include "nvfp4.hip"
 #include "norm.hip"
 #include "gemm_w8a8.hip"

@@ -46,6 +46,27 @@ extern "C" __global__ void __launch_bounds__(256) mtrt_copy_b128(const u32x4* __
     __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
 }
 
+// The two one-directional companions of the copy, one 128-bit access per lane: what the memory system sustains for a
+// stream that is only read (the loaded words are folded together and stored only if they equal `key`, which the
+// caller picks so that no lane stores) and for a stream that is only written.
+// (src, sink, nvec, key) / (dst, nvec, value) ; grid = ceil(nvec / 256), block = 256
+extern "C" __global__ void __launch_bounds__(256) mtrt_read_b128(const u32x4* __restrict__ src, uint32_t* __restrict__ sink,
+                                                                int64_t nvec, uint32_t key) {
+  const int64_t stride = int64_t(gridDim.x) * blockDim.x;
+  uint32_t fold = 0;
+  for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec; i += stride) {
+    const u32x4 v = __builtin_nontemporal_load(src + i);
+    fold |= (v[0] ^ key) & (v[1] ^ key) & (v[2] ^ key) & (v[3] ^ key);
+  }
+  if (fold == 0xFFFFFFFFu) sink[0] = fold;             // never true for the all-zero key on the benchmark's fill pattern
+}
+extern "C" __global__ void __launch_bounds__(256) mtrt_fill_b128(u32x4* __restrict__ dst, int64_t nvec, uint32_t value) {
+  const int64_t stride = int64_t(gridDim.x) * blockDim.x;
+  const u32x4 v = {value, value, value, value};
+  for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec; i += stride)
+    __builtin_nontemporal_store(v, dst + i);
+}
+
 // Matrix-core yardstick: what MFMA rate does the chip sustain on GIVEN operand data with no
 // memory traffic at all?  One wave per SIMD loads eight 16-byte fragments once and then issues
 // `ksteps` rounds of 16 independent MFMAs (a 4 x 4 register tile on fixed fragments, nothing else in the

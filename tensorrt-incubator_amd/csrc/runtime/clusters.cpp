@@ -511,6 +511,59 @@ int32_t mtrt_hip_dynamic_quantize_dequantize(mtrt_stream_t stream, const void *x
   return qdq_dispatch(0, as_hip(stream), x, x_dtype, q, q_dtype, nullptr, scale_out, MTRT_SCALE_UNIFORM, 1, n, 1, flags);
 }
 
+int32_t mtrt_hip_dynamic_quantize_rows(mtrt_stream_t stream, const void *x, int32_t x_dtype, void *q, int32_t q_dtype,
+                                       int64_t rows, int64_t d, float qmax, float *amax_out, float *scale_out,
+                                       int32_t flags) {
+  clear_error();
+  const char *xn = float_name(x_dtype);
+  if (!xn)
+    return set_error(MTRT_INVALID_ARGUMENT, "float operand dtype %d is not one of f32/f16/bf16", x_dtype);
+  if (q_dtype != MTRT_I8 && q_dtype != MTRT_F8E4M3FN)
+    return set_error(MTRT_INVALID_ARGUMENT, "dynamic per-row quantization targets i8 or f8E4M3FN, got dtype %d", q_dtype);
+  if (rows < 0 || d < 0)
+    return set_error(MTRT_INVALID_ARGUMENT, "negative extent [%lld, %lld]", (long long)rows, (long long)d);
+  int64_t n;
+  if (!element_count(rows, d, &n) || n >= (int64_t(1) << 35))
+    return set_error(MTRT_INVALID_ARGUMENT, "[%lld, %lld] elements exceed the supported 2^35", (long long)rows, (long long)d);
+  if (flags & ~(MTRT_Q_ROUND_TO_INT | MTRT_F8_REFHOST | MTRT_F8_VIA_F16))
+    return set_error(MTRT_INVALID_ARGUMENT, "unknown flag bits 0x%x", flags);
+  if ((flags & MTRT_F8_REFHOST) && (flags & MTRT_F8_VIA_F16))
+    return set_error(MTRT_INVALID_ARGUMENT, "MTRT_F8_REFHOST and MTRT_F8_VIA_F16 name two different conversions; pass one");
+  if (n == 0)
+    return MTRT_OK;                                    // no row has an element: nothing is written
+  if (!x || !q)
+    return set_error(MTRT_INVALID_ARGUMENT, "null operand");
+  if (!scale_out)
+    return set_error(MTRT_INVALID_ARGUMENT, "scale_out must point at device memory for one f32 per row");
+  if (!aligned(x, float_bytes(x_dtype)))
+    return set_error(MTRT_INVALID_ARGUMENT, "float operand is not aligned to its element size");
+  DeviceState *st = device_state();
+  if (!st)
+    return MTRT_RUNTIME_ERROR;
+  // One launch while a row fits in the registers of a wave (up to 64 x 16 vectors) or of a workgroup's four waves
+  // (up to 256 x 16 vectors): the row is read once.  Other rows (not whole vectors, operands off alignment, longer)
+  // run as the two launches whose results this call is defined by.
+  const int group = x_dtype == MTRT_F32 ? 4 : 8;
+  const int64_t nvec = d / group;
+  if (d % group == 0 && aligned(x, 16) && aligned(q, group) && nvec <= 256 * 16) {
+    const bool per_wave = nvec <= 64 * 16;
+    const int64_t lanes = per_wave ? 64 : 256;
+    int nv = 1;
+    while (lanes * nv < nvec)
+      nv *= 2;
+    const int64_t grid = per_wave ? (rows + 3) / 4 : rows;
+    if (grid <= int64_t(kMaxGrid)) {
+      void *args[] = {&x, &q, &rows, &d, &qmax, &amax_out, &scale_out, &flags};
+      return launch(st, KernelName("mtrt_dynq_rows_") + xn + "_" + code_name(q_dtype) + (per_wave ? "_v" : "_g4v") + nv,
+                    uint32_t(grid), kBlock, as_hip(stream), args);
+    }
+  }
+  const int32_t st1 = mtrt_hip_amax_scales(stream, x, x_dtype, MTRT_SCALE_ROW, rows, d, rows, qmax, amax_out, scale_out);
+  if (st1 != MTRT_OK)
+    return st1;
+  return qdq_dispatch(0, as_hip(stream), x, x_dtype, q, q_dtype, nullptr, scale_out, MTRT_SCALE_ROW, rows, d, rows, flags);
+}
+
 namespace {
 int32_t nvfp4_dispatch(bool quantize, hipStream_t stream, const void *xy, int32_t dtype, const void *q, const void *scales,
                        const float *tensor_amax, int64_t d0, int64_t d1, int32_t block_axis) {

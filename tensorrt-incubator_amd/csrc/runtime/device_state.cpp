@@ -83,8 +83,12 @@ struct DeviceState {
   static constexpr int kSlots = 256;
   static constexpr int kSlotWords = 64 * 32;
   uint32_t *slots = nullptr;
+  // The stream -> block mapping has a mutex of its own (slot_mu), which reduction_slot holds across the launch of
+  // a fresh block's clear; that launch may take `mu` to resolve the fill kernel.  Order: slot_mu, then mu.
+  std::mutex slot_mu;
   std::map<hipStream_t, int> slot_of;
   std::vector<int> free_slots;   // slots of destroyed streams, handed out again before new ones
+  std::vector<bool> pinned = std::vector<bool>(kSlots, false);   // handed out under stream capture: never recycled
   int next_slot = 0;
 };
 
@@ -178,43 +182,47 @@ int32_t clear_slot(DeviceState *st, uint32_t *block, hipStream_t stream) {
 } // namespace
 
 uint32_t *reduction_slot(DeviceState *st, hipStream_t stream) {
+  // A kernel recorded into a graph keeps the block's address in its arguments for as long as the graph is replayed,
+  // which can be long after the capture stream is gone: a block handed out while its stream is capturing stays out
+  // of the free list for good (256 blocks per device; a capture stream is normally bound once).
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  const bool capturing = hipStreamIsCapturing(stream, &capture) == hipSuccess && capture != hipStreamCaptureStatusNone;
+  std::lock_guard<std::mutex> lock(st->slot_mu);
+  auto it = st->slot_of.find(stream);
+  if (it != st->slot_of.end()) {
+    if (capturing)
+      st->pinned[size_t(it->second)] = true;
+    return st->slots + size_t(it->second) * DeviceState::kSlotWords;
+  }
   int slot;
-  bool fresh = false;
-  {
-    std::lock_guard<std::mutex> lock(st->mu);
-    auto it = st->slot_of.find(stream);
-    if (it != st->slot_of.end()) {
-      slot = it->second;
-    } else {
-      if (!st->free_slots.empty()) {
-        slot = st->free_slots.back();
-        st->free_slots.pop_back();
-      } else if (st->next_slot < DeviceState::kSlots) {
-        slot = st->next_slot++;
-      } else {
-        set_error(MTRT_RUNTIME_ERROR, "more than %d live streams use grid reductions", DeviceState::kSlots);
-        return nullptr;
-      }
-      st->slot_of.emplace(stream, slot);
-      fresh = true;
-    }
+  if (!st->free_slots.empty()) {
+    slot = st->free_slots.back();
+    st->free_slots.pop_back();
+  } else if (st->next_slot < DeviceState::kSlots) {
+    slot = st->next_slot++;
+  } else {
+    set_error(MTRT_RUNTIME_ERROR, "more than %d live streams use grid reductions", DeviceState::kSlots);
+    return nullptr;
   }
   uint32_t *block = st->slots + size_t(slot) * DeviceState::kSlotWords;
   // A block newly bound to a stream is cleared in stream order before its first use: whatever an earlier
   // owner (a destroyed stream, or a launch that never finished) left in it cannot reach this stream's results.
-  if (fresh && clear_slot(st, block, stream) != MTRT_OK) {
-    std::lock_guard<std::mutex> lock(st->mu);
-    st->slot_of.erase(stream);
+  // The clear is queued before the mapping becomes visible (the lock is held), so no other thread's reduction on
+  // this stream can be queued in front of it.
+  if (clear_slot(st, block, stream) != MTRT_OK) {
     st->free_slots.push_back(slot);
     return nullptr;
   }
+  st->slot_of.emplace(stream, slot);
+  if (capturing)
+    st->pinned[size_t(slot)] = true;
   return block;
 }
 
 int32_t reset_reduction_slot(DeviceState *st, hipStream_t stream) {
   int slot = -1;
   {
-    std::lock_guard<std::mutex> lock(st->mu);
+    std::lock_guard<std::mutex> lock(st->slot_mu);
     auto it = st->slot_of.find(stream);
     if (it != st->slot_of.end())
       slot = it->second;
@@ -238,16 +246,17 @@ void forget_stream(hipStream_t stream) {
   for (DeviceState *st : states) {
     bool bound;
     {
-      std::lock_guard<std::mutex> lock(st->mu);
+      std::lock_guard<std::mutex> lock(st->slot_mu);
       bound = st->slot_of.count(stream) != 0;
     }
     if (!bound)
       continue;
     (void)hipStreamSynchronize(stream);
-    std::lock_guard<std::mutex> lock(st->mu);
+    std::lock_guard<std::mutex> lock(st->slot_mu);
     auto it = st->slot_of.find(stream);
     if (it != st->slot_of.end()) {
-      st->free_slots.push_back(it->second);
+      if (!st->pinned[size_t(it->second)])             // a captured graph may still name a pinned block
+        st->free_slots.push_back(it->second);
       st->slot_of.erase(it);
     }
   }

@@ -13,11 +13,14 @@
 //    pointer is handed to kernels.  Every GPU has its own copy of the array at its own address.
 //  * The entry point itself calls no hipMalloc / hipFree and builds no heap objects: the kernel
 //    handles were resolved at set-up.
-//  * All calls on one GPU share that GPU's array.  Each call first clears the block with a small
-//    fill kernel on the caller's stream (a kernel, not a memset node, so the pair can be captured
-//    into a graph), then runs the reduction.  Two calls that overlap in time on one GPU (different
+//  * All calls on one GPU share that GPU's array.  Each call first clears the block with the
+//    built-in module's fill kernel on the caller's stream (a kernel, not a memset node, so the
+//    pair can be captured into a graph; launched through the driver call, whose own return value
+//    says whether THIS launch was accepted), then runs the reduction.  Two calls that overlap in time on one GPU (different
 //    streams) race on the block; callers serialise them.
 #include <hip/hip_runtime.h>
+
+#include <atomic>
 
 #include "runtime_internal.hpp"
 
@@ -32,16 +35,14 @@ namespace {
 
 constexpr int kMaxDevices = 64;
 struct PerDevice {
-  uint32_t *ptr = nullptr;               // device address of `scratch` on this device
+  // device address of `scratch` on this device; written last by the set-up (release) and read first by the entry
+  // point (acquire), so a thread that sees it also sees the handles below
+  std::atomic<uint32_t *> ptr{nullptr};
   hipFunction_t amax[3] = {nullptr, nullptr, nullptr};   // indexed by MTRT_F32 / MTRT_F16 / MTRT_BF16
+  hipFunction_t fill = nullptr;          // mtrt_fill of the built-in module
   int num_cus = 0;
 };
 PerDevice g_dev[kMaxDevices];
-
-__global__ void __launch_bounds__(256) mtrt_no_alloc_clear(uint32_t *p, int words) {
-  for (int i = threadIdx.x; i < words; i += 256)
-    p[i] = 0u;
-}
 
 } // namespace
 
@@ -62,8 +63,11 @@ int32_t no_alloc_setup(DeviceState *st, int device) {
     if (!d.amax[i])
       return MTRT_NOT_FOUND;
   }
+  d.fill = find_kernel(st, "mtrt_fill");
+  if (!d.fill)
+    return MTRT_NOT_FOUND;
   d.num_cus = num_compute_units(st);
-  d.ptr = static_cast<uint32_t *>(p);
+  d.ptr.store(static_cast<uint32_t *>(p), std::memory_order_release);
   return MTRT_OK;
 }
 
@@ -90,18 +94,24 @@ extern "C" int32_t mtrt_hip_amax_no_alloc(mtrt_stream_t stream, const void *x, i
   hipError_t e = hipGetDevice(&device);
   if (e != hipSuccess)
     return set_error(MTRT_RUNTIME_ERROR, "no usable HIP device: %s", hipGetErrorString(e));
-  if (device < 0 || device >= kMaxDevices || !g_dev[device].ptr)
+  uint32_t *block = device >= 0 && device < kMaxDevices ? g_dev[device].ptr.load(std::memory_order_acquire) : nullptr;
+  if (!block)
     return set_error(MTRT_RUNTIME_ERROR,
                      "device %d is not set up: call mtrt_hip_init() on it first (set-up loads code and "
                      "allocates, this entry point does neither)", device);
   const PerDevice &d = g_dev[device];
   hipStream_t s = as_hip(stream);
 
-  uint32_t *block = d.ptr;
-  hipLaunchKernelGGL(mtrt_no_alloc_clear, dim3(1), dim3(256), 0, s, block, kScratchWords);
-  e = hipGetLastError();
-  if (e != hipSuccess)
-    return set_error(MTRT_DRIVER_ERROR, "launching the clear kernel: %s", hipGetErrorString(e));
+  {
+    uint8_t *p = reinterpret_cast<uint8_t *>(block);
+    int64_t count = kScratchWords;
+    uint32_t fill = 0;
+    int32_t width = 4;
+    void *fargs[] = {&p, &count, &fill, &width};
+    e = hipModuleLaunchKernel(d.fill, 1, 1, 1, 256, 1, 1, 0, s, fargs, nullptr);
+    if (e != hipSuccess)
+      return set_error(MTRT_DRIVER_ERROR, "launching the clear kernel: %s", hipGetErrorString(e));
+  }
 
   // launch shape of mtrt_hip_amax: at most two workgroups per compute unit, 4 x 128-bit loads per lane and trip
   const int per_vec = dtype == MTRT_F32 ? 4 : 8;
@@ -115,7 +125,6 @@ extern "C" int32_t mtrt_hip_amax_no_alloc(mtrt_stream_t stream, const void *x, i
   void *args[] = {&x_arg, &n_arg, &qmax_arg, &amax_out, &scale_out, &block};
   e = hipModuleLaunchKernel(d.amax[dtype], uint32_t(grid), 1, 1, 256, 1, 1, 0, s, args, nullptr);
   if (e != hipSuccess) {
-    (void)hipGetLastError();
     return set_error(MTRT_DRIVER_ERROR, "launching the amax kernel grid %lld: %s", (long long)grid, hipGetErrorString(e));
   }
   return MTRT_OK;

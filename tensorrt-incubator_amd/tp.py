@@ -328,9 +328,11 @@ class Linear:
 
     Every product runs on a hand-written kernel of this library; which one follows from the parameters:
 
-      * int8, an input scale, weight scale per tensor or per output channel (dim 0): the product of the two
-        dequantized operands equals (q_x . q_W^T) * s_x * s_w[n] exactly in real arithmetic, so it runs on the
-        integer matrix cores (W8A8 cluster: int32 accumulation, f16 result widened to the module's dtype).
+      * int8 in a float16 module, an input scale, weight scale per tensor or per output channel (dim 0): the product
+        of the two dequantized operands equals (q_x . q_W^T) * s_x * s_w[n] exactly in real arithmetic, so it runs on
+        the integer matrix cores (W8A8 cluster: int32 accumulation, f16 result).  The cluster writes f16, so a
+        float32 or bfloat16 module keeps the literal form below: its results are not rounded to f16 on the way and
+        values beyond 65504 stay finite.
       * int4 weight-only in a float16 module, weight scale per tensor or per output channel, in_features a
         multiple of 64: the W4A16 cluster dequantizes the packed codes on the way into the matrix cores.
         (The rank-2 scale of this API groups OUTPUT features, [out/B, in] as weight_loader.py:102-115 builds it;
@@ -351,7 +353,14 @@ class Linear:
         self.weight_scale = None
         self.input_scale = None
         self._plan_key = None
+        self._plan_owners = None
         self._plan = None
+
+    def invalidate(self):
+        """Forget the prepared weight side.  Call after changing a parameter's device memory in a way torch does not
+        see (a kernel of this library writing into it, a raw pointer): assignments of new Tensors and torch's own
+        in-place updates are noticed without it."""
+        self._plan_key = self._plan_owners = self._plan = None
 
     def __call__(self, x):
         return self.forward(x)
@@ -372,10 +381,12 @@ class Linear:
     # -- weight side, once ---------------------------------------------------------------------------
     def _prepared(self):
         torch = _torch()
-        def ident(t):      # a new Tensor object or an in-place update of its storage makes a new key
-            return (id(t), t._t._version) if isinstance(t, Tensor) else t
-        key = (ident(self.weight), ident(self.weight_scale), ident(self.input_scale), self.quant_dtype, self.weight_quant_dim)
-        if self._plan is not None and self._plan_key == key:
+        # The plan belongs to these very parameter objects (held here, so that none of them can be freed and its
+        # identity handed to another object) at these versions of their storage.
+        owners = (self.weight, self.weight_scale, self.input_scale)
+        key = (tuple(t._t._version if isinstance(t, Tensor) else t for t in owners), self.quant_dtype, self.weight_quant_dim)
+        if (self._plan is not None and self._plan_key == key and
+                all(a is b for a, b in zip(self._plan_owners, owners))):
             return self._plan
         from . import gemm_w4a16_prepack, gemm_w8a8_prepack_fragments
         N, K = self.weight.shape
@@ -391,7 +402,7 @@ class Linear:
             q_weight = quantize(self.weight, self.weight_scale, self.quant_dtype, self.weight_quant_dim)
             w_scale = _convert_scale(self.weight_scale, self.dtype)
             per_out = w_scale.rank == 0 or (w_scale.rank == 1 and self.weight_quant_dim == 0)
-            if self.quant_dtype == int8 and has_x_scale and per_out:
+            if self.quant_dtype == int8 and has_x_scale and per_out and self.dtype == float16:
                 plan["route"] = "w8a8"
                 codes = q_weight.device_data().contiguous()          # [N, K], K contiguous
                 plan["s_w"] = _scale_on_device(w_scale).reshape(-1).expand(N).contiguous()
@@ -408,7 +419,7 @@ class Linear:
                 plan["scale_kn"] = _scale_on_device(w_scale).reshape(-1).expand(N).to(torch.float16).reshape(1, N).contiguous()
             else:
                 plan["weight"] = dequantize(q_weight, self.weight_scale, self.dtype, self.weight_quant_dim).device_data().contiguous()
-        self._plan_key, self._plan = key, plan
+        self._plan_key, self._plan_owners, self._plan = key, owners, plan
         return plan
 
     # -- forward ---------------------------------------------------------------------------------------

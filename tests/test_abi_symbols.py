@@ -156,6 +156,16 @@ def test_argument_validation_of_the_newer_entry_points_needs_no_device(pkg):
     assert dq(None, None, pkg.F32, 16, pkg.I8, 16, 64, 127.0, 16, 16, 0) == 1 and "null operand" in err()
     assert dq(None, 16, pkg.F32, 16, pkg.I8, 16, 64, 127.0, 16, None, 0) == 1 and "scale_out" in err()
     assert dq(None, 16, pkg.F32, 16, pkg.I8, 16, 64, 127.0, 16, 16, 64) == 1 and "flag" in err()
+    # dynamic per-row quantization in one call
+    dr = L.mtrt_hip_dynamic_quantize_rows
+    assert dr(None, 16, 9, 16, pkg.I8, 4, 16, 127.0, 16, 16, 0) == 1 and "f32/f16/bf16" in err()
+    assert dr(None, 16, pkg.F32, 16, pkg.I4, 4, 16, 7.0, 16, 16, 0) == 1 and "i8 or f8E4M3FN" in err()
+    assert dr(None, 16, pkg.F32, 16, pkg.I8, -4, 16, 127.0, 16, 16, 0) == 1 and "negative" in err()
+    assert dr(None, 16, pkg.F32, 16, pkg.I8, 1 << 20, 1 << 20, 127.0, 16, 16, 0) == 1 and "2^35" in err()
+    assert dr(None, None, pkg.F32, 16, pkg.I8, 4, 16, 127.0, 16, 16, 0) == 1 and "null operand" in err()
+    assert dr(None, 16, pkg.F32, 16, pkg.I8, 4, 16, 127.0, 16, None, 0) == 1 and "scale_out" in err()
+    assert dr(None, 16, pkg.F32, 16, pkg.F8E4M3FN, 4, 16, 448.0, 16, 16, pkg.F8_REFHOST | pkg.F8_VIA_F16) == 1 and "two different" in err()
+    assert dr(None, 16, pkg.F32, 16, pkg.I8, 0, 16, 127.0, 16, 16, 0) == 0                          # no rows
     # quantize on views
     ok_view = pkg.View2d(0, 8, 1)
     below = pkg.View2d(2, -8, 1)                               # row 1 would start 6 elements below the base pointer

@@ -5,12 +5,15 @@ fixed chain of correctly rounded f32 operations followed by one f16 narrowing, s
 f16 outputs must be BIT-IDENTICAL to the oracle's.
 
 W4A16: the dequantised weights are bit-exact (one f16 rounding, checked by reading them
-back through one-hot activations); the f32 accumulation runs in the matrix cores' order,
-not the host's left-to-right order, so outputs are compared under a tolerance:
-    |got - ref| <= 1e-3 * |ref| + 1 ulp_f16(ref) + 1e-3 * sqrt(K) * rms(a_row) * rms(wd_col)
-The last term is the scale of the rounding noise of a length-K f32 dot product whose terms
-cancel; without it results near zero could not be compared relatively at all.  The same bound
-is applied against a float64 evaluation.
+back through one-hot activations, once per tile kernel); the f32 accumulation runs in the
+matrix cores' order, not the host's left-to-right order, so outputs are compared under two bounds:
+    against the oracle, every element:   |got - ref| <= 1 ulp_f16(ref) + noise
+    against float64, every element:      |got - exact| <= 1e-3 * |exact| + 1 ulp_f16(exact) + noise
+    noise = 1e-5 * sqrt(K) * rms(a_row) * rms(wd_col)
+and the share of outputs whose bits differ from the oracle's is bounded (kMaxShare).  The noise term is the size of
+the rounding error of a length-K f32 dot product (measured on the host at K = 4096: 0.7e-5 in these units); it is
+what lets an output whose terms cancel to nearly zero be compared at all, and it is far below one f16 ulp of a
+typical output, so a kernel that rounded once too often per product would not pass.
 """
 import numpy as np
 import pytest
@@ -59,9 +62,8 @@ def test_w8a8_small_m_kernel_on_row_major_weights(pkg, orc, shape):
     a, w, a_s, w_s = _w8a8_inputs(rng(M + K + N), M, K, N)
     print("case: w8a8 small M, row-major weights", shape, flush=True)
     y, kernel = _run_w8a8(pkg, a, w, a_s, w_s)
-    # while streaming the weights at this kernel's rate is shorter than one tile's K loop
-    small = 3.0 + N * K / 3.4e6 < (8.0 + 0.006 * K) * -(-((N + 255) // 256) // 256)
-    assert kernel == ("mtrt_gemm_w8a8_nk_rows32" if small else "mtrt_gemm_w8a8_nk")
+    # the kernel that reads the weights once, or the tile loop where the host's estimate puts very wide weights
+    assert kernel in ("mtrt_gemm_w8a8_nk_rows32", "mtrt_gemm_w8a8_nk")
     orc.set_threads(16)
     ref = orc.gemm_w8a8(a, w, a_s, w_s)
     orc.set_threads(1)
@@ -80,10 +82,18 @@ def test_w8a8_33_to_128_rows_on_row_major_weights(pkg, orc, shape):
     assert np.array_equal(bits16(y).reshape(M, N), orc.gemm_w8a8(a, w, a_s, w_s))
 
 
-def _frag_small_kernel(M, N, units=256):
-    """Up to 32 rows on fragment-order weights: the four-wave kernel with hand-counted waits for up to 16 rows and more
-    32-column tiles than half the compute units, the wave-private eight-wave kernel otherwise."""
-    return "mtrt_gemm_w8a8_frag_rows32" if M > 16 or 2 * ((N + 31) // 32) <= units else "mtrt_gemm_w8a8_small16"
+# Up to 32 rows on fragment-order weights: the four-wave kernel with hand-counted waits (up to 16 rows) or the
+# wave-private eight-wave kernel; which of the two depends on the number of compute units, the results do not.
+_FRAG_SMALL = {"mtrt_gemm_w8a8_frag_rows32", "mtrt_gemm_w8a8_small16"}
+
+
+def _frag_small_ok(kernel, M):
+    return kernel in _FRAG_SMALL and (M <= 16 or kernel == "mtrt_gemm_w8a8_frag_rows32")
+
+
+# the tile kernels on fragment-order weights (one launch in rounds of tiles, or one workgroup per compute unit walking
+# its share of the columns)
+_FRAG_TILE = {"mtrt_gemm_w8a8_frag", "mtrt_gemm_w8a8_frag_strips"}
 
 
 def _run_w8a8_frag(pkg, a, w, a_s, w_s, from_nk=False):
@@ -102,7 +112,8 @@ def test_w8a8_weights_in_registers_kernel(pkg, orc, shape):
     a, w, a_s, w_s = _w8a8_inputs(rng(M + K + N), M, K, N)
     print("case: w8a8 fragments", shape, flush=True)
     y, kernel = _run_w8a8_frag(pkg, a, w, a_s, w_s, from_nk=(M % 2 == 1))
-    assert kernel == (_frag_small_kernel(M, N) if M <= 32 else "mtrt_gemm_w8a8_frag_rows64" if M <= 64 else "mtrt_gemm_w8a8_frag")
+    assert (_frag_small_ok(kernel, M) if M <= 32 else kernel in ("mtrt_gemm_w8a8_frag_rows64", "mtrt_gemm_w8a8_frag") if M <= 64
+            else kernel in _FRAG_TILE), kernel
     orc.set_threads(16)
     ref = orc.gemm_w8a8(a, w, a_s, w_s)
     orc.set_threads(1)
@@ -119,17 +130,11 @@ def test_w8a8_small_m_kernel(pkg, orc, shape):
     M, K, N = shape
     a, w, a_s, w_s = _w8a8_inputs(rng(M + K + N), M, K, N)
     y, kernel = _run_w8a8_frag(pkg, a, w, a_s, w_s, from_nk=(M % 2 == 1))
-    assert kernel == _frag_small_kernel(M, N)
+    assert _frag_small_ok(kernel, M), kernel
     orc.set_threads(16)
     ref = orc.gemm_w8a8(a, w, a_s, w_s)
     orc.set_threads(1)
     assert np.array_equal(bits16(y).reshape(M, N), ref)
-
-
-def _frag_rows_estimates(M, K, N, units=256):
-    tile = max(5.0 + 0.004 * K, N * K / 4.5e6) * -(-((N + 255) // 256) // units)
-    rows = 5.0 + N * K / 4.0e6 if M <= 64 else 3.0 + 0.0032 * K * -(-((N + 31) // 32) // units)
-    return rows, tile
 
 
 @pytest.mark.parametrize("shape", [(64, 512, 4100), (50, 256, 8192), (33, 1024, 520), (64, 4096, 4096), (41, 128, 31), (48, 4096, 11008),
@@ -143,8 +148,7 @@ def test_w8a8_33_to_128_rows_on_fragment_order_weights(pkg, orc, shape):
     a, w, a_s, w_s = _w8a8_inputs(rng(M + K + N), M, K, N)
     print("case: w8a8 fragments, 33..128 rows", shape, flush=True)
     y, kernel = _run_w8a8_frag(pkg, a, w, a_s, w_s, from_nk=(M % 2 == 1))
-    rows_us, tile_us = _frag_rows_estimates(M, K, N)
-    assert kernel == (("mtrt_gemm_w8a8_frag_rows64" if M <= 64 else "mtrt_gemm_w8a8_frag_rows128") if rows_us < tile_us else "mtrt_gemm_w8a8_frag")
+    assert kernel in (("mtrt_gemm_w8a8_frag_rows64" if M <= 64 else "mtrt_gemm_w8a8_frag_rows128"),) + tuple(_FRAG_TILE), kernel
     orc.set_threads(16)
     ref = orc.gemm_w8a8(a, w, a_s, w_s)
     orc.set_threads(1)
@@ -229,7 +233,7 @@ def test_c4_w8a8_full_size(pkg, orc):
     assert torch.equal(y, expect)
     # the weights-in-registers kernel gives the same bits
     y2, kernel2 = _run_w8a8_frag(pkg, a, w, a_s, w_s)
-    assert kernel2 == "mtrt_gemm_w8a8_frag"
+    assert kernel2 in _FRAG_TILE
     assert torch.equal(y2, expect)
 
 
@@ -263,20 +267,28 @@ def _run_w4a16(pkg, a, wp_host, s, K, N, B, prepack=True):
     return y, pkg.last_kernel()
 
 
-def _check_w4a16(orc, y, a, w, s, K, N, B, ref_bits):
+kNoise = 1e-5        # f32 accumulation noise, in units of sqrt(K) * rms(a_row) * rms(wd_col)
+kMaxShare = 0.02     # largest share of outputs that may differ from the oracle's bits (by one f16 ulp)
+
+
+def _ulp16(v):
+    return 2.0 ** np.floor(np.log2(np.maximum(np.abs(v), 2.0 ** -14))) * 2.0 ** -10
+
+
+def _check_w4a16(orc, y, a, w, s, K, N, B, ref_bits, max_share=kMaxShare):
     got = bits16(y).reshape(-1, N).view(np.float16).astype(np.float64)
     ref = ref_bits.view(np.float16).astype(np.float64)
     af = a.view(np.float16).astype(np.float64)
     wdf = (w.astype(np.float16) * np.repeat(s.view(np.float16), B, axis=0)).astype(np.float64)
     exact = af @ wdf
-    noise = 1e-3 * np.sqrt(K) * np.sqrt((af ** 2).mean(axis=1))[:, None] * np.sqrt((wdf ** 2).mean(axis=0))[None, :]
-    def ulp(v):
-        return 2.0 ** np.floor(np.log2(np.maximum(np.abs(v), 2.0 ** -14))) * 2.0 ** -10
-    for name, target in (("oracle", ref), ("float64", exact)):
-        bound = 1e-3 * np.abs(target) + ulp(target) + noise
+    noise = kNoise * np.sqrt(K) * np.sqrt((af ** 2).mean(axis=1))[:, None] * np.sqrt((wdf ** 2).mean(axis=0))[None, :]
+    for name, target, rel in (("oracle", ref, 0.0), ("float64", exact, 1e-3)):
+        bound = rel * np.abs(target) + _ulp16(target) + noise
         err = np.abs(got - target)
         assert np.all(err <= bound), "%s: worst excess %g at %s" % (name, (err - bound).max(), np.unravel_index(np.argmax(err - bound), err.shape))
-    return np.count_nonzero(got != ref) / got.size
+    share = np.count_nonzero(got != ref) / got.size
+    assert share <= max(max_share, 2.0 / got.size), "share of outputs that differ from the oracle: %g" % share
+    return share
 
 
 @pytest.mark.parametrize("shape", [(16, 256, 64), (1, 128, 32), (32, 1024, 96), (7, 512, 40), (33, 256, 64), (128, 512, 64),
@@ -307,6 +319,25 @@ def test_w4a16_dequantised_weights_are_bit_exact(pkg, orc):
         a = orc.narrow(eye[rows], orc.F16)
         y, kernel = _run_w4a16(pkg, a, orc.pack_int4(w), s, K, N, B)
         assert np.array_equal(bits16(y).reshape(-1, N), wd[rows]), kernel
+
+
+@pytest.mark.parametrize("case", [(2048, 8192, "mtrt_gemm_w4a16_t256x256"), (512, 1024, "mtrt_gemm_w4a16_t128x128")])
+def test_w4a16_tile_kernels_dequantise_bit_exactly(pkg, orc, case):
+    """Identity activations (M = K) through the 256 x 256 and the 128 x 128 tile kernels: every output is one product
+    1 x wd plus zeros, so y must equal the dequantised weights bit for bit whatever the order of the sums: pins the
+    fragment order of the re-laid weights, the nibble decoding, the scale row of every K block and the single f16
+    rounding in the kernels that carry the benchmark."""
+    K, N, want = case
+    B = 128
+    g = rng(K + N)
+    w = g.integers(-8, 8, (K, N)).astype(np.int8)
+    s = orc.narrow(g.uniform(0.005, 0.02, (K // B, N)).astype(np.float32), orc.F16)
+    eye = np.zeros((K, K), np.float32)
+    np.fill_diagonal(eye, 1.0)
+    wd = (w.astype(np.float16) * np.repeat(s.view(np.float16), B, axis=0)).view(np.uint16)
+    y, kernel = _run_w4a16(pkg, orc.narrow(eye, orc.F16), orc.pack_int4(w), s, K, N, B)
+    assert kernel == want
+    assert np.array_equal(bits16(y).reshape(K, N), wd)
 
 
 @pytest.mark.parametrize("case", [(5, 48, 7, 16), (9, 100, 33, 20), (3, 128, 6, 128), (130, 256, 200, 32), (70, 192, 131, 16),
@@ -372,7 +403,7 @@ def test_c5_w4a16_full_size(pkg, orc, M):
     wd = (torch.from_numpy(w.astype(np.float16)).to(dev) *
           torch.from_numpy(s.view(np.float16).copy()).to(dev).repeat_interleave(B, dim=0)).double()
     exact = af @ wd
-    noise = 1e-3 * np.sqrt(K) * (af ** 2).mean(dim=1).sqrt()[:, None] * (wd ** 2).mean(dim=0).sqrt()[None, :]
+    noise = kNoise * np.sqrt(K) * (af ** 2).mean(dim=1).sqrt()[:, None] * (wd ** 2).mean(dim=0).sqrt()[None, :]
     ulp = torch.exp2(torch.floor(torch.log2(exact.abs().clamp_min(2.0 ** -14)))) * 2.0 ** -10
     err = (y.double() - exact).abs()
     excess = err - (1e-3 * exact.abs() + ulp + noise)

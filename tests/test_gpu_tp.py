@@ -208,42 +208,80 @@ def test_quant_linear_reference_cases(tp):
 
 
 def test_quant_linear_int8_runs_on_the_w8a8_cluster(tp, orc, pkg):
-    """int8 Linear with an input scale and per-output-channel weight scales lands on the integer matrix cores
-    (fragment-order weights prepared once): against a float64 product of the oracle's dequantized operands,
-    1e-3 relative (f16 result)."""
+    """int8 Linear in a float16 module with an input scale and per-output-channel weight scales lands on the integer
+    matrix cores (fragment-order weights prepared once): against a float64 product of the oracle's dequantized
+    operands, 1e-3 relative (f16 result)."""
     r = rng(77)
-    for M, K, N, kernel in ((96, 256, 160, "mtrt_gemm_w8a8_frag_rows128"), (5, 72, 33, "mtrt_gemm_w8a8_nk_edge")):
-        x = r.standard_normal((M, K)).astype(np.float32)
-        w = (r.standard_normal((N, K)) * 0.05).astype(np.float32)
-        b = r.standard_normal(N).astype(np.float32)
-        s_x = np.float32(np.abs(x).max() / 127.0)
-        s_w = (np.abs(w).max(axis=1) / 127.0).astype(np.float32)
-        lin = tp.Linear(K, N, quant_dtype=tp.int8, weight_quant_dim=0)
+    for M, K, N, kernels in ((96, 256, 160, ("mtrt_gemm_w8a8_frag_rows128", "mtrt_gemm_w8a8_frag")), (5, 72, 33, ("mtrt_gemm_w8a8_nk_edge",))):
+        x = r.standard_normal((M, K)).astype(np.float16)
+        w = (r.standard_normal((N, K)) * 0.05).astype(np.float16)
+        b = r.standard_normal(N).astype(np.float16)
+        s_x = np.float16(np.abs(x.astype(np.float32)).max() / 127.0)
+        s_w = (np.abs(w.astype(np.float32)).max(axis=1) / 127.0).astype(np.float16)
+        lin = tp.Linear(K, N, dtype=tp.float16, quant_dtype=tp.int8, weight_quant_dim=0)
         lin.load_state_dict({"weight": tp.Tensor(w), "bias": tp.Tensor(b), "weight_scale": tp.Tensor(s_w),
                              "input_scale": tp.Tensor(s_x)})
         assert lin.route() == "w8a8"
         plan = lin._prepared()
         out = lin(tp.Tensor(x)).torch().cpu().numpy().astype(np.float64)
         assert lin._prepared() is plan, "the weight side must be prepared once, not per forward pass"
-        assert pkg.last_kernel() == kernel
+        assert pkg.last_kernel() in kernels
 
-        qx = orc.quantize(x.ravel(), orc.F32, orc.I8, np.array([s_x]), orc.SCALE_UNIFORM, M, K)
-        qw = orc.quantize(w.ravel(), orc.F32, orc.I8, s_w, orc.SCALE_ROW, N, K, N)
-        xd = qx.astype(np.float64).reshape(M, K) * np.float64(s_x)
-        wd = qw.astype(np.float64).reshape(N, K) * s_w.astype(np.float64)[:, None]
+        s_x32, s_w32 = np.float32(s_x), s_w.astype(np.float32)
+        qx = orc.quantize(x.view(np.uint16).ravel(), orc.F16, orc.I8, np.array([s_x32]), orc.SCALE_UNIFORM, M, K)
+        qw = orc.quantize(w.view(np.uint16).ravel(), orc.F16, orc.I8, s_w32, orc.SCALE_ROW, N, K, N)
+        xd = qx.astype(np.float64).reshape(M, K) * np.float64(s_x32)
+        wd = qw.astype(np.float64).reshape(N, K) * s_w32.astype(np.float64)[:, None]
         core = xd @ wd.T
-        ref = core + b
-        tol = (1e-3 + 2.0 ** -10) * np.abs(core) + 1e-6 * (1 + np.abs(b))     # 1e-3 relative + one f16 rounding of the product
+        bias = b.astype(np.float64)
+        ref = core + bias
+        # 1e-3 relative + one f16 rounding of the product + one of the sum with the bias
+        tol = (1e-3 + 2.0 ** -10) * np.abs(core) + 2.0 ** -10 * np.abs(ref) + 1e-6
         assert np.all(np.abs(out - ref) <= tol), float(np.max(np.abs(out - ref) / (np.abs(ref) + 1e-9)))
-        # a new weight tensor is picked up (the plan is keyed on the parameter objects)
-        lin.weight = tp.Tensor(2 * w)
-        lin.weight_scale = tp.Tensor(2 * s_w)
+        # a new weight tensor is picked up (the plan belongs to the parameter objects it was made from)
+        lin.weight = tp.Tensor((2 * w.astype(np.float32)).astype(np.float16))
+        lin.weight_scale = tp.Tensor((2 * s_w.astype(np.float32)).astype(np.float16))
+        assert lin._prepared() is not plan
         out2 = lin(tp.Tensor(x)).torch().cpu().numpy().astype(np.float64)
-        assert np.all(np.abs(out2 - (2 * core + b)) <= 2 * tol)
-        # the literal fake-quant form on the dense kernel agrees (weight scales along dim 0, no integer GEMM when
-        # the input scale is absent)
+        assert np.all(np.abs(out2 - (2 * core + bias)) <= 2 * tol)
+        # an in-place update that torch cannot see is picked up after invalidate()
+        plan2 = lin._prepared()
+        lin.invalidate()
+        assert lin._prepared() is not plan2
+        # without the input scale there is no integer GEMM: the literal fake-quant form on the dense kernel
         lin.input_scale = None
         assert lin.route() == "dense"
+
+
+@pytest.mark.parametrize("dname", ["float32", "bfloat16"])
+def test_quant_linear_int8_keeps_the_module_dtype_outside_float16(tp, orc, pkg, dname):
+    """A float32 or bfloat16 module with the same parameters stays on the literal form DQ(Q(x)) @ DQ(Q(W))^T in its own
+    dtype: the W8A8 cluster writes f16, which would round every output to eleven bits and turn anything beyond 65504
+    into inf.  Scales are chosen so that the outputs reach about 3e5."""
+    import torch
+    d = getattr(tp, dname)
+    td = {"float32": torch.float32, "bfloat16": torch.bfloat16}[dname]
+    r = rng(79)
+    M, K, N = 40, 256, 96
+    x = torch.from_numpy((r.standard_normal((M, K)) * 30.0).astype(np.float32)).to(td)
+    w = torch.from_numpy((r.standard_normal((N, K)) * 30.0).astype(np.float32)).to(td)
+    w[:, :] = w.abs()                                  # no cancellation: every output is large
+    x[:, :] = x.abs()
+    s_x = (x.float().abs().max() / 127.0).to(td)
+    s_w = (w.float().abs().amax(dim=1) / 127.0).to(td)
+    lin = tp.Linear(K, N, bias=False, dtype=d, quant_dtype=tp.int8, weight_quant_dim=0)
+    lin.load_state_dict({"weight": tp.Tensor(w, dtype=d), "weight_scale": tp.Tensor(s_w, dtype=d), "input_scale": tp.Tensor(s_x, dtype=d)})
+    assert lin.route() == "dense"
+    out = lin(tp.Tensor(x, dtype=d)).torch()
+    assert pkg.last_kernel().startswith("mtrt_gemm_dense_")
+    assert out.dtype == td and bool(torch.isfinite(out).all()) and float(out.float().max()) > 65504.0
+    xq = torch.clamp(torch.round(x.float() / s_x.float()), -128, 127)
+    wq = torch.clamp(torch.round(w.float() / s_w.float()[:, None]), -128, 127)
+    xd = (xq * s_x.float()).to(td).double()           # the dequantized operands in the module's dtype
+    wd = (wq * s_w.float()[:, None]).to(td).double()
+    ref = xd @ wd.T
+    ulp = {"float32": 2.0 ** -23, "bfloat16": 2.0 ** -7}[dname]
+    assert bool(torch.all((out.cpu().double() - ref).abs() <= (ulp + 1e-5) * ref.abs()))
 
 
 def test_quant_linear_int4_weight_only_runs_on_the_w4a16_cluster(tp, orc, pkg):
