@@ -309,8 +309,8 @@ MTRT_CAPI_EXPORTED int32_t mtrt_hip_dynamic_quantize_dequantize(mtrt_stream_t st
  * scale_out: f32 [rows], required; amax_out: f32 [rows] or NULL; flags as for mtrt_hip_quantize.  Results are
  * bit-identical to mtrt_hip_amax_scales(MTRT_SCALE_ROW, nb = rows) followed by mtrt_hip_quantize(MTRT_SCALE_ROW,
  * nb = rows).  Rows of whole 128-bit vectors (d % 4 == 0 for f32, d % 8 == 0 for f16 / bf16, x 16-byte aligned, q
- * aligned to 4 / 8 bytes) of up to 16384 (f32) or 32768 elements run as ONE launch that reads x once, the row held in
- * registers between the reduction and the quantization; other shapes run as those two launches. */
+ * aligned to 4 / 8 bytes) of up to 16384 elements (32768 for f16 / bf16 to int8) run as ONE launch that reads x once,
+ * the row held in registers between the reduction and the quantization; other shapes run as those two launches. */
 MTRT_CAPI_EXPORTED int32_t mtrt_hip_dynamic_quantize_rows(mtrt_stream_t stream, const void *x, int32_t x_dtype,
                                                           void *q, int32_t q_dtype, int64_t rows, int64_t d,
                                                           float qmax, float *amax_out, float *scale_out,

@@ -171,6 +171,9 @@ __device__ __forceinline__ void dynqdq_body(const typename X::storage* __restric
 MTRT_DYNQ_KERNELS(f32, F32, i8, I8)
 MTRT_DYNQ_KERNELS(f32, F32, f8, F8)
 MTRT_DYNQ_KERNELS(f16, F16, i8, I8)
-MTRT_DYNQ_KERNELS(f16, F16, f8, F8)
 MTRT_DYNQ_KERNELS(bf16, BF16, i8, I8)
-MTRT_DYNQ_KERNELS(bf16, BF16, f8, F8)
+// 16-bit -> f8: four vectors per lane only.  With sixteen the 128 registers a lane of a 1024-lane workgroup has do not
+// hold the chunk and part of it goes to scratch memory, whose allocation costs a launch some 10 us (measured: f16
+// [32 Mi] to f8 55.8 us against 35.5 us to int8); such tensors take the two launches instead.
+MTRT_DYNQ_KERNEL(f16, F16, f8, F8, 4)
+MTRT_DYNQ_KERNEL(bf16, BF16, f8, F8, 4)

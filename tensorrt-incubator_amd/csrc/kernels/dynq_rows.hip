@@ -10,7 +10,7 @@
 // activations and the per-token scales a_scale[m] of the W8A8 GEMM.
 //
 // The two-launch form (amax per row, then quantize with row scales) reads the activations twice.  Here the row
-// stays in registers between the reduction and the quantization: a wave owns a row (NV 128-bit vectors per lane,
+// stays in registers between the reduction and the quantization: a wave owns a row (NV <= 8 128-bit vectors per lane,
 // up to 64 * NV vectors per row) or, for longer rows, the four waves of a workgroup share one and meet in LDS;
 // the row maximum is a cross-lane exchange, the quotient the short exact division of qdq.hip (ExactDivisor), so
 // codes and scales are bit-identical to the two launches.  Loads are unconditional (lanes past the end of the row
@@ -85,21 +85,29 @@ __device__ __forceinline__ void body(const typename X::storage* __restrict__ x, 
 // (x [rows, d], q [rows, d], rows, d, qmax, amax_out [rows] or null, scale_out [rows], flags)
 //   d % G == 0 (G = 4 for f32, 8 for f16 / bf16), 0 < d / G <= 64 * NV (`_v`) or 256 * NV (`_g4v`), x 16-byte aligned,
 //   q aligned to G codes; grid = ceil(rows / 4) (`_v`: a wave per row) or rows (`_g4v`: a workgroup per row), block = 256.
-#define MTRT_DYNQ_ROWS_KERNEL(XN, XT, QN, QT, NV)                                                                        \
+// A wave holds up to 8 vectors per lane (more rows per compute unit in flight than with 16), the workgroup form 4 to 16.
+// The 16-vector form of the 16-bit -> f8 pairs needs scratch memory (the host does not launch it: a kernel with more
+// than a little scratch pays about 10 us per launch for its allocation) and is not built.
+#define MTRT_DYNQ_ROWS_WAVE(XN, XT, QN, QT, NV)                                                                          \
   extern "C" __global__ void __launch_bounds__(256) mtrt_dynq_rows_##XN##_##QN##_v##NV(                                   \
       const XT::storage* x, QT::storage* q, int64_t rows, int64_t d, float qmax, float* amax_out, float* scale_out,       \
       int32_t flags) {                                                                                                    \
-    dynq_rows_cluster::body<XT, QT, NV, 1>(x, q, rows, d, qmax, amax_out, scale_out, flags); }                            \
+    dynq_rows_cluster::body<XT, QT, NV, 1>(x, q, rows, d, qmax, amax_out, scale_out, flags); }
+#define MTRT_DYNQ_ROWS_GROUP(XN, XT, QN, QT, NV)                                                                         \
   extern "C" __global__ void __launch_bounds__(256) mtrt_dynq_rows_##XN##_##QN##_g4v##NV(                                 \
       const XT::storage* x, QT::storage* q, int64_t rows, int64_t d, float qmax, float* amax_out, float* scale_out,       \
       int32_t flags) {                                                                                                    \
     dynq_rows_cluster::body<XT, QT, NV, 4>(x, q, rows, d, qmax, amax_out, scale_out, flags); }
 #define MTRT_DYNQ_ROWS_KERNELS(XN, XT, QN, QT)                                                                            \
-  MTRT_DYNQ_ROWS_KERNEL(XN, XT, QN, QT, 1) MTRT_DYNQ_ROWS_KERNEL(XN, XT, QN, QT, 2) MTRT_DYNQ_ROWS_KERNEL(XN, XT, QN, QT, 4) \
-  MTRT_DYNQ_ROWS_KERNEL(XN, XT, QN, QT, 8) MTRT_DYNQ_ROWS_KERNEL(XN, XT, QN, QT, 16)
+  MTRT_DYNQ_ROWS_WAVE(XN, XT, QN, QT, 1) MTRT_DYNQ_ROWS_WAVE(XN, XT, QN, QT, 2) MTRT_DYNQ_ROWS_WAVE(XN, XT, QN, QT, 4)     \
+  MTRT_DYNQ_ROWS_WAVE(XN, XT, QN, QT, 8) MTRT_DYNQ_ROWS_GROUP(XN, XT, QN, QT, 4) MTRT_DYNQ_ROWS_GROUP(XN, XT, QN, QT, 8)
 MTRT_DYNQ_ROWS_KERNELS(f32, F32, i8, I8)
 MTRT_DYNQ_ROWS_KERNELS(f32, F32, f8, F8)
 MTRT_DYNQ_ROWS_KERNELS(f16, F16, i8, I8)
 MTRT_DYNQ_ROWS_KERNELS(f16, F16, f8, F8)
 MTRT_DYNQ_ROWS_KERNELS(bf16, BF16, i8, I8)
 MTRT_DYNQ_ROWS_KERNELS(bf16, BF16, f8, F8)
+MTRT_DYNQ_ROWS_GROUP(f32, F32, i8, I8, 16)
+MTRT_DYNQ_ROWS_GROUP(f32, F32, f8, F8, 16)
+MTRT_DYNQ_ROWS_GROUP(f16, F16, i8, I8, 16)
+MTRT_DYNQ_ROWS_GROUP(bf16, BF16, i8, I8, 16)

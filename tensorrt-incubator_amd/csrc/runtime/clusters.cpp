@@ -172,6 +172,15 @@ int32_t pick_nv(int64_t nvec_per_row) {
   return 0;
 }
 
+// Some element-aligned (`_u`) kernels on f32 rows with eight vectors per lane come out of the compiler badly: the
+// LayerNorm ones with 230 registers per lane (one wave per SIMD: f32 [4096, 8190] took 114 us against softmax's 45),
+// the 1024-lane ones of both families with 1.4 KB of scratch memory per lane (whose allocation costs a launch some
+// 10 us).  Their 16-vector forms take under 130 registers and no scratch, so those rows use them (a lane past the
+// end of the row holds nothing).
+int unaligned_nv(int32_t dtype, int nv, int lanes, bool layernorm) {
+  return dtype == MTRT_F32 && nv == 8 && (layernorm || lanes == 1024) ? 16 : nv;
+}
+
 // Rows too long for one wave: a workgroup of 256 or 1024 lanes with 8 or 16 vectors per lane owns the row.
 // Returns false when the row is longer than 1024 * 16 vectors.
 bool pick_group(int64_t nvec_per_row, int *threads, int *nv) {
@@ -489,8 +498,12 @@ int32_t mtrt_hip_dynamic_quantize_dequantize(mtrt_stream_t stream, const void *x
   const int group = x_dtype == MTRT_F32 ? 4 : 8;
   // one workgroup per compute unit at most, and one slot of the exchange per workgroup (256 of them)
   const int64_t nvec = n / group, units = std::min(num_compute_units(st), 256);
+  // (The 16-vector form of the 16-bit -> f8 pairs does not fit the 128 registers a lane of a 1024-lane workgroup has
+  // and would keep some of the row in scratch memory; a kernel that needs more than a little scratch pays some 10 us
+  // per launch for its allocation, more than the second launch costs, so those pairs stop at 4 vectors per lane.)
+  const int max_nv = group == 8 && q_dtype == MTRT_F8E4M3FN ? 4 : 16;
   const bool one_launch = n > 0 && n % group == 0 && aligned(x, 16) && aligned(q, group) && (!y || aligned(y, 16)) &&
-                          nvec <= units * 1024 * 16 && !((flags & MTRT_F8_REFHOST) && (flags & MTRT_F8_VIA_F16));
+                          nvec <= units * 1024 * max_nv && !((flags & MTRT_F8_REFHOST) && (flags & MTRT_F8_VIA_F16));
   if (one_launch) {
     uint32_t *slot = reduction_slot(st, as_hip(stream));
     if (!slot)
@@ -545,8 +558,11 @@ int32_t mtrt_hip_dynamic_quantize_rows(mtrt_stream_t stream, const void *x, int3
   // run as the two launches whose results this call is defined by.
   const int group = x_dtype == MTRT_F32 ? 4 : 8;
   const int64_t nvec = d / group;
-  if (d % group == 0 && aligned(x, 16) && aligned(q, group) && nvec <= 256 * 16) {
-    const bool per_wave = nvec <= 64 * 16;
+  // A wave holds up to 8 vectors per lane, a workgroup's lanes up to 16; the 16-bit -> f8 pairs stop at 8 (their
+  // 16-vector form would spill to scratch memory, whose allocation costs a launch some 10 us).
+  const int max_group_nv = group == 8 && q_dtype == MTRT_F8E4M3FN ? 8 : 16;
+  if (d % group == 0 && aligned(x, 16) && aligned(q, group) && nvec <= 256 * max_group_nv) {
+    const bool per_wave = nvec <= 64 * 8;
     const int64_t lanes = per_wave ? 64 : 256;
     int nv = 1;
     while (lanes * nv < nvec)
@@ -678,11 +694,13 @@ int32_t mtrt_hip_layernorm(mtrt_stream_t stream, const void *x, const void *gamm
   // Row lengths that are not whole vectors, or operands that are not 16-byte aligned: the same two schemes with
   // 128-bit accesses at element alignment and the last d % per_vec elements of a row moved one by one.
   if (!vec_ok && d >= per_vec) {
-    const int rnv = pick_nv(d / per_vec);
-    if (rnv && rows <= kMaxRowsPerWaveKernels)
+    int rnv = pick_nv(d / per_vec);
+    if (rnv && rows <= kMaxRowsPerWaveKernels) {
+      rnv = unaligned_nv(dtype, rnv, 64, true);
       return launch(st, KernelName("mtrt_layernorm_") + xn + "_u64v" + rnv, blocks_for(rows, kBlock / 64), kBlock, as_hip(stream), args);
+    }
     if (!rnv && rows <= int64_t(kMaxGrid) * 1024 && pick_group(d / per_vec, &threads, &gnv))
-      return launch(st, KernelName("mtrt_layernorm_") + xn + "_u" + threads + "v" + gnv, uint32_t(rows), uint32_t(threads),
+      return launch(st, KernelName("mtrt_layernorm_") + xn + "_u" + threads + "v" + unaligned_nv(dtype, gnv, threads, true), uint32_t(rows), uint32_t(threads),
                     as_hip(stream), args);
   }
   return launch(st, KernelName("mtrt_layernorm_") + xn + "_any",
@@ -729,11 +747,13 @@ int32_t mtrt_hip_softmax(mtrt_stream_t stream, const void *x, void *y, int32_t d
   // Row lengths that are not whole vectors, or operands that are not 16-byte aligned: the same two schemes with
   // 128-bit accesses at element alignment and the last d % per_vec elements of a row moved one by one.
   if (!vec_ok && d >= per_vec) {
-    const int rnv = pick_nv(d / per_vec);
-    if (rnv && rows <= kMaxRowsPerWaveKernels)
+    int rnv = pick_nv(d / per_vec);
+    if (rnv && rows <= kMaxRowsPerWaveKernels) {
+      rnv = unaligned_nv(dtype, rnv, 64, false);
       return launch(st, KernelName("mtrt_softmax_") + xn + "_u64v" + rnv, blocks_for(rows, kBlock / 64), kBlock, as_hip(stream), args);
+    }
     if (!rnv && rows <= int64_t(kMaxGrid) * 1024 && pick_group(d / per_vec, &threads, &gnv))
-      return launch(st, KernelName("mtrt_softmax_") + xn + "_u" + threads + "v" + gnv, uint32_t(rows), uint32_t(threads),
+      return launch(st, KernelName("mtrt_softmax_") + xn + "_u" + threads + "v" + unaligned_nv(dtype, gnv, threads, false), uint32_t(rows), uint32_t(threads),
                     as_hip(stream), args);
   }
   return launch(st, KernelName("mtrt_softmax_") + xn + "_any",

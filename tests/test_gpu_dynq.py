@@ -64,7 +64,11 @@ def test_type_pairs_and_grid_sizes(pkg, orc, xname, qname):
     for n, kernel in ((grp * 37, k + "v4"), (grp * (1024 * 4 * 3 + 555), k + "v4"), (grp * 1024 * 4 * 256 + grp * 1024 * 16 * 3, k + "v16")):
         x = (g.standard_normal(n) * 3).astype(np.float32)
         orc.set_threads(16)
-        _check(pkg, orc, x, xname, qname, kernel)
+        if kernel.endswith("v16") and grp == 8 and qname == "f8":
+            # no 16-vector form for the 16-bit -> f8 pairs (it would need scratch memory): the two launches
+            assert _check(pkg, orc, x, xname, qname).startswith("mtrt_qdq_")
+        else:
+            _check(pkg, orc, x, xname, qname, kernel)
         orc.set_threads(1)
 
 

@@ -60,9 +60,13 @@ def test_type_pairs_and_row_lengths(pkg, orc, xname, qname):
     k = "mtrt_dynq_rows_%s_%s_" % (xname, qname)
     orc.set_threads(16)
     for rows, nvec, kernel in ((1, 1, "v1"), (5, 37, "v1"), (7, 64, "v1"), (6, 65, "v2"), (9, 200, "v4"), (3, 512, "v8"),
-                               (10, 1000, "v16"), (2, 1024, "v16"), (3, 1025, "g4v8"), (5, 300 * 4 + 7, "g4v8"),
+                               (10, 1000, "g4v4"), (2, 1024, "g4v4"), (3, 1025, "g4v8"), (5, 300 * 4 + 7, "g4v8"),
                                (2, 4096, "g4v16"), (131, 96, "v2")):
         x = (g.standard_normal((rows, nvec * grp)) * g.uniform(0.1, 30.0, (rows, 1))).astype(np.float32)
+        if kernel == "g4v16" and grp == 8 and qname == "f8":
+            # the 16-vector form of the 16-bit -> f8 pairs is not built (it would need scratch memory): two launches
+            assert _check(pkg, orc, x, xname, qname).startswith("mtrt_q_row")
+            continue
         _check(pkg, orc, x, xname, qname, k + kernel)
     orc.set_threads(1)
 

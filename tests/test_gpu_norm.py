@@ -273,11 +273,20 @@ def test_softmax_rows_owned_by_a_workgroup(pkg, orc, name):
         _run_softmax(pkg, orc, name, 3, d, 70 + d % 89, "mtrt_softmax_" + name + suffix, frac=2e-2 if d <= 40000 else 5e-2)
 
 
-def _ragged_cases(name):
+def _ragged_cases(name, layernorm=False):
     """(row length, kernel suffix): lengths that are not whole vectors (attention rows of 77, 197, 1500 keys; a
     50257-entry vocabulary) in every scheme, from one vector plus one element up to 1024 x 16 vectors plus a tail;
     rows of at most 32 vectors share a wave (8, 16 or 32 lanes each) whether or not they are whole vectors."""
     e = 4 if name == "f32" else 8
+    cases = _ragged_cases_by_length(e)
+    if name == "f32" and layernorm:
+        # the eight-vector f32 LayerNorm kernels at element alignment compile to 230 registers: the host takes the
+        # sixteen-vector forms for those rows
+        cases = [(d, s.replace("v8", "v16")) for d, s in cases]
+    return cases
+
+
+def _ragged_cases_by_length(e):
     return [(1, "_u8v1"), (2, "_u8v1"), (e - 1, "_u8v1"), (e + 1, "_u8v1"), (77, "_u16v1" if e == 8 else "_u32v1"), (197, "_u32v1" if e == 8 else "_u64v1"), (e * 8, "_u8v1"),
             (e * 32, "_u32v1"), (e * 32 + 1, "_u32v1"), (e * 33 + 1, "_u64v1"), (e * 64 + 3, "_u64v1"), (e * 65 + 3, "_u64v2"), (1500 if e == 8 else 1501, "_u64v4" if e == 8 else "_u64v8"),
             (e * 512 + e - 1, "_u64v8"), (e * 1024 + 1, "_u64v16"), (e * 1025 + 2, "_u256v8"), (e * 4096 + 3, "_u256v16"),
@@ -286,7 +295,7 @@ def _ragged_cases(name):
 
 @pytest.mark.parametrize("name", ["f32", "f16", "bf16"])
 def test_layernorm_ragged_rows(pkg, orc, name):
-    for d, suffix in _ragged_cases(name):
+    for d, suffix in _ragged_cases(name, layernorm=True):
         _run_layernorm(pkg, orc, name, 5, d, 80 + d % 89, "mtrt_layernorm_" + name + suffix, frac=2e-2 if d <= 40000 else 5e-2,
                        oracle_slack=4.0 if d > 40000 else 1.0)
 
