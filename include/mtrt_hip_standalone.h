@@ -87,12 +87,12 @@ inline void abort_on_error(Status st) {
 /* MTRTRuntimeCore.h:46-59 */
 template <class To, class From>
 To bit_cast(From src) {
-  static_assert(sizeof(From) == sizeof(To), "Types must have matching sizes");
-  static_assert(std::is_trivially_copyable<From>::value, "Source type must be trivially copyable");
-  static_assert(std::is_trivially_copyable<To>::value, "Destination type must be trivially copyable");
-  To dst;
-  std::memcpy(std::addressof(dst), std::addressof(src), sizeof(To));
-  return dst;
+  static_assert(sizeof(To) == sizeof(From) && std::is_trivially_copyable<To>::value &&
+                    std::is_trivially_copyable<From>::value,
+                "mtrt::bit_cast needs two trivially copyable types of one size");
+  To result;                               /* the object representation copied over: defined for any such pair */
+  std::memcpy(static_cast<void *>(&result), static_cast<const void *>(&src), sizeof result);
+  return result;
 }
 
 /* MTRTRuntimeCore.h:67-88: offset, shape and strides count ELEMENTS, not bytes. */

@@ -24,6 +24,38 @@ constexpr uint32_t kMaxGrid = 1u << 20;
 // kMaxGrid.  Tensors with more rows take the `_any` kernels, which loop over rows.
 constexpr int64_t kMaxRowsPerWaveKernels = int64_t(kMaxGrid) * (kBlock / 64);
 
+// ---- launch-time estimates behind the GEMM dispatch ------------------------------------------------------------
+// Every choice between two GEMM kernels compares two estimates of the launch time in microseconds.  All constants
+// live here, each with the measurement that set it (one MI355X, 256 compute units, times from HIP events over
+// rotating operands; `rounds` = ceil(tiles / compute units), `row bytes` = K * element size).  They are fits to a
+// few points, good to about 10 %: near a crossover either kernel is within that of the other, so a box whose power
+// state moves the times by a few per cent picks differently without losing more than that.
+namespace tuning {
+// Tile loop against [N,K] operands (both panels through LDS), per round of 256 x 256 tiles: a fixed part plus the
+// K loop.  int8: M = 16, K = 4096, N = 11008 32.7 us; M = 1, K = N = 4096 27.6 us; M = 32, K = N = 8192 57.1 us
+// (8 + 0.006 * 4096 = 32.6, 8 + 0.006 * 8192 = 57.2).
+constexpr double kTileFixedUs = 8.0, kTileUsPerRowByte = 0.006;
+// Tile loop on fragment-order int8 weights (weights straight into registers), per round: M = 64 at (K, N) =
+// (4096, 4096) 21.0 us, (4096, 11008) 23.2 us, (8192, 8192) 38.4 us; never below streaming the weights at 4.5 TB/s
+// ((11008, 4096) 34.1 us for 45 MB + the fixed part).
+constexpr double kFragTileFixedUs = 5.0, kFragTileUsPerK = 0.004, kFragTileBytesPerUs = 4.5e6;
+// Wave-private kernels that read the weights once (gemm_core::rows32), up to 64 rows: a fixed part plus the weight
+// bytes at the rate the kernel streams them.  [N,K] int8 weights 3.4 TB/s (M = 16, K = 4096, N = 11008 13.0 us;
+// M = 32, K = N = 8192 18.2 us); f16 / bf16 / f32 [N,K] weights and fragment-order int8 weights 4.0 TB/s
+// (dense f16 M = 16, K = 4096, N = 11008 23.4 us; fragment order M = 64 (4096, 4096) 9.3 us, (11008, 4096) 17.1 us).
+constexpr double kRowsFixedUs = 3.0, kRowsBytesPerUs = 3.4e6, kRowsWideBytesPerUs = 4.0e6, kFragRowsFixedUs = 5.0;
+// The same kernels with four row tiles (65 to 128 rows): one workgroup per compute unit at a time, so rounds of 32-column
+// tiles, each the length of its K loop.  [N,K] operands 3.7 ns per row byte (int8 M = 128, K = N = 4096 18.4 us,
+// K = N = 8192 30.7 us); fragment-order weights 3.2 ns per k (16.1 us / 28.1 us at the same shapes).
+constexpr double kRows128FixedUs = 3.0, kRows128UsPerRowByte = 0.0037, kFragRows128UsPerK = 0.0032;
+// W4A16 tile choice: a full round of 256 x 256 tiles takes 3.25 times a full round of 128 x 128 tiles (for four times
+// the work), and a last round filled to a fraction f of the units takes 0.56 + 0.44 f^2 of a full one (fewer units
+// share the power budget).  Fitted over M = 48 ... 4096 at (K, N) = (4096, 4096), (4096, 11008), (11008, 4096),
+// (8192, 8192), (5120, 13824), (4096, 14336), (8192, 28672), (4096, 2048), 16 to 256 tiles in the last round; where
+// the rule changed the choice: K = N = 4096, M = 2048 83.6 -> 77.1 us; N = 11008, M = 1536 193.2 -> 175.0 us.
+constexpr double kW4BigRoundPerSmallRound = 3.25, kW4PartialRoundBase = 0.56, kW4PartialRoundSlope = 0.44;
+} // namespace tuning
+
 const char *float_name(int32_t dt) {
   switch (dt) {
   case MTRT_F32: return "f32";
@@ -806,12 +838,14 @@ int32_t mtrt_hip_gemm_w8a8(mtrt_stream_t stream, const void *a, const void *w_nk
     // 32.7 us against 13.4; M = 32, K = N = 8192 57.1 against 18.6; M = 1, K = N = 4096 27.6 against 11.2), so it
     // only wins on very large weights.  33 to 64 rows take the form with two activation row tiles per weight fragment.
     const double tile_rounds = double(((N + 255) / 256 + num_compute_units(st) - 1) / num_compute_units(st));
-    const double small_us = 3.0 + double(N) * double(K) / 3.4e6, tile_us = (8.0 + 0.006 * double(K)) * tile_rounds;
+    const double small_us = tuning::kRowsFixedUs + double(N) * double(K) / tuning::kRowsBytesPerUs;
+    const double tile_us = (tuning::kTileFixedUs + tuning::kTileUsPerRowByte * double(K)) * tile_rounds;
     // 65 to 128 rows: four row tiles per weight fragment, one workgroup of four waves per compute unit at a time, so
     // the launch runs in rounds of about 3.7 ns per k (M = 128, K = N = 4096: 33 -> 18.4 us; K = N = 8192: 57 -> 30.7;
     // N = 11008 needs two rounds and equals the tile launch)
     const int64_t tiles32 = (N + 31) / 32;
-    const double mid_us = 3.0 + 0.0037 * double(K) * double((tiles32 + num_compute_units(st) - 1) / num_compute_units(st));
+    const double mid_us = tuning::kRows128FixedUs + tuning::kRows128UsPerRowByte * double(K) *
+                                                        double((tiles32 + num_compute_units(st) - 1) / num_compute_units(st));
     if (M <= 64 ? small_us < tile_us : M <= 128 && mid_us < tile_us) {
       return launch(st, KernelName(M <= 32 ? "mtrt_gemm_w8a8_nk_rows32" : M <= 64 ? "mtrt_gemm_w8a8_nk_rows64" : "mtrt_gemm_w8a8_nk_rows128"),
                     uint32_t(std::min<int64_t>(tiles32, int64_t(kMaxGrid) * 1024)), M <= 64 ? 512 : 256, as_hip(stream), args);
@@ -898,8 +932,10 @@ int32_t mtrt_hip_gemm_w8a8_fragments(mtrt_stream_t stream, const void *a, const 
     // stays on the tiles at 23.9).
     const int64_t tiles32 = (N + 31) / 32, units = num_compute_units(st);
     const double weights = double(N) * double(K);
-    const double tile_us = std::max(5.0 + 0.004 * double(K), weights / 4.5e6) * double(((N + 255) / 256 + units - 1) / units);
-    const double rows_us = M <= 64 ? 5.0 + weights / 4.0e6 : 3.0 + 0.0032 * double(K) * double((tiles32 + units - 1) / units);
+    const double tile_us = std::max(tuning::kFragTileFixedUs + tuning::kFragTileUsPerK * double(K), weights / tuning::kFragTileBytesPerUs) *
+                           double(((N + 255) / 256 + units - 1) / units);
+    const double rows_us = M <= 64 ? tuning::kFragRowsFixedUs + weights / tuning::kRowsWideBytesPerUs
+                                   : tuning::kRows128FixedUs + tuning::kFragRows128UsPerK * double(K) * double((tiles32 + units - 1) / units);
     if (rows_us < tile_us) {
       void *rargs[] = {&a, &w_frag, &a_scale, &w_scale, &y, &M, &K, &N};
       return launch(st, KernelName(M <= 64 ? "mtrt_gemm_w8a8_frag_rows64" : "mtrt_gemm_w8a8_frag_rows128"),
@@ -968,12 +1004,14 @@ int32_t mtrt_hip_linear_dense(mtrt_stream_t stream, const void *x, const void *w
   // 473 -> 50 us); 33 to 64 rows the form with two activation row tiles per weight fragment; the tile loop (about
   // 8 us + 6 ns per byte of a row, per round) only wins on very large weights.
   const bool whole_slices = K > 0 && (K * eb) % 128 == 0 && aligned(x, 16) && aligned(w_nk, 16);
-  const double tile_us = (8.0 + 0.006 * double(K * eb)) * double(((N + 255) / 256 + num_compute_units(st) - 1) / num_compute_units(st));
-  const double small_us = 3.0 + double(N) * double(K * eb) / 4.0e6;
+  const double tile_us = (tuning::kTileFixedUs + tuning::kTileUsPerRowByte * double(K * eb)) *
+                         double(((N + 255) / 256 + num_compute_units(st) - 1) / num_compute_units(st));
+  const double small_us = tuning::kRowsFixedUs + double(N) * double(K * eb) / tuning::kRowsWideBytesPerUs;
   const int64_t tiles32 = (N + 31) / 32;
   // 65 to 128 rows: four row tiles per weight fragment, rounds of one workgroup per compute unit (3.7 ns per byte of a row);
   // f32 operands are bound by their matrix instructions there, which the tile loop is as well, at eight times the rows
-  const double mid_us = 3.0 + 0.0037 * double(K * eb) * double((tiles32 + num_compute_units(st) - 1) / num_compute_units(st));
+  const double mid_us = tuning::kRows128FixedUs + tuning::kRows128UsPerRowByte * double(K * eb) *
+                                                      double((tiles32 + num_compute_units(st) - 1) / num_compute_units(st));
   if (whole_slices && (M <= 64 ? small_us < tile_us : M <= 128 && (dtype == MTRT_F32 || mid_us < tile_us))) {
     void *rargs[] = {&x, &w_nk, &bias, &y, &M, &K, &N};
     return launch(st, KernelName(M <= 32 ? "mtrt_gemm_dense_rows32_" : M <= 64 ? "mtrt_gemm_dense_rows64_" : "mtrt_gemm_dense_rows128_") + xn,
@@ -1110,11 +1148,11 @@ int32_t mtrt_hip_gemm_w4a16(mtrt_stream_t stream, const void *a, const void *w_k
       const int64_t wide_panels = (N + 127) / 128, wide_m = (M + 127) / 128, wide_tiles = wide_panels * wide_m;
       auto rounds = [units](int64_t tiles) {
         const double f = double(tiles % units) / double(units);
-        return double(tiles / units) + (tiles % units ? 0.56 + 0.44 * f * f : 0.0);
+        return double(tiles / units) + (tiles % units ? tuning::kW4PartialRoundBase + tuning::kW4PartialRoundSlope * f * f : 0.0);
       };
       const int64_t big = 8 * ((panels + 7) / 8) * tiles_m, wide = 8 * ((wide_panels + 7) / 8) * wide_m;
       const int64_t narrow = 8 * ((((N + 63) / 64) + 7) / 8) * wide_m;
-      if (3.25 * rounds(big_tiles) < rounds(wide_tiles) && big <= int64_t(kMaxGrid) * 1024)
+      if (tuning::kW4BigRoundPerSmallRound * rounds(big_tiles) < rounds(wide_tiles) && big <= int64_t(kMaxGrid) * 1024)
         return launch(st, KernelName("mtrt_gemm_w4a16_t256x256"), uint32_t(big), 256, as_hip(stream), args);
       if (N <= 64 && narrow <= int64_t(kMaxGrid) * 1024)
         return launch(st, KernelName("mtrt_gemm_w4a16_t128x64"), uint32_t(narrow), kBlock, as_hip(stream), args);

@@ -268,7 +268,8 @@ def _run_w4a16(pkg, a, wp_host, s, K, N, B, prepack=True):
 
 
 kNoise = 1e-5        # f32 accumulation noise, in units of sqrt(K) * rms(a_row) * rms(wd_col)
-kMaxShare = 0.02     # largest share of outputs that may differ from the oracle's bits (by one f16 ulp)
+kMaxShare = 0.015    # largest share of outputs that may differ from the oracle's bits, by one f16 ulp (measured: at
+                     # most 0.61 %, 0.50 % at K = 4096: sums that land within the two orders' f32 difference of an f16 tie)
 
 
 def _ulp16(v):
@@ -287,6 +288,7 @@ def _check_w4a16(orc, y, a, w, s, K, N, B, ref_bits, max_share=kMaxShare):
         err = np.abs(got - target)
         assert np.all(err <= bound), "%s: worst excess %g at %s" % (name, (err - bound).max(), np.unravel_index(np.argmax(err - bound), err.shape))
     share = np.count_nonzero(got != ref) / got.size
+    print("w4a16: %d outputs, %.4f %% differ from the oracle's bits" % (got.size, 100.0 * share), flush=True)
     assert share <= max(max_share, 2.0 / got.size), "share of outputs that differ from the oracle: %g" % share
     return share
 
