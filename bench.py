@@ -504,8 +504,9 @@ def extra_clusters(pkg, torch, reps):
         return run
     out = []
     work = 3.0 * rows * d + 8.0 * rows
-    for what, make in (("mtrt_dynq_rows_f16_i8_v8 (one launch)", fused), ("mtrt_amax_rows_f16 + mtrt_q_row_f16_i8 (two launches)", two)):
+    for what, make in (("%s (one launch)", fused), ("mtrt_amax_rows_f16 + %s (two launches)", two)):
         us = time_kernel(pkg, torch, dict(make=make, nslots=ns), reps)
+        what = what % pkg.last_kernel()
         out.append(dict(kernel=what, config="per-token int8 quantization of C4's activations, f16 [2048, 4096]", bound="hbm",
                         us=round(us, 2), achieved=round(work / us / 1e3, 1), peak=HBM_PEAK, unit="GB/s",
                         frac=round(work / us / 1e3 / HBM_PEAK, 4), work=work))

@@ -100,7 +100,8 @@ __device__ __forceinline__ void body(const typename X::storage* __restrict__ x, 
     dynq_rows_cluster::body<XT, QT, NV, 4>(x, q, rows, d, qmax, amax_out, scale_out, flags); }
 #define MTRT_DYNQ_ROWS_KERNELS(XN, XT, QN, QT)                                                                            \
   MTRT_DYNQ_ROWS_WAVE(XN, XT, QN, QT, 1) MTRT_DYNQ_ROWS_WAVE(XN, XT, QN, QT, 2) MTRT_DYNQ_ROWS_WAVE(XN, XT, QN, QT, 4)     \
-  MTRT_DYNQ_ROWS_WAVE(XN, XT, QN, QT, 8) MTRT_DYNQ_ROWS_GROUP(XN, XT, QN, QT, 4) MTRT_DYNQ_ROWS_GROUP(XN, XT, QN, QT, 8)
+  MTRT_DYNQ_ROWS_WAVE(XN, XT, QN, QT, 8) MTRT_DYNQ_ROWS_GROUP(XN, XT, QN, QT, 1) MTRT_DYNQ_ROWS_GROUP(XN, XT, QN, QT, 2)  \
+  MTRT_DYNQ_ROWS_GROUP(XN, XT, QN, QT, 4) MTRT_DYNQ_ROWS_GROUP(XN, XT, QN, QT, 8)
 MTRT_DYNQ_ROWS_KERNELS(f32, F32, i8, I8)
 MTRT_DYNQ_ROWS_KERNELS(f32, F32, f8, F8)
 MTRT_DYNQ_ROWS_KERNELS(f16, F16, i8, I8)

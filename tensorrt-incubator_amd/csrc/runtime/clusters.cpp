@@ -594,7 +594,12 @@ int32_t mtrt_hip_dynamic_quantize_rows(mtrt_stream_t stream, const void *x, int3
   // 16-vector form would spill to scratch memory, whose allocation costs a launch some 10 us).
   const int max_group_nv = group == 8 && q_dtype == MTRT_F8E4M3FN ? 8 : 16;
   if (d % group == 0 && aligned(x, 16) && aligned(q, group) && nvec <= 256 * max_group_nv) {
-    const bool per_wave = nvec <= 64 * 8;
+    // A wave per row while that fills the chip (at least four waves per SIMD); with fewer rows the four waves of a
+    // workgroup share each row, which puts four times the waves on the same loads (f16 [2048, 4096] 8.5 -> 7.5 us,
+    // [4096, 4096] 12.7 -> 11.8 us; [8192, 4096] 22.7 against 23.4 us the other way).  Rows shorter than one vector
+    // per lane of a workgroup stay with the wave form.
+    const bool few_rows = rows <= int64_t(16) * num_compute_units(st) && nvec >= 256;
+    const bool per_wave = nvec <= 64 * 8 && !few_rows;
     const int64_t lanes = per_wave ? 64 : 256;
     int nv = 1;
     while (lanes * nv < nvec)

@@ -46,7 +46,8 @@ def test_c4_activations_full_size(pkg, orc):
     """The activations of BASELINE config 4 before quantization: f16 [2048, 4096], per-token int8 codes and scales."""
     x = (rng(4).standard_normal((2048, 4096), dtype=np.float32) * 3.0)
     orc.set_threads(16)
-    assert _check(pkg, orc, x, "f16", "i8", "mtrt_dynq_rows_f16_i8_v8") == "mtrt_dynq_rows_f16_i8_v8"
+    # (few enough rows that the four waves of a workgroup share each one)
+    assert _check(pkg, orc, x, "f16", "i8") in ("mtrt_dynq_rows_f16_i8_g4v2", "mtrt_dynq_rows_f16_i8_v8")
     orc.set_threads(1)
 
 
@@ -55,13 +56,15 @@ def test_c4_activations_full_size(pkg, orc):
 def test_type_pairs_and_row_lengths(pkg, orc, xname, qname):
     """One vector per row up to the longest row a wave holds, then the workgroup form up to its longest; row counts
     that leave the last workgroup of the wave form partly filled."""
+    import torch
     g = rng(sum(map(ord, xname + qname)))
     grp = 4 if xname == "f32" else 8
+    many = 16 * torch.cuda.get_device_properties(0).multi_processor_count + 3   # more rows than the workgroup form is used for
     k = "mtrt_dynq_rows_%s_%s_" % (xname, qname)
     orc.set_threads(16)
-    for rows, nvec, kernel in ((1, 1, "v1"), (5, 37, "v1"), (7, 64, "v1"), (6, 65, "v2"), (9, 200, "v4"), (3, 512, "v8"),
-                               (10, 1000, "g4v4"), (2, 1024, "g4v4"), (3, 1025, "g4v8"), (5, 300 * 4 + 7, "g4v8"),
-                               (2, 4096, "g4v16"), (131, 96, "v2")):
+    for rows, nvec, kernel in ((1, 1, "v1"), (5, 37, "v1"), (7, 64, "v1"), (6, 65, "v2"), (9, 200, "v4"), (3, 512, "g4v2"),
+                               (4, 256, "g4v1"), (10, 1000, "g4v4"), (2, 1024, "g4v4"), (3, 1025, "g4v8"), (5, 300 * 4 + 7, "g4v8"),
+                               (2, 4096, "g4v16"), (131, 96, "v2"), (many, 264, "v8"), (many + 1, 136, "v4")):
         x = (g.standard_normal((rows, nvec * grp)) * g.uniform(0.1, 30.0, (rows, 1))).astype(np.float32)
         if kernel == "g4v16" and grp == 8 and qname == "f8":
             # the 16-vector form of the 16-bit -> f8 pairs is not built (it would need scratch memory): two launches
