@@ -33,9 +33,9 @@
 // (SQ_LDS_BANK_CONFLICT reads 0 for these kernels).
 //
 // Tile order: the hardware deals consecutive workgroup ids round-robin to the 8 XCDs,
-// each with its own L2.  XCD x is given the N panels x, x+8, ... and walks down all M
-// tiles of a panel before the next, so a B panel is fetched into one L2 only.  The
-// grid is padded to 8 * ceil(panels / 8) * tiles_m; surplus workgroups leave at once.
+// each with its own L2.  Every XCD is given the same number of tiles, neighbours in an order
+// that keeps a B panel's M tiles together (tile_of_even); the grid is padded to a multiple
+// of 8, surplus workgroups leave at once.
 //
 // Epilogue: in a 32 x 32 accumulator tile lane l holds column (l & 31) and rows
 // 8*(r/4) + 4*(l >> 5) + (r % 4): 16 values in 16 different rows.  Each wave parks its
@@ -130,7 +130,6 @@ __device__ __forceinline__ void write_tile(Acc (&acc)[IT][JT], Epilogue& epi, ui
   static_assert(IT % 4 == 0, "waves cover whole groups of 128 rows");
   constexpr int WCOLS = 32 * JT;
   constexpr int HC = JT >= 2 ? 2 : 1;                  // column tiles staged at a time: 64 or 32 columns
-  constexpr int CHUNKS = HC * 4;                       // 16-byte chunks per staged row
   const int lane = threadIdx.x & 63;
   const int wm = slot / NWN, wn = slot % NWN;
   const int frow = lane & 31, fhalf = lane >> 5;
@@ -140,26 +139,29 @@ __device__ __forceinline__ void write_tile(Acc (&acc)[IT][JT], Epilogue& epi, ui
   if (!active) return;
   int8_t* out = lds + slot * kOutWave;
   const bool vec_ok = (N % 8 == 0) && ((reinterpret_cast<uintptr_t>(y) & 15) == 0);
-  // the whole tile of the workgroup lies inside y (rows of all SLOTS / NWN wave rows, columns of all NWN wave columns)
-  const bool inside = vec_ok && m0 + (SLOTS / NWN) * (32 * IT) <= M && n0 + NWN * WCOLS <= N;
-#pragma unroll
-  for (int ib = 0; ib < IT / 4; ++ib)
-#pragma unroll
-  for (int half = 0; half < JT / HC; ++half) {
+  // all rows of the workgroup's tile lie inside y (the rows of all SLOTS / NWN wave rows)
+  const bool rows_inside = vec_ok && m0 + (SLOTS / NWN) * (32 * IT) <= M;
+  // one pass: 128 rows (row group ib) x HCP column tiles starting at column tile jt0 of the wave
+  auto pass = [&](auto hcp, int ib, int jt0) {
+    constexpr int HCP = decltype(hcp)::value;
+    constexpr int CHUNKS = HCP * 4;                    // 16-byte chunks per staged row
     const int wrow = wm * (32 * IT) + ib * 128;         // first row of this pass inside the workgroup's tile
+    const int64_t pcol = n0 + wn * WCOLS + jt0 * 32;    // first column of this pass
+    if (pcol >= N) return;                             // a tile that hangs over the last column: nothing to store
+    const bool inside = rows_inside && pcol + 32 * HCP <= N;
     // what the epilogue needs per column (the same for every row of the pass) is fetched once, before the rows
-    epi.template columns<HC>(wn * WCOLS + half * (32 * HC) + fhalf * 4);
+    epi.template columns<HCP>(wn * WCOLS + jt0 * 32 + fhalf * 4);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int lrow = i * 32 + frow;
       epi.row(wrow + lrow);
 #pragma unroll
-      for (int jj = 0; jj < HC; ++jj)
+      for (int jj = 0; jj < HCP; ++jj)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const int lcol = jj * 32 + q * 8 + fhalf * 4;  // columns lcol .. lcol+3 of this group <-> r = 4q .. 4q+3
           uint32_t bits[4];
-          epi.convert4(acc[ib * 4 + i][half * HC + jj], q, jj, bits);
+          epi.convert4(acc[ib * 4 + i][jt0 + jj], q, jj, bits);
           u32x2 packed;
           packed[0] = bits[0] | (bits[1] << 16);
           packed[1] = bits[2] | (bits[3] << 16);
@@ -171,7 +173,7 @@ __device__ __forceinline__ void write_tile(Acc (&acc)[IT][JT], Epilogue& epi, ui
       // every row and column of the tile exists and whole vectors can be stored: no test per store, and the address
       // moves on by a constant (the general form below costs about ten branches and a 64-bit multiply per store)
       const int r0 = lane / CHUNKS, ch = lane % CHUNKS;
-      uint16_t* dst = y + (m0 + wrow + r0) * N + (n0 + wn * WCOLS + half * (32 * HC) + ch * 8);
+      uint16_t* dst = y + (m0 + wrow + r0) * N + (n0 + wn * WCOLS + jt0 * 32 + ch * 8);
       const int64_t step = int64_t(64 / CHUNKS) * N;
 #pragma unroll
       for (int it = 0; it < 128 * CHUNKS / 64; ++it) {
@@ -179,13 +181,13 @@ __device__ __forceinline__ void write_tile(Acc (&acc)[IT][JT], Epilogue& epi, ui
         __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dst));
         dst += step;
       }
-      continue;
+      return;
     }
 #pragma unroll
     for (int it = 0; it < 128 * CHUNKS / 64; ++it) {
       const int lrow = it * (64 / CHUNKS) + lane / CHUNKS, ch = lane % CHUNKS;
       const int64_t row = m0 + wrow + lrow;
-      const int64_t col = n0 + wn * WCOLS + half * (32 * HC) + ch * 8;
+      const int64_t col = n0 + wn * WCOLS + jt0 * 32 + ch * 8;
       const u32x4 v = *reinterpret_cast<const u32x4*>(out + lrow * kOutRow + ch * 16);
       if (row < M) {
         if (vec_ok) {
@@ -197,6 +199,12 @@ __device__ __forceinline__ void write_tile(Acc (&acc)[IT][JT], Epilogue& epi, ui
         }
       }
     }
+  };
+#pragma unroll
+  for (int ib = 0; ib < IT / 4; ++ib) {
+#pragma unroll
+    for (int half = 0; half < JT / HC; ++half) pass(IntC<HC>{}, ib, half * HC);
+    if constexpr (JT % HC != 0) pass(IntC<1>{}, ib, JT - 1);   // an odd tile left over: 32 columns
   }
 }
 
@@ -350,53 +358,44 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, const int8_t* 
   finish_tile<JT>(acc, epi, y, M, N, m0, n0, lds, wave);
 }
 
-// Tile order: the hardware deals consecutive workgroup ids round-robin to the 8 XCDs, each with
-// its own L2.  XCD x is given the N panels x, x+8, ... and walks down all M tiles of a panel
-// before the next, so a B panel is fetched into one L2 only.  A set of `panels` panels takes
-// padded_blocks(panels, tiles_m) ids; surplus ids get no tile.
-__device__ __host__ __forceinline__ int64_t padded_blocks(int64_t panels, int64_t tiles_m) { return 8 * ((panels + 7) / 8) * tiles_m; }
+// Tile order.  The hardware deals consecutive workgroup ids round-robin to the 8 XCDs, each with its own L2, so
+// workgroup id belongs to XCD id % 8.  All tiles are put in ONE order: M tiles in groups of `group`; inside a group the
+// panels one after the other, a panel's M tiles of the group next to each other.  An XCD's 32 units then work on
+// `group` M tiles x 32 / group panels at a time, and what its L2 has to fetch per K slice is group x (A panel slice)
+// + 32 / group x (B panel slice): the group size that minimises it depends on the bytes per row of the two operands
+// (for 4-bit weights under f16 activations a B slice is a quarter of an A slice, so few M tiles and many panels
+// re-read far less; group >= tiles_m walks down all M tiles of a panel before the next).
+// XCD x takes the tiles [x * per, (x + 1) * per) of that order, per = nblocks / 8 = ceil(tiles / 8): every XCD gets the
+// same number of tiles, give or take one.  Dealing whole panels to the XCDs (panel p to XCD p % 8: a panel is then
+// fetched into one L2 only) leaves some XCDs with a panel more than others, and on real data a launch lasts as long
+// as its busiest XCD, whose clock follows its load: W4A16 M = 4096 with 43 panels, XCDs with 96 and with 80 tiles,
+// 324 us; 86 each, 297 us (on zero operands the same either way).  A panel that straddles two XCDs' ranges is fetched
+// into two L2s.
+// nblocks = even_blocks(tiles): ids of this section of the grid (8 * per); surplus ids get no tile.
 // (Tile counts fit 32 bits: the index arithmetic is 32-bit on purpose.  As 64-bit divisions, which the hardware does
 // not have, it was some 500 scalar instructions, over a microsecond, in front of the first load of every workgroup.)
-__device__ __forceinline__ bool tile_of(int64_t id64, int64_t tiles_m64, int64_t panels64, int64_t& tile_m, int64_t& panel) {
-  const uint32_t id = uint32_t(id64), tiles_m = uint32_t(tiles_m64), panels = uint32_t(panels64);
-  const uint32_t xcd = id & 7, local = id >> 3;
-  const uint32_t q = local / tiles_m;
-  panel = q * 8 + xcd;
-  tile_m = local - q * tiles_m;
-  return q * 8 + xcd < panels;
-}
-// The same, with the M tiles walked in groups of `group` rows of tiles: an XCD's 32 units then
-// work on `group` M tiles x 32/group panels at a time instead of on all M tiles of a few panels.
-// What an XCD's L2 has to fetch per K slice is group x (A panel slice) + 32/group x (B panel
-// slice); the group size that minimises it depends on the bytes per row of the two operands
-// (for 4-bit weights under f16 activations a B slice is a quarter of an A slice, so few M tiles and
-// many panels re-read far less).  group >= tiles_m gives tile_of's order.
-__device__ __forceinline__ bool tile_of_grouped(int64_t id64, int64_t tiles_m64, int64_t panels64, int64_t group64, int64_t& tile_m,
-                                                int64_t& panel) {
-  const uint32_t id = uint32_t(id64), tiles_m = uint32_t(tiles_m64), panels = uint32_t(panels64), group = uint32_t(group64);
-  const uint32_t xcd = id & 7, local = id >> 3;
-  const uint32_t slots = (panels + 7) / 8;               // panel slots of one XCD
+__device__ __host__ __forceinline__ int64_t even_blocks(int64_t tiles) { return 8 * ((tiles + 7) / 8); }
+__device__ __forceinline__ bool tile_of_even(uint32_t id, uint32_t nblocks, int64_t tiles_m64, int64_t panels64, int64_t group64,
+                                             int64_t& tile_m, int64_t& panel) {
+  const uint32_t tiles_m = uint32_t(tiles_m64), panels = uint32_t(panels64);
+  const uint32_t group = uint32_t(group64) < tiles_m ? uint32_t(group64) : tiles_m;
+  const uint32_t per = nblocks >> 3;
+  const uint32_t at = (id & 7) * per + (id >> 3);
+  if (at >= tiles_m * panels) return false;
+  const uint32_t per_group = panels * group;
   const uint32_t full = tiles_m / group;                 // whole groups; a last group holds the remainder
-  const uint32_t per_group = slots * group;
-  uint32_t g = local / per_group, r, size;
+  uint32_t g = at / per_group, r, size;
   if (g < full) {
-    r = local - g * per_group;
+    r = at - g * per_group;
     size = group;
   } else {
     g = full;
-    r = local - full * per_group;
+    r = at - full * per_group;
     size = tiles_m - full * group;
   }
   const uint32_t q = r / size;
-  panel = q * 8 + xcd;
+  panel = q;
   tile_m = g * group + (r - q * size);
-  return q * 8 + xcd < panels;
-}
-__device__ __forceinline__ bool tile_origin(int64_t M, int64_t N, int64_t& m0, int64_t& n0) {
-  int64_t tile_m, panel;
-  if (!tile_of(blockIdx.x, (M + BM - 1) / BM, (N + BN - 1) / BN, tile_m, panel)) return false;
-  m0 = tile_m * BM;
-  n0 = panel * BN;
   return true;
 }
 

@@ -162,17 +162,19 @@ __device__ __forceinline__ void dense_mfma_body(const typename X::storage* __res
                                                 const typename X::storage* __restrict__ bias, uint16_t* __restrict__ y, int64_t M,
                                                 int64_t K, int64_t N, int64_t full_panels, int8_t* lds) {
   const int64_t tiles_m = (M + gemm_core::BM - 1) / gemm_core::BM;
-  const int64_t full_blocks = gemm_core::padded_blocks(full_panels, tiles_m);
+  const int64_t full_blocks = gemm_core::even_blocks(full_panels * tiles_m);
   BiasEpilogue<X> epi{bias, nullptr, {}};
   const int8_t* a8 = reinterpret_cast<const int8_t*>(x);
   const int8_t* w8 = reinterpret_cast<const int8_t*>(w);
   int64_t tile_m, panel;
   if (int64_t(blockIdx.x) < full_blocks) {
-    if (!gemm_core::tile_of(blockIdx.x, tiles_m, full_panels, tile_m, panel)) return;
+    if (!gemm_core::tile_of_even(blockIdx.x, uint32_t(full_blocks), tiles_m, full_panels, tiles_m, tile_m, panel)) return;
     gemm_core::run<HalfTraits<X>, 4>(a8, w8, K * 2, epi, y, M, N, K * 2 / gemm_core::BKB, tile_m * 256, panel * 256, lds);
   } else {
     const int64_t n_full = full_panels * 256;
-    if (!gemm_core::tile_of(blockIdx.x - full_blocks, tiles_m, (N - n_full + 127) / 128, tile_m, panel)) return;
+    if (!gemm_core::tile_of_even(blockIdx.x - uint32_t(full_blocks), gridDim.x - uint32_t(full_blocks), tiles_m, (N - n_full + 127) / 128,
+                                 tiles_m, tile_m, panel))
+      return;
     gemm_core::run<HalfTraits<X>, 2>(a8, w8, K * 2, epi, y, M, N, K * 2 / gemm_core::BKB, tile_m * 256, n_full + panel * 128, lds);
   }
 }
@@ -181,17 +183,19 @@ __device__ __forceinline__ void dense_mfma_f32_body(const float* __restrict__ x,
                                                     float* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t full_panels,
                                                     int8_t* lds) {
   const int64_t tiles_m = (M + gemm_core::BM - 1) / gemm_core::BM;
-  const int64_t full_blocks = gemm_core::padded_blocks(full_panels, tiles_m);
+  const int64_t full_blocks = gemm_core::even_blocks(full_panels * tiles_m);
   BiasF32Epilogue epi{bias};
   const int8_t* a8 = reinterpret_cast<const int8_t*>(x);
   const int8_t* w8 = reinterpret_cast<const int8_t*>(w);
   int64_t tile_m, panel;
   if (int64_t(blockIdx.x) < full_blocks) {
-    if (!gemm_core::tile_of(blockIdx.x, tiles_m, full_panels, tile_m, panel)) return;
+    if (!gemm_core::tile_of_even(blockIdx.x, uint32_t(full_blocks), tiles_m, full_panels, tiles_m, tile_m, panel)) return;
     gemm_core::run<F32Traits, 4>(a8, w8, K * 4, epi, y, M, N, K * 4 / gemm_core::BKB, tile_m * 256, panel * 256, lds);
   } else {
     const int64_t n_full = full_panels * 256;
-    if (!gemm_core::tile_of(blockIdx.x - full_blocks, tiles_m, (N - n_full + 127) / 128, tile_m, panel)) return;
+    if (!gemm_core::tile_of_even(blockIdx.x - uint32_t(full_blocks), gridDim.x - uint32_t(full_blocks), tiles_m, (N - n_full + 127) / 128,
+                                 tiles_m, tile_m, panel))
+      return;
     gemm_core::run<F32Traits, 2>(a8, w8, K * 4, epi, y, M, N, K * 4 / gemm_core::BKB, tile_m * 256, n_full + panel * 128, lds);
   }
 }

@@ -403,8 +403,8 @@ __device__ __forceinline__ void weight_regs_kernel(const uint16_t* __restrict__ 
                                                    int64_t K, int64_t N, int64_t block, int8_t* lds) {
   int64_t tile_m, panel;
   // A slice of a 4-bit weight panel is a quarter of the bytes of an activation panel slice of the same
-  // width: groups of four M tiles, eight panels at a time per XCD
-  if (!gemm_core::tile_of_grouped(blockIdx.x, (M + S::kBM - 1) / S::kBM, (N + S::kBN - 1) / S::kBN, 4, tile_m, panel)) return;
+  // width: groups of four M tiles, eight panels at a time per XCD; every XCD the same number of tiles
+  if (!gemm_core::tile_of_even(blockIdx.x, gridDim.x, (M + S::kBM - 1) / S::kBM, (N + S::kBN - 1) / S::kBN, 4, tile_m, panel)) return;
   const int64_t m0 = tile_m * S::kBM, n0 = panel * S::kBN;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int slot = wave % S::kSlots;
@@ -418,7 +418,7 @@ __device__ __forceinline__ void weight_regs_kernel(const uint16_t* __restrict__ 
 }
 
 // (a [M,K] f16, w_prepacked, scale [K/block, N] f16, y [M,N] f16, M, K, N, block) ; K % 64 == 0, block % 64 == 0,
-// a 16-byte aligned and below 4 GiB.  grid = 8 * ceil(ceil(N/256) / 8) * ceil(M/256), block = 256.
+// a 16-byte aligned and below 4 GiB.  grid = 8 * ceil(ceil(N/256) * ceil(M/256) / 8), block = 256.
 // Four waves, each a whole 256-row column of the tile (256 x 64, one wave per SIMD, 256 accumulator registers):
 // a weight fragment is dequantised once per workgroup and a wave issues 16 MFMAs per k-step.  Against eight
 // waves of 128 x 64 (every weight fragment dequantised by two waves) in one process: 343 -> 330 us at
@@ -431,7 +431,7 @@ extern "C" __global__ void __launch_bounds__(256, 1) mtrt_gemm_w4a16_t256x256(
   weight_regs_kernel<BigShape>(a, wp, scale, y, M, K, N, block, lds);
 }
 // Medium M: 128 x 64 tiles so that the grid still fills the chip, two wave sets splitting each slice.
-// Same argument list.  grid = 8 * ceil(ceil(N/64) / 8) * ceil(M/128), block = 256.
+// Same argument list.  grid = 8 * ceil(ceil(N/64) * ceil(M/128) / 8), block = 256.
 using MidShape = Shape<1, 2, 1, 2, 4, 5>;              // 128 x 64, 4 waves, four slices ahead (two workgroups share a CU's LDS)
 extern "C" __global__ void __launch_bounds__(256) mtrt_gemm_w4a16_t128x64(
     const uint16_t* __restrict__ a, const uint32_t* __restrict__ wp, const uint16_t* __restrict__ scale,

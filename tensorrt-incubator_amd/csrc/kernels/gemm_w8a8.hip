@@ -31,19 +31,19 @@ struct I8Traits {
   static __device__ __forceinline__ Acc mfma(v4i a, v4i b, Acc c) { return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0); }
 };
 
-struct ScaleEpilogue {
+// BN: columns of the workgroup's tile (the scratch holds 256 + BN floats)
+template <int BN>
+struct ScaleEpilogueT {
   const float* a_scale;
   const float* w_scale;
   const float* sa;                                   // a_scale of this tile's 256 rows, in LDS
-  const float* sw;                                   // w_scale of this tile's 256 columns, in LDS
+  const float* sw;                                   // w_scale of this tile's BN columns, in LDS
   float as;
   __device__ __forceinline__ void setup(int8_t* scratch, int64_t m0, int64_t M, int64_t n0, int64_t N) {
     float* dst = reinterpret_cast<float*>(scratch);
-    const int64_t row = m0 + threadIdx.x, col = n0 + threadIdx.x;   // the first 256 threads: 256 rows, 256 columns
-    if (threadIdx.x < 256) {
-      dst[threadIdx.x] = row < M ? a_scale[row] : 0.0f;
-      dst[256 + threadIdx.x] = col < N ? w_scale[col] : 0.0f;
-    }
+    const int64_t row = m0 + threadIdx.x;              // the first 256 threads: 256 rows
+    if (threadIdx.x < 256) dst[threadIdx.x] = row < M ? a_scale[row] : 0.0f;
+    for (int c = threadIdx.x; c < BN; c += blockDim.x) dst[256 + c] = n0 + c < N ? w_scale[n0 + c] : 0.0f;
     sa = dst;
     sw = dst + 256;
   }
@@ -63,6 +63,7 @@ struct ScaleEpilogue {
   }
   f32x4 wsr[2][4];
 };
+using ScaleEpilogue = ScaleEpilogueT<256>;
 
 // The entry points below have C linkage; they sit inside the namespace only so that
 // its helper names do not meet those of the other clusters in the one-module build.
@@ -71,21 +72,24 @@ struct ScaleEpilogue {
 // a and w_nk 16-byte aligned, both below 4 GiB.  The first full_panels * 256 columns are computed in
 // 256 x 256 tiles, the rest in 256 x 128 tiles: with one workgroup per compute unit a launch runs in
 // rounds, and a last round that would use few of the units is cut into twice as many tiles of half
-// the length.  grid = padded_blocks(full_panels, tiles_m) + padded_blocks(half panels, tiles_m), block = 256.
+// the length.  grid = even_blocks(full_panels * tiles_m) + even_blocks(half panels * tiles_m), block = 256 (each kind
+// of tile dealt evenly to the XCDs, gemm_core::tile_of_even).
 extern "C" __global__ void __launch_bounds__(gemm_core::THREADS, 1) mtrt_gemm_w8a8_nk(
     const int8_t* __restrict__ a, const int8_t* __restrict__ w, const float* __restrict__ a_scale,
     const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t full_panels) {
   __shared__ __attribute__((aligned(16))) int8_t lds[gemm_core::LDS_BYTES];
   const int64_t tiles_m = (M + gemm_core::BM - 1) / gemm_core::BM;
-  const int64_t full_blocks = gemm_core::padded_blocks(full_panels, tiles_m);
+  const int64_t full_blocks = gemm_core::even_blocks(full_panels * tiles_m);
   ScaleEpilogue epi{a_scale, w_scale, nullptr, nullptr, 0.0f, {}};
   int64_t tile_m, panel;
   if (int64_t(blockIdx.x) < full_blocks) {
-    if (!gemm_core::tile_of(blockIdx.x, tiles_m, full_panels, tile_m, panel)) return;
+    if (!gemm_core::tile_of_even(blockIdx.x, uint32_t(full_blocks), tiles_m, full_panels, tiles_m, tile_m, panel)) return;
     gemm_core::run<I8Traits, 4>(a, w, K, epi, y, M, N, K / gemm_core::BKB, tile_m * 256, panel * 256, lds);
   } else {
     const int64_t n_full = full_panels * 256;
-    if (!gemm_core::tile_of(blockIdx.x - full_blocks, tiles_m, (N - n_full + 127) / 128, tile_m, panel)) return;
+    if (!gemm_core::tile_of_even(blockIdx.x - uint32_t(full_blocks), gridDim.x - uint32_t(full_blocks), tiles_m, (N - n_full + 127) / 128,
+                                 tiles_m, tile_m, panel))
+      return;
     gemm_core::run<I8Traits, 2>(a, w, K, epi, y, M, N, K / gemm_core::BKB, tile_m * 256, n_full + panel * 128, lds);
   }
 }
@@ -280,6 +284,164 @@ __device__ __forceinline__ void run(const int8_t* __restrict__ a, int64_t a_row_
   write_tile<JT, kNWN, kWaves>(acc, epi, y, M, N, m0, n0, lds, slot, true);
 }
 
+
+// ---- 256 x 384 tiles: four waves of 256 x 96 -------------------------------------------------------------
+// The widest tile the register file holds: 384 accumulator registers per lane.  Every wave owns all 256 rows of 96
+// columns, so each weight fragment is loaded by ONE wave (the 2 x 2 waves above load each twice) and a workgroup
+// moves 80 KiB per slice for 384 MFMAs where the 256 x 256 tile moves 96 KiB for 256: on zero operands the loop runs at
+// 95 % of its MFMA time.  What it takes:
+//   * With one wave per SIMD the compiler gives the matrix instructions accumulation registers only, 256 per lane.
+//     The third column tile's accumulators therefore live in ordinary vector registers, through MFMAs written as
+//     instructions (the compiler does not see inside: s_nops in front of the epilogue let the matrix cores finish).
+//   * That leaves about 120 vector registers for everything else.  Activation fragments are read HALF a k-step
+//     ahead (two sets of four: chunks 0..3 of a k-step read its row tiles 4..7, chunks 4..7 row tiles 0..3 of the
+//     next k-step); the weights of a k-step (3 x 16 bytes per lane) sit in a ring of four k-steps and are asked for
+//     again as soon as the k-step is over, three k-steps before their next use.
+//   * Memory instructions are issued in a fixed order per k-step (chunk 0: activations, chunks 1..3: weights,
+//     chunk 4: activations) and waited for by count: when a k-step starts, eleven have been issued since its weights
+//     were asked for; the activations of slice s+1 were asked for during slice s-1 and have landed by the same count
+//     in front of k-step 3, where the workgroup meets.
+// Measured against mtrt_gemm_w8a8_frag in one process at M = 2048, K = 4096, N = 11008 (232 tiles, one round, against
+// 1.5 rounds of the smaller tile): 83.5 -> 77.9 us on the benchmark's data, 64.0 -> 58.1 us on zeros, same bits.
+constexpr int kWideBN = 384;
+constexpr int kWideOut = 4 * gemm_core::kOutWave + (256 + kWideBN) * 4;
+constexpr int kWideLds = kWideOut > 4 * kStageBytes ? kWideOut : 4 * kStageBytes;
+
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(gemm_core::IntC<I>{});
+    static_for<I + 1, N>(f);
+  }
+}
+// 16 bytes per lane of k-step T of a weight slice: scalar base, 32-bit lane offset, the k-step as the instruction's offset
+template <int T>
+__device__ __forceinline__ void load_w(v4i& dst, uint32_t lane_off, const int8_t* base) {
+  __asm__ volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "=v"(dst) : "v"(lane_off), "s"(base), "n"(T * 1024) : "memory");
+}
+
+template <class Epilogue>
+__device__ __forceinline__ void run_wide(const int8_t* __restrict__ a, int64_t a_row_bytes, const v4i* __restrict__ wfrag,
+                                         int64_t ntiles, Epilogue& epi, uint16_t* __restrict__ y, int64_t M, int64_t N,
+                                         int64_t slices, int64_t m0, int64_t n0, int8_t* lds) {
+  using namespace gemm_core;
+  constexpr int IT = 8, JT = 3, AN = 4, kG = 8;
+  constexpr int JA = 2;                                // column tiles whose accumulators the compiler places
+  constexpr int kFly = 11;                             // memory instructions issued since a k-step's weights were asked for
+  const int lane = threadIdx.x & 63;
+  const int slot = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // = the wave's column: 1 x 4 waves
+  const int frow = lane & 31, fhalf = lane >> 5;
+
+  v16i acc[IT][JT];
+  const uint32_t nslices = uint32_t(slices), last = nslices - 1;
+  DmaLoaderT<kG> al;
+  al.init(a, M, a_row_bytes, m0);
+  v4i fa[2][AN];
+  v4i wr[4][JT];
+  const int8_t* wsrc[JT];                              // slice 0 of each column tile (uniform)
+  uint32_t wlane = uint32_t(lane) * 16;
+#pragma unroll
+  for (int j = 0; j < JT; ++j) {
+    int64_t tile = n0 / 32 + slot * JT + j;
+    tile = tile < ntiles ? tile : ntiles - 1;          // tiles past N: some valid data, never stored
+    wsrc[j] = reinterpret_cast<const int8_t*>(wfrag + tile * slices * 256);
+  }
+  auto fetch_w = [&](auto tt, v4i& dst, int j, uint32_t slice) {
+    load_w<decltype(tt)::value>(dst, wlane, wsrc[j] + uint64_t(slice) * 4096);
+  };
+  const uint32_t lds_base = uint32_t(uintptr_t((lds_void_t*)lds));
+  uint32_t a_lane[4];
+#pragma unroll
+  for (int p = 0; p < 4; ++p) a_lane[p] = lds_base + uint32_t(lds_off(frow, 2 * p + fhalf));
+  auto read_a = [&](v4i& dst, uint32_t addr, auto tile) {
+    constexpr int I = decltype(tile)::value;
+    __asm__ volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(I * 4096) : "memory");
+  };
+  // the reads form one stream, four chunks ahead of their use: three younger ones may be outstanding
+  auto landed_a = [&](v4i& frag) { __asm__ volatile("s_waitcnt lgkmcnt(3)" : "+v"(frag)::"memory"); };
+  auto stage_off = [&](uint32_t slice) { return uint32_t(slice & 3) * uint32_t(kStageBytes); };
+  auto stage = [&](uint32_t slice) { return lds + stage_off(slice); };
+  auto at_most_last = [&](uint32_t slice) { return slice - ((uint32_t(last - slice) >> 31) * (slice - last)); };  // scalar min
+
+  // slice 0 and its weights for k-steps 0..2 (k-step 3's are asked for in k-step 0, like every slice's), then slice 1
+  const uint32_t one = at_most_last(1);
+#pragma unroll
+  for (int g = 0; g < kG; ++g) al.dma_at(al.slice_base(0), stage(0), g);
+  static_for<0, 3>([&](auto t) {
+    constexpr int T = decltype(t)::value;
+#pragma unroll
+    for (int j = 0; j < JT; ++j) fetch_w(t, wr[T][j], j, 0);
+  });
+#pragma unroll
+  for (int g = 0; g < kG; ++g) al.dma_at(al.slice_base(one), stage(1), g);
+  __builtin_amdgcn_sched_barrier(0);
+  {                                                    // accumulators cleared by the matrix cores under those loads
+    v4i none = {0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < IT; ++i)
+#pragma unroll
+      for (int j = 0; j < JT; ++j) {
+        __asm__ volatile("" : "+v"(none));
+        if (j < JA) acc[i][j] = I8Traits::mfma(none, none, I8Traits::zero());
+        else __asm__ volatile("v_mfma_i32_32x32x32_i8 %0, %1, %1, 0" : "=v"(acc[i][j]) : "v"(none));
+      }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+#pragma unroll
+  for (int t = 0; t < 3; ++t) __asm__ volatile("s_waitcnt vmcnt(0)" : "+v"(wr[t][0]), "+v"(wr[t][1]), "+v"(wr[t][2])::"memory");
+  drain_and_barrier();
+  static_for<0, AN>([&](auto i) { read_a(fa[0][decltype(i)::value], a_lane[0] + stage_off(0), i); });
+
+  // k-step T of slice s0 (the next slice: s1): eight fenced chunks; chunk c multiplies row tile c by the three weight
+  // fragments of the k-step.  ca: LDS offset of the stage this k-step reads, ra: of the stage the next k-step reads.
+  auto kstep = [&](auto step, uint32_t ca, uint32_t ra, uint32_t s0, uint32_t s1, const int8_t* src, int8_t* nd) {
+    constexpr int T = decltype(step)::value;
+    const uint32_t raddr = a_lane[(T + 1) & 3] + ra, caddr = a_lane[T] + ca;
+    __asm__ volatile("s_waitcnt vmcnt(%3)" : "+v"(wr[T][0]), "+v"(wr[T][1]), "+v"(wr[T][2]) : "n"(kFly) : "memory");
+    static_for<0, IT>([&](auto cc) {
+      constexpr int c = decltype(cc)::value;
+      constexpr int ASET = c / AN, AI = c % AN;
+      landed_a(fa[ASET][AI]);
+#pragma unroll
+      for (int j = 0; j < JT; ++j) {
+        if (j < JA) acc[c][j] = I8Traits::mfma(wr[T][j], fa[ASET][AI], acc[c][j]);
+        else __asm__ volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+v"(acc[c][j]) : "v"(wr[T][j]), "v"(fa[ASET][AI]));
+      }
+      if constexpr (c < AN) read_a(fa[1][c], caddr, IntC<c + AN>{});           // row tile c + 4 of this k-step
+      else read_a(fa[0][c - AN], raddr, IntC<c - AN>{});                       // row tile c - 4 of the next
+      if constexpr (c == 0) al.dma_at(src, nd, 2 * T);
+      if constexpr (c == 4) al.dma_at(src, nd, 2 * T + 1);
+      if constexpr (c >= 1 && c <= 3) {                // the registers of the k-step before this one, for their next use
+        if constexpr (T == 0) fetch_w(IntC<3>{}, wr[3][c - 1], c - 1, s0);
+        else fetch_w(IntC<T - 1>{}, wr[T - 1][c - 1], c - 1, s1);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+  for (uint32_t s = 0; s < nslices; ++s) {
+    const uint32_t pa = stage_off(s);
+    const uint32_t s1 = at_most_last(s + 1), s2 = at_most_last(s + 2);
+    const int8_t* src = al.slice_base(s2);             // the slice fetched during this one (past the end: the last again,
+    int8_t* nd = stage(s + 2);                         //  into a stage nobody reads)
+    kstep(IntC<0>{}, pa, pa, s, s1, src, nd);
+    kstep(IntC<1>{}, pa, pa, s, s1, src, nd);
+    kstep(IntC<2>{}, pa, pa, s, s1, src, nd);
+    // the activations of slice s+1 have landed (fifteen memory instructions were issued since the last of them); the
+    // fragment reads in flight belong to stages that are not written before the next barrier but one
+    __asm__ volatile("s_waitcnt vmcnt(%0)" ::"n"(kFly) : "memory");
+    __asm__ volatile("s_barrier" ::: "memory");
+    kstep(IntC<3>{}, pa, stage_off(s + 1), s, s1, src, nd);
+  }
+  __builtin_amdgcn_s_waitcnt(0x0070);                  // the surplus loads and fragment reads have landed: their
+#pragma unroll                                         // registers stay allocated up to here
+  for (int i = 0; i < AN; ++i) __asm__ volatile("s_waitcnt lgkmcnt(0)" ::"v"(fa[0][i]), "v"(fa[1][i]) : "memory");
+#pragma unroll
+  for (int t = 0; t < 4; ++t) __asm__ volatile("s_waitcnt vmcnt(0)" ::"v"(wr[t][0]), "v"(wr[t][1]), "v"(wr[t][2]) : "memory");
+  __asm__ volatile("s_nop 15\n\ts_nop 15" ::: "memory");   // the matrix cores are done with the accumulators in vector registers
+
+  write_tile<JT, 4, 4>(acc, epi, y, M, N, m0, n0, lds, slot, true);
+}
+
 }  // namespace frag
 
 // (a [M,K] i8, w_frag (fragment order), a_scale [M] f32, w_scale [N] f32, y [M,N] f16, M, K, N, full_panels) ;
@@ -291,15 +453,17 @@ __device__ __forceinline__ void frag_kernel(const int8_t* __restrict__ a, const 
                                             int64_t full_panels, int8_t* lds) {
   constexpr int JT = 8 / NWN;                          // column tiles per wave in a full tile; half of it in a half tile
   const int64_t tiles_m = (M + 255) / 256, ntiles = (N + 31) / 32;
-  const int64_t full_blocks = gemm_core::padded_blocks(full_panels, tiles_m);
+  const int64_t full_blocks = gemm_core::even_blocks(full_panels * tiles_m);
   ScaleEpilogue epi{a_scale, w_scale, nullptr, nullptr, 0.0f, {}};
   int64_t tile_m, panel;
   if (int64_t(blockIdx.x) < full_blocks) {
-    if (!gemm_core::tile_of(blockIdx.x, tiles_m, full_panels, tile_m, panel)) return;
+    if (!gemm_core::tile_of_even(blockIdx.x, uint32_t(full_blocks), tiles_m, full_panels, tiles_m, tile_m, panel)) return;
     frag::run<NWN, JT>(a, K, w_frag, ntiles, epi, y, M, N, K / 128, tile_m * 256, panel * 256, lds);
   } else {
     const int64_t n_full = full_panels * 256;
-    if (!gemm_core::tile_of(blockIdx.x - full_blocks, tiles_m, (N - n_full + 127) / 128, tile_m, panel)) return;
+    if (!gemm_core::tile_of_even(blockIdx.x - uint32_t(full_blocks), gridDim.x - uint32_t(full_blocks), tiles_m, (N - n_full + 127) / 128,
+                                 tiles_m, tile_m, panel))
+      return;
     frag::run<NWN, JT / 2>(a, K, w_frag, ntiles, epi, y, M, N, K / 128, tile_m * 256, n_full + panel * 128, lds);
   }
 }
@@ -309,6 +473,18 @@ extern "C" __global__ void __launch_bounds__(frag::Waves<2>::kThreads, 1) mtrt_g
     const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t full_panels) {
   __shared__ __attribute__((aligned(16))) int8_t lds[frag::Waves<2>::kLds];
   frag_kernel<2>(a, w_frag, a_scale, w_scale, y, M, K, N, full_panels, lds);
+}
+// 256 x 384 tiles (frag::run_wide).  (a, w_frag, a_scale, w_scale, y, M, K, N) as above.
+// grid = 8 * ceil(ceil(M/256) * ceil(N/384) / 8), block = 256: the tiles dealt evenly to the XCDs, a panel's M tiles neighbours.
+extern "C" __global__ void __launch_bounds__(256, 1) mtrt_gemm_w8a8_frag_t256x384(
+    const int8_t* __restrict__ a, const v4i* __restrict__ w_frag, const float* __restrict__ a_scale,
+    const float* __restrict__ w_scale, uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N) {
+  __shared__ __attribute__((aligned(16))) int8_t lds[frag::kWideLds];
+  const int64_t tiles_m = (M + 255) / 256, ntiles = (N + 31) / 32, panels = (N + frag::kWideBN - 1) / frag::kWideBN;
+  ScaleEpilogueT<frag::kWideBN> epi{a_scale, w_scale, nullptr, nullptr, 0.0f, {}};
+  int64_t tile_m, panel;
+  if (!gemm_core::tile_of_even(blockIdx.x, gridDim.x, tiles_m, panels, tiles_m, tile_m, panel)) return;
+  frag::run_wide(a, K, w_frag, ntiles, epi, y, M, N, K / 128, tile_m * 256, panel * frag::kWideBN, lds);
 }
 // Weight re-layout into fragment order, from [K,N] (nk = 0) or [N,K] (nk = 1).  One 16-byte chunk per
 // thread.  (w, w_frag, K, N, nk) ; K % 128 == 0 ; w_frag holds 32 * ceil(N/32) * K bytes.

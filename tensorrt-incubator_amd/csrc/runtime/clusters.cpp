@@ -54,6 +54,10 @@ constexpr double kRows128FixedUs = 3.0, kRows128UsPerRowByte = 0.0037, kFragRows
 // (8192, 8192), (5120, 13824), (4096, 14336), (8192, 28672), (4096, 2048), 16 to 256 tiles in the last round; where
 // the rule changed the choice: K = N = 4096, M = 2048 83.6 -> 77.1 us; N = 11008, M = 1536 193.2 -> 175.0 us.
 constexpr double kW4BigRoundPerSmallRound = 3.25, kW4PartialRoundBase = 0.56, kW4PartialRoundSlope = 0.44;
+// W8A8 on fragment-order weights: a round of 256 x 384 tiles, in rounds of 256 x 256 tiles.  One and a half times the
+// MFMAs at 0.93 of the time per MFMA (M = 2048, K = 4096, N = 11008: 232 wide tiles in one round 77.9 us, 344 tiles
+// in one and a half rounds 83.5 us, interleaved in one process on the benchmark's data).
+constexpr double kW8WideRoundPerRound = 1.5 * 0.93;
 } // namespace tuning
 
 const char *float_name(int32_t dt) {
@@ -867,7 +871,7 @@ int32_t mtrt_hip_gemm_w8a8(mtrt_stream_t stream, const void *a, const void *w_nk
     else if (rest > 0 && rest * 2 <= units)
       full_panels = panels - (rest + tiles_m - 1) / tiles_m;
     const int64_t half_panels = (N - full_panels * 256 + 127) / 128;
-    const int64_t grid = 8 * ((full_panels + 7) / 8) * tiles_m + 8 * ((half_panels + 7) / 8) * tiles_m;
+    const int64_t grid = 8 * ((full_panels * tiles_m + 7) / 8) + 8 * ((half_panels * tiles_m + 7) / 8);   // each kind dealt evenly to the XCDs
     if (grid <= int64_t(kMaxGrid) * 1024) {
       void *fast_args[] = {&a, &w_nk, &a_scale, &w_scale, &y, &M, &K, &N, &full_panels};
       return launch(st, KernelName("mtrt_gemm_w8a8_nk"), uint32_t(grid), kBlock, as_hip(stream), fast_args);
@@ -969,13 +973,25 @@ int32_t mtrt_hip_gemm_w8a8_fragments(mtrt_stream_t stream, const void *a, const 
   // a last round that would use at most half of the units is cut into 128-wide half tiles.
   const int64_t panels = (N + 255) / 256, tiles_m = (M + 255) / 256, units = num_compute_units(st);
   const int64_t tiles = panels * tiles_m, rest = tiles % units;
+  {
+    // ... or 256 x 384 tiles (fewer bytes moved per MFMA, every weight fragment loaded once per workgroup) where their
+    // rounds come out shorter
+    const double rounds = tiles * 2 <= units ? 0.5 : double(tiles / units) + (rest == 0 ? 0.0 : rest * 2 <= units ? 0.5 : 1.0);
+    const int64_t wide_tiles = ((N + 383) / 384) * tiles_m;
+    const double wide_rounds = tuning::kW8WideRoundPerRound * double((wide_tiles + units - 1) / units);
+    const int64_t wide_grid = 8 * ((wide_tiles + 7) / 8);
+    if (wide_rounds < rounds && wide_grid <= int64_t(kMaxGrid) * 1024) {
+      void *wargs[] = {&a, &w_frag, &a_scale, &w_scale, &y, &M, &K, &N};
+      return launch(st, KernelName("mtrt_gemm_w8a8_frag_t256x384"), uint32_t(wide_grid), 256, as_hip(stream), wargs);
+    }
+  }
   int64_t full_panels = panels;
   if (tiles * 2 <= units)
     full_panels = 0;
   else if (rest > 0 && rest * 2 <= units)
     full_panels = panels - (rest + tiles_m - 1) / tiles_m;
   const int64_t half_panels = (N - full_panels * 256 + 127) / 128;
-  const int64_t grid = 8 * ((full_panels + 7) / 8) * tiles_m + 8 * ((half_panels + 7) / 8) * tiles_m;
+  const int64_t grid = 8 * ((full_panels * tiles_m + 7) / 8) + 8 * ((half_panels * tiles_m + 7) / 8);   // each kind dealt evenly to the XCDs
   if (grid > int64_t(kMaxGrid) * 1024)
     return set_error(MTRT_INVALID_ARGUMENT, "problem [%lld, %lld] needs too many tiles", (long long)M, (long long)N);
   void *args[] = {&a, &w_frag, &a_scale, &w_scale, &y, &M, &K, &N, &full_panels};
@@ -1034,7 +1050,7 @@ int32_t mtrt_hip_linear_dense(mtrt_stream_t stream, const void *x, const void *w
     else if (rest > 0 && rest * 2 <= units)
       full_panels = panels - (rest + tiles_m - 1) / tiles_m;
     const int64_t half_panels = (N - full_panels * 256 + 127) / 128;
-    const int64_t grid = 8 * ((full_panels + 7) / 8) * tiles_m + 8 * ((half_panels + 7) / 8) * tiles_m;
+    const int64_t grid = 8 * ((full_panels * tiles_m + 7) / 8) + 8 * ((half_panels * tiles_m + 7) / 8);   // each kind dealt evenly to the XCDs
     if (grid <= int64_t(kMaxGrid) * 1024) {
       void *margs[] = {&x, &w_nk, &bias, &y, &M, &K, &N, &full_panels};
       return launch(st, KernelName("mtrt_gemm_dense_mfma_") + xn, uint32_t(grid), kBlock, as_hip(stream), margs);
@@ -1155,8 +1171,9 @@ int32_t mtrt_hip_gemm_w4a16(mtrt_stream_t stream, const void *a, const void *w_k
         const double f = double(tiles % units) / double(units);
         return double(tiles / units) + (tiles % units ? tuning::kW4PartialRoundBase + tuning::kW4PartialRoundSlope * f * f : 0.0);
       };
-      const int64_t big = 8 * ((panels + 7) / 8) * tiles_m, wide = 8 * ((wide_panels + 7) / 8) * wide_m;
-      const int64_t narrow = 8 * ((((N + 63) / 64) + 7) / 8) * wide_m;
+      // (grids: the tiles dealt evenly to the eight XCDs, gemm_core::tile_of_even)
+      const int64_t big = 8 * ((big_tiles + 7) / 8), wide = 8 * ((wide_tiles + 7) / 8);
+      const int64_t narrow = 8 * ((((N + 63) / 64) * wide_m + 7) / 8);
       if (tuning::kW4BigRoundPerSmallRound * rounds(big_tiles) < rounds(wide_tiles) && big <= int64_t(kMaxGrid) * 1024)
         return launch(st, KernelName("mtrt_gemm_w4a16_t256x256"), uint32_t(big), 256, as_hip(stream), args);
       if (N <= 64 && narrow <= int64_t(kMaxGrid) * 1024)

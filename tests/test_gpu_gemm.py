@@ -93,7 +93,7 @@ def _frag_small_ok(kernel, M):
 
 # the tile kernels on fragment-order weights (one launch in rounds of tiles, or one workgroup per compute unit walking
 # its share of the columns)
-_FRAG_TILE = {"mtrt_gemm_w8a8_frag", "mtrt_gemm_w8a8_frag_strips"}
+_FRAG_TILE = {"mtrt_gemm_w8a8_frag", "mtrt_gemm_w8a8_frag_t256x384"}
 
 
 def _run_w8a8_frag(pkg, a, w, a_s, w_s, from_nk=False):
@@ -235,6 +235,63 @@ def test_c4_w8a8_full_size(pkg, orc):
     y2, kernel2 = _run_w8a8_frag(pkg, a, w, a_s, w_s)
     assert kernel2 in _FRAG_TILE
     assert torch.equal(y2, expect)
+
+
+def _launch_wide_w8a8(pkg, a, w, a_s, w_s):
+    """mtrt_gemm_w8a8_frag_t256x384 launched by hand from the built-in module (the entry point takes it only where its
+    rounds come out shorter), with the grid its comment gives."""
+    import ctypes
+    import torch
+    L = pkg.lib()
+    pkg.check(L.mtrt_hip_init())
+    M, K = a.shape
+    N = w.shape[1]
+    ad, wd = torch.from_numpy(a).cuda(), torch.from_numpy(w).cuda()
+    wf = pkg.gemm_w8a8_prepack_fragments(wd)
+    asd, wsd = torch.from_numpy(a_s).cuda(), torch.from_numpy(w_s).cuda()
+    y = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+    name = b"mtrt_gemm_w8a8_frag_t256x384"
+    fn = L.mtrt_cuda_module_get_function(L.mtrt_hip_builtin_module(), name, len(name))
+    assert fn
+    vals = [ctypes.c_void_p(ad.data_ptr()), ctypes.c_void_p(wf.data_ptr()), ctypes.c_void_p(asd.data_ptr()), ctypes.c_void_p(wsd.data_ptr()),
+            ctypes.c_void_p(y.data_ptr()), ctypes.c_int64(M), ctypes.c_int64(K), ctypes.c_int64(N)]
+    args = (ctypes.c_void_p * len(vals))(*[ctypes.cast(ctypes.pointer(v), ctypes.c_void_p) for v in vals])
+    tiles = ((M + 255) // 256) * ((N + 383) // 384)
+    L.mtrt_cuda_launch_kernel(fn, 8 * ((tiles + 7) // 8), 1, 1, 256, 1, 1, 0, torch.cuda.current_stream().cuda_stream, args)
+    torch.cuda.synchronize()
+    return y
+
+
+@pytest.mark.parametrize("shape", [(256, 128, 384), (1, 128, 1), (300, 256, 200), (257, 384, 385), (512, 1024, 1160), (700, 256, 8200),
+                                   (130, 512, 4001), (2048, 128, 11008)])
+def test_w8a8_wide_tile_kernel(pkg, orc, shape):
+    """The 256 x 384 tile kernel on its own: one slice (K = 128: nothing but the first loads and the surplus ones), three
+    slices, many; one tile and several rounds' worth; M and N that leave the last row and column tiles ragged, N that is
+    not a whole vector (the element-wise stores), panels whose last waves have no column at all.  Integer sums: bit-exact."""
+    M, K, N = shape
+    a, w, a_s, w_s = _w8a8_inputs(rng(M + K + N + 1), M, K, N)
+    print("case: w8a8 wide tile", shape, flush=True)
+    y = _launch_wide_w8a8(pkg, a, w, a_s, w_s)
+    orc.set_threads(16)
+    ref = orc.gemm_w8a8(a, w, a_s, w_s)
+    orc.set_threads(1)
+    assert np.array_equal(bits16(y).reshape(M, N), ref)
+
+
+def test_w8a8_wide_tile_is_taken_where_its_rounds_are_shorter(pkg, orc):
+    """At the shape of BASELINE config 4 (344 tiles of 256 x 256 = one and a half rounds on 256 compute units, 232 of
+    256 x 384 = one) the entry point launches the wide kernel; the result is the oracle's either way."""
+    import torch
+    M, K, N = 2048, 256, 11008
+    a, w, a_s, w_s = _w8a8_inputs(rng(44), M, K, N)
+    y, kernel = _run_w8a8_frag(pkg, a, w, a_s, w_s)
+    if torch.cuda.get_device_properties(0).multi_processor_count == 256:
+        assert kernel == "mtrt_gemm_w8a8_frag_t256x384", kernel
+    assert kernel in _FRAG_TILE
+    orc.set_threads(16)
+    ref = orc.gemm_w8a8(a, w, a_s, w_s)
+    orc.set_threads(1)
+    assert np.array_equal(bits16(y).reshape(M, N), ref)
 
 
 def test_w8a8_argument_checks(pkg):
