@@ -232,7 +232,7 @@ def build_workloads(pkg, torch, which):
                     def zero(i, az5=az5, wz5=wz5, s5=s5, y5=y5, M=M):
                         a = (az5.data_ptr(), None, wz5.data_ptr(), s5[i].data_ptr(), y5[i].data_ptr(), M, K, N, B)
                         return lambda: pkg.check(L.mtrt_hip_gemm_w4a16(stream(), *a))
-                out.append(dict(name=kname, config="C5 M=%d" % M, bound="mfma", work=2.0 * M * K * N, peak=F16_PEAK,
+                out.append(dict(name=kname, dispatched=True, config="C5 M=%d" % M, bound="mfma", work=2.0 * M * K * N, peak=F16_PEAK,
                                 unit="TFLOP/s", nslots=ns, make=gemm4, keep=(a5, w5, s5, y5),
                                 probe=("mtrt_mfma_probe_f16", a5[0], 32768.0) if M == 4096 else None, zero_operands=zero))
 

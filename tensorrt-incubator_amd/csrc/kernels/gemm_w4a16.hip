@@ -97,6 +97,17 @@ struct F16Traits {
     ua.i = a; ub.i = b;
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(ua.h, ub.h, c, 0, 0, 0);
   }
+  // The same with the accumulator held in ordinary vector registers.  With one wave per SIMD the compiler gives the
+  // matrix instructions accumulation registers only (256 per lane); a tile with more than 256 accumulators keeps the
+  // rest in the other half of the register file through these.  The compiler does not see inside: whoever reads such
+  // an accumulator with another instruction waits for the matrix core first (settle_vgpr).
+  static __device__ __forceinline__ void mfma_vgpr(gemm_core::v4i a, gemm_core::v4i b, Acc& c) {
+    __asm__ volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void clear_vgpr(gemm_core::v4i a, gemm_core::v4i b, Acc& c) {
+    __asm__ volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=v"(c) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void settle_vgpr() { __asm__ volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
 };
 
 struct PlainEpilogue {
@@ -183,9 +194,12 @@ struct WeightRegs {
 // stages in LDS, at least DEPTH + 1.  A tile with little work per slice needs the deeper ring: its loads
 // must be issued a memory latency (about 2000 cycles under load) ahead, however few MFMA cycles a slice is.
 // IT: 32-row tiles per wave (4: 128 rows; 8: 256 rows, one wave per SIMD owning a whole column of the tile).
-template <int MW, int NWN, int JT, int KW, int DEPTH = 2, int STAGES = 4, int IT = 4>
+// HS: 1 = the activation fragments of a whole k-step are read one k-step ahead (two sets of IT fragments);
+// 2 = half a k-step ahead (two sets of IT / 2: the registers that a tile with more accumulators cannot spare).
+template <int MW, int NWN, int JT, int KW, int DEPTH = 2, int STAGES = 4, int IT = 4, int HS = 1>
 struct Shape {
-  static constexpr int kMW = MW, kNWN = NWN, kJT = JT, kKW = KW, kDepth = DEPTH, kStages = STAGES, kIT = IT;
+  static constexpr int kMW = MW, kNWN = NWN, kJT = JT, kKW = KW, kDepth = DEPTH, kStages = STAGES, kIT = IT, kHS = HS;
+  static_assert(HS == 1 || (HS == 2 && IT % 2 == 0), "fragments are read a whole or half a k-step ahead");
   static_assert(STAGES >= DEPTH + 1, "the stage being filled must not be one that is read");
   static constexpr int kSlots = MW * NWN, kWaves = KW * kSlots;
   static constexpr int kBM = 32 * IT * MW, kBN = 32 * JT * NWN;
@@ -223,6 +237,9 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
   const int frow = lane & 31, fhalf = lane >> 5;
 
   v16f acc[IT][JT];
+  // column tiles whose accumulators the compiler places (accumulation registers); those of the others are pinned to
+  // ordinary vector registers (F16Traits::mfma_vgpr)
+  constexpr int JA = IT * JT * 16 > 256 ? 256 / (IT * 16) : JT;
 
   const uint32_t nslices = uint32_t(slices), last = nslices - 1;
   DmaLoaderT<G> al;
@@ -241,10 +258,11 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
     frem &= wrap - 1u;
     fsrow += wrap * scale_row_bytes;
   };
-  struct FragSet {
-    v4i a[IT];
-    u4 b[JT];
-  } f0, f1;
+  // Activation fragments: set P holds row tiles [0, IT) of the k-steps of parity P (HS == 1) or row tiles
+  // [P * IT / 2, (P + 1) * IT / 2) of every k-step (HS == 2).  Weight fragments: set P for the k-steps of parity P.
+  constexpr int HS = S::kHS, AN = IT / HS;
+  v4i fa[2][AN];
+  u4 fb[2][JT];
   // Fragment reads are issued as opaque instructions and waited for by count.  Left to the compiler every
   // k-step got one s_waitcnt lgkmcnt(0) placed right behind a read that had just been issued (its bookkeeping
   // of the in-order LDS counter gives up across the loop edge), so each k-step exposed one LDS round trip with
@@ -255,12 +273,13 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
   uint32_t a_lane[4];
 #pragma unroll
   for (int p = 0; p < 4; ++p) a_lane[p] = lds_base + uint32_t(lds_off(wm * (32 * IT) + frow, 2 * p + fhalf));
-  auto read_a = [&](FragSet& f, uint32_t addr, auto tile) {
+  auto read_a = [&](v4i& dst, uint32_t addr, auto tile) {
     constexpr int I = decltype(tile)::value;
-    __asm__ volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(f.a[I]) : "v"(addr), "n"(I * 4096) : "memory");
+    __asm__ volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(I * 4096) : "memory");
   };
-  auto landed_a = [&](FragSet& f, int i) {
-    __asm__ volatile("s_waitcnt lgkmcnt(%1)" : "+v"(f.a[i]) : "n"(IT - 1) : "memory");
+  // the reads form one stream, AN chunks ahead of their use: AN - 1 younger ones may be outstanding
+  auto landed_a = [&](v4i& frag) {
+    __asm__ volatile("s_waitcnt lgkmcnt(%1)" : "+v"(frag) : "n"(AN - 1) : "memory");
   };
   auto stage_off = [&](uint32_t slice) { return uint32_t(slice % uint32_t(NS)) * uint32_t(S::kStageBytes); };
   auto stage = [&](uint32_t slice) { return lds + stage_off(slice); };
@@ -285,7 +304,8 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
 #pragma unroll
       for (int j = 0; j < JT; ++j) {
         __asm__ volatile("" : "+v"(none));             // one MFMA per accumulator, not one result copied around
-        acc[i][j] = F16Traits::mfma(none, none, F16Traits::zero());
+        if (j < JA) acc[i][j] = F16Traits::mfma(none, none, F16Traits::zero());
+        else F16Traits::clear_vgpr(none, none, acc[i][j]);
       }
     __builtin_amdgcn_sched_barrier(0);
   }
@@ -294,11 +314,11 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
   // itself), the direct-to-LDS loads stay where they are written, and slice 0's are the oldest of all.
   __builtin_amdgcn_s_waitcnt(0x0070 | (((D - 1) * G) & 15) | ((((D - 1) * G) >> 4) << 14));
   __asm__ volatile("s_barrier" ::: "memory");
-  static_for<0, IT>([&](auto i) { read_a(f0, a_lane[KH] + stage_off(0), i); });
+  static_for<0, AN>([&](auto i) { read_a(fa[0][decltype(i)::value], a_lane[KH] + stage_off(0), i); });
 #pragma unroll
   for (int j = 0; j < JT; ++j) {
-    wr.template half<0, KH>(j, 0, f0.b[j]);
-    wr.template half<0, KH>(j, 1, f0.b[j]);
+    wr.template half<0, KH>(j, 0, fb[0][j]);
+    wr.template half<0, KH>(j, 1, fb[0][j]);
   }
 
   // Step T (of NK) of a slice of parity PAR: MFMAs on `cur`, everything for this wave's next
@@ -306,21 +326,31 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
   // fragment read, its share of the 2 * JT halves of the next weights' dequantisation and, in
   // step 0, G/4 direct-to-LDS loads.  Raw nibbles and scales of slice s+2 are fetched in the
   // last step into the register set that the step before finished with.
-  auto kstep = [&](auto par, auto step, FragSet& cur, FragSet& nxt, uint32_t ra, const int8_t* src, int8_t* nd) {
+  // ca: LDS offset of the stage this k-step reads (HS == 2 only: its second half of row tiles is read during its first);
+  // ra: of the stage the next k-step reads.
+  auto kstep = [&](auto par, auto step, uint32_t ca, uint32_t ra, const int8_t* src, int8_t* nd) {
     constexpr int PAR = decltype(par)::value, T = decltype(step)::value;
     constexpr bool kLast = T == NK - 1;
     constexpr int NSET = kLast ? (PAR + 1) % D : PAR;  // register set and dword the next k-step's weights come from
     constexpr int NP = kLast ? KH : KH + (T + 1) * KW;
+    constexpr int CUR = T % 2, NXT = 1 - CUR;          // weight fragment sets (and activation sets with HS == 1)
     const uint32_t raddr = a_lane[NP] + ra;
+    const uint32_t caddr = a_lane[KH + T * KW] + ca;
     static_for<0, IT>([&](auto cc) {
       constexpr int c = decltype(cc)::value;
-      landed_a(cur, c);
+      constexpr int ASET = HS == 1 ? CUR : c / AN, AI = c % AN;
+      landed_a(fa[ASET][AI]);
 #pragma unroll
-      for (int j = 0; j < JT; ++j) acc[c][j] = F16Traits::mfma(__builtin_bit_cast(v4i, cur.b[j]), cur.a[c], acc[c][j]);
-      read_a(nxt, raddr, cc);
+      for (int j = 0; j < JT; ++j) {
+        if (j < JA) acc[c][j] = F16Traits::mfma(__builtin_bit_cast(v4i, fb[CUR][j]), fa[ASET][AI], acc[c][j]);
+        else F16Traits::mfma_vgpr(__builtin_bit_cast(v4i, fb[CUR][j]), fa[ASET][AI], acc[c][j]);
+      }
+      if constexpr (HS == 1) read_a(fa[NXT][c], raddr, cc);
+      else if constexpr (c < AN) read_a(fa[1][c], caddr, IntC<c + AN>{});          // row tile c + AN of this k-step
+      else read_a(fa[0][c - AN], raddr, IntC<c - AN>{});                           // row tile c - AN of the next
 #pragma unroll
       for (int u = 0; u < 2 * JT; ++u)
-        if ((u * IT) / (2 * JT) == c) wr.template half<NSET, NP>(u >> 1, u & 1, nxt.b[u >> 1]);
+        if ((u * IT) / (2 * JT) == c) wr.template half<NSET, NP>(u >> 1, u & 1, fb[NXT][u >> 1]);
       if (T == 0) {
         if constexpr (G >= IT) {
 #pragma unroll
@@ -338,11 +368,11 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
     const int8_t* src = al.slice_base(fslice);         // the slice fetched during this one: s + D, or the last
     int8_t* nd = stage(s + D);
     if (NK == 4) {
-      kstep(par, IntC<0>{}, f0, f1, pa, src, nd);
-      kstep(par, IntC<1>{}, f1, f0, pa, src, nd);
-      kstep(par, IntC<NK == 4 ? 2 : 0>{}, f0, f1, pa, src, nd);
+      kstep(par, IntC<0>{}, pa, pa, src, nd);
+      kstep(par, IntC<1>{}, pa, pa, src, nd);
+      kstep(par, IntC<NK == 4 ? 2 : 0>{}, pa, pa, src, nd);
     } else {
-      kstep(par, IntC<0>{}, f0, f1, pa, src, nd);
+      kstep(par, IntC<0>{}, pa, pa, src, nd);
     }
     // slice s+1 and the registers of slice s+1 have landed; only younger loads may still fly
     // With a ring of at least D + 2 stages the fragment reads in flight belong to a stage that is not written before the
@@ -351,7 +381,7 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
     constexpr int kLgkm = NS >= D + 2 ? 0x0F00 : 0x0000;
     __builtin_amdgcn_s_waitcnt(0x0070 | kLgkm | (kFly & 15) | ((kFly >> 4) << 14));   // vmcnt(kFly) [lgkmcnt(0)]
     __asm__ volatile("s_barrier" ::: "memory");
-    kstep(par, IntC<NK - 1>{}, f1, f0, stage_off(s + 1), src, nd);
+    kstep(par, IntC<NK - 1>{}, pa, stage_off(s + 1), src, nd);
     advance();
   };
 
@@ -364,8 +394,9 @@ __device__ __forceinline__ void run_weight_regs(const int8_t* __restrict__ a, in
   __builtin_amdgcn_s_waitcnt(0x0070);                  // the surplus loads of the last slices have landed
   // ... and so have the surplus fragment reads: their registers stay allocated up to here
 #pragma unroll
-  for (int i = 0; i < IT; ++i) __asm__ volatile("s_waitcnt lgkmcnt(0)" ::"v"(f0.a[i]), "v"(f1.a[i]) : "memory");
+  for (int i = 0; i < AN; ++i) __asm__ volatile("s_waitcnt lgkmcnt(0)" ::"v"(fa[0][i]), "v"(fa[1][i]) : "memory");
 
+  if (JA < JT) F16Traits::settle_vgpr();
   if (KW == 2) {                                       // second set hands its sums to the first through LDS
     __syncthreads();
     float* sum = reinterpret_cast<float*>(lds) + slot * ((32 * IT) * 32 * JT);
@@ -429,6 +460,20 @@ extern "C" __global__ void __launch_bounds__(256, 1) mtrt_gemm_w4a16_t256x256(
     uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t block) {
   __shared__ __attribute__((aligned(16))) int8_t lds[BigShape::kLds];
   weight_regs_kernel<BigShape>(a, wp, scale, y, M, K, N, block, lds);
+}
+// 256 x 384 tiles: four waves of 256 x 96, 384 accumulator registers per lane, a third of them in ordinary vector
+// registers (F16Traits::mfma_vgpr), activation fragments read half a k-step ahead.  A workgroup moves 44 KiB per
+// slice for 384 MFMAs where the 256 x 256 tile moves 40 KiB for 256, and reads each activation fragment from LDS for
+// three MFMAs instead of two.  Same argument list, grid = 8 * ceil(ceil(N/384) * ceil(M/256) / 8), block = 256.
+// Against mtrt_gemm_w4a16_t256x256 in one process (K = 4096, N = 11008, the benchmark's data / zeros): M = 4096
+// 298.4 -> 286.8 / 214.7 -> 207.1 us, M = 2048 (one round instead of two) 181 -> 145 / 141 -> 104, M = 8192 600 -> 571 /
+// 430 -> 411; same bits.
+using WideShape = Shape<1, 4, 3, 1, 2, 4, 8, 2>;       // 256 x 384, 4 waves
+extern "C" __global__ void __launch_bounds__(256, 1) mtrt_gemm_w4a16_t256x384(
+    const uint16_t* __restrict__ a, const uint32_t* __restrict__ wp, const uint16_t* __restrict__ scale,
+    uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t block) {
+  __shared__ __attribute__((aligned(16))) int8_t lds[WideShape::kLds];
+  weight_regs_kernel<WideShape>(a, wp, scale, y, M, K, N, block, lds);
 }
 // Medium M: 128 x 64 tiles so that the grid still fills the chip, two wave sets splitting each slice.
 // Same argument list.  grid = 8 * ceil(ceil(N/64) * ceil(M/128) / 8), block = 256.

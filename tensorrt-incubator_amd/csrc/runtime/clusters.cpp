@@ -54,10 +54,15 @@ constexpr double kRows128FixedUs = 3.0, kRows128UsPerRowByte = 0.0037, kFragRows
 // (8192, 8192), (5120, 13824), (4096, 14336), (8192, 28672), (4096, 2048), 16 to 256 tiles in the last round; where
 // the rule changed the choice: K = N = 4096, M = 2048 83.6 -> 77.1 us; N = 11008, M = 1536 193.2 -> 175.0 us.
 constexpr double kW4BigRoundPerSmallRound = 3.25, kW4PartialRoundBase = 0.56, kW4PartialRoundSlope = 0.44;
+// ... and a round of 256 x 384 tiles takes 1.5 x 0.95 of a round of 256 x 256 tiles (K = 4096, N = 11008, the benchmark's
+// data, old and new in one process: M = 4096, 3 rounds against 2, 298.4 -> 286.8 us; M = 8192 600 -> 571; M = 2048, two
+// rounds against one, 181 -> 145).
+constexpr double kW4WideRoundPerBigRound = 1.5 * 0.95;
 // W8A8 on fragment-order weights: a round of 256 x 384 tiles, in rounds of 256 x 256 tiles.  One and a half times the
-// MFMAs at 0.93 of the time per MFMA (M = 2048, K = 4096, N = 11008: 232 wide tiles in one round 77.9 us, 344 tiles
-// in one and a half rounds 83.5 us, interleaved in one process on the benchmark's data).
-constexpr double kW8WideRoundPerRound = 1.5 * 0.93;
+// MFMAs at 0.9 of the time per MFMA (K = 4096, N = 11008, the benchmark's data, both kernels in one process: M = 2048,
+// one round against one and a half, 77.9 against 83.5 us; M = 4096, two against three, 158 / 165; M = 8192, four
+// against five and a half, 321 / 338; M = 3072, two against two and a half, 137 / 135).
+constexpr double kW8WideRoundPerRound = 1.5 * 0.9;
 } // namespace tuning
 
 const char *float_name(int32_t dt) {
@@ -1156,7 +1161,7 @@ int32_t mtrt_hip_gemm_w4a16(mtrt_stream_t stream, const void *a, const void *w_k
       const uint32_t grid = uint32_t(M > 8 && tiles > cus && tiles <= 2 * cus ? cus : tiles);
       return launch(st, KernelName(M <= 16 ? "mtrt_gemm_w4a16_skinny16" : "mtrt_gemm_w4a16_skinny"), grid, kBlock, as_hip(stream), args);
     }
-    // 256 x 256 tiles (four waves) or 128 x 128 tiles (eight waves), one workgroup per compute unit at a time.  A
+    // 256 x 384 or 256 x 256 tiles (four waves) or 128 x 128 tiles (eight waves), one workgroup per compute unit at a time.  A
     // launch runs in rounds of one tile per unit; a full round of the large tile takes 3.25 times a full round of
     // the small one for four times the work, and a partly filled last round is shorter than a full one (fewer
     // units share the power budget): 0.56 + 0.44 f^2 of it at fill f (measured over M = 48 ... 4096 at (K, N) =
@@ -1174,7 +1179,12 @@ int32_t mtrt_hip_gemm_w4a16(mtrt_stream_t stream, const void *a, const void *w_k
       // (grids: the tiles dealt evenly to the eight XCDs, gemm_core::tile_of_even)
       const int64_t big = 8 * ((big_tiles + 7) / 8), wide = 8 * ((wide_tiles + 7) / 8);
       const int64_t narrow = 8 * ((((N + 63) / 64) * wide_m + 7) / 8);
-      if (tuning::kW4BigRoundPerSmallRound * rounds(big_tiles) < rounds(wide_tiles) && big <= int64_t(kMaxGrid) * 1024)
+      const int64_t huge_tiles = ((N + 383) / 384) * tiles_m, huge = 8 * ((huge_tiles + 7) / 8);
+      const double big_cost = tuning::kW4BigRoundPerSmallRound * rounds(big_tiles);
+      const double huge_cost = tuning::kW4BigRoundPerSmallRound * tuning::kW4WideRoundPerBigRound * rounds(huge_tiles);
+      if (huge_cost < big_cost && huge_cost < rounds(wide_tiles) && huge <= int64_t(kMaxGrid) * 1024)
+        return launch(st, KernelName("mtrt_gemm_w4a16_t256x384"), uint32_t(huge), 256, as_hip(stream), args);
+      if (big_cost < rounds(wide_tiles) && big <= int64_t(kMaxGrid) * 1024)
         return launch(st, KernelName("mtrt_gemm_w4a16_t256x256"), uint32_t(big), 256, as_hip(stream), args);
       if (N <= 64 && narrow <= int64_t(kMaxGrid) * 1024)
         return launch(st, KernelName("mtrt_gemm_w4a16_t128x64"), uint32_t(narrow), kBlock, as_hip(stream), args);

@@ -380,9 +380,10 @@ def test_w4a16_dequantised_weights_are_bit_exact(pkg, orc):
         assert np.array_equal(bits16(y).reshape(-1, N), wd[rows]), kernel
 
 
-@pytest.mark.parametrize("case", [(2048, 8192, "mtrt_gemm_w4a16_t256x256"), (512, 1024, "mtrt_gemm_w4a16_t128x128")])
+@pytest.mark.parametrize("case", [(2048, 8192, "mtrt_gemm_w4a16_t256x256"), (512, 1024, "mtrt_gemm_w4a16_t128x128"),
+                                  (2048, 11008, "mtrt_gemm_w4a16_t256x384")])
 def test_w4a16_tile_kernels_dequantise_bit_exactly(pkg, orc, case):
-    """Identity activations (M = K) through the 256 x 256 and the 128 x 128 tile kernels: every output is one product
+    """Identity activations (M = K) through the 256 x 384, the 256 x 256 and the 128 x 128 tile kernels: every output is one product
     1 x wd plus zeros, so y must equal the dequantised weights bit for bit whatever the order of the sums: pins the
     fragment order of the re-laid weights, the nibble decoding, the scale row of every K block and the single f16
     rounding in the kernels that carry the benchmark."""
@@ -395,8 +396,50 @@ def test_w4a16_tile_kernels_dequantise_bit_exactly(pkg, orc, case):
     np.fill_diagonal(eye, 1.0)
     wd = (w.astype(np.float16) * np.repeat(s.view(np.float16), B, axis=0)).view(np.uint16)
     y, kernel = _run_w4a16(pkg, orc.narrow(eye, orc.F16), orc.pack_int4(w), s, K, N, B)
-    assert kernel == want
+    import torch
+    if torch.cuda.get_device_properties(0).multi_processor_count == 256:    # (the tile is chosen by rounds of the compute units)
+        assert kernel == want
     assert np.array_equal(bits16(y).reshape(K, N), wd)
+
+
+def _launch_wide_w4a16(pkg, a, wp_host, s, K, N, B):
+    """mtrt_gemm_w4a16_t256x384 launched by hand from the built-in module (the entry point takes it only where its
+    rounds come out shorter), with the grid its comment gives."""
+    import ctypes
+    import torch
+    L = pkg.lib()
+    pkg.check(L.mtrt_hip_init())
+    M = a.shape[0]
+    ad = torch.from_numpy(a.view(np.int16)).view(torch.float16).cuda()
+    sd = torch.from_numpy(s.view(np.int16)).view(torch.float16).cuda()
+    pre = pkg.gemm_w4a16_prepack(torch.from_numpy(wp_host).cuda(), K, N)
+    y = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+    name = b"mtrt_gemm_w4a16_t256x384"
+    fn = L.mtrt_cuda_module_get_function(L.mtrt_hip_builtin_module(), name, len(name))
+    assert fn
+    vals = [ctypes.c_void_p(ad.data_ptr()), ctypes.c_void_p(pre.data_ptr()), ctypes.c_void_p(sd.data_ptr()), ctypes.c_void_p(y.data_ptr()),
+            ctypes.c_int64(M), ctypes.c_int64(K), ctypes.c_int64(N), ctypes.c_int64(B)]
+    args = (ctypes.c_void_p * len(vals))(*[ctypes.cast(ctypes.pointer(v), ctypes.c_void_p) for v in vals])
+    tiles = ((M + 255) // 256) * ((N + 383) // 384)
+    L.mtrt_cuda_launch_kernel(fn, 8 * ((tiles + 7) // 8), 1, 1, 256, 1, 1, 0, torch.cuda.current_stream().cuda_stream, args)
+    torch.cuda.synchronize()
+    return y
+
+
+@pytest.mark.parametrize("case", [(256, 64, 384, 64), (1, 128, 1, 128), (300, 256, 200, 64), (257, 192, 385, 64), (512, 1024, 1160, 128),
+                                  (700, 256, 8200, 256), (130, 512, 4001, 128)])
+def test_w4a16_wide_tile_kernel(pkg, orc, case):
+    """The 256 x 384 tile kernel on its own: one slice (K = 64), three, many; blocks of one slice and of several; one tile
+    and several rounds' worth; ragged last row and column tiles, N that is not a whole vector, panels whose last waves
+    have no column at all.  Against the oracle and float64 within the bound of the tile kernels."""
+    M, K, N, B = case
+    a, w, wp, s = _w4a16_inputs(orc, rng(M * K + N + 1), M, K, N, B)
+    print("case: w4a16 wide tile", case, flush=True)
+    y = _launch_wide_w4a16(pkg, a, wp, s, K, N, B)
+    orc.set_threads(16)
+    ref = orc.gemm_w4a16(a, wp, s, K, N, B)
+    orc.set_threads(1)
+    _check_w4a16(orc, y, a, w, s, K, N, B, ref)
 
 
 @pytest.mark.parametrize("case", [(5, 48, 7, 16), (9, 100, 33, 20), (3, 128, 6, 128), (130, 256, 200, 32), (70, 192, 131, 16),
@@ -445,7 +488,8 @@ def test_c5_w4a16_full_size(pkg, orc, M):
     K, N, B = 4096, 11008, 128
     a, w, wp, s = _w4a16_inputs(orc, rng(5), M, K, N, B)
     y, kernel = _run_w4a16(pkg, a, wp, s, K, N, B)
-    assert kernel == {16: "mtrt_gemm_w4a16_strips16", 256: "mtrt_gemm_w4a16_t128x128", 4096: "mtrt_gemm_w4a16_t256x256"}[M]
+    assert kernel in {16: ("mtrt_gemm_w4a16_strips16",), 256: ("mtrt_gemm_w4a16_t128x128",),
+                      4096: ("mtrt_gemm_w4a16_t256x384", "mtrt_gemm_w4a16_t256x256")}[M]
     rows = sorted(set([0, M - 1] + list(range(0, M, max(1, M // 38)))))[:40]
     orc.set_threads(16)
     import torch
@@ -525,13 +569,18 @@ def test_w4a16_narrow_mid_tile_kernel(pkg, orc):
     _check_w4a16(orc, y[rows].contiguous(), a[rows], w, s, K, N, B, ref)
 
 
-def test_w4a16_big_tile_kernel_ragged_edges(pkg, orc):
-    """The 256 x 256-tile kernel on a shape whose M and N are not multiples of the tile
-    (M = 2000, N = 16416 = 513 column tiles of 32), K = 256 so the oracle stays cheap."""
-    M, K, N, B = 2000, 256, 16416, 128
+@pytest.mark.parametrize("N,want", [(8000, "mtrt_gemm_w4a16_t256x256"), (16416, "mtrt_gemm_w4a16_t256x384")])
+def test_w4a16_big_tile_kernel_ragged_edges(pkg, orc, N, want):
+    """The 256-row tile kernels on shapes whose M and N are not multiples of the tile (M = 2000; N = 8000 = 250 column
+    tiles of 32: one full round of 256 x 256 tiles on 256 compute units; N = 16416 = 513 column tiles: 256 x 384 tiles
+    save a round), K = 256 so the oracle stays cheap."""
+    import torch
+    M, K, B = 2000, 256, 128
     a, w, wp, s = _w4a16_inputs(orc, rng(77), M, K, N, B)
     y, kernel = _run_w4a16(pkg, a, wp, s, K, N, B)
-    assert kernel == "mtrt_gemm_w4a16_t256x256"
+    if torch.cuda.get_device_properties(0).multi_processor_count == 256:
+        assert kernel == want
+    assert kernel in ("mtrt_gemm_w4a16_t256x256", "mtrt_gemm_w4a16_t256x384")
     rows = sorted(set([0, 1, 127, 128, 255, 256, 1023, 1791, 1792, 1998, 1999] + list(range(5, M, 97))))
     orc.set_threads(16)
     ref = np.concatenate([orc.gemm_w4a16(a, wp, s, K, N, B, m0=r, mcount=1) for r in rows])
@@ -540,16 +589,19 @@ def test_w4a16_big_tile_kernel_ragged_edges(pkg, orc):
 
 
 @pytest.mark.parametrize("shape,kernel", [((1536, 4096), "t128x128"), ((600, 8480), "t128x128"), ((2048, 4096), "t128x128"),
-                                          ((768, 11008), "t256x256"), ((1536, 11008), "t128x128"), ((3072, 4096), "t256x256")])
+                                          ((768, 11008), "t256x256"), ((1536, 11008), "t256x384"), ((3072, 4096), "t256x256")])
 def test_w4a16_tile_choice_and_results_at_mid_m(pkg, orc, shape, kernel):
     """The tile is chosen by the estimated number of rounds of one tile per compute unit: 128 x 128 tiles where the
-    256 x 256 ones would fill half of the units or spill a few tiles into another round.  Sampled rows against the
-    oracle for each choice."""
+    larger ones would fill half of the units or spill a few tiles into another round, 256 x 384 where they save a
+    round.  Sampled rows against the oracle for each choice (the expected choice is that of 256 compute units)."""
     M, N = shape
     K, B = 256, 128
     a, w, wp, s = _w4a16_inputs(orc, rng(M + N), M, K, N, B)
     y, k = _run_w4a16(pkg, a, wp, s, K, N, B)
-    assert k == "mtrt_gemm_w4a16_" + kernel
+    import torch
+    if torch.cuda.get_device_properties(0).multi_processor_count == 256:
+        assert k == "mtrt_gemm_w4a16_" + kernel
+    assert k in ("mtrt_gemm_w4a16_t128x128", "mtrt_gemm_w4a16_t256x256", "mtrt_gemm_w4a16_t256x384")
     rows = sorted(set([0, 1, 127, 128, 255, 256, M - 2, M - 1] + list(range(7, M, 113))))
     orc.set_threads(16)
     ref = np.concatenate([orc.gemm_w4a16(a, wp, s, K, N, B, m0=r, mcount=1) for r in rows])
