@@ -55,6 +55,19 @@ __device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
   c.h = (_Float16)f;                     // v_cvt_f16_f32: RNE, overflow -> inf, subnormals kept
   return c.u;
 }
+// Two at once into one word (lo in bits 0..15): v_cvt_pk_f16_f32, the same rounding; half the instructions of
+// two single conversions and no merge of the halves.
+__device__ __forceinline__ uint32_t f32x2_to_f16x2_bits(float lo, float hi) {
+  __asm__("" : "+v"(lo), "+v"(hi));      // as above: no merging of the producers into a single rounding
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+  union { f16x2_t h; uint32_t u; } c;
+  c.h = __builtin_convertvector((f32x2_t){lo, hi}, f16x2_t);
+  return c.u;
+}
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2_bits(float lo, float hi) {
+  return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+}
 
 // f8E4M3FN (OCP) pair conversion in hardware: RNE.  Inputs are pre-clamped to
 // [-448, 448] by every caller, so the saturation rule of the instruction is

@@ -160,11 +160,11 @@ __device__ __forceinline__ void write_tile(Acc (&acc)[IT][JT], Epilogue& epi, ui
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const int lcol = jj * 32 + q * 8 + fhalf * 4;  // columns lcol .. lcol+3 of this group <-> r = 4q .. 4q+3
-          uint32_t bits[4];
-          epi.convert4(acc[ib * 4 + i][jt0 + jj], q, jj, bits);
+          uint32_t words[2];                             // four 16-bit outputs, the first in the low half of words[0]
+          epi.convert4(acc[ib * 4 + i][jt0 + jj], q, jj, words);
           u32x2 packed;
-          packed[0] = bits[0] | (bits[1] << 16);
-          packed[1] = bits[2] | (bits[3] << 16);
+          packed[0] = words[0];
+          packed[1] = words[1];
           *reinterpret_cast<u32x2*>(out + lrow * kOutRow + lcol * 2) = packed;
         }
     }
@@ -259,7 +259,7 @@ __device__ __forceinline__ void finish_tile(Acc (&acc)[4][JT], Epilogue& epi, fl
 // tile that fills the last, partial round of a launch.
 // Traits: Acc (16-wide accumulator vector), mfma(first, second, acc), zero().
 // Epilogue: setup(lds scratch, m0, M, n0, N), columns<HC>(first column of the lane in the tile), row(row in tile),
-// convert4(acc, q, column tile of the pass, bits).
+// convert4(acc, q, column tile of the pass, words): outputs 4q .. 4q+3 of the accumulator as two words of two.
 // Y: uint16_t (16-bit outputs through the staged epilogue) or float (direct stores, see write_tile_f32).
 template <class Traits, int JT, class Epilogue, typename Y>
 __device__ __forceinline__ void run(const int8_t* __restrict__ a, const int8_t* __restrict__ b, int64_t row_bytes, Epilogue& epi,

@@ -126,6 +126,9 @@ struct BiasF32Epilogue {
 template <typename X> __device__ __forceinline__ uint32_t narrow16(float v);
 template <> __device__ __forceinline__ uint32_t narrow16<F16>(float v) { return f32_to_f16_bits(v); }
 template <> __device__ __forceinline__ uint32_t narrow16<BF16>(float v) { return f32_to_bf16_bits(v); }
+template <typename X> __device__ __forceinline__ uint32_t narrow16x2(float lo, float hi);
+template <> __device__ __forceinline__ uint32_t narrow16x2<F16>(float lo, float hi) { return f32x2_to_f16x2_bits(lo, hi); }
+template <> __device__ __forceinline__ uint32_t narrow16x2<BF16>(float lo, float hi) { return f32x2_to_bf16x2_bits(lo, hi); }
 
 // y = narrow(acc + f32(bias[n])) (no addition without a bias, as in the kernel above)
 template <typename X>
@@ -147,12 +150,15 @@ struct BiasEpilogue {
 #pragma unroll
       for (int q = 0; q < 4; ++q) br[jj][q] = *reinterpret_cast<const f32x4*>(sb + first_col_in_tile + jj * 32 + q * 8);
   }
-  __device__ __forceinline__ void convert4(const v16f& acc, int q, int jj, uint32_t (&bits)[4]) const {
+  __device__ __forceinline__ void convert4(const v16f& acc, int q, int jj, uint32_t (&words)[2]) const {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      float v = acc[4 * q + e];
-      if (bias) v = v + br[jj][q][e];
-      bits[e] = narrow16<X>(v);
+    for (int e = 0; e < 4; e += 2) {
+      float v0 = acc[4 * q + e], v1 = acc[4 * q + e + 1];
+      if (bias) {
+        v0 = v0 + br[jj][q][e];
+        v1 = v1 + br[jj][q][e + 1];
+      }
+      words[e >> 1] = narrow16x2<X>(v0, v1);
     }
   }
 };

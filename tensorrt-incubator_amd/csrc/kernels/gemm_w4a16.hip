@@ -115,9 +115,9 @@ struct PlainEpilogue {
   __device__ __forceinline__ void row(int) {}
   template <int HC>
   __device__ __forceinline__ void columns(int) {}
-  __device__ __forceinline__ void convert4(const v16f& acc, int q, int, uint32_t (&bits)[4]) const {
+  __device__ __forceinline__ void convert4(const v16f& acc, int q, int, uint32_t (&words)[2]) const {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) bits[e] = f32_to_f16_bits(acc[4 * q + e]);
+    for (int e = 0; e < 4; e += 2) words[e >> 1] = f32x2_to_f16x2_bits(acc[4 * q + e], acc[4 * q + e + 1]);
   }
 };
 

@@ -57,9 +57,10 @@ struct ScaleEpilogueT {
 #pragma unroll
       for (int q = 0; q < 4; ++q) wsr[jj][q] = *reinterpret_cast<const f32x4*>(sw + first_col_in_tile + jj * 32 + q * 8);
   }
-  __device__ __forceinline__ void convert4(const v16i& acc, int q, int jj, uint32_t (&bits)[4]) const {
+  __device__ __forceinline__ void convert4(const v16i& acc, int q, int jj, uint32_t (&words)[2]) const {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) bits[e] = f32_to_f16_bits((float(acc[4 * q + e]) * as) * wsr[jj][q][e]);
+    for (int e = 0; e < 4; e += 2)
+      words[e >> 1] = f32x2_to_f16x2_bits((float(acc[4 * q + e]) * as) * wsr[jj][q][e], (float(acc[4 * q + e + 1]) * as) * wsr[jj][q][e + 1]);
   }
   f32x4 wsr[2][4];
 };

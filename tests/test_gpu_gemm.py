@@ -211,6 +211,24 @@ def test_w8a8_extreme_values_do_not_overflow(pkg, orc):
     assert got[0, 1] == 4096 * 128 * 128 / 2.0 ** 24 and got[0, 0] == -4096 * 128 * 127 / 2.0 ** 24
 
 
+def test_w8a8_tile_epilogue_over_the_whole_f16_range(pkg, orc):
+    """Row scales from 2^-34 to 2^6 put the outputs of the tile kernels' epilogue (two f32 roundings, then a pair of f16
+    conversions in one instruction) everywhere between f16 subnormals, ties at the subnormal boundary and overflow to
+    infinity; the bits are the oracle's."""
+    M, K, N = 320, 128, 416
+    a, w, _, w_s = _w8a8_inputs(rng(61), M, K, N)
+    a_s = (2.0 ** np.linspace(-34, 6, M)).astype(np.float32)
+    for run in (_run_w8a8, _run_w8a8_frag):
+        y, kernel = run(pkg, a, w, a_s, w_s)
+        got = bits16(y).reshape(M, N)
+        ref = orc.gemm_w8a8(a, w, a_s, w_s)
+        assert np.array_equal(got, ref), kernel
+    f = ref.view(np.float16)
+    assert np.isinf(f).any() and ((np.abs(f) < 6.0e-5) & (f != 0)).any()
+    y = _launch_wide_w8a8(pkg, a, w, a_s, w_s)
+    assert np.array_equal(bits16(y).reshape(M, N), ref)
+
+
 def test_c4_w8a8_full_size(pkg, orc):
     """BASELINE config 4: M=2048 K=4096 N=11008, values clip(rint(N(0,40))), seed 4.  The oracle
     evaluates one whole 256-row tile (every lane/accumulator position of the kernel) plus rows
