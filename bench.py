@@ -30,7 +30,8 @@ own operand data (the published dense peaks hold for idle data only: the clock d
 the board's power limit); GEMM entries carry "frac_of_sustained" beside "frac".
 "hbm_sustained" is the matching yardstick for the memory-bound kernels: a stream that is only read, one that is only
 written and a plain copy, over 1 GiB each; HBM entries carry "frac_of_sustained" against the yardstick with their
-access mix ("sustained_mix").
+access mix ("sustained_mix"), and "same_size_yardstick_us": the time of ONE launch of that yardstick moving as many
+bytes as the workload does (the 1 GiB rate is out of reach of any launch of a few tens of MB).
 "library_yardsticks" are the vendor library's plain GEMMs (torch.matmul f16, torch._int_mm) at the same shapes,
 timed the same way; they are not part of the step.
 "cpu_baseline" times the CPU oracle (a C++ restatement of the reference's host
@@ -305,7 +306,7 @@ def mfma_sustained(pkg, torch, kernel, operand, ops_per_mfma):
     return ksteps * 16.0 * units * 4 * ops_per_mfma / us / 1e6
 
 
-def hbm_sustained(pkg, torch, nbytes=1 << 30):
+def hbm_sustained(pkg, torch, sizes=(), reps=200, nbytes=1 << 30):
     """What the memory system sustains on this box for the three access mixes of the memory-bound clusters, each as
     one launch of a yardstick kernel over `nbytes` (one 128-bit access per lane, one-shot grid, buffers far larger than
     the 256 MiB Infinity Cache): {"read": GB/s of a stream that is only read, "write": only written, "copy": bytes
@@ -347,9 +348,32 @@ def hbm_sustained(pkg, torch, nbytes=1 << 30):
         for e in events:
             L.mtrt_cuda_event_release(e)
         out[kind] = round(moved / (0.5 * (us[4] + us[5])) / 1e3, 1)
+    # The same yardsticks at the SIZE of each memory-bound workload (`sizes`: (key, bytes moved, mix)): one launch
+    # moving as many bytes as the workload's algorithmic traffic (a copy: half read, half written), on rotating
+    # windows of the 1 GiB buffers, timed like the workloads (batches of back-to-back launches, median).  A launch of
+    # a few tens of MB is far from the 1 GiB rate for any kernel: the chip takes microseconds to fill and drain.
+    same_size = {}
+    for key, moved, mix in sizes:
+        per_stream = (int(moved) // (1 if mix == "read" else 2)) // 4096 * 4096
+        if per_stream < 4096 or per_stream > nbytes:
+            continue
+        nv = per_stream // 16
+        nslots = max(1, min(48, nbytes // per_stream))
+        name = b"mtrt_read_b128" if mix == "read" else b"mtrt_copy_b128"
+        fn = L.mtrt_cuda_module_get_function(yardstick_module(pkg), name, len(name))
+        calls = []
+        for j in range(nslots):
+            if mix == "read":
+                vals = (ctypes.c_void_p(src.data_ptr() + j * per_stream), ctypes.c_void_p(sink.data_ptr()), ctypes.c_int64(nv), ctypes.c_uint32(0))
+            else:
+                vals = (ctypes.c_void_p(src.data_ptr() + j * per_stream), ctypes.c_void_p(dst.data_ptr() + j * per_stream), ctypes.c_int64(nv))
+            args = (ctypes.c_void_p * len(vals))(*[ctypes.cast(ctypes.pointer(v), ctypes.c_void_p) for v in vals])
+            calls.append(lambda keep=(vals, args), args=args, fn=fn, g=nv // 256: L.mtrt_cuda_launch_kernel(fn, g, 1, 1, 256, 1, 1, 0, s, args))
+        us = time_kernel(pkg, torch, dict(make=lambda i, calls=calls: calls[i], nslots=nslots), reps)
+        same_size[key] = round(us, 2)
     assert int(sink[0]) == 0
     del src, dst
-    return out
+    return out, same_size
 
 
 def kernel_sources_digest():
@@ -714,12 +738,16 @@ def main():
     # what the memory system sustains on this box (pure read, pure write, copy); HBM rows are also given as a fraction
     # of the yardstick with their access mix (amax only reads; every other cluster reads and writes, like the copy;
     # the small-M GEMM reads 60 bytes for every byte it writes)
-    hbm = hbm_sustained(pkg, torch)
-    for w, k in zip(wl, kernels):
+    hbm, same_size = hbm_sustained(pkg, torch, [(i, w["work"], w.get("mix", "copy")) for i, w in enumerate(wl) if w["bound"] == "hbm"],
+                                   args.kernel_reps)
+    for i, (w, k) in enumerate(zip(wl, kernels)):
         if k["bound"] == "hbm":
             mix = w.get("mix", "copy")
             k["frac_of_sustained"] = round(k["achieved"] / hbm[mix], 4)
             k["sustained_mix"] = mix
+            if i in same_size:     # a plain read / copy launch moving the same number of bytes
+                k["same_size_yardstick_us"] = same_size[i]
+                k["frac_of_same_size_yardstick"] = round(same_size[i] / k["us"], 4)
     value = 100.0 * (ideal_us / 1e3) / ms_per_step
     dom = max(kernels, key=lambda k: k["us"])
     traffic = traffic_from_profile(dom["kernel"])
