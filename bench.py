@@ -672,7 +672,7 @@ def main():
     ap.add_argument("--kernel-reps", type=int, default=100, help="launches per kernel for the per-kernel timing")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-cache-variants", action="store_true",
-                    help="skip the warm-cache and 16x-rows launches (they reuse kernel names: keeps a profile's per-kernel averages clean)")
+                    help="skip the warm-cache, 16x-rows and same-size yardstick launches (they reuse kernel names: keeps a profile's per-kernel averages clean)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: every box of this build has one, and the hot path has no "
@@ -738,8 +738,8 @@ def main():
     # what the memory system sustains on this box (pure read, pure write, copy); HBM rows are also given as a fraction
     # of the yardstick with their access mix (amax only reads; every other cluster reads and writes, like the copy;
     # the small-M GEMM reads 60 bytes for every byte it writes)
-    hbm, same_size = hbm_sustained(pkg, torch, [(i, w["work"], w.get("mix", "copy")) for i, w in enumerate(wl) if w["bound"] == "hbm"],
-                                   args.kernel_reps)
+    hbm, same_size = hbm_sustained(pkg, torch, [] if args.no_cache_variants else
+                                   [(i, w["work"], w.get("mix", "copy")) for i, w in enumerate(wl) if w["bound"] == "hbm"], args.kernel_reps)
     for i, (w, k) in enumerate(zip(wl, kernels)):
         if k["bound"] == "hbm":
             mix = w.get("mix", "copy")
