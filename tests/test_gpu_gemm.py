@@ -296,6 +296,23 @@ def test_w8a8_wide_tile_kernel(pkg, orc, shape):
     assert np.array_equal(bits16(y).reshape(M, N), ref)
 
 
+def test_w8a8_wide_tile_kernel_equals_the_entry_point_on_random_shapes(pkg):
+    """Integer sums are exact in any order, so whichever kernel the entry point picks for a shape (wave-private rows
+    kernels, 256 x 256 tiles, half tiles) must give the wide tile kernel's bits: 24 seeded shapes with ragged M, N and
+    one to sixteen slices."""
+    import torch
+    g = rng(2024)
+    for case in range(24):
+        M = int(g.integers(1, 1400))
+        K = 128 * int(g.integers(1, 17))
+        N = int(g.integers(1, 2600))
+        a, w, a_s, w_s = _w8a8_inputs(g, M, K, N)
+        print("case: w8a8 wide vs entry point", (M, K, N), flush=True)
+        y_wide = _launch_wide_w8a8(pkg, a, w, a_s, w_s)
+        y_api, kernel = _run_w8a8_frag(pkg, a, w, a_s, w_s)
+        assert torch.equal(y_wide, y_api), ((M, K, N), kernel)
+
+
 def test_w8a8_wide_tile_is_taken_where_its_rounds_are_shorter(pkg, orc):
     """At the shape of BASELINE config 4 (344 tiles of 256 x 256 = one and a half rounds on 256 compute units, 232 of
     256 x 384 = one) the entry point launches the wide kernel; the result is the oracle's either way."""
@@ -458,6 +475,38 @@ def test_w4a16_wide_tile_kernel(pkg, orc, case):
     ref = orc.gemm_w4a16(a, wp, s, K, N, B)
     orc.set_threads(1)
     _check_w4a16(orc, y, a, w, s, K, N, B, ref)
+
+
+def test_w4a16_wide_tile_kernel_equals_the_256_x_256_tile_on_random_shapes(pkg, orc):
+    """Both 256-row tile kernels add a row's products in the same order (k ascending, one f32 accumulator per output),
+    so their results are the same bits: 16 seeded shapes with ragged M and N, blocks of one to four slices.  (The
+    entry point is steered to the 256 x 256 tile by launching it by hand, like the wide one.)"""
+    import ctypes
+    import torch
+    L = pkg.lib()
+    g = rng(2025)
+    name = b"mtrt_gemm_w4a16_t256x256"
+    fn = L.mtrt_cuda_module_get_function(L.mtrt_hip_builtin_module(), name, len(name))
+    assert fn
+    for case in range(16):
+        M = int(g.integers(1, 1200))
+        B = 64 * int(g.integers(1, 5))
+        K = B * int(g.integers(1, 9))
+        N = int(g.integers(1, 2400))
+        a, w, wp, s = _w4a16_inputs(orc, g, M, K, N, B)
+        print("case: w4a16 wide vs 256 x 256", (M, K, N, B), flush=True)
+        y_wide = _launch_wide_w4a16(pkg, a, wp, s, K, N, B)
+        ad = torch.from_numpy(a.view(np.int16)).view(torch.float16).cuda()
+        sd = torch.from_numpy(s.view(np.int16)).view(torch.float16).cuda()
+        pre = pkg.gemm_w4a16_prepack(torch.from_numpy(wp).cuda(), K, N)
+        y = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+        vals = [ctypes.c_void_p(ad.data_ptr()), ctypes.c_void_p(pre.data_ptr()), ctypes.c_void_p(sd.data_ptr()), ctypes.c_void_p(y.data_ptr()),
+                ctypes.c_int64(M), ctypes.c_int64(K), ctypes.c_int64(N), ctypes.c_int64(B)]
+        args = (ctypes.c_void_p * len(vals))(*[ctypes.cast(ctypes.pointer(v), ctypes.c_void_p) for v in vals])
+        tiles = ((M + 255) // 256) * ((N + 255) // 256)
+        L.mtrt_cuda_launch_kernel(fn, 8 * ((tiles + 7) // 8), 1, 1, 256, 1, 1, 0, torch.cuda.current_stream().cuda_stream, args)
+        torch.cuda.synchronize()
+        assert torch.equal(y_wide.view(torch.int16), y.view(torch.int16)), (M, K, N, B)
 
 
 @pytest.mark.parametrize("case", [(5, 48, 7, 16), (9, 100, 33, 20), (3, 128, 6, 128), (130, 256, 200, 32), (70, 192, 131, 16),
