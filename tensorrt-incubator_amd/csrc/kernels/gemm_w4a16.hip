@@ -497,6 +497,19 @@ extern "C" __global__ void __launch_bounds__(512) mtrt_gemm_w4a16_t128x128(
   weight_regs_kernel<MidWideShape>(a, wp, scale, y, M, K, N, block, lds);
 }
 
+// Medium M, twice as wide: 128 x 256 tiles, the same eight waves with two column tiles each.  An activation fragment
+// read from LDS serves two MFMAs and the activation panel is fetched for half as many workgroups; a slice takes 0.48 us
+// against 0.37 us for twice the MFMAs, so a full round of these tiles costs 1.9 rounds of the 128 x 128 ones: ahead where
+// it saves a round (K = 4096, N = 11008: M = 512 56.9 -> 51.3 us, M = 300 53.8 -> 47.5; K = N = 8192, M = 1024 124.9 -> 115.9),
+// behind where the narrower tile fits one round anyway (M = 256: 43.6 against 27.3 us).
+using MidWide2Shape = Shape<1, 4, 2, 2, 4, 8>;         // 128 x 256, 8 waves (two sets of four), four slices ahead
+extern "C" __global__ void __launch_bounds__(512) mtrt_gemm_w4a16_t128x256(
+    const uint16_t* __restrict__ a, const uint32_t* __restrict__ wp, const uint16_t* __restrict__ scale,
+    uint16_t* __restrict__ y, int64_t M, int64_t K, int64_t N, int64_t block) {
+  __shared__ __attribute__((aligned(16))) int8_t lds[MidWide2Shape::kLds];
+  weight_regs_kernel<MidWide2Shape>(a, wp, scale, y, M, K, N, block, lds);
+}
+
 // Small M (<= 32): one workgroup per 32 columns, four waves split K.
 // G: groups of 8 activation rows kept per stage (M <= 8 * G); WAVES: waves that split K;
 // JT: column tiles of the workgroup (blockIdx.x, blockIdx.x + gridDim.x), sharing the activations.

@@ -58,6 +58,10 @@ constexpr double kW4BigRoundPerSmallRound = 3.25, kW4PartialRoundBase = 0.56, kW
 // data, old and new in one process: M = 4096, 3 rounds against 2, 298.4 -> 286.8 us; M = 8192 600 -> 571; M = 2048, two
 // rounds against one, 181 -> 145).
 constexpr double kW4WideRoundPerBigRound = 1.5 * 0.95;
+// ... and a round of 128 x 256 tiles 1.9 rounds of 128 x 128 tiles (0.48 against 0.37 us per 64-k slice and a longer
+// start and end; at 15 shapes with M = 300 ... 2048, (K, N) = (4096, 11008), (4096, 4096), (11008, 4096), (8192, 8192),
+// (5120, 13824) the estimate takes the fastest of the four tiles at every one).
+constexpr double kW4Mid256RoundPerSmallRound = 1.9;
 // W8A8 on fragment-order weights: a round of 256 x 384 tiles, in rounds of 256 x 256 tiles.  One and a half times the
 // MFMAs at 0.9 of the time per MFMA (K = 4096, N = 11008, the benchmark's data, both kernels in one process: M = 2048,
 // one round against one and a half, 77.9 against 83.5 us; M = 4096, two against three, 158 / 165; M = 8192, four
@@ -1161,7 +1165,7 @@ int32_t mtrt_hip_gemm_w4a16(mtrt_stream_t stream, const void *a, const void *w_k
       const uint32_t grid = uint32_t(M > 8 && tiles > cus && tiles <= 2 * cus ? cus : tiles);
       return launch(st, KernelName(M <= 16 ? "mtrt_gemm_w4a16_skinny16" : "mtrt_gemm_w4a16_skinny"), grid, kBlock, as_hip(stream), args);
     }
-    // 256 x 384 or 256 x 256 tiles (four waves) or 128 x 128 tiles (eight waves), one workgroup per compute unit at a time.  A
+    // 256 x 384 or 256 x 256 tiles (four waves) or 128 x 256 / 128 x 128 tiles (eight waves), one workgroup per compute unit at a time.  A
     // launch runs in rounds of one tile per unit; a full round of the large tile takes 3.25 times a full round of
     // the small one for four times the work, and a partly filled last round is shorter than a full one (fewer
     // units share the power budget): 0.56 + 0.44 f^2 of it at fill f (measured over M = 48 ... 4096 at (K, N) =
@@ -1180,12 +1184,17 @@ int32_t mtrt_hip_gemm_w4a16(mtrt_stream_t stream, const void *a, const void *w_k
       const int64_t big = 8 * ((big_tiles + 7) / 8), wide = 8 * ((wide_tiles + 7) / 8);
       const int64_t narrow = 8 * ((((N + 63) / 64) * wide_m + 7) / 8);
       const int64_t huge_tiles = ((N + 383) / 384) * tiles_m, huge = 8 * ((huge_tiles + 7) / 8);
+      const int64_t mid_tiles = panels * wide_m, mid = 8 * ((mid_tiles + 7) / 8);   // 128 x 256
       const double big_cost = tuning::kW4BigRoundPerSmallRound * rounds(big_tiles);
       const double huge_cost = tuning::kW4BigRoundPerSmallRound * tuning::kW4WideRoundPerBigRound * rounds(huge_tiles);
-      if (huge_cost < big_cost && huge_cost < rounds(wide_tiles) && huge <= int64_t(kMaxGrid) * 1024)
+      const double mid_cost = tuning::kW4Mid256RoundPerSmallRound * rounds(mid_tiles);
+      const double small_cost = std::min(rounds(wide_tiles), mid_cost);
+      if (huge_cost < big_cost && huge_cost < small_cost && huge <= int64_t(kMaxGrid) * 1024)
         return launch(st, KernelName("mtrt_gemm_w4a16_t256x384"), uint32_t(huge), 256, as_hip(stream), args);
-      if (big_cost < rounds(wide_tiles) && big <= int64_t(kMaxGrid) * 1024)
+      if (big_cost < small_cost && big <= int64_t(kMaxGrid) * 1024)
         return launch(st, KernelName("mtrt_gemm_w4a16_t256x256"), uint32_t(big), 256, as_hip(stream), args);
+      if (mid_cost < rounds(wide_tiles) && N > 64 && mid <= int64_t(kMaxGrid) * 1024)
+        return launch(st, KernelName("mtrt_gemm_w4a16_t128x256"), uint32_t(mid), 512, as_hip(stream), args);
       if (N <= 64 && narrow <= int64_t(kMaxGrid) * 1024)
         return launch(st, KernelName("mtrt_gemm_w4a16_t128x64"), uint32_t(narrow), kBlock, as_hip(stream), args);
       if (wide <= int64_t(kMaxGrid) * 1024)

@@ -98,7 +98,7 @@ def test_embedded_code_object_is_gfx950_and_has_the_kernels(pkg):
             names += ["mtrt_q_view_%s_%s" % (x, q), "mtrt_dq_view_%s_%s" % (x, q), "mtrt_q_viewt_%s_%s" % (x, q), "mtrt_dq_viewt_%s_%s" % (x, q)]
     names += ["mtrt_fill", "mtrt_gemm_dense_f32", "mtrt_gemm_dense_f16", "mtrt_gemm_dense_bf16", "mtrt_gemm_dense_mfma_f16", "mtrt_gemm_dense_mfma_bf16", "mtrt_gemm_dense_mfma_f32", "mtrt_gemm_dense_edge_f32", "mtrt_gemm_dense_edge_f16", "mtrt_gemm_dense_edge_bf16", "mtrt_gemm_w8a8_frag", "mtrt_gemm_w8a8_frag_t256x384",
               "mtrt_gemm_w8a8_small16", "mtrt_gemm_w8a8_frag_rows32", "mtrt_gemm_w8a8_nk", "mtrt_gemm_w8a8_nk_rows32", "mtrt_gemm_dense_rows32_f32", "mtrt_gemm_dense_rows32_f16", "mtrt_gemm_dense_rows32_bf16", "mtrt_gemm_w8a8_nk_rows64", "mtrt_gemm_w8a8_frag_rows64", "mtrt_gemm_w8a8_frag_rows128", "mtrt_gemm_w8a8_nk_rows128", "mtrt_gemm_dense_rows128_f32", "mtrt_gemm_dense_rows128_f16", "mtrt_gemm_dense_rows128_bf16", "mtrt_gemm_dense_rows64_f32", "mtrt_gemm_dense_rows64_f16", "mtrt_gemm_dense_rows64_bf16", "mtrt_gemm_w8a8_nk_edge", "mtrt_gemm_w8a8_nk_any", "mtrt_gemm_w4a16_t256x256", "mtrt_gemm_w4a16_t256x384",
-              "mtrt_gemm_w4a16_t128x128", "mtrt_gemm_w4a16_t128x64", "mtrt_gemm_w4a16_skinny", "mtrt_gemm_w4a16_skinny16",
+              "mtrt_gemm_w4a16_t128x128", "mtrt_gemm_w4a16_t128x256", "mtrt_gemm_w4a16_t128x64", "mtrt_gemm_w4a16_skinny", "mtrt_gemm_w4a16_skinny16",
               "mtrt_gemm_w4a16_strips16", "mtrt_gemm_w4a16_edge", "mtrt_gemm_w4a16_any"]
     for n in names:
         assert n.encode() + b"\x00" in blob, "kernel %s is not in the code object" % n

@@ -416,9 +416,9 @@ def test_w4a16_dequantised_weights_are_bit_exact(pkg, orc):
 
 
 @pytest.mark.parametrize("case", [(2048, 8192, "mtrt_gemm_w4a16_t256x256"), (512, 1024, "mtrt_gemm_w4a16_t128x128"),
-                                  (2048, 11008, "mtrt_gemm_w4a16_t256x384")])
+                                  (2048, 11008, "mtrt_gemm_w4a16_t256x384"), (1536, 4096, "mtrt_gemm_w4a16_t128x256")])
 def test_w4a16_tile_kernels_dequantise_bit_exactly(pkg, orc, case):
-    """Identity activations (M = K) through the 256 x 384, the 256 x 256 and the 128 x 128 tile kernels: every output is one product
+    """Identity activations (M = K) through the 256 x 384, 256 x 256, 128 x 256 and 128 x 128 tile kernels: every output is one product
     1 x wd plus zeros, so y must equal the dequantised weights bit for bit whatever the order of the sums: pins the
     fragment order of the re-laid weights, the nibble decoding, the scale row of every K block and the single f16
     rounding in the kernels that carry the benchmark."""
@@ -655,12 +655,12 @@ def test_w4a16_big_tile_kernel_ragged_edges(pkg, orc, N, want):
     _check_w4a16(orc, y[rows].contiguous(), a[rows], w, s, K, N, B, ref)
 
 
-@pytest.mark.parametrize("shape,kernel", [((1536, 4096), "t128x128"), ((600, 8480), "t128x128"), ((2048, 4096), "t128x128"),
+@pytest.mark.parametrize("shape,kernel", [((1536, 4096), "t128x256"), ((600, 8480), "t128x256"), ((2048, 4096), "t128x256"), ((1024, 4096), "t128x128"),
                                           ((768, 11008), "t256x256"), ((1536, 11008), "t256x384"), ((3072, 4096), "t256x256")])
 def test_w4a16_tile_choice_and_results_at_mid_m(pkg, orc, shape, kernel):
     """The tile is chosen by the estimated number of rounds of one tile per compute unit: 128 x 128 tiles where the
-    larger ones would fill half of the units or spill a few tiles into another round, 256 x 384 where they save a
-    round.  Sampled rows against the oracle for each choice (the expected choice is that of 256 compute units)."""
+    larger ones would fill half of the units or spill a few tiles into another round, 128 x 256 and 256 x 384 where
+    they save a round.  Sampled rows against the oracle for each choice (the expected choice is that of 256 compute units)."""
     M, N = shape
     K, B = 256, 128
     a, w, wp, s = _w4a16_inputs(orc, rng(M + N), M, K, N, B)
@@ -668,7 +668,7 @@ def test_w4a16_tile_choice_and_results_at_mid_m(pkg, orc, shape, kernel):
     import torch
     if torch.cuda.get_device_properties(0).multi_processor_count == 256:
         assert k == "mtrt_gemm_w4a16_" + kernel
-    assert k in ("mtrt_gemm_w4a16_t128x128", "mtrt_gemm_w4a16_t256x256", "mtrt_gemm_w4a16_t256x384")
+    assert k in ("mtrt_gemm_w4a16_t128x128", "mtrt_gemm_w4a16_t128x256", "mtrt_gemm_w4a16_t256x256", "mtrt_gemm_w4a16_t256x384")
     rows = sorted(set([0, 1, 127, 128, 255, 256, M - 2, M - 1] + list(range(7, M, 113))))
     orc.set_threads(16)
     ref = np.concatenate([orc.gemm_w4a16(a, wp, s, K, N, B, m0=r, mcount=1) for r in rows])
